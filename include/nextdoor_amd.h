@@ -1,0 +1,135 @@
+/*
+ * C ABI of the MI355X transit-parallel sampling engine (libnextdoor_amd.so).
+ *
+ * Plain pointers and sizes only.  Every function that can fail returns 0 on success and
+ * a negative value on failure; nd_last_error() then describes the failure (per thread).
+ * Nothing here aborts the process.  The library owns every buffer it returns a pointer
+ * to; such pointers stay valid until the owning object is freed or the call that
+ * produced them is repeated.  One caller at a time per sampler (the reference's
+ * single-host-thread contract); all device work of a sampler runs on its private stream.
+ *
+ * Citations (file:line) name the reference interface each entry point stands for;
+ * paths are relative to the plasma-umass/NextDoor tree.
+ */
+#ifndef NEXTDOOR_AMD_H
+#define NEXTDOOR_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nd_graph nd_graph;     /* host CSR: the reference's CSR* (src/csr.hpp:46-196) */
+typedef struct nd_sampler nd_sampler; /* NextDoorData<SampleType, App> + engine state (src/libNextDoor.hpp:13-37) */
+
+const char* nd_last_error(void);
+
+/* Apps compiled into the library (the reference builds one binary per app; here one
+ * library holds all of them and the app is chosen by name, e.g. "DeepWalk", "KHop"). */
+int nd_num_apps(void);
+const char* nd_app_name(int index);
+
+/* ---- graphs ------------------------------------------------------------------------ */
+
+/* loadGraph(graph, file, type, format), src/nextdoor.cu:1845-1891.
+ * type: "edge-list" | "adj-list"; format: "binary" | "text". */
+int nd_graph_load(const char* path, const char* graph_type, const char* graph_format, nd_graph** out);
+/* csr_from_graph, src/csr.hpp:399-424, from in-memory edges (sorted per vertex by
+ * (dst, weight), duplicates kept).  n_vertices <= 0: largest id + 1.  weight may be NULL. */
+int nd_graph_from_edges(int32_t n_vertices, int64_t n_edges, const int32_t* src, const int32_t* dst,
+                        const float* weight, nd_graph** out);
+/* Same from CSR arrays (row_ptr[n_vertices + 1], col[n_edges], weight[n_edges] or NULL). */
+int nd_graph_from_csr(int32_t n_vertices, int64_t n_edges, const int32_t* row_ptr, const int32_t* col,
+                      const float* weight, nd_graph** out);
+/* Seeded synthetic graphs used by the benchmark configurations (no counterpart in the
+ * reference, which downloads its datasets: downloadDataset.sh:1). */
+int nd_graph_rmat(int scale, int edge_factor, double a, double b, double c, uint64_t seed, int symmetrise,
+                  nd_graph** out);
+int nd_graph_chung_lu(int32_t n_vertices, int64_t n_edges, double exponent, uint64_t seed, nd_graph** out);
+int32_t nd_graph_num_vertices(const nd_graph* g);
+int64_t nd_graph_num_edges(const nd_graph* g);
+const int32_t* nd_graph_row_ptr(const nd_graph* g);
+const int32_t* nd_graph_col(const nd_graph* g);
+const float* nd_graph_weight(const nd_graph* g);
+const float* nd_graph_max_weight(const nd_graph* g); /* src/graph.hpp:71-80 */
+void nd_graph_free(nd_graph* g);
+
+/* ---- sampler: the libNextDoor.hpp host API ------------------------------------------ */
+
+int nd_sampler_create(const char* app_name, nd_sampler** out);
+/* transferCSRToGPUs(data, csr), src/nextdoor.cu:1893-1911.  The graph must outlive the sampler. */
+int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g);
+/* allocNextDoorDataOnGPU(csr, data), src/nextdoor.cu:1931-2086.  seed keys the Philox
+ * stream that replaces init_curand_states (src/nextdoor.cu:1838-1843). */
+int nd_sampler_alloc(nd_sampler* s, uint64_t seed);
+/* doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006. */
+int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing);
+/* getFinalSamples(data), src/nextdoor.cu:3211-3237: copies device -> host and returns the
+ * host vector (num_samples * final_sample_size int32, INVALID = n_vertices). */
+int nd_sampler_get_final_samples(nd_sampler* s, const int32_t** data, int64_t* length);
+/* getFinalSampleSize<App>(), src/nextdoor.cu:1913-1929. */
+int nd_sampler_final_sample_size(const nd_sampler* s);
+/* App::numSamples(csr) as fixed by alloc. */
+int64_t nd_sampler_num_samples(const nd_sampler* s);
+/* NextDoorData::initialContents (src/libNextDoor.hpp:18): the roots of every sample. */
+int nd_sampler_initial_contents(const nd_sampler* s, const int32_t** data, int64_t* length);
+/* NextDoorData::INVALID_VERTEX and ::maxBits (src/libNextDoor.hpp:35-36). */
+int32_t nd_sampler_invalid_vertex(const nd_sampler* s);
+int nd_sampler_max_bits(const nd_sampler* s);
+/* App().steps(), App().stepSize(k), App().initialSampleSize(), App().samplingType(). */
+int nd_sampler_steps(const nd_sampler* s);
+int nd_sampler_step_size(const nd_sampler* s, int step);
+int nd_sampler_initial_sample_size(const nd_sampler* s);
+int nd_sampler_sampling_type(const nd_sampler* s);
+/* NextDoorData::dOutputSamples (src/libNextDoor.hpp:23) copied to the host: num_samples
+ * SampleType structs.  nd_sampler_sample_state_bytes is 0 for an empty SampleType. */
+int64_t nd_sampler_sample_state_bytes(const nd_sampler* s);
+int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
+/* The per-phase wall-clock breakdown the reference prints (src/nextdoor.cu:2963-2966),
+ * measured with events on the sampler's stream when profiling is on.
+ * out[0] end to end, [1] inversion, [2] load balancing, [3] flat (identity / sub-wavefront)
+ * kernel, [4] workgroup + grid-wide kernel, all in milliseconds; [5] flat launches,
+ * [6] workgroup launches, [7] sort passes. */
+int nd_sampler_set_profiling(nd_sampler* s, int on);
+int nd_sampler_phase_times(const nd_sampler* s, float out[8]);
+/* freeDeviceData(data), src/nextdoor.cu:2088-2115. */
+void nd_sampler_free_device(nd_sampler* s);
+void nd_sampler_destroy(nd_sampler* s);
+
+/* ---- module-level functions (src/nextDoorPythonModule.cu:40-102) --------------------- */
+/* One process-wide sampler, as the reference's static NextDoorData per module. */
+
+/* initSampling(graph): binary edge-list path (nextDoorPythonModule.cu:40-52).  The
+ * reference compiles one module per app; here the app is named.  seed as above. */
+int nd_init_sampling(const char* app_name, const char* graph_path, uint64_t seed);
+/* sample() (nextDoorPythonModule.cu:54-58); runs the load-balanced transit-parallel engine. */
+int nd_sample(void);
+/* finalSampleLength() (nextDoorPythonModule.cu:75-81): total length of the final-samples vector. */
+int64_t nd_final_sample_length(void);
+/* finalSamplesArray() (nextDoorPythonModule.cu:90-94): borrowed pointer into the host vector. */
+const int32_t* nd_final_samples_array(void);
+/* freeDeviceMemory() (nextDoorPythonModule.cu:83-87). */
+void nd_free_device_memory(void);
+
+/* ---- building blocks, exposed for parity tests ---------------------------------------- */
+/* All take HOST buffers, run the device kernel the engine uses, and copy the result back. */
+
+/* The random-number buffer of one step: out[slot * draws_per_slot + d] = uniform draw d of
+ * output slot (first_slot + slot) at `step` (replaces curand_uniform over per-thread
+ * states, src/rand_num_gen.cuh:117-122). */
+int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, int64_t n_slots,
+                           int draws_per_slot, float* out);
+/* cub::DeviceRadixSort::SortPairs as called at src/nextdoor.cu:2930-2933: stable sort of
+ * (key, value) by the low key_bits bits.  vals == NULL: value = index. */
+int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_bits, int32_t* keys_out,
+                  int32_t* vals_out);
+/* invalidVertexStartPos + DeviceRunLengthEncode::Encode + DeviceScan::ExclusiveSum
+ * (src/nextdoor.cu:1804-1836, 2535-2545, 2560-2567) over a sorted key array. */
+int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
+                       int32_t* offsets, int64_t* n_runs, int64_t* n_valid);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

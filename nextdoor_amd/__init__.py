@@ -1,0 +1,273 @@
+"""Host-side mirror of the NextDoor sampling interface over libnextdoor_amd.so.
+
+The compute path is the HIP library (csrc/, C ABI in include/nextdoor_amd.h).  This
+package only loads it and mirrors, for Python callers, the two surfaces of the reference:
+
+* the libNextDoor host API (src/libNextDoor.hpp:39-50): ``loadGraph`` ->
+  :meth:`Graph.load`, ``transferCSRToGPUs`` + ``allocNextDoorDataOnGPU`` ->
+  :meth:`Sampler.__init__`, ``doTransitParallelSampling`` ->
+  :meth:`Sampler.do_transit_parallel`, ``getFinalSamples`` -> :meth:`Sampler.final_samples`,
+  ``freeDeviceData`` -> :meth:`Sampler.free_device`;
+* the per-app Python module functions (src/nextDoorPythonModule.cu:40-102):
+  ``initSampling / sample / finalSamples / finalSampleLength / freeDeviceMemory /
+  finalSamplesArray`` -> :class:`SamplingModule`.
+
+There is no CPU fallback: without the built library and a GPU every sampling call raises.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _capi
+from ._capi import NextDoorError, check, lib
+
+__all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
+           "sort_pairs", "unique_transits"]
+
+
+def app_names():
+    L = lib()
+    return [L.nd_app_name(i).decode() for i in range(L.nd_num_apps())]
+
+
+def _as(arr, dtype):
+    return np.ascontiguousarray(arr, dtype=dtype)
+
+
+def _ptr(arr, ctype):
+    return arr.ctypes.data_as(C.POINTER(ctype))
+
+
+class Graph:
+    """Host CSR graph (the reference's ``CSR*``)."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    @classmethod
+    def load(cls, path, graph_type="edge-list", graph_format="binary"):
+        h = C.c_void_p()
+        check(lib().nd_graph_load(str(path).encode(), graph_type.encode(), graph_format.encode(), C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_edges(cls, src, dst, weight=None, n_vertices=0):
+        src, dst = _as(src, np.int32), _as(dst, np.int32)
+        w = None if weight is None else _as(weight, np.float32)
+        h = C.c_void_p()
+        check(lib().nd_graph_from_edges(n_vertices, len(src), _ptr(src, C.c_int32), _ptr(dst, C.c_int32),
+                                        None if w is None else _ptr(w, C.c_float), C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_csr(cls, row_ptr, col, weight=None):
+        row_ptr, col = _as(row_ptr, np.int32), _as(col, np.int32)
+        w = None if weight is None else _as(weight, np.float32)
+        h = C.c_void_p()
+        check(lib().nd_graph_from_csr(len(row_ptr) - 1, len(col), _ptr(row_ptr, C.c_int32), _ptr(col, C.c_int32),
+                                      None if w is None else _ptr(w, C.c_float), C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def rmat(cls, scale, edge_factor, a=0.57, b=0.19, c=0.19, seed=42, symmetrise=False):
+        h = C.c_void_p()
+        check(lib().nd_graph_rmat(scale, edge_factor, a, b, c, seed, int(symmetrise), C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def chung_lu(cls, n_vertices, n_edges, exponent, seed=42):
+        h = C.c_void_p()
+        check(lib().nd_graph_chung_lu(n_vertices, n_edges, exponent, seed, C.byref(h)))
+        return cls(h)
+
+    @property
+    def n_vertices(self):
+        return lib().nd_graph_num_vertices(self._h)
+
+    @property
+    def n_edges(self):
+        return lib().nd_graph_num_edges(self._h)
+
+    def _view(self, fn, n, dtype):
+        if n == 0:
+            return np.zeros(0, dtype=dtype)
+        return np.ctypeslib.as_array(fn(self._h), shape=(n,))
+
+    # zero-copy views into the library-owned arrays (valid while the Graph lives)
+    @property
+    def row_ptr(self):
+        return self._view(lib().nd_graph_row_ptr, self.n_vertices + 1, np.int32)
+
+    @property
+    def col(self):
+        return self._view(lib().nd_graph_col, self.n_edges, np.int32)
+
+    @property
+    def weight(self):
+        return self._view(lib().nd_graph_weight, self.n_edges, np.float32)
+
+    @property
+    def max_weight(self):
+        return self._view(lib().nd_graph_max_weight, self.n_vertices, np.float32)
+
+    def close(self):
+        if self._h:
+            lib().nd_graph_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Sampler:
+    """``NextDoorData<SampleType, App>`` plus the engine, for one app and one graph."""
+
+    def __init__(self, app, graph, seed=42):
+        self._h = C.c_void_p()
+        self.graph = graph  # keeps the host CSR alive
+        check(lib().nd_sampler_create(app.encode(), C.byref(self._h)))
+        try:
+            check(lib().nd_sampler_set_graph(self._h, graph._h))
+            check(lib().nd_sampler_alloc(self._h, seed))
+        except Exception:
+            self.close()
+            raise
+
+    # shape algebra of the app
+    @property
+    def num_samples(self):
+        return lib().nd_sampler_num_samples(self._h)
+
+    @property
+    def final_sample_size(self):
+        return lib().nd_sampler_final_sample_size(self._h)
+
+    @property
+    def steps(self):
+        return lib().nd_sampler_steps(self._h)
+
+    def step_size(self, k):
+        return lib().nd_sampler_step_size(self._h, k)
+
+    @property
+    def initial_sample_size(self):
+        return lib().nd_sampler_initial_sample_size(self._h)
+
+    @property
+    def invalid_vertex(self):
+        return lib().nd_sampler_invalid_vertex(self._h)
+
+    @property
+    def max_bits(self):
+        return lib().nd_sampler_max_bits(self._h)
+
+    @property
+    def initial_contents(self):
+        p, n = C.POINTER(C.c_int32)(), C.c_int64()
+        check(lib().nd_sampler_initial_contents(self._h, C.byref(p), C.byref(n)))
+        return np.ctypeslib.as_array(p, shape=(n.value,)).copy()
+
+    def do_transit_parallel(self, load_balancing=True):
+        check(lib().nd_sampler_do_transit_parallel(self._h, int(load_balancing)))
+
+    def final_samples(self):
+        """(num_samples, final_sample_size) int32 array; INVALID entries equal n_vertices."""
+        p, n = C.POINTER(C.c_int32)(), C.c_int64()
+        check(lib().nd_sampler_get_final_samples(self._h, C.byref(p), C.byref(n)))
+        flat = np.ctypeslib.as_array(p, shape=(n.value,)).copy()
+        return flat.reshape(self.num_samples, self.final_sample_size)
+
+    def sample_states(self):
+        nbytes = lib().nd_sampler_sample_state_bytes(self._h)
+        if nbytes <= 0:
+            return None
+        buf = np.empty(nbytes, dtype=np.uint8)
+        check(lib().nd_sampler_get_sample_states(self._h, buf.ctypes.data_as(C.c_void_p), nbytes))
+        return buf
+
+    def set_profiling(self, on):
+        check(lib().nd_sampler_set_profiling(self._h, int(on)))
+
+    def phase_times(self):
+        out = (C.c_float * 8)()
+        check(lib().nd_sampler_phase_times(self._h, out))
+        keys = ["end_to_end_ms", "inversion_ms", "load_balancing_ms", "flat_kernel_ms", "workgroup_kernel_ms",
+                "flat_launches", "workgroup_launches", "sort_passes"]
+        return dict(zip(keys, list(out)))
+
+    def free_device(self):
+        lib().nd_sampler_free_device(self._h)
+
+    def close(self):
+        if self._h:
+            lib().nd_sampler_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class SamplingModule:
+    """The functions of one per-app Python module of the reference
+    (src/nextDoorPythonModule.cu:40-102), e.g. ``SamplingModule("KHop")`` for
+    ``KHopSamplingPy3``.  State is process-wide, as in the reference."""
+
+    def __init__(self, app, seed=42):
+        self.app, self.seed = app, seed
+
+    def initSampling(self, graph_path):
+        check(lib().nd_init_sampling(self.app.encode(), str(graph_path).encode(), self.seed))
+
+    def sample(self):
+        check(lib().nd_sample())
+
+    def finalSampleLength(self):
+        return lib().nd_final_sample_length()
+
+    def finalSamplesArray(self):
+        """numpy view of the library's host vector (no copy), like wrapping the reference's
+        ``int* finalSamplesArray()``."""
+        p = lib().nd_final_samples_array()
+        if not p:
+            raise NextDoorError(lib().nd_last_error().decode())
+        return np.ctypeslib.as_array(p, shape=(lib().nd_final_sample_length(),))
+
+    def finalSamples(self):
+        return self.finalSamplesArray().tolist()
+
+    def freeDeviceMemory(self):
+        lib().nd_free_device_memory()
+
+
+# ---- building blocks (device kernels behind host buffers) ---------------------------------
+
+def philox_fill_uniform(seed, step, first_slot, n_slots, draws_per_slot=1):
+    out = np.empty(n_slots * draws_per_slot, dtype=np.float32)
+    check(lib().nd_philox_fill_uniform(seed, step, first_slot, n_slots, draws_per_slot, _ptr(out, C.c_float)))
+    return out.reshape(n_slots, draws_per_slot)
+
+
+def sort_pairs(keys, vals, key_bits):
+    keys = _as(keys, np.int32)
+    v = None if vals is None else _as(vals, np.int32)
+    ko, vo = np.empty_like(keys), np.empty_like(keys)
+    check(lib().nd_sort_pairs(_ptr(keys, C.c_int32), None if v is None else _ptr(v, C.c_int32), len(keys), key_bits,
+                              _ptr(ko, C.c_int32), _ptr(vo, C.c_int32)))
+    return ko, vo
+
+
+def unique_transits(sorted_keys, invalid):
+    k = _as(sorted_keys, np.int32)
+    n = len(k)
+    uniq, counts, offsets = (np.empty(max(n, 1), dtype=np.int32) for _ in range(3))
+    n_runs, n_valid = C.c_int64(), C.c_int64()
+    check(lib().nd_unique_transits(_ptr(k, C.c_int32), n, invalid, _ptr(uniq, C.c_int32), _ptr(counts, C.c_int32),
+                                   _ptr(offsets, C.c_int32), C.byref(n_runs), C.byref(n_valid)))
+    r = n_runs.value
+    return uniq[:r], counts[:r], offsets[:r], n_valid.value

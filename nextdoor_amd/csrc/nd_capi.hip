@@ -1,0 +1,376 @@
+// C ABI of the sampling engine (declarations and reference citations: include/nextdoor_amd.h).
+#include "../../include/nextdoor_amd.h"
+
+#include <string.h>
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "nd_apps_khop.hpp"
+#include "nd_apps_walks.hpp"
+#include "nd_engine.hpp"
+#include "nd_graph.hpp"
+
+struct nd_graph {
+  CSR csr;
+};
+
+struct nd_sampler {
+  std::unique_ptr<nd::EngineBase> engine;
+  const nd_graph* graph = nullptr;
+};
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(const std::string& msg, int code = -1) {
+  g_error = msg;
+  return code;
+}
+
+struct AppEntry {
+  const char* name;
+  nd::EngineBase* (*make)(const char*);
+};
+
+template <class SampleType, class App>
+nd::EngineBase* make_engine(const char* name) {
+  return new nd::Engine<SampleType, App>(name);
+}
+
+// name -> instantiation.  The first block carries the reference's app names and sizes.
+const AppEntry kApps[] = {
+    {"UniformRandomWalk", make_engine<UniformRandomWalkSample, UniformRandomWalkApp>},
+    {"DeepWalk", make_engine<DummySample, DeepWalkApp>},
+    {"PPR", make_engine<DummySample, PPRApp>},
+    {"Node2Vec", make_engine<Node2VecSample, Node2VecApp>},
+    {"KHop", make_engine<KHopSample, KHopApp>},
+    // one walk per vertex (benchmark configurations) and the weighted second-order walk
+    {"DeepWalkPerVertex", make_engine<DummySample, DeepWalkPerVertexApp>},
+    {"PPRPerVertex", make_engine<DummySample, PPRPerVertexApp>},
+    {"Node2VecPerVertex", make_engine<Node2VecSample, Node2VecPerVertexApp>},
+    {"WeightedNode2Vec", make_engine<Node2VecSample, WeightedNode2VecApp>},
+    // short variants for quick checks
+    {"UniformRandomWalk8", make_engine<UniformRandomWalkSample, UniformRandomWalkAppT<8>>},
+    {"WeightedNode2Vec8", make_engine<Node2VecSample, WeightedNode2VecAppT<8>>},
+    {"KHop3x2", make_engine<KHopSample, KHopAppT<3, 2>>},
+    {"KHop4x3x2", make_engine<KHopSample, KHopAppT<4, 3, 2>>},
+};
+constexpr int kNumApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
+
+nd_sampler* g_module_sampler = nullptr;
+nd_graph* g_module_graph = nullptr;
+
+struct DeviceBuffer {
+  void* p = nullptr;
+  ~DeviceBuffer() { if (p) (void)hipFree(p); }
+  hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 4); }
+  template <class T> T* as() { return (T*)p; }
+};
+
+__global__ void philox_fill_kernel(uint64_t seed, uint32_t step, uint64_t first_slot, size_t n_slots,
+                                   int draws_per_slot, float* out) {
+  const size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= n_slots) return;
+  nd::RandState rng;
+  rng.reset(seed, first_slot + slot, step);
+  for (int d = 0; d < draws_per_slot; ++d) out[slot * draws_per_slot + d] = rng.next_uniform();
+}
+
+__global__ void run_counts_kernel(const uint32_t* run_start, const nd::RunsMeta* meta, uint32_t* counts) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < meta->n_runs) counts[r] = run_start[r + 1] - run_start[r];
+}
+
+#define CAPI_HIP(expr)                                                                        \
+  do {                                                                                        \
+    hipError_t e_ = (expr);                                                                   \
+    if (e_ != hipSuccess) return fail(std::string(#expr) + ": " + hipGetErrorString(e_));     \
+  } while (0)
+
+}  // namespace
+
+extern "C" {
+
+const char* nd_last_error(void) { return g_error.c_str(); }
+
+int nd_num_apps(void) { return kNumApps; }
+const char* nd_app_name(int index) { return index >= 0 && index < kNumApps ? kApps[index].name : nullptr; }
+
+// ---- graphs ---------------------------------------------------------------------------
+
+int nd_graph_load(const char* path, const char* graph_type, const char* graph_format, nd_graph** out) {
+  if (!out) return fail("null out");
+  std::unique_ptr<nd_graph> g(new nd_graph);
+  std::string err;
+  if (nd::load_graph_file(g->csr, path, graph_type, graph_format, &err) != 0) return fail(err);
+  *out = g.release();
+  return 0;
+}
+
+int nd_graph_from_edges(int32_t n_vertices, int64_t n_edges, const int32_t* src, const int32_t* dst,
+                        const float* weight, nd_graph** out) {
+  if (!out || n_edges < 0 || (n_edges > 0 && (!src || !dst))) return fail("bad argument");
+  std::unique_ptr<nd_graph> g(new nd_graph);
+  std::string err;
+  if (nd::csr_from_edges(g->csr, n_vertices, (size_t)n_edges, src, dst, weight, &err) != 0) return fail(err);
+  *out = g.release();
+  return 0;
+}
+
+int nd_graph_from_csr(int32_t n_vertices, int64_t n_edges, const int32_t* row_ptr, const int32_t* col,
+                      const float* weight, nd_graph** out) {
+  if (!out || !row_ptr || (n_edges > 0 && !col)) return fail("bad argument");
+  std::unique_ptr<nd_graph> g(new nd_graph);
+  std::string err;
+  if (nd::csr_from_arrays(g->csr, n_vertices, n_edges, row_ptr, col, weight, &err) != 0) return fail(err);
+  *out = g.release();
+  return 0;
+}
+
+int nd_graph_rmat(int scale, int edge_factor, double a, double b, double c, uint64_t seed, int symmetrise,
+                  nd_graph** out) {
+  if (!out) return fail("null out");
+  std::unique_ptr<nd_graph> g(new nd_graph);
+  std::string err;
+  if (nd::generate_rmat(g->csr, scale, edge_factor, a, b, c, seed, symmetrise != 0, &err) != 0) return fail(err);
+  *out = g.release();
+  return 0;
+}
+
+int nd_graph_chung_lu(int32_t n_vertices, int64_t n_edges, double exponent, uint64_t seed, nd_graph** out) {
+  if (!out) return fail("null out");
+  std::unique_ptr<nd_graph> g(new nd_graph);
+  std::string err;
+  if (nd::generate_chung_lu(g->csr, n_vertices, n_edges, exponent, seed, &err) != 0) return fail(err);
+  *out = g.release();
+  return 0;
+}
+
+int32_t nd_graph_num_vertices(const nd_graph* g) { return g ? g->csr.get_n_vertices() : 0; }
+int64_t nd_graph_num_edges(const nd_graph* g) { return g ? (int64_t)g->csr.col.size() : 0; }
+const int32_t* nd_graph_row_ptr(const nd_graph* g) { return g ? g->csr.row_ptr.data() : nullptr; }
+const int32_t* nd_graph_col(const nd_graph* g) { return g ? g->csr.col.data() : nullptr; }
+const float* nd_graph_weight(const nd_graph* g) { return g ? g->csr.weight.data() : nullptr; }
+const float* nd_graph_max_weight(const nd_graph* g) { return g ? g->csr.max_weight.data() : nullptr; }
+void nd_graph_free(nd_graph* g) { delete g; }
+
+// ---- sampler --------------------------------------------------------------------------
+
+int nd_sampler_create(const char* app_name, nd_sampler** out) {
+  if (!app_name || !out) return fail("null argument");
+  for (int i = 0; i < kNumApps; ++i) {
+    if (strcmp(kApps[i].name, app_name) == 0) {
+      nd_sampler* s = new nd_sampler;
+      s->engine.reset(kApps[i].make(kApps[i].name));
+      *out = s;
+      return 0;
+    }
+  }
+  return fail(std::string("unknown app '") + app_name + "'");
+}
+
+int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g) {
+  if (!s || !g) return fail("null argument");
+  int n_devices = 0;
+  if (hipGetDeviceCount(&n_devices) != hipSuccess || n_devices < 1) return fail("no HIP device available");
+  s->graph = g;
+  const int rc = s->engine->set_graph(&g->csr);
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
+int nd_sampler_alloc(nd_sampler* s, uint64_t seed) {
+  if (!s) return fail("null sampler");
+  const int rc = s->engine->alloc(seed);
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
+int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing) {
+  if (!s) return fail("null sampler");
+  const int rc = s->engine->sample(enable_load_balancing ? nd::kTransitParallelLoadBalanced : nd::kTransitParallel);
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
+int nd_sampler_get_final_samples(nd_sampler* s, const int32_t** data, int64_t* length) {
+  if (!s || !data || !length) return fail("null argument");
+  const int rc = s->engine->fetch_final_samples();
+  if (rc != 0) return fail(s->engine->last_error, rc);
+  *data = s->engine->hFinalSamples.data();
+  *length = (int64_t)s->engine->hFinalSamples.size();
+  return 0;
+}
+
+int nd_sampler_final_sample_size(const nd_sampler* s) { return s ? s->engine->final_sample_size() : -1; }
+int64_t nd_sampler_num_samples(const nd_sampler* s) { return s ? s->engine->num_samples() : -1; }
+
+int nd_sampler_initial_contents(const nd_sampler* s, const int32_t** data, int64_t* length) {
+  if (!s || !data || !length) return fail("null argument");
+  *data = s->engine->initialContents.data();
+  *length = (int64_t)s->engine->initialContents.size();
+  return 0;
+}
+
+int32_t nd_sampler_invalid_vertex(const nd_sampler* s) { return s ? s->engine->invalid_vertex() : -1; }
+int nd_sampler_max_bits(const nd_sampler* s) { return s ? s->engine->max_bits() : -1; }
+int nd_sampler_steps(const nd_sampler* s) { return s ? s->engine->steps() : -1; }
+int nd_sampler_step_size(const nd_sampler* s, int step) {
+  return s && step >= 0 && step < s->engine->steps() ? s->engine->step_size(step) : -1;
+}
+int nd_sampler_initial_sample_size(const nd_sampler* s) { return s ? s->engine->initial_sample_size() : -1; }
+int nd_sampler_sampling_type(const nd_sampler* s) { return s ? s->engine->sampling_type() : -1; }
+
+int64_t nd_sampler_sample_state_bytes(const nd_sampler* s) { return s ? (int64_t)s->engine->sample_state_bytes() : -1; }
+
+int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes) {
+  if (!s || !dst) return fail("null argument");
+  const int rc = s->engine->fetch_sample_states(dst, (size_t)bytes);
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
+int nd_sampler_set_profiling(nd_sampler* s, int on) {
+  if (!s) return fail("null sampler");
+  s->engine->profiling = on != 0;
+  return 0;
+}
+
+int nd_sampler_phase_times(const nd_sampler* s, float out[8]) {
+  if (!s || !out) return fail("null argument");
+  const nd::PhaseTimes& t = s->engine->times;
+  out[0] = t.end_to_end; out[1] = t.inversion; out[2] = t.load_balancing; out[3] = t.flat_kernel;
+  out[4] = t.workgroup_kernel; out[5] = (float)t.flat_launches; out[6] = (float)t.workgroup_launches;
+  out[7] = (float)t.sort_launches;
+  return 0;
+}
+
+void nd_sampler_free_device(nd_sampler* s) {
+  if (s) s->engine->free_device();
+}
+
+void nd_sampler_destroy(nd_sampler* s) { delete s; }
+
+// ---- module-level functions ---------------------------------------------------------------
+
+void nd_free_device_memory(void) {
+  if (g_module_sampler) nd_sampler_destroy(g_module_sampler);
+  g_module_sampler = nullptr;
+  if (g_module_graph) nd_graph_free(g_module_graph);
+  g_module_graph = nullptr;
+}
+
+int nd_init_sampling(const char* app_name, const char* graph_path, uint64_t seed) {
+  nd_free_device_memory();
+  int rc = nd_graph_load(graph_path, "edge-list", "binary", &g_module_graph);
+  if (rc != 0) return rc;
+  rc = nd_sampler_create(app_name, &g_module_sampler);
+  if (rc == 0) rc = nd_sampler_set_graph(g_module_sampler, g_module_graph);
+  if (rc == 0) rc = nd_sampler_alloc(g_module_sampler, seed);
+  if (rc != 0) {
+    const std::string keep = g_error;
+    nd_free_device_memory();
+    g_error = keep;
+  }
+  return rc;
+}
+
+int nd_sample(void) {
+  if (!g_module_sampler) return fail("sample() before initSampling()");
+  return nd_sampler_do_transit_parallel(g_module_sampler, 1);
+}
+
+int64_t nd_final_sample_length(void) {
+  return g_module_sampler ? (int64_t)g_module_sampler->engine->hFinalSamples.size() : 0;
+}
+
+const int32_t* nd_final_samples_array(void) {
+  if (!g_module_sampler) { fail("finalSamplesArray() before initSampling()"); return nullptr; }
+  const int32_t* data = nullptr;
+  int64_t len = 0;
+  if (nd_sampler_get_final_samples(g_module_sampler, &data, &len) != 0) return nullptr;
+  return data;
+}
+
+// ---- building blocks ------------------------------------------------------------------------
+
+int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, int64_t n_slots, int draws_per_slot,
+                           float* out) {
+  if (n_slots < 0 || draws_per_slot < 1 || (n_slots > 0 && !out)) return fail("bad argument");
+  if (n_slots == 0) return 0;
+  DeviceBuffer d;
+  const size_t bytes = sizeof(float) * (size_t)n_slots * draws_per_slot;
+  CAPI_HIP(d.alloc(bytes));
+  philox_fill_kernel<<<dim3((unsigned)((n_slots + 255) / 256)), dim3(256), 0, 0>>>(seed, step, first_slot,
+                                                                                  (size_t)n_slots, draws_per_slot,
+                                                                                  d.as<float>());
+  CAPI_HIP(hipGetLastError());
+  CAPI_HIP(hipMemcpy(out, d.p, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_bits, int32_t* keys_out,
+                  int32_t* vals_out) {
+  if (n < 0 || key_bits < 1 || key_bits > 32 || (n > 0 && (!keys || !keys_out || !vals_out)))
+    return fail("bad argument");
+  if (n == 0) return 0;
+  if (n >= (int64_t)1 << 31) return fail("too many pairs");
+  const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);
+  DeviceBuffer k_in, v_in, k_a, v_a, k_b, v_b, hist, scratch;
+  const size_t bytes = sizeof(uint32_t) * (size_t)n;
+  CAPI_HIP(k_in.alloc(bytes));
+  CAPI_HIP(k_a.alloc(bytes));
+  CAPI_HIP(v_a.alloc(bytes));
+  CAPI_HIP(k_b.alloc(bytes));
+  CAPI_HIP(v_b.alloc(bytes));
+  CAPI_HIP(hist.alloc(sizeof(uint32_t) * plan.hist_elems));
+  CAPI_HIP(scratch.alloc(sizeof(uint32_t) * plan.scratch_elems));
+  CAPI_HIP(hipMemcpy(k_in.p, keys, bytes, hipMemcpyHostToDevice));
+  if (vals) {
+    CAPI_HIP(v_in.alloc(bytes));
+    CAPI_HIP(hipMemcpy(v_in.p, vals, bytes, hipMemcpyHostToDevice));
+  }
+  uint32_t *k_sorted = nullptr, *v_sorted = nullptr;
+  CAPI_HIP(nd::radix_sort_pairs(plan, k_in.as<uint32_t>(), vals ? v_in.as<uint32_t>() : nullptr, k_a.as<uint32_t>(),
+                                v_a.as<uint32_t>(), k_b.as<uint32_t>(), v_b.as<uint32_t>(), hist.as<uint32_t>(),
+                                scratch.as<uint32_t>(), 0, &k_sorted, &v_sorted));
+  CAPI_HIP(hipDeviceSynchronize());
+  CAPI_HIP(hipMemcpy(keys_out, k_sorted, bytes, hipMemcpyDeviceToHost));
+  CAPI_HIP(hipMemcpy(vals_out, v_sorted, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
+                       int32_t* offsets, int64_t* n_runs, int64_t* n_valid) {
+  if (n < 0 || !n_runs || !n_valid || (n > 0 && (!sorted_keys || !uniq || !counts || !offsets)))
+    return fail("bad argument");
+  *n_runs = 0;
+  *n_valid = 0;
+  if (n == 0) return 0;
+  const size_t bytes = sizeof(uint32_t) * (size_t)n;
+  DeviceBuffer keys, run_key, run_start, run_count, meta, scratch;
+  CAPI_HIP(keys.alloc(bytes));
+  CAPI_HIP(run_key.alloc(bytes));
+  CAPI_HIP(run_start.alloc(bytes + sizeof(uint32_t)));
+  CAPI_HIP(run_count.alloc(bytes));
+  CAPI_HIP(meta.alloc(sizeof(nd::RunsMeta)));
+  CAPI_HIP(scratch.alloc(sizeof(uint32_t) * nd::runs_scratch_elems((size_t)n)));
+  CAPI_HIP(hipMemcpy(keys.p, sorted_keys, bytes, hipMemcpyHostToDevice));
+  CAPI_HIP(nd::find_transit_runs(keys.as<uint32_t>(), (size_t)n, (uint32_t)invalid, run_key.as<uint32_t>(),
+                                 run_start.as<uint32_t>(), meta.as<nd::RunsMeta>(), scratch.as<uint32_t>(), 0));
+  run_counts_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(run_start.as<uint32_t>(),
+                                                                           meta.as<nd::RunsMeta>(),
+                                                                           run_count.as<uint32_t>());
+  CAPI_HIP(hipGetLastError());
+  nd::RunsMeta h;
+  CAPI_HIP(hipMemcpy(&h, meta.p, sizeof(h), hipMemcpyDeviceToHost));
+  *n_runs = h.n_runs;
+  *n_valid = h.n_valid;
+  if (h.n_runs) {
+    CAPI_HIP(hipMemcpy(uniq, run_key.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(counts, run_count.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(offsets, run_start.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+// The compile-time App contract of the sampling engine, for gfx950.
+//
+// An application is a stateless struct (the engine constructs it on the fly as App())
+// with the member functions of the reference's apps (example/uniformRandWalk.cu:15-93):
+//   steps(), stepSize(k), next(...), samplingType(), outputFormat(), numSamples(CSR*),
+//   initialSample(idx, CSR*, SampleType&), initialSampleSize(CSR*), hasExplicitTransits(),
+//   stepTransits(...), initializeSample(CSR*, id).
+// This header supplies, in the global namespace and under the spellings those app sources
+// use, every type and helper they refer to: VertexID / VertexID_t / EdgePos_t, CSR and
+// CSRPartition, SamplingType / OutputFormat, RandNumGen::rand_int, utils::binarySearch and
+// the random-state handle.  The handle is the engine's own Philox cursor (nd::RandState);
+// it only carries the name the app signature spells.  No vendor RNG library is involved.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "nd_philox.hpp"
+
+typedef int32_t VertexID;
+typedef int32_t EdgePos_t;
+typedef VertexID VertexID_t;
+
+// src/nextdoor.cu:62-71
+enum SamplingType { IndividualNeighborhood, CollectiveNeighborhood };
+enum OutputFormat { SampledVertices, AdjacencyMatrix };
+// src/nextdoor.cu:48
+constexpr int ALL_NEIGHBORS = -1;
+
+// Host-side graph in CSR form.  Plays the role of the reference's CSR class
+// (src/csr.hpp:46-196) for the host members of an App (numSamples, initialSample ...).
+// Stored as structure-of-arrays: row_ptr[V+1], col[E], weight[E], max_weight[V];
+// the adjacency of every vertex is sorted ascending by (destination, weight) with
+// duplicates kept (src/graph.hpp:38,156) and max_weight[v] = max(0, weights of v)
+// (src/graph.hpp:71-80).
+class CSR {
+ public:
+  typedef VertexID Edge;
+
+  std::vector<EdgePos_t> row_ptr;
+  std::vector<Edge> col;
+  std::vector<float> weight;
+  std::vector<float> max_weight;
+
+  VertexID get_n_vertices() const { return row_ptr.empty() ? 0 : (VertexID)(row_ptr.size() - 1); }
+  EdgePos_t get_n_edges() const { return (EdgePos_t)col.size(); }
+  bool has_vertex(VertexID v) const { return 0 <= v && v < get_n_vertices(); }
+  EdgePos_t n_edges_for_vertex(VertexID v) const { return row_ptr[v + 1] - row_ptr[v]; }
+  EdgePos_t get_start_edge_idx(VertexID v) const { return row_ptr[v]; }
+  // inclusive end, -1 for a vertex without edges (src/csr.hpp:75-77, 413-416)
+  EdgePos_t get_end_edge_idx(VertexID v) const { return n_edges_for_vertex(v) == 0 ? -1 : row_ptr[v + 1] - 1; }
+  const Edge* get_edges() const { return col.data(); }
+  const float* get_weights() const { return weight.data(); }
+};
+
+// Device view of the graph, handed to App::next as `CSRPartition* csr`
+// (accessor names of src/csr.hpp:198-385).  Lives in kernel arguments, not in
+// constant memory.
+class CSRPartition {
+ public:
+  const EdgePos_t* row_ptr;
+  const CSR::Edge* edges;
+  const float* weights;
+  const float* max_weights;
+  VertexID n_vertices;
+  EdgePos_t n_edges;
+
+  __host__ __device__ __forceinline__ VertexID get_n_vertices() const { return n_vertices; }
+  __host__ __device__ __forceinline__ EdgePos_t get_n_edges() const { return n_edges; }
+  __host__ __device__ __forceinline__ bool has_vertex(int v) const { return v >= 0 && v < n_vertices; }
+  __host__ __device__ __forceinline__ EdgePos_t get_start_edge_idx(int v) const { return row_ptr[v]; }
+  __host__ __device__ __forceinline__ EdgePos_t get_end_edge_idx(int v) const {
+    const EdgePos_t b = row_ptr[v], e = row_ptr[v + 1];
+    return e == b ? -1 : e - 1;
+  }
+  __host__ __device__ __forceinline__ EdgePos_t get_n_edges_for_vertex(VertexID v) const {
+    return row_ptr[v + 1] - row_ptr[v];
+  }
+  __host__ __device__ __forceinline__ float get_max_weight(int v) const { return max_weights[v]; }
+  __host__ __device__ __forceinline__ CSR::Edge get_edge(EdgePos_t idx) const { return edges[idx]; }
+  __host__ __device__ __forceinline__ float get_weight(EdgePos_t idx) const { return weights[idx]; }
+  __host__ __device__ __forceinline__ const CSR::Edge* get_edges() const { return edges; }
+  __host__ __device__ __forceinline__ const float* get_weights() const { return weights; }
+  __host__ __device__ __forceinline__ const CSR::Edge* get_edges(VertexID v) const { return edges + row_ptr[v]; }
+  __host__ __device__ __forceinline__ const float* get_weights(VertexID v) const { return weights + row_ptr[v]; }
+
+  // src/csr.hpp:342-359: binary search of dst in the sorted adjacency of src
+  __host__ __device__ __forceinline__ bool has_edge_logn(VertexID src, VertexID dst) const {
+    EdgePos_t l = row_ptr[src];
+    EdgePos_t r = row_ptr[src + 1] - 1;
+    while (l <= r) {
+      const EdgePos_t m = l + (r - l) / 2;
+      const CSR::Edge e = edges[m];
+      if (e == dst) return true;
+      if (e < dst) l = m + 1; else r = m - 1;
+    }
+    return false;
+  }
+};
+
+// The random-state handle named in App::next / App::stepTransits.
+typedef nd::RandState curandState;
+
+// Uniform variate in [0, 1) from the engine's Philox cursor.
+__host__ __device__ __forceinline__ float curand_uniform(curandState* state) { return state->next_uniform(); }
+
+// src/rand_num_gen.cuh:117-122
+struct RandNumGen {
+  __host__ __device__ __forceinline__ static EdgePos_t rand_int(curandState* state, const EdgePos_t n) {
+    return nd::rand_int_from_uniform(state->next_uniform(), n);
+  }
+};
+
+namespace utils {
+// src/utils.hpp:30-48
+template <typename F, typename T>
+__host__ __device__ __forceinline__ bool binarySearch(F& array, T x, int size) {
+  EdgePos_t l = 0;
+  EdgePos_t r = size - 1;
+  while (l <= r) {
+    const EdgePos_t m = l + (r - l) / 2;
+    const auto probe = array[m];
+    if (probe == x) return true;
+    if (probe < x) l = m + 1; else r = m - 1;
+  }
+  return false;
+}
+}  // namespace utils
+
+namespace nd {
+
+// Adjacency of the current transit staged in LDS: entries [0, cached) come from LDS,
+// the rest from HBM.  One of the two EdgeArray / WeightArray types an App::next is
+// instantiated with (the other is a plain pointer); only operator[] is required
+// (the reference's CachedArray, src/nextdoor.cu:76-124, plays this role).
+template <typename T>
+struct LdsBackedArray {
+  const T* lds;
+  const T* global;
+  EdgePos_t cached;
+  __device__ __forceinline__ T operator[](EdgePos_t i) const { return i < cached ? lds[i] : global[i]; }
+};
+
+// Optional compile-time hints an App may carry; absent members mean `false`.
+//   static constexpr bool kUsesEdgeWeights = true;  -> stage weights in LDS as well
+template <typename App, typename = void>
+struct app_uses_weights { static constexpr bool value = false; };
+template <typename App>
+struct app_uses_weights<App, decltype((void)App::kUsesEdgeWeights)> { static constexpr bool value = App::kUsesEdgeWeights; };
+
+}  // namespace nd

@@ -1,0 +1,638 @@
+// Transit-parallel sampling engine for one MI355X (gfx950, wave64).
+//
+// What this implements, against the reference (file:line in the reference tree):
+//   allocNextDoorDataOnGPU     src/nextdoor.cu:1931-2086   -> Engine::alloc
+//   transferCSRToGPUs          src/nextdoor.cu:1893-1911   -> Engine::set_graph
+//   doTransitParallelSampling  src/nextdoor.cu:2191-3006   -> Engine::sample
+//   getFinalSamples            src/nextdoor.cu:3211-3237   -> Engine::final_samples
+//   freeDeviceData             src/nextdoor.cu:2088-2115   -> Engine::free_device
+//   samplingKernel / identityKernel / gridKernel  212-336 / 338-504 / 976-1204
+//                                                      -> step_flat_kernel / step_workgroup_kernel
+//   partitionTransitsInKernels 1520-1802               -> classify_runs
+//
+// Differences that are deliberate:
+//  * The (sample -> transit) map stores only the transit; the map index IS the slot
+//    (sample * transitsPerSample + j).  The inversion sorts (transit, slot) and the step
+//    kernels write output (slot * stepSize + nbr) of sample slot / transitsPerSample at a
+//    fixed place: final[sample * F + segBase + j * stepSize + nbr].  The reference places
+//    k-hop outputs with an atomic cursor per sample (nextdoor.cu:304, 473), i.e. in no
+//    fixed order; this order is one it can produce, and it never changes between runs or
+//    kernel classes.
+//  * Random numbers are Philox draws keyed by the output slot and the step (nd_philox.hpp),
+//    so load balancing on/off, kernel class and lane assignment cannot change a result.
+//  * No host round trip inside the step loop: run counts, work lists and the
+//    valid-prefix length stay in device memory; kernels whose work size is only known on
+//    the device are launched with a fixed grid and stride over the device-side count.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "nd_contract.hpp"
+#include "nd_radix_sort.hpp"
+#include "nd_transit_runs.hpp"
+
+namespace nd {
+
+// ---------------------------------------------------------------------------------------
+// Host-visible, app-independent interface (what the C ABI talks to)
+// ---------------------------------------------------------------------------------------
+
+enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1 };
+
+struct PhaseTimes {  // milliseconds, accumulated over one sample() call when profiling is on
+  float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0;
+  int flat_launches = 0, workgroup_launches = 0, sort_launches = 0;
+};
+
+class EngineBase {
+ public:
+  virtual ~EngineBase() {}
+  virtual const char* app_name() const = 0;
+  virtual int set_graph(const CSR* graph) = 0;
+  virtual int alloc(uint64_t seed) = 0;
+  virtual int sample(int mode) = 0;
+  virtual int fetch_final_samples() = 0;
+  virtual void free_device() = 0;
+  virtual int64_t num_samples() const = 0;
+  virtual int final_sample_size() const = 0;
+  virtual int steps() const = 0;
+  virtual int step_size(int k) const = 0;
+  virtual int initial_sample_size() const = 0;
+  virtual int sampling_type() const = 0;
+  virtual int32_t invalid_vertex() const = 0;
+  virtual int max_bits() const = 0;
+  virtual size_t sample_state_bytes() const = 0;
+  virtual int fetch_sample_states(void* dst, size_t bytes) = 0;
+
+  std::vector<VertexID_t> hFinalSamples;       // as NextDoorData::hFinalSamples (libNextDoor.hpp:17)
+  std::vector<VertexID_t> initialContents;     // as NextDoorData::initialContents (libNextDoor.hpp:18)
+  std::string last_error;
+  bool profiling = false;
+  PhaseTimes times;
+};
+
+#define ND_HIP_TRY(expr)                                                                  \
+  do {                                                                                    \
+    hipError_t nd_e_ = (expr);                                                            \
+    if (nd_e_ != hipSuccess) {                                                            \
+      last_error = std::string(#expr) + ": " + hipGetErrorString(nd_e_);                  \
+      return -1;                                                                          \
+    }                                                                                     \
+  } while (0)
+
+// ---------------------------------------------------------------------------------------
+// Step kernels
+// ---------------------------------------------------------------------------------------
+
+struct StepParams {
+  CSRPartition csr;
+  int step;
+  uint32_t step_size;            // m_k
+  uint32_t transits_per_sample;  // T_k
+  uint32_t seg_base;             // offset of this step's segment inside a final sample
+  uint32_t final_size;           // F
+  int32_t invalid;
+  int is_last;
+  uint64_t seed;
+  uint64_t first_slot;           // RNG slot of local output 0 (first sample of this device)
+  uint32_t first_sample;
+  uint32_t n_pairs;              // S * T_k
+  const uint32_t* pair_keys;     // transit of each pair (sorted, or the raw map at step 0)
+  const uint32_t* pair_slots;    // slot of each pair; nullptr: slot == index
+  int32_t* next_transits;        // map for step k+1, indexed by output slot
+  int32_t* final_samples;
+  void* samples;                 // SampleType[S] or nullptr
+};
+
+constexpr int kStepThreads = 256;
+// LDS adjacency cache of the workgroup kernel, in edges.
+constexpr int kCacheEdges = 8192;
+// A transit goes to the workgroup kernel when at least this many outputs are drawn from it.
+constexpr uint32_t kWorkgroupWork = 256;
+// Outputs one work item of the workgroup kernel covers at most; larger runs are split
+// over several workgroups (the grid-wide case).
+constexpr uint32_t kChunkOutputs = 2048;
+
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit,
+                                               uint32_t pair_slot, uint32_t nbr, EdgePos_t n_edges, float max_weight,
+                                               EdgeArray& edges, WeightArray& weights) {
+  const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
+  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
+  VertexID neighbor = P.invalid;
+  // next() only runs for a real transit that has edges (nextdoor.cu:250-262)
+  if (transit != P.invalid && n_edges != 0) {
+    curandState rng;
+    rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+    SampleType local_state;
+    SampleType* state = std::is_empty<SampleType>::value ? &local_state : (SampleType*)P.samples + sample;
+    const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
+        P.step, &csr, &transit, (VertexID)(P.first_sample + sample), state, max_weight, edges, weights, n_edges,
+        (VertexID_t)nbr, &rng);
+    neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
+  }
+  if (!P.is_last) P.next_transits[out_slot] = neighbor;
+  const uint64_t within = out_slot - (uint64_t)sample * P.transits_per_sample * P.step_size;
+  P.final_samples[(size_t)sample * P.final_size + P.seg_base + within] = neighbor;
+}
+
+// One lane per output: lane i draws neighbour (i % m) for pair (i / m).  With the map
+// sorted by transit, neighbouring lanes share row extents and adjacency lines.
+// skip_flag (nullable): per-vertex marker of transits the workgroup kernel handles.
+template <class SampleType, class App>
+__global__ __launch_bounds__(kStepThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
+  const uint64_t total = (uint64_t)P.n_pairs * P.step_size;
+  const uint64_t i = (uint64_t)blockIdx.x * kStepThreads + threadIdx.x;
+  if (i >= total) return;
+  CSRPartition csr = P.csr;
+  const uint32_t pair = P.step_size == 1 ? (uint32_t)i : (uint32_t)(i / P.step_size);
+  const uint32_t nbr = (uint32_t)(i - (uint64_t)pair * P.step_size);
+  const VertexID transit = (VertexID)P.pair_keys[pair];
+  const uint32_t slot = P.pair_slots ? P.pair_slots[pair] : pair;
+  EdgePos_t n_edges = 0;
+  float max_weight = 0.0f;
+  const CSR::Edge* edges = nullptr;
+  const float* weights = nullptr;
+  if (transit != P.invalid) {
+    if (skip_flag && skip_flag[transit]) return;
+    const EdgePos_t begin = csr.row_ptr[transit];
+    n_edges = csr.row_ptr[transit + 1] - begin;
+    edges = csr.edges + begin;
+    weights = csr.weights + begin;
+    max_weight = csr.max_weights[transit];
+  }
+  produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, slot, nbr, n_edges, max_weight,
+                                                                 edges, weights);
+}
+
+// One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
+// transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
+// with coalesced reads and every draw of the stretch gathers from LDS.
+template <class SampleType, class App>
+__global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams P,
+                                                                      const uint32_t* __restrict__ chunks,
+                                                                      const RunsMeta* __restrict__ meta,
+                                                                      uint32_t chunk_capacity,
+                                                                      uint8_t* __restrict__ skip_flag) {
+  constexpr bool kWeights = app_uses_weights<App>::value;
+  __shared__ CSR::Edge s_edges[kCacheEdges];
+  __shared__ float s_weights[kWeights ? kCacheEdges : 1];
+  CSRPartition csr = P.csr;
+  const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
+  for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+    const uint32_t first_pair = chunks[2 * c];
+    const uint32_t n_pairs = chunks[2 * c + 1];
+    const VertexID transit = (VertexID)P.pair_keys[first_pair];
+    const EdgePos_t begin = csr.row_ptr[transit];
+    const EdgePos_t n_edges = csr.row_ptr[transit + 1] - begin;
+    const float max_weight = csr.max_weights[transit];
+    const EdgePos_t cached = n_edges < kCacheEdges ? n_edges : kCacheEdges;
+    __syncthreads();  // the previous work item is done with the cache
+    for (EdgePos_t e = threadIdx.x; e < cached; e += kStepThreads) {
+      s_edges[e] = csr.edges[begin + e];
+      if (kWeights) s_weights[e] = csr.weights[begin + e];
+    }
+    if (threadIdx.x == 0) skip_flag[transit] = 0;  // leave the marker array clean for the next step
+    __syncthreads();
+    LdsBackedArray<CSR::Edge> edges{s_edges, csr.edges + begin, cached};
+    LdsBackedArray<float> lds_weights{s_weights, csr.weights + begin, kWeights ? cached : 0};
+    const uint32_t outputs = n_pairs * P.step_size;
+    for (uint32_t o = threadIdx.x; o < outputs; o += kStepThreads) {
+      const uint32_t p = P.step_size == 1 ? o : o / P.step_size;
+      const uint32_t nbr = o - p * P.step_size;
+      const uint32_t slot = P.pair_slots[first_pair + p];
+      produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
+          P, csr, transit, slot, nbr, n_edges, max_weight, edges, lds_weights);
+    }
+  }
+}
+
+// One lane per unique transit: decide which kernel class serves it and emit work items.
+// Classes by neighbour-work (outputs drawn from the transit = count * stepSize):
+//   work <  kWorkgroupWork                      -> flat kernel (sub-wavefront: the lanes of a
+//                                                  wave that share the transit share its lines)
+//   work >= kWorkgroupWork, one work item       -> workgroup kernel
+//   work >  kChunkOutputs, several work items   -> grid-wide: the transit is split over workgroups
+// A transit whose adjacency does not fit the LDS cache, or is much longer than the number
+// of draws taken from it, is cheaper to gather directly and stays with the flat kernel.
+__global__ __launch_bounds__(256) void classify_runs(const uint32_t* __restrict__ run_key,
+                                                     const uint32_t* __restrict__ run_start, RunsMeta* meta,
+                                                     const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
+                                                     uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
+                                                     uint8_t* __restrict__ skip_flag) {
+  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= meta->n_runs) return;
+  const uint32_t start = run_start[r];
+  const uint32_t count = run_start[r + 1] - start;
+  const uint32_t transit = run_key[r];
+  const uint64_t work = (uint64_t)count * step_size;
+  if (work < kWorkgroupWork) return;
+  const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
+  if (degree == 0 || degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) return;
+  uint32_t pairs_per_chunk = kChunkOutputs / step_size;
+  if (pairs_per_chunk == 0) pairs_per_chunk = 1;
+  const uint32_t n_items = (count + pairs_per_chunk - 1) / pairs_per_chunk;
+  // Work items are claimed with one atomic; their order in the list is irrelevant to the
+  // results.  The list is sized so that every claim fits (see Engine::alloc); should one
+  // not fit, the transit is left to the flat kernel and the entries that did fit are
+  // processed twice with identical results.
+  const uint32_t base = atomicAdd(&meta->n_chunks, n_items);
+  const bool fits = base + n_items <= chunk_capacity;
+  for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
+    const uint32_t off = g * pairs_per_chunk;
+    chunks[2 * (base + g)] = start + off;
+    chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+  }
+  if (fits) {
+    skip_flag[transit] = 1;
+    atomicAdd(&meta->n_big_pairs, count);
+  }
+}
+
+__global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
+// ---------------------------------------------------------------------------------------
+// Shape algebra (nextdoor.cu:126-197, 1913-1929)
+// ---------------------------------------------------------------------------------------
+
+template <class App>
+inline bool is_collective() { return App().samplingType() == CollectiveNeighborhood; }
+
+template <class App>
+inline int64_t step_size_at_step(int step) {
+  if (step == -1) return 0;
+  int64_t n = is_collective<App>() ? 0 : (int64_t)App().initialSampleSize(nullptr);
+  for (int i = 0; i <= step; ++i) {
+    if (is_collective<App>()) n += App().stepSize(i); else n *= App().stepSize(i);
+  }
+  return n;
+}
+
+template <class App>
+inline int final_sample_size() {
+  int64_t total = 0, per_step = 1;
+  for (int k = 0; k < App().steps(); ++k) {
+    if (is_collective<App>()) per_step = App().stepSize(k); else per_step *= App().stepSize(k);
+    total += per_step;
+  }
+  return (int)total;
+}
+
+// ---------------------------------------------------------------------------------------
+// Engine
+// ---------------------------------------------------------------------------------------
+
+template <class SampleType, class App>
+class Engine : public EngineBase {
+ public:
+  explicit Engine(const char* name) : name_(name) {}
+  ~Engine() override { free_device(); }
+
+  const char* app_name() const override { return name_; }
+  int64_t num_samples() const override { return n_samples_; }
+  int final_sample_size() const override { return nd::final_sample_size<App>(); }
+  int steps() const override { return App().steps(); }
+  int step_size(int k) const override { return App().stepSize(k); }
+  int initial_sample_size() const override { return App().initialSampleSize(nullptr); }
+  int sampling_type() const override { return App().samplingType(); }
+  int32_t invalid_vertex() const override { return invalid_; }
+  int max_bits() const override { return max_bits_; }
+  size_t sample_state_bytes() const override {
+    return std::is_empty<SampleType>::value ? 0 : sizeof(SampleType) * (size_t)n_samples_;
+  }
+
+  // transferCSRToGPUs: the whole graph is resident on the device.
+  int set_graph(const CSR* graph) override {
+    free_graph();
+    graph_ = graph;
+    const size_t V = (size_t)graph->get_n_vertices();
+    const size_t E = graph->col.size();
+    if (V == 0) { last_error = "graph has no vertices"; return -1; }
+    if (E >= (size_t)INT32_MAX) { last_error = "edge count does not fit int32 edge positions"; return -1; }
+    ND_HIP_TRY(hipMalloc(&d_row_ptr_, sizeof(EdgePos_t) * (V + 1)));
+    ND_HIP_TRY(hipMalloc(&d_col_, sizeof(VertexID) * (E ? E : 1)));
+    ND_HIP_TRY(hipMalloc(&d_weight_, sizeof(float) * (E ? E : 1)));
+    ND_HIP_TRY(hipMalloc(&d_max_weight_, sizeof(float) * V));
+    ND_HIP_TRY(hipMemcpy(d_row_ptr_, graph->row_ptr.data(), sizeof(EdgePos_t) * (V + 1), hipMemcpyHostToDevice));
+    if (E) {
+      ND_HIP_TRY(hipMemcpy(d_col_, graph->col.data(), sizeof(VertexID) * E, hipMemcpyHostToDevice));
+      ND_HIP_TRY(hipMemcpy(d_weight_, graph->weight.data(), sizeof(float) * E, hipMemcpyHostToDevice));
+    }
+    ND_HIP_TRY(hipMemcpy(d_max_weight_, graph->max_weight.data(), sizeof(float) * V, hipMemcpyHostToDevice));
+    view_.row_ptr = d_row_ptr_;
+    view_.edges = d_col_;
+    view_.weights = d_weight_;
+    view_.max_weights = d_max_weight_;
+    view_.n_vertices = (VertexID)V;
+    view_.n_edges = (EdgePos_t)E;
+    return 0;
+  }
+
+  // allocNextDoorDataOnGPU: run the host half of the App (numSamples, initializeSample,
+  // initialSample) and allocate every per-run buffer once.
+  int alloc(uint64_t seed) override {
+    if (!graph_) { last_error = "alloc before set_graph"; return -1; }
+    free_run_buffers();
+    seed_ = seed;
+    CSR* csr = const_cast<CSR*>(graph_);
+    App app;
+    if (app.hasExplicitTransits()) { last_error = "apps with explicit transits are not supported"; return -2; }
+    if (is_collective<App>()) { last_error = "collective apps need the layer engine"; return -2; }
+    const int n_steps = app.steps();
+    for (int k = 0; k < n_steps; ++k)
+      if (app.stepSize(k) <= 0) { last_error = "stepSize must be positive (ALL_NEIGHBORS is not supported)"; return -2; }
+    n_samples_ = app.numSamples(csr);
+    init_size_ = app.initialSampleSize(csr);
+    if (n_samples_ <= 0 || init_size_ <= 0) { last_error = "app yields no samples"; return -2; }
+    invalid_ = graph_->get_n_vertices();  // nextdoor.cu:1993
+    max_bits_ = 0;
+    while ((invalid_ >> max_bits_) != 0) max_bits_++;
+
+    samples_.clear();
+    initialContents.clear();
+    samples_.reserve((size_t)n_samples_);
+    initialContents.reserve((size_t)n_samples_ * init_size_);
+    for (int64_t s = 0; s < n_samples_; ++s) {
+      samples_.push_back(app.template initializeSample<SampleType>(csr, (VertexID_t)s));
+      std::vector<VertexID_t> roots = app.initialSample((int)s, csr, samples_.back());
+      if ((EdgePos_t)roots.size() != init_size_) {
+        last_error = "initialSample size differs from initialSampleSize";  // nextdoor.cu:1964-1969
+        return -2;
+      }
+      initialContents.insert(initialContents.end(), roots.begin(), roots.end());
+    }
+
+    // largest map: transits entering the last step
+    uint64_t max_pairs = (uint64_t)n_samples_ * init_size_;
+    uint64_t outputs = max_pairs;
+    uint64_t max_outputs = 0;
+    for (int k = 0; k < n_steps; ++k) {
+      outputs *= (uint64_t)app.stepSize(k);
+      if (outputs > max_outputs) max_outputs = outputs;
+      if (k < n_steps - 1) max_pairs = outputs;
+    }
+    if (max_outputs >= (1ull << 32) || max_pairs >= (1ull << 31)) {
+      last_error = "a step has 2^32 or more outputs; split the samples over several runs";
+      return -2;
+    }
+    max_pairs_ = (size_t)max_pairs;
+    const size_t F = (size_t)final_sample_size();
+    hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
+
+    ND_HIP_TRY(hipStreamCreate(&stream_));
+    ND_HIP_TRY(hipMalloc(&d_initial_, sizeof(VertexID_t) * initialContents.size()));
+    ND_HIP_TRY(hipMemcpy(d_initial_, initialContents.data(), sizeof(VertexID_t) * initialContents.size(),
+                         hipMemcpyHostToDevice));
+    if (!std::is_empty<SampleType>::value) {
+      ND_HIP_TRY(hipMalloc(&d_samples_, sizeof(SampleType) * (size_t)n_samples_));
+    }
+    ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
+    ND_HIP_TRY(hipMalloc(&d_map_, sizeof(int32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * max_pairs_));
+    const SortPlan plan = make_sort_plan(max_pairs_, max_bits_);
+    ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * plan.hist_elems));
+    size_t scratch = plan.scratch_elems;
+    if (runs_scratch_elems(max_pairs_) > scratch) scratch = runs_scratch_elems(max_pairs_);
+    ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
+    ND_HIP_TRY(hipMalloc(&d_run_key_, sizeof(uint32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_run_start_, sizeof(uint32_t) * (max_pairs_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta)));
+    ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta)));
+    // work-item list: a run of `count` pairs emits ceil(count / pairsPerChunk) items and at
+    // most outputs / kWorkgroupWork runs qualify, so this bound holds at every step
+    {
+      uint64_t cap = 0, pairs = (uint64_t)n_samples_ * init_size_;
+      for (int k = 0; k < n_steps; ++k) {
+        const uint64_t mk = (uint64_t)app.stepSize(k);
+        uint64_t per_chunk = kChunkOutputs / mk;
+        if (per_chunk == 0) per_chunk = 1;
+        const uint64_t need = pairs / per_chunk + pairs * mk / kWorkgroupWork + 2;
+        if (need > cap) cap = need;
+        pairs *= mk;
+      }
+      chunk_capacity_ = (uint32_t)cap;
+    }
+    ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
+    ND_HIP_TRY(hipMalloc(&d_skip_flag_, (size_t)invalid_ + 1));
+    ND_HIP_TRY(hipMemset(d_skip_flag_, 0, (size_t)invalid_ + 1));
+    ND_HIP_TRY(hipEventCreate(&ev_a_));
+    ND_HIP_TRY(hipEventCreate(&ev_b_));
+    ND_HIP_TRY(hipEventCreate(&ev_begin_));
+    ND_HIP_TRY(hipEventCreate(&ev_end_));
+    allocated_ = true;
+    return 0;
+  }
+
+  // doTransitParallelSampling: the step loop.  Everything is enqueued on one stream;
+  // the only host wait is at the end.
+  int sample(int mode) override {
+    if (!allocated_) { last_error = "sample before alloc"; return -1; }
+    const bool balance = mode == kTransitParallelLoadBalanced;
+    App app;
+    const int n_steps = app.steps();
+    const size_t F = (size_t)final_sample_size();
+    times = PhaseTimes();
+    if (!std::is_empty<SampleType>::value) {
+      ND_HIP_TRY(hipMemcpyAsync(d_samples_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
+                                hipMemcpyHostToDevice, stream_));
+    }
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
+
+    uint32_t transits_per_sample = (uint32_t)init_size_;
+    uint32_t seg_base = 0;
+    for (int step = 0; step < n_steps; ++step) {
+      const uint32_t m = (uint32_t)app.stepSize(step);
+      const uint32_t n_pairs = (uint32_t)((uint64_t)n_samples_ * transits_per_sample);
+      StepParams P;
+      P.csr = view_;
+      P.step = step;
+      P.step_size = m;
+      P.transits_per_sample = transits_per_sample;
+      P.seg_base = seg_base;
+      P.final_size = (uint32_t)F;
+      P.invalid = invalid_;
+      P.is_last = step == n_steps - 1;
+      P.seed = seed_;
+      P.first_slot = 0;
+      P.first_sample = 0;
+      P.n_pairs = n_pairs;
+      P.next_transits = d_map_;
+      P.final_samples = d_final_;
+      P.samples = d_samples_;
+      const uint64_t outputs = (uint64_t)n_pairs * m;
+      const unsigned flat_grid = (unsigned)((outputs + kStepThreads - 1) / kStepThreads);
+
+      if (step == 0) {
+        // roots are used in sample order (the reference also feeds step 0 an unsorted map
+        // when there is more than one step, nextdoor.cu:2400 and the FIXME at 2372)
+        P.pair_keys = (const uint32_t*)d_initial_;
+        P.pair_slots = nullptr;
+        tick();
+        step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, nullptr);
+        tock(&times.flat_kernel);
+        times.flat_launches++;
+      } else {
+        // inversion: sort (transit, slot) by transit
+        const SortPlan plan = make_sort_plan(n_pairs, max_bits_);
+        uint32_t *sorted_keys = nullptr, *sorted_slots = nullptr;
+        tick();
+        ND_HIP_TRY(radix_sort_pairs(plan, (const uint32_t*)d_map_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_,
+                                    d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots));
+        tock(&times.inversion);
+        times.sort_launches += plan.passes;
+        P.pair_keys = sorted_keys;
+        P.pair_slots = sorted_slots;
+        if (!balance) {
+          tick();
+          step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, nullptr);
+          tock(&times.flat_kernel);
+          times.flat_launches++;
+        } else {
+          tick();
+          ND_HIP_TRY(find_transit_runs(sorted_keys, n_pairs, (uint32_t)invalid_, d_run_key_, d_run_start_, d_meta_,
+                                       d_scratch_, stream_));
+          const unsigned max_runs = n_pairs < (uint32_t)invalid_ ? n_pairs : (uint32_t)invalid_;
+          classify_runs<<<dim3((max_runs + 255) / 256), dim3(256), 0, stream_>>>(
+              d_run_key_, d_run_start_, d_meta_, d_row_ptr_, m, d_chunks_, chunk_capacity_, d_skip_flag_);
+          tock(&times.load_balancing);
+          tick();
+          step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, d_skip_flag_);
+          tock(&times.flat_kernel);
+          times.flat_launches++;
+          tick();
+          unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
+          step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
+              P, d_chunks_, d_meta_, chunk_capacity_, d_skip_flag_);
+          tock(&times.workgroup_kernel);
+          times.workgroup_launches++;
+        }
+      }
+      ND_HIP_TRY(hipGetLastError());
+      seg_base += transits_per_sample * m;
+      transits_per_sample *= m;
+    }
+    ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
+    return 0;
+  }
+
+  // getFinalSamples: device -> hFinalSamples
+  int fetch_final_samples() override {
+    if (!allocated_) { last_error = "no device data"; return -1; }
+    ND_HIP_TRY(hipMemcpy(hFinalSamples.data(), d_final_, sizeof(VertexID_t) * hFinalSamples.size(),
+                         hipMemcpyDeviceToHost));
+    return 0;
+  }
+
+  int fetch_sample_states(void* dst, size_t bytes) override {
+    if (!allocated_ || std::is_empty<SampleType>::value) { last_error = "no sample state"; return -1; }
+    if (bytes != sample_state_bytes()) { last_error = "sample state size mismatch"; return -1; }
+    ND_HIP_TRY(hipMemcpy(dst, d_samples_, bytes, hipMemcpyDeviceToHost));
+    return 0;
+  }
+
+  void free_device() override {
+    free_run_buffers();
+    free_graph();
+  }
+
+ private:
+  void tick() {
+    if (profiling) (void)hipEventRecord(ev_a_, stream_);
+  }
+  void tock(float* acc) {
+    if (!profiling) return;
+    (void)hipEventRecord(ev_b_, stream_);
+    (void)hipEventSynchronize(ev_b_);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, ev_a_, ev_b_);
+    *acc += ms;
+  }
+
+  template <class T>
+  static void release(T*& p) {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+  }
+
+  void free_graph() {
+    release(d_row_ptr_);
+    release(d_col_);
+    release(d_weight_);
+    release(d_max_weight_);
+  }
+
+  void free_run_buffers() {
+    release(d_initial_);
+    release(d_samples_);
+    release(d_final_);
+    release(d_map_);
+    release(d_keys_a_);
+    release(d_vals_a_);
+    release(d_keys_b_);
+    release(d_vals_b_);
+    release(d_hist_);
+    release(d_scratch_);
+    release(d_run_key_);
+    release(d_run_start_);
+    release(d_meta_);
+    release(d_chunks_);
+    release(d_skip_flag_);
+    if (allocated_) {
+      (void)hipEventDestroy(ev_a_);
+      (void)hipEventDestroy(ev_b_);
+      (void)hipEventDestroy(ev_begin_);
+      (void)hipEventDestroy(ev_end_);
+      (void)hipStreamDestroy(stream_);
+    }
+    allocated_ = false;
+  }
+
+  const char* name_;
+  const CSR* graph_ = nullptr;
+  CSRPartition view_{};
+  EdgePos_t* d_row_ptr_ = nullptr;
+  VertexID* d_col_ = nullptr;
+  float* d_weight_ = nullptr;
+  float* d_max_weight_ = nullptr;
+
+  std::vector<SampleType> samples_;
+  int64_t n_samples_ = 0;
+  int init_size_ = 0;
+  int32_t invalid_ = 0;
+  int max_bits_ = 0;
+  uint64_t seed_ = 0;
+  size_t max_pairs_ = 0;
+  uint32_t chunk_capacity_ = 0;
+  bool allocated_ = false;
+
+  hipStream_t stream_ = nullptr;
+  hipEvent_t ev_a_ = nullptr, ev_b_ = nullptr, ev_begin_ = nullptr, ev_end_ = nullptr;
+  VertexID_t* d_initial_ = nullptr;
+  SampleType* d_samples_ = nullptr;
+  VertexID_t* d_final_ = nullptr;
+  int32_t* d_map_ = nullptr;
+  uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
+  uint32_t* d_hist_ = nullptr;
+  uint32_t* d_scratch_ = nullptr;
+  uint32_t* d_run_key_ = nullptr;
+  uint32_t* d_run_start_ = nullptr;
+  RunsMeta* d_meta_ = nullptr;
+  uint32_t* d_chunks_ = nullptr;
+  uint8_t* d_skip_flag_ = nullptr;
+};
+
+}  // namespace nd

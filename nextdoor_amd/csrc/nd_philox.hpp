@@ -1,0 +1,111 @@
+// Counter-based random numbers for the sampling engine (host + gfx950 device).
+//
+// Replaces the reference's per-thread-slot XORWOW states (src/nextdoor.cu:1838-1843,
+// src/rand_num_gen.cuh:117-122): 48 bytes of state per launch thread are traded for a
+// stateless Philox4x32-10 block keyed by WHAT is being sampled, so results do not depend
+// on which kernel, workgroup or lane happens to execute an output slot.
+//
+//   block(slot, step, b) = Philox4x32-10(counter = {slot_lo, slot_hi, step, b},
+//                                        key     = {seed_lo, seed_hi})
+//   draw d of (slot, step) = word (d & 3) of block(slot, step, d >> 2)
+//   uniform = (word >> 8) * 2^-24   in [0, 1)
+//
+// `slot` is the global index of the output being produced at `step`:
+// ((sample * transitsPerSample + transitIdx) * stepSize + neighbourIdx).
+#pragma once
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#include <hip/hip_runtime.h>
+#define ND_HD __host__ __device__ __forceinline__
+#else
+#define ND_HD inline
+#endif
+
+namespace nd {
+
+struct PhiloxBlock {
+  uint32_t w[4];
+};
+
+ND_HD uint32_t mul_hi_u32(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __umulhi(a, b);
+#else
+  return (uint32_t)(((uint64_t)a * (uint64_t)b) >> 32);
+#endif
+}
+
+ND_HD PhiloxBlock philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                uint32_t k0, uint32_t k1) {
+  constexpr uint32_t kMulA = 0xD2511F53u, kMulB = 0xCD9E8D57u;
+  constexpr uint32_t kWeylA = 0x9E3779B9u, kWeylB = 0xBB67AE85u;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi_a = mul_hi_u32(kMulA, c0), lo_a = kMulA * c0;
+    const uint32_t hi_b = mul_hi_u32(kMulB, c2), lo_b = kMulB * c2;
+    c0 = hi_b ^ c1 ^ k0;
+    c1 = lo_b;
+    c2 = hi_a ^ c3 ^ k1;
+    c3 = lo_a;
+    k0 += kWeylA;
+    k1 += kWeylB;
+  }
+  PhiloxBlock out;
+  out.w[0] = c0; out.w[1] = c1; out.w[2] = c2; out.w[3] = c3;
+  return out;
+}
+
+ND_HD float u32_to_unit_float(uint32_t word) {
+  return (float)(word >> 8) * 5.9604644775390625e-08f;  // 2^-24, exact
+}
+
+// Cursor over the draws of one (slot, step).  This is the object an App's next()
+// receives as its random-state handle.
+struct RandState {
+  uint32_t slot_lo, slot_hi, step, draw;
+  uint32_t key0, key1;
+  PhiloxBlock cache;
+
+  ND_HD void reset(uint64_t seed, uint64_t slot, uint32_t step_) {
+    slot_lo = (uint32_t)slot;
+    slot_hi = (uint32_t)(slot >> 32);
+    step = step_;
+    draw = 0;
+    key0 = (uint32_t)seed;
+    key1 = (uint32_t)(seed >> 32);
+  }
+
+  ND_HD uint32_t next_word() {
+    const uint32_t lane = draw & 3u;
+    if (lane == 0) cache = philox4x32_10(slot_lo, slot_hi, step, draw >> 2, key0, key1);
+    ++draw;
+    // select without dynamic register indexing
+    uint32_t word = cache.w[0];
+    word = lane == 1 ? cache.w[1] : word;
+    word = lane == 2 ? cache.w[2] : word;
+    word = lane == 3 ? cache.w[3] : word;
+    return word;
+  }
+
+  ND_HD float next_uniform() { return u32_to_unit_float(next_word()); }
+};
+
+// One-shot form used by fills and host code.
+ND_HD float uniform_at(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw) {
+  PhiloxBlock b = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, draw >> 2,
+                                (uint32_t)seed, (uint32_t)(seed >> 32));
+  return u32_to_unit_float(b.w[draw & 3u]);
+}
+
+// min((int)(u * n), n - 1): the reference's RandNumGen::rand_int
+// (src/rand_num_gen.cuh:117-122) with u in [0,1).  The clamp still matters: u * n
+// rounds up to n for u = 1 - 2^-24 and large n.
+ND_HD int32_t rand_int_from_uniform(float u, int32_t n) {
+  const float scaled = u * (float)n;
+  const int32_t id = (int32_t)scaled;
+  return id < n - 1 ? id : n - 1;
+}
+
+}  // namespace nd

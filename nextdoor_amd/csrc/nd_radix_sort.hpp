@@ -1,0 +1,207 @@
+// Sample -> transit inversion: stable LSD radix sort of (transit vertex, slot) pairs.
+//
+// Takes the place of cub::DeviceRadixSort::SortPairs in the reference's step loop
+// (src/nextdoor.cu:2924-2939; key width maxBits from 1993-1999): keys are transit vertex
+// ids in [0, V] (V = INVALID_VERTEX sorts last), only the low `key_bits` bits are sorted.
+// The value is the SLOT of the pair in the unsorted map (sample * transitsPerSample + j),
+// not the sample id, so the step kernels can place outputs without atomics; on the first
+// pass the values are generated from the index instead of being read.
+//
+// Per 8-bit digit pass: (1) per-tile digit histogram, (2) exclusive scan of the
+// digit-major histogram table, (3) scatter.  The scatter ranks keys inside a tile with
+// wave64 ballots (match-any on the digit), keeps one running counter per wave and digit in
+// LDS, stages the tile digit-sorted in LDS and writes runs of equal digits to HBM.
+// No spinning, no inter-workgroup waiting.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "nd_device_scan.hpp"
+
+namespace nd {
+
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSortItems = 16;
+constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs per workgroup
+constexpr int kRadixBits = 8;
+constexpr int kRadix = 1 << kRadixBits;
+constexpr uint32_t kPadKey = 0xFFFFFFFFu;  // never a real key: keys are <= V < 2^31
+
+// Element `it` of lane `lane` in wave `wave` sits at this offset inside the tile: each
+// wave owns a contiguous chunk and reads it 64 keys (256 B) at a time, so the order
+// (wave, it, lane) is the input order and one running counter per wave keeps it stable.
+__device__ __forceinline__ int tile_offset(int wave, int it, int lane) {
+  return wave * (kWave * kSortItems) + it * kWave + lane;
+}
+
+__global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* __restrict__ keys, size_t n, int shift,
+                                                                uint32_t mask, uint32_t* __restrict__ hist,
+                                                                uint32_t num_tiles) {
+  __shared__ uint32_t s_hist[kRadix];
+  s_hist[threadIdx.x] = 0;
+  __syncthreads();
+  const size_t tile_start = (size_t)blockIdx.x * kSortTile;
+#pragma unroll
+  for (int it = 0; it < kSortItems; ++it) {
+    const size_t idx = tile_start + (size_t)it * kSortThreads + threadIdx.x;
+    if (idx < n) atomicAdd(&s_hist[(keys[idx] >> shift) & mask], 1u);
+  }
+  __syncthreads();
+  if (threadIdx.x <= mask) hist[(size_t)threadIdx.x * num_tiles + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+template <bool kIotaValues>
+__global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __restrict__ keys_in,
+                                                              const uint32_t* __restrict__ vals_in,
+                                                              uint32_t* __restrict__ keys_out,
+                                                              uint32_t* __restrict__ vals_out, size_t n, int shift,
+                                                              uint32_t mask, int digit_bits,
+                                                              const uint32_t* __restrict__ scanned_hist,
+                                                              uint32_t num_tiles) {
+  __shared__ uint32_t s_keys[kSortTile];
+  __shared__ uint32_t s_vals[kSortTile];
+  __shared__ uint32_t s_wave_count[kSortWaves][kRadix];
+  __shared__ uint32_t s_digit_base[kRadix];
+  __shared__ uint32_t s_global_base[kRadix];
+  __shared__ uint32_t s_scan_tmp[kSortWaves];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const size_t tile_start = (size_t)blockIdx.x * kSortTile;
+  const uint32_t in_tile = (uint32_t)((n - tile_start) < (size_t)kSortTile ? (n - tile_start) : (size_t)kSortTile);
+
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) s_wave_count[w][tid] = 0;
+  __syncthreads();
+
+  uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
+#pragma unroll
+  for (int it = 0; it < kSortItems; ++it) {
+    const uint32_t off = (uint32_t)tile_offset(wave, it, lane);
+    const bool live = off < in_tile;
+    key[it] = live ? keys_in[tile_start + off] : kPadKey;
+    if (kIotaValues) val[it] = (uint32_t)(tile_start + off);
+    else val[it] = live ? vals_in[tile_start + off] : 0u;
+  }
+
+  const uint64_t lanes_below = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int it = 0; it < kSortItems; ++it) {
+    const uint32_t digit = (key[it] >> shift) & mask;
+    // peers = lanes of this wave holding the same digit
+    uint64_t peers = ~0ull;
+    for (int b = 0; b < digit_bits; ++b) {
+      const bool bit = (digit >> b) & 1u;
+      const uint64_t vote = __ballot(bit);
+      peers &= bit ? vote : ~vote;
+    }
+    const int leader = __ffsll((unsigned long long)peers) - 1;
+    uint32_t before = 0;
+    if (lane == leader) before = atomicAdd(&s_wave_count[wave][digit], (uint32_t)__popcll(peers));
+    before = __shfl(before, leader, kWave);
+    rank[it] = before + (uint32_t)__popcll(peers & lanes_below);
+  }
+  __syncthreads();
+
+  // per digit: turn the per-wave counts into exclusive prefixes over waves, then scan
+  // the tile totals over digits.
+  uint32_t digit_total = 0;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) {
+    const uint32_t c = s_wave_count[w][tid];
+    s_wave_count[w][tid] = digit_total;
+    digit_total += c;
+  }
+  uint32_t tile_total;
+  const uint32_t digit_base = block_exclusive_scan_256(digit_total, s_scan_tmp, &tile_total);
+  s_digit_base[tid] = digit_base;
+  if ((uint32_t)tid <= mask) s_global_base[tid] = scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
+  __syncthreads();
+
+#pragma unroll
+  for (int it = 0; it < kSortItems; ++it) {
+    const uint32_t digit = (key[it] >> shift) & mask;
+    const uint32_t pos = s_digit_base[digit] + s_wave_count[wave][digit] + rank[it];
+    s_keys[pos] = key[it];
+    s_vals[pos] = val[it];
+  }
+  __syncthreads();
+
+  // pad keys carry the largest digit and come last in input order, so the live keys
+  // occupy positions [0, in_tile)
+  for (uint32_t p = tid; p < in_tile; p += kSortThreads) {
+    const uint32_t k = s_keys[p];
+    const uint32_t out = s_global_base[(k >> shift) & mask] + p;
+    keys_out[out] = k;
+    vals_out[out] = s_vals[p];
+  }
+}
+
+struct SortPlan {
+  size_t n = 0;
+  int key_bits = 0;
+  int passes = 0;
+  uint32_t num_tiles = 0;
+  size_t hist_elems = 0;     // kRadix * num_tiles
+  size_t scratch_elems = 0;  // scan scratch
+};
+
+inline SortPlan make_sort_plan(size_t n, int key_bits) {
+  SortPlan p;
+  p.n = n;
+  p.key_bits = key_bits < 1 ? 1 : key_bits;
+  p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
+  p.num_tiles = (uint32_t)((n + kSortTile - 1) / kSortTile);
+  p.hist_elems = (size_t)kRadix * p.num_tiles;
+  p.scratch_elems = scan_scratch_elems(p.hist_elems);
+  return p;
+}
+
+// Sorts n pairs by the low key_bits bits of the key.  keys_in is not modified.
+// vals_in == nullptr means "value = index".  Two ping-pong buffer pairs (a, b) of n
+// elements each; the result lands in *keys_sorted / *vals_sorted (one of a / b).
+// hist needs plan.hist_elems and scratch plan.scratch_elems uint32.
+inline hipError_t radix_sort_pairs(const SortPlan& plan, const uint32_t* keys_in, const uint32_t* vals_in,
+                                   uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
+                                   uint32_t* hist, uint32_t* scratch, hipStream_t stream,
+                                   uint32_t** keys_sorted, uint32_t** vals_sorted) {
+  *keys_sorted = keys_a;
+  *vals_sorted = vals_a;
+  if (plan.n == 0) return hipSuccess;
+  // digits as even as possible: 23 bits -> 8, 8, 7
+  const uint32_t* src_k = keys_in;
+  const uint32_t* src_v = vals_in;
+  uint32_t* dst_k = keys_a;
+  uint32_t* dst_v = vals_a;
+  int shift = 0;
+  for (int pass = 0; pass < plan.passes; ++pass) {
+    const int remaining = plan.key_bits - shift;
+    const int passes_left = plan.passes - pass;
+    const int bits = (remaining + passes_left - 1) / passes_left;
+    const uint32_t mask = (1u << bits) - 1u;
+    const size_t table = ((size_t)mask + 1) * plan.num_tiles;
+    radix_histogram<<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(src_k, plan.n, shift, mask, hist,
+                                                                            plan.num_tiles);
+    hipError_t e = exclusive_scan_u32(hist, hist, table, scratch, stream);
+    if (e != hipSuccess) return e;
+    if (pass == 0 && src_v == nullptr)
+      radix_scatter<true><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
+          src_k, nullptr, dst_k, dst_v, plan.n, shift, mask, bits, hist, plan.num_tiles);
+    else
+      radix_scatter<false><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
+          src_k, src_v, dst_k, dst_v, plan.n, shift, mask, bits, hist, plan.num_tiles);
+    *keys_sorted = dst_k;
+    *vals_sorted = dst_v;
+    src_k = dst_k;
+    src_v = dst_v;
+    if (dst_k == keys_a) { dst_k = keys_b; dst_v = vals_b; }
+    else { dst_k = keys_a; dst_v = vals_a; }
+    shift += bits;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace nd

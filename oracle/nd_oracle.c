@@ -1,0 +1,503 @@
+/*
+ * CPU oracle for the transit-parallel sampling path.  TEST INFRASTRUCTURE ONLY:
+ * see nd_oracle.h.  Plain C, compiled with -ffp-contract=off so that every float
+ * operation is the single IEEE operation written here.
+ */
+#include "nd_oracle.h"
+
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* Philox4x32-10                                                              */
+/* ------------------------------------------------------------------------- */
+
+void ndo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  /* multipliers and Weyl key increments as published for philox4x32 */
+  const uint64_t mul_a = 0xD2511F53u, mul_b = 0xCD9E8D57u;
+  const uint32_t weyl_a = 0x9E3779B9u, weyl_b = 0xBB67AE85u;
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+  uint32_t k0 = key[0], k1 = key[1];
+  for (int round = 0; round < 10; ++round) {
+    uint64_t pa = mul_a * (uint64_t)c0;
+    uint64_t pb = mul_b * (uint64_t)c2;
+    uint32_t n0 = (uint32_t)(pb >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)pb;
+    uint32_t n2 = (uint32_t)(pa >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)pa;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += weyl_a; k1 += weyl_b;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+float ndo_uniform(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw) {
+  uint32_t ctr[4] = {(uint32_t)slot, (uint32_t)(slot >> 32), step, draw >> 2};
+  uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  uint32_t out[4];
+  ndo_philox4x32_10(ctr, key, out);
+  return (float)(out[draw & 3u] >> 8) * 5.9604644775390625e-08f; /* 2^-24 */
+}
+
+int32_t ndo_rand_int(float u, int32_t n) {
+  /* rand_num_gen.cuh:118-121: ff = u * n (float multiply, n converted to float),
+   * id = min((EdgePos_t)ff, n-1) */
+  float ff = u * (float)n;
+  int32_t id = (int32_t)ff;
+  return id < n - 1 ? id : n - 1;
+}
+
+/* A cursor over the draws of one (slot, step): what the device RandState is. */
+typedef struct {
+  uint64_t seed, slot;
+  uint32_t step, draw;
+  ndo_stats* st;
+} rng_cursor;
+
+static float next_uniform(rng_cursor* c) {
+  float u = ndo_uniform(c->seed, c->slot, c->step, c->draw);
+  c->draw++;
+  if (c->st) c->st->draws++;
+  return u;
+}
+
+static int32_t next_int(rng_cursor* c, int32_t n) { return ndo_rand_int(next_uniform(c), n); }
+
+/* ------------------------------------------------------------------------- */
+/* Shape algebra                                                              */
+/* ------------------------------------------------------------------------- */
+
+int ndo_is_collective(const ndo_app_desc* app) {
+  return app->kind == NDO_LAYER_LITERAL || app->kind == NDO_FASTGCN_IMPORTANCE ||
+         app->kind == NDO_LADIES_IMPORTANCE;
+}
+
+int64_t ndo_step_size_at_step(const ndo_app_desc* app, int step) {
+  /* nextdoor.cu:162-186 */
+  if (step == -1) return 0;
+  if (!ndo_is_collective(app)) {
+    int64_t n = app->initial_size;
+    for (int i = 0; i <= step; ++i) n *= app->step_size[i];
+    return n;
+  }
+  int64_t n = 0;
+  for (int i = 0; i <= step; ++i) n += app->step_size[i];
+  return n;
+}
+
+int64_t ndo_number_of_transits(const ndo_app_desc* app, int step) {
+  /* nextdoor.cu:188-197 */
+  if (ndo_is_collective(app)) return app->step_size[step];
+  return ndo_step_size_at_step(app, step);
+}
+
+int64_t ndo_sub_warp_size_at_step(const ndo_app_desc* app, int step) {
+  /* nextdoor.cu:133-160: next power of two >= stepSize(step) */
+  if (step == -1) return 0;
+  int64_t x = app->step_size[step];
+  int64_t w = 1;
+  while (w < x) w <<= 1;
+  return w;
+}
+
+int64_t ndo_final_sample_size(const ndo_app_desc* app) {
+  /* nextdoor.cu:1913-1929 */
+  int64_t total = 0, per_step = 1;
+  for (int k = 0; k < app->steps; ++k) {
+    if (ndo_is_collective(app)) per_step = app->step_size[k];
+    else per_step *= app->step_size[k];
+    total += per_step;
+  }
+  return total;
+}
+
+int ndo_max_bits(int32_t n_vertices) {
+  /* nextdoor.cu:1993-1999 with INVALID_VERTEX = n_vertices */
+  int bits = 0;
+  while (((int64_t)n_vertices >> bits) != 0) bits++;
+  return bits;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Graph accessors                                                            */
+/* ------------------------------------------------------------------------- */
+
+static inline int32_t degree_of(const ndo_graph* g, int32_t v) { return g->row_ptr[v + 1] - g->row_ptr[v]; }
+
+/* utils::binarySearch (utils.hpp:30-48) */
+static int sorted_contains(const int32_t* a, int32_t x, int32_t n, ndo_stats* st) {
+  int32_t l = 0, r = n - 1;
+  while (l <= r) {
+    int32_t m = l + (r - l) / 2;
+    if (st) st->search_probes++;
+    if (a[m] == x) return 1;
+    if (a[m] < x) l = m + 1; else r = m - 1;
+  }
+  return 0;
+}
+
+int ndo_has_edge(const ndo_graph* g, int32_t src, int32_t dst) {
+  return sorted_contains(g->col + g->row_ptr[src], dst, degree_of(g, src), 0);
+}
+
+/* ------------------------------------------------------------------------- */
+/* next() of the IndividualNeighborhood apps                                  */
+/* ------------------------------------------------------------------------- */
+
+static int32_t next_individual(const ndo_graph* g, const ndo_app_desc* app, int step, int32_t transit,
+                               int32_t* t_state, rng_cursor* rc) {
+  ndo_stats* st = rc->st;
+  const int32_t n = degree_of(g, transit);
+  const int32_t* edges = g->col + g->row_ptr[transit];
+  const float* weights = g->weight + g->row_ptr[transit];
+  const float max_w = g->max_weight[transit];
+  if (st) st->next_calls++;
+
+  switch (app->kind) {
+    case NDO_UNIFORM_WALK: {
+      /* example/uniformRandWalk.cu:35-36 (never called with n == 0: nextdoor.cu:257) */
+      int32_t x = next_int(rc, n);
+      if (st) st->edge_reads++;
+      return edges[x];
+    }
+    case NDO_KHOP: {
+      /* khop.cu:18-22 */
+      if (n == 0) return -1;
+      int32_t x = next_int(rc, n);
+      if (st) st->edge_reads++;
+      return edges[x];
+    }
+    case NDO_DEEPWALK:
+    case NDO_PPR: {
+      if (n == 0) return -1;
+      if (app->kind == NDO_PPR) {
+        /* randomWalks.cu:105-109 */
+        float stop = next_uniform(rc);
+        if (stop < 0.01f) return -1;
+      }
+      if (n == 1) { if (st) st->edge_reads++; return edges[0]; }
+      /* randomWalks.cu:81-88: rejection against the vertex's max edge weight */
+      int32_t x = next_int(rc, n);
+      float y = next_uniform(rc) * max_w;
+      if (st) st->weight_reads++;
+      while (y > weights[x]) {
+        x = next_int(rc, n);
+        y = next_uniform(rc) * max_w;
+        if (st) st->weight_reads++;
+      }
+      if (st) st->edge_reads++;
+      return edges[x];
+    }
+    case NDO_NODE2VEC: {
+      /* randomWalks.cu:141-172, literally: the return-edge test compares the edge
+       * INDEX x with the vertex id t (randomWalks.cu:159). */
+      if (n == 0) return -1;
+      if (n == 1 || step == 0) { *t_state = transit; if (st) st->edge_reads++; return edges[0]; }
+      const float p = app->p, q = app->q;
+      float envelope = p > 1.0f / q ? p : 1.0f / q;
+      if (envelope < 1.0f) envelope = 1.0f;
+      for (;;) {
+        int32_t x = next_int(rc, n);
+        int32_t v = edges[x];
+        if (st) st->edge_reads++;
+        float y = next_uniform(rc) * envelope;
+        int32_t t = *t_state;
+        float h;
+        if (x == t) h = p;
+        else if (sorted_contains(g->col + g->row_ptr[t], v, degree_of(g, t), st)) h = 1.0f / q;
+        else h = 1.0f;
+        if (y < h) { *t_state = transit; return v; }
+      }
+    }
+    case NDO_WEIGHTED_NODE2VEC: {
+      /* Own definition (the reference has no weighted node2vec): second-order bias h
+       * as above but with the return test on the VERTEX (v == t), multiplied by the
+       * edge weight, rejected against max_weight * max(p, 1/q, 1).  Step 0 has no
+       * previous vertex: h = 1, i.e. a DeepWalk step. */
+      if (n == 0) return -1;
+      if (n == 1) { *t_state = transit; if (st) st->edge_reads++; return edges[0]; }
+      const float p = app->p, q = app->q;
+      float hmax = p > 1.0f / q ? p : 1.0f / q;
+      if (hmax < 1.0f) hmax = 1.0f;
+      const float envelope = max_w * hmax;
+      for (;;) {
+        int32_t x = next_int(rc, n);
+        int32_t v = edges[x];
+        float wx = weights[x];
+        if (st) { st->edge_reads++; st->weight_reads++; }
+        float y = next_uniform(rc) * envelope;
+        float h;
+        if (step == 0) h = 1.0f;
+        else {
+          int32_t t = *t_state;
+          if (v == t) h = p;
+          else if (sorted_contains(g->col + g->row_ptr[t], v, degree_of(g, t), st)) h = 1.0f / q;
+          else h = 1.0f;
+        }
+        if (y < h * wx) { *t_state = transit; return v; }
+      }
+    }
+    default:
+      return -1;
+  }
+}
+
+int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                          int64_t n_samples, int64_t first_sample,
+                          const int32_t* initial, int32_t* final_samples,
+                          int32_t* state_t, ndo_stats* stats, int n_threads) {
+  if (ndo_is_collective(app) || app->steps <= 0 || app->steps > NDO_MAX_STEPS) return -1;
+  const int32_t invalid = g->n_vertices;
+  const int64_t F = ndo_final_sample_size(app);
+  const int init = app->initial_size;
+  if (stats) memset(stats, 0, sizeof(*stats));
+  if (n_threads < 1) n_threads = 1;
+
+  ndo_stats* per_thread = (ndo_stats*)calloc((size_t)n_threads, sizeof(ndo_stats));
+  if (!per_thread) return -2;
+
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 256) num_threads(n_threads)
+#endif
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int tid = 0;
+#ifdef _OPENMP
+    tid = omp_get_thread_num();
+#endif
+    ndo_stats* st = stats ? &per_thread[tid] : 0;
+    int32_t* out = final_samples + s * F;
+    int32_t t_state = -1;
+    const int32_t* prev = initial + s * init;  /* transits of step k */
+    int64_t T = init;                          /* numberOfTransits of step k-1 / transits per sample */
+    int64_t seg_base = 0;
+    for (int k = 0; k < app->steps; ++k) {
+      const int m = app->step_size[k];
+      int32_t* seg = out + seg_base;
+      for (int64_t j = 0; j < T; ++j) {
+        const int32_t transit = prev[j];
+        for (int nbr = 0; nbr < m; ++nbr) {
+          int32_t neighbor = invalid;
+          /* nextdoor.cu:250-262: next() only runs for a valid transit with edges */
+          if (transit != invalid && transit != -1 && degree_of(g, transit) != 0) {
+            rng_cursor rc;
+            rc.seed = seed;
+            rc.slot = (uint64_t)(((first_sample + s) * T + j) * m + nbr);
+            rc.step = (uint32_t)k;
+            rc.draw = 0;
+            rc.st = st;
+            int32_t r = next_individual(g, app, k, transit, &t_state, &rc);
+            neighbor = (r == -1) ? invalid : r;  /* nextdoor.cu:288 */
+          }
+          seg[j * m + nbr] = neighbor;
+          if (st && neighbor != invalid) st->valid_outputs++;
+        }
+      }
+      prev = seg;
+      seg_base += T * m;
+      T *= m;
+    }
+    if (state_t) state_t[s] = t_state;
+  }
+
+  if (stats) {
+    for (int i = 0; i < n_threads; ++i) {
+      stats->next_calls += per_thread[i].next_calls;
+      stats->draws += per_thread[i].draws;
+      stats->search_probes += per_thread[i].search_probes;
+      stats->valid_outputs += per_thread[i].valid_outputs;
+      stats->edge_reads += per_thread[i].edge_reads;
+      stats->weight_reads += per_thread[i].weight_reads;
+    }
+  }
+  free(per_thread);
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Inversion / RLE / scan / binning                                           */
+/* ------------------------------------------------------------------------- */
+
+void ndo_sort_pairs(const int32_t* keys_in, const int32_t* vals_in, int64_t n,
+                    int32_t* keys_out, int32_t* vals_out) {
+  /* stable counting-free merge sort on indices: simple and obviously stable */
+  if (n <= 0) return;
+  int64_t* idx = (int64_t*)malloc(sizeof(int64_t) * (size_t)n);
+  int64_t* tmp = (int64_t*)malloc(sizeof(int64_t) * (size_t)n);
+  for (int64_t i = 0; i < n; ++i) idx[i] = i;
+  for (int64_t width = 1; width < n; width *= 2) {
+    for (int64_t lo = 0; lo < n; lo += 2 * width) {
+      int64_t mid = lo + width < n ? lo + width : n;
+      int64_t hi = lo + 2 * width < n ? lo + 2 * width : n;
+      int64_t a = lo, b = mid, o = lo;
+      while (a < mid && b < hi) {
+        /* take from the left run on ties: stability */
+        if ((uint32_t)keys_in[idx[b]] < (uint32_t)keys_in[idx[a]]) tmp[o++] = idx[b++];
+        else tmp[o++] = idx[a++];
+      }
+      while (a < mid) tmp[o++] = idx[a++];
+      while (b < hi) tmp[o++] = idx[b++];
+    }
+    int64_t* sw = idx; idx = tmp; tmp = sw;
+  }
+  for (int64_t i = 0; i < n; ++i) {
+    keys_out[i] = keys_in[idx[i]];
+    vals_out[i] = vals_in[idx[i]];
+  }
+  free(idx);
+  free(tmp);
+}
+
+int64_t ndo_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid,
+                            int32_t* uniq, int32_t* counts, int32_t* offsets,
+                            int64_t* n_valid) {
+  /* invalidVertexStartPos (nextdoor.cu:1804-1836) + RunLengthEncode (2535-2545)
+   * + ExclusiveSum (2560-2567) */
+  int64_t valid = 0;
+  while (valid < n && sorted_keys[valid] != invalid) valid++;
+  if (n_valid) *n_valid = valid;
+  int64_t runs = 0;
+  for (int64_t i = 0; i < valid;) {
+    int64_t j = i;
+    while (j < valid && sorted_keys[j] == sorted_keys[i]) j++;
+    uniq[runs] = sorted_keys[i];
+    counts[runs] = (int32_t)(j - i);
+    offsets[runs] = (int32_t)i;
+    runs++;
+    i = j;
+  }
+  return runs;
+}
+
+int ndo_kernel_class(int64_t count, int64_t sub_warp_size) {
+  int64_t work = count * sub_warp_size;
+  if (work >= 256) return 1;
+  if (work >= 32) return 2;
+  if (work >= 8) return 3;
+  return 4;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Distinct                                                                   */
+/* ------------------------------------------------------------------------- */
+
+static int cmp_i32(const void* a, const void* b) {
+  int32_t x = *(const int32_t*)a, y = *(const int32_t*)b;
+  return (x > y) - (x < y);
+}
+
+void ndo_distinct(const ndo_app_desc* app, int64_t n_samples, int32_t invalid,
+                  int32_t* final_samples, int32_t* counts) {
+  const int64_t F = ndo_final_sample_size(app);
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int64_t base = 0;
+    for (int k = 0; k < app->steps; ++k) {
+      int64_t len = ndo_step_size_at_step(app, k);
+      int32_t* seg = final_samples + s * F + base;
+      /* invalid == n_vertices is larger than every vertex id, so it sorts last */
+      qsort(seg, (size_t)len, sizeof(int32_t), cmp_i32);
+      int64_t kept = 0;
+      for (int64_t i = 0; i < len; ++i) {
+        if (seg[i] == invalid) break;
+        if (kept == 0 || seg[kept - 1] != seg[i]) seg[kept++] = seg[i];
+      }
+      for (int64_t i = kept; i < len; ++i) seg[i] = invalid;
+      if (counts) counts[s * app->steps + k] = (int32_t)kept;
+      base += len;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Validators                                                                 */
+/* ------------------------------------------------------------------------- */
+
+/* numNeighborsSampledAtStep (check_results.cu:4-29), as written */
+static int64_t neighbors_sampled_at_step(const ndo_app_desc* app, int step) {
+  if (step < 0) return 0;
+  int64_t n = app->step_size[0];
+  for (int i = 1; i <= step; ++i) {
+    if (app->step_size[i] == 1) n += app->step_size[i];
+    else n += n * app->step_size[i];
+  }
+  return n;
+}
+
+int ndo_check_sampled_vertices(const ndo_graph* g, const ndo_app_desc* app,
+                               int64_t n_samples, const int32_t* initial,
+                               const int32_t* final_samples, int32_t invalid, int n_threads) {
+  const int64_t F = ndo_final_sample_size(app);
+  const int max_steps = 4; /* check_results.cu:173 */
+  const int steps = app->steps < max_steps ? app->steps : max_steps;
+  int ok = 1;
+  if (n_threads < 1) n_threads = 1;
+  for (int step = 0; step < steps; ++step) {
+    int bad = 0;
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(n_threads) reduction(| : bad)
+#endif
+    for (int64_t s = 0; s < n_samples; ++s) {
+      const int32_t* fs = final_samples + s * F;
+      if (step == 0) {
+        /* check_results.cu:185-232 (fixed step sizes only) */
+        const int32_t root = initial[s]; /* literal: initialSamples[sampleId] */
+        int64_t valid = 0;
+        for (int64_t v = 0; v < app->step_size[0]; ++v) {
+          int32_t x = fs[v];
+          if (x != invalid) {
+            valid++;
+            if (!ndo_has_edge(g, root, x)) bad |= 1;
+          }
+        }
+        if (valid == 0 && degree_of(g, root) > 0) bad |= 1;
+      } else {
+        /* check_results.cu:234-291 */
+        const int64_t prev_lo = neighbors_sampled_at_step(app, step - 2);
+        const int64_t prev_hi = neighbors_sampled_at_step(app, step - 1);
+        const int64_t cur_hi = (step == app->steps - 1) ? F : neighbors_sampled_at_step(app, step);
+        int64_t prev_edges = 0, valid = 0;
+        for (int64_t v = prev_lo; v < prev_hi; ++v)
+          if (fs[v] != invalid) prev_edges += degree_of(g, fs[v]);
+        for (int64_t v = prev_hi; v < cur_hi; ++v) {
+          int32_t x = fs[v];
+          if (x == invalid) continue;
+          valid++;
+          int found = 0;
+          for (int64_t v1 = prev_lo; v1 < prev_hi && !found; ++v1)
+            if (fs[v1] != invalid && ndo_has_edge(g, fs[v1], x)) found = 1;
+          if (!found) bad |= 1;
+        }
+        if (valid == 0 && prev_edges > 0) bad |= 1;
+      }
+    }
+    if (bad) { ok = 0; break; }
+  }
+  return ok;
+}
+
+int ndo_check_exact_transits(const ndo_graph* g, const ndo_app_desc* app,
+                             int64_t n_samples, const int32_t* initial,
+                             const int32_t* final_samples, int32_t invalid) {
+  const int64_t F = ndo_final_sample_size(app);
+  for (int64_t s = 0; s < n_samples; ++s) {
+    const int32_t* prev = initial + s * app->initial_size;
+    int64_t T = app->initial_size, base = 0;
+    for (int k = 0; k < app->steps; ++k) {
+      const int m = app->step_size[k];
+      const int32_t* seg = final_samples + s * F + base;
+      for (int64_t j = 0; j < T; ++j)
+        for (int nbr = 0; nbr < m; ++nbr) {
+          int32_t x = seg[j * m + nbr];
+          if (x < 0 || x > invalid) return 0;
+          if (x == invalid) continue;
+          if (prev[j] == invalid || !ndo_has_edge(g, prev[j], x)) return 0;
+        }
+      prev = seg;
+      base += T * m;
+      T *= m;
+    }
+  }
+  return 1;
+}

@@ -1,0 +1,157 @@
+/*
+ * CPU oracle for the transit-parallel sampling path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This is a plain-C restatement of the sampler semantics of plasma-umass/NextDoor
+ * (file:line citations are relative to the reference checkout) evaluated the
+ * obvious way: one sample after the other, one transit after the other.  It is
+ * the checker for the HIP engine; nothing that ships may link, import or call it.
+ * Only tests, the smoke check and the cpu_baseline leg of the benchmark use it.
+ *
+ * Parity status of each function is stated next to its declaration:
+ *   "pinned by ..."     - an independent check exists in tests/ (KAT, closed form,
+ *                         brute force, special case reducing to a library routine)
+ *   "parity unpinned"   - semantics are this repo's own definition; the reference
+ *                         holds no vector or test for it.
+ */
+#ifndef ND_ORACLE_H
+#define ND_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NDO_MAX_STEPS 128
+
+/* App identifiers (the structs under src/apps and example/ of the reference). */
+enum ndo_app_kind {
+  NDO_UNIFORM_WALK = 0,      /* example/uniformRandWalk.cu:27-37            */
+  NDO_DEEPWALK = 1,          /* src/apps/randomwalks/randomWalks.cu:65-91   */
+  NDO_PPR = 2,               /* src/apps/randomwalks/randomWalks.cu:93-125  */
+  NDO_NODE2VEC = 3,          /* src/apps/randomwalks/randomWalks.cu:132-173 */
+  NDO_WEIGHTED_NODE2VEC = 4, /* this repo's weighted variant; parity unpinned */
+  NDO_KHOP = 5,              /* src/apps/khop/khop.cu:10-23                 */
+  NDO_LAYER_LITERAL = 6,     /* src/apps/fastgcn/fastgcnSampling.cu:23-47 and
+                                src/apps/ladies/ladiessampling.cu:23-47 (identical bodies) */
+  NDO_FASTGCN_IMPORTANCE = 7,/* this repo's degree^2 importance sampler; parity unpinned */
+  NDO_LADIES_IMPORTANCE = 8  /* this repo's column-norm^2 sampler; parity unpinned */
+};
+
+typedef struct {
+  int32_t n_vertices;
+  int64_t n_edges;
+  const int32_t* row_ptr;    /* [n_vertices+1]; adjacency of v is col[row_ptr[v] .. row_ptr[v+1]) */
+  const int32_t* col;        /* sorted ascending by (dst, weight) per vertex, duplicates kept (graph.hpp:38,156) */
+  const float* weight;
+  const float* max_weight;   /* [n_vertices]; max(0, weights of v) (graph.hpp:71-80) */
+} ndo_graph;
+
+typedef struct {
+  int kind;                       /* enum ndo_app_kind */
+  int steps;                      /* App::steps() */
+  int step_size[NDO_MAX_STEPS];   /* App::stepSize(k) */
+  int initial_size;               /* App::initialSampleSize() */
+  float p, q;                     /* node2vec parameters (reference hard-codes 2.0 / 0.5) */
+} ndo_app_desc;
+
+typedef struct {
+  int64_t next_calls;     /* times the app's next() ran */
+  int64_t draws;          /* uniform variates consumed */
+  int64_t search_probes;  /* binary-search loop iterations */
+  int64_t valid_outputs;  /* output slots != INVALID (reference: totalSampledVertices, nextdoor.cu:3284-3299) */
+  int64_t edge_reads;     /* neighbour-id loads */
+  int64_t weight_reads;   /* edge-weight loads */
+} ndo_stats;
+
+/* ---- random numbers (replaces cuRAND XORWOW; rand_num_gen.cuh:117-122) ---- */
+
+/* Philox4x32-10 block function (Salmon et al., SC'11; Random123 1.09).
+ * pinned by the Random123 known-answer vectors in tests/test_oracle_philox.py. */
+void ndo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+
+/* The draw-th uniform of (slot, step): word (draw & 3) of the block with counter
+ * (slot_lo, slot_hi, step, draw >> 2) and key (seed_lo, seed_hi), mapped to [0,1) as
+ * (word >> 8) * 2^-24.  pinned by KAT + range/closed-form tests. */
+float ndo_uniform(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw);
+
+/* RandNumGen::rand_int (rand_num_gen.cuh:117-122): min((int)(u*n), n-1) in float.
+ * pinned by closed-form cases incl. the u*n == n rounding case. */
+int32_t ndo_rand_int(float u, int32_t n);
+
+/* ---- shape algebra (nextdoor.cu:126-197, 1913-1929) ---- */
+int64_t ndo_step_size_at_step(const ndo_app_desc* app, int step);    /* stepSizeAtStep   */
+int64_t ndo_number_of_transits(const ndo_app_desc* app, int step);   /* numberOfTransits */
+int64_t ndo_sub_warp_size_at_step(const ndo_app_desc* app, int step);/* subWarpSizeAtStep */
+int64_t ndo_final_sample_size(const ndo_app_desc* app);              /* getFinalSampleSize */
+int ndo_is_collective(const ndo_app_desc* app);
+int ndo_max_bits(int32_t n_vertices);                                /* nextdoor.cu:1993-1999 */
+
+/* ---- IndividualNeighborhood sampling (walks, k-hop) ----
+ * Step semantics: samplingKernel nextdoor.cu:212-336; output layout: step-k segment
+ * starts at sum_{i<k} (outputs of step i per sample); inside it slot j*m_k + nbr holds
+ * the nbr-th neighbour drawn for the j-th transit (the j-th entry of the step k-1
+ * segment; roots for k = 0).  The reference places entries inside a segment with an
+ * atomic cursor (nextdoor.cu:304,473), i.e. in no fixed order; this canonical order
+ * is one of the orders it can produce.  RNG slot of that output:
+ * ((first_sample + s) * T_k + j) * m_k + nbr.
+ * final[n_samples * F] is fully written (INVALID = n_vertices where nothing was sampled).
+ * state_t (may be NULL): Node2VecSample::t per sample after the last step.
+ * Uniform/k-hop: pinned by closed forms on path/star/complete graphs;
+ * DeepWalk: pinned by equal-weight reduction + chi-square; Node2Vec literal: pinned by
+ * hand-traced cases; weighted node2vec: parity unpinned (own definition) beyond
+ * distribution checks. */
+int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                          int64_t n_samples, int64_t first_sample,
+                          const int32_t* initial, int32_t* final_samples,
+                          int32_t* state_t, ndo_stats* stats, int n_threads);
+
+/* ---- inversion, run-length encode, scan, binning (nextdoor.cu:2924-2939, 2529-2572,
+ *      1520-1802; utils.hpp:491-497) ---- */
+
+/* Stable sort of (key, value) pairs by key (cub::DeviceRadixSort::SortPairs semantics).
+ * pinned by comparison with numpy's stable argsort in tests. */
+void ndo_sort_pairs(const int32_t* keys_in, const int32_t* vals_in, int64_t n,
+                    int32_t* keys_out, int32_t* vals_out);
+
+/* Unique keys of the sorted prefix whose keys != invalid, their counts and start
+ * offsets (RLE + exclusive sum).  Returns the number of runs.
+ * pinned by numpy.unique in tests. */
+int64_t ndo_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid,
+                            int32_t* uniq, int32_t* counts, int32_t* offsets,
+                            int64_t* n_valid);
+
+/* Kernel class of a transit that count samples sit on, sub-warp size W:
+ * count*W >= 256 -> 1 (grid), >= 32 -> 2 (block), >= 8 -> 3 (sub-warp), else 4 (identity)
+ * (utils.hpp:491-497, nextdoor.cu:55-61, 1560-1600). pinned by threshold table test. */
+int ndo_kernel_class(int64_t count, int64_t sub_warp_size);
+
+/* ---- distinct post-pass for k-hop (behavioural hint: src/distinct.cuh:1-111) ----
+ * Per sample, per hop segment: ascending unique valid ids packed left, rest = invalid;
+ * counts[s*steps + k] = number kept.  Own definition: parity unpinned by the reference;
+ * pinned by sort+unique brute force and idempotence. */
+void ndo_distinct(const ndo_app_desc* app, int64_t n_samples, int32_t invalid,
+                  int32_t* final_samples, int32_t* counts);
+
+/* ---- validators (src/check_results.cu) ---- */
+
+/* checkSampledVerticesResult (check_results.cu:162-299) as written: first 4 steps,
+ * "adjacent to some valid vertex of the previous step's segment", and "segment all
+ * INVALID only if the previous segment has no edges".  Returns 1 when it passes. */
+int ndo_check_sampled_vertices(const ndo_graph* g, const ndo_app_desc* app,
+                               int64_t n_samples, const int32_t* initial,
+                               const int32_t* final_samples, int32_t invalid, int n_threads);
+
+/* Stronger check used by this repo's tests: all steps, and each output must be a
+ * neighbour of exactly the transit it was drawn for (canonical layout). */
+int ndo_check_exact_transits(const ndo_graph* g, const ndo_app_desc* app,
+                             int64_t n_samples, const int32_t* initial,
+                             const int32_t* final_samples, int32_t invalid);
+
+/* CSRPartition::has_edge_logn (csr.hpp:342-359). */
+int ndo_has_edge(const ndo_graph* g, int32_t src, int32_t dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

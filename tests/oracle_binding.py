@@ -1,0 +1,198 @@
+"""ctypes binding of the CPU oracle (oracle/libnd_oracle.so).  Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ORACLE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+LIB = os.path.join(ORACLE_DIR, "libnd_oracle.so")
+
+MAX_STEPS = 128
+
+UNIFORM_WALK, DEEPWALK, PPR, NODE2VEC, WEIGHTED_NODE2VEC, KHOP, LAYER_LITERAL, FASTGCN_IMPORTANCE, \
+    LADIES_IMPORTANCE = range(9)
+
+i32p = C.POINTER(C.c_int32)
+f32p = C.POINTER(C.c_float)
+
+
+class GraphStruct(C.Structure):
+    _fields_ = [("n_vertices", C.c_int32), ("n_edges", C.c_int64), ("row_ptr", i32p), ("col", i32p),
+                ("weight", f32p), ("max_weight", f32p)]
+
+
+class AppDesc(C.Structure):
+    _fields_ = [("kind", C.c_int), ("steps", C.c_int), ("step_size", C.c_int * MAX_STEPS),
+                ("initial_size", C.c_int), ("p", C.c_float), ("q", C.c_float)]
+
+
+class Stats(C.Structure):
+    _fields_ = [("next_calls", C.c_int64), ("draws", C.c_int64), ("search_probes", C.c_int64),
+                ("valid_outputs", C.c_int64), ("edge_reads", C.c_int64), ("weight_reads", C.c_int64)]
+
+    def as_dict(self):
+        return {k: getattr(self, k) for k, _ in self._fields_}
+
+
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", ORACLE_DIR, "-s"], check=True)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            build()
+        L = C.CDLL(LIB)
+        L.ndo_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+        L.ndo_uniform.restype = C.c_float
+        L.ndo_uniform.argtypes = [C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32]
+        L.ndo_rand_int.restype = C.c_int32
+        L.ndo_rand_int.argtypes = [C.c_float, C.c_int32]
+        for name in ("ndo_step_size_at_step", "ndo_number_of_transits", "ndo_sub_warp_size_at_step"):
+            getattr(L, name).restype = C.c_int64
+            getattr(L, name).argtypes = [C.POINTER(AppDesc), C.c_int]
+        L.ndo_final_sample_size.restype = C.c_int64
+        L.ndo_final_sample_size.argtypes = [C.POINTER(AppDesc)]
+        L.ndo_max_bits.argtypes = [C.c_int32]
+        L.ndo_sample_individual.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64, C.c_int64,
+                                            C.c_int64, i32p, i32p, i32p, C.POINTER(Stats), C.c_int]
+        L.ndo_sort_pairs.argtypes = [i32p, i32p, C.c_int64, i32p, i32p]
+        L.ndo_unique_transits.restype = C.c_int64
+        L.ndo_unique_transits.argtypes = [i32p, C.c_int64, C.c_int32, i32p, i32p, i32p, C.POINTER(C.c_int64)]
+        L.ndo_kernel_class.argtypes = [C.c_int64, C.c_int64]
+        L.ndo_distinct.argtypes = [C.POINTER(AppDesc), C.c_int64, C.c_int32, i32p, i32p]
+        L.ndo_check_sampled_vertices.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
+                                                 C.c_int32, C.c_int]
+        L.ndo_check_exact_transits.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
+                                               C.c_int32]
+        L.ndo_has_edge.argtypes = [C.POINTER(GraphStruct), C.c_int32, C.c_int32]
+        _lib = L
+    return _lib
+
+
+def _p(a, ct):
+    return a.ctypes.data_as(C.POINTER(ct))
+
+
+class Graph:
+    """CSR arrays held as numpy, plus the struct the oracle takes."""
+
+    def __init__(self, row_ptr, col, weight=None, max_weight=None):
+        self.row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+        self.col = np.ascontiguousarray(col, dtype=np.int32)
+        self.weight = (np.ones(len(self.col), np.float32) if weight is None
+                       else np.ascontiguousarray(weight, dtype=np.float32))
+        V = len(self.row_ptr) - 1
+        if max_weight is None:
+            mw = np.zeros(V, np.float32)
+            for v in range(V):
+                seg = self.weight[self.row_ptr[v]:self.row_ptr[v + 1]]
+                if len(seg):
+                    mw[v] = max(np.float32(0), seg.max())
+            max_weight = mw
+        self.max_weight = np.ascontiguousarray(max_weight, dtype=np.float32)
+        self.n_vertices = V
+        self.struct = GraphStruct(V, len(self.col), _p(self.row_ptr, C.c_int32), _p(self.col, C.c_int32),
+                                  _p(self.weight, C.c_float), _p(self.max_weight, C.c_float))
+
+    @classmethod
+    def from_adjacency(cls, adj, weights=None):
+        """adj: list of neighbour lists; sorted here by (dst, weight) like the reference loader."""
+        row_ptr, col, w = [0], [], []
+        for v, nb in enumerate(adj):
+            ws = [1.0] * len(nb) if weights is None else list(weights[v])
+            pairs = sorted(zip(nb, ws))
+            col += [p[0] for p in pairs]
+            w += [p[1] for p in pairs]
+            row_ptr.append(len(col))
+        return cls(row_ptr, col, w)
+
+
+def app_desc(kind, steps, step_sizes, initial_size=1, p=2.0, q=0.5):
+    d = AppDesc()
+    d.kind, d.steps, d.initial_size, d.p, d.q = kind, steps, initial_size, p, q
+    if isinstance(step_sizes, int):
+        step_sizes = [step_sizes] * steps
+    for i, s in enumerate(step_sizes):
+        d.step_size[i] = s
+    return d
+
+
+def philox(ctr, key):
+    c = (C.c_uint32 * 4)(*ctr)
+    k = (C.c_uint32 * 2)(*key)
+    o = (C.c_uint32 * 4)()
+    lib().ndo_philox4x32_10(c, k, o)
+    return list(o)
+
+
+def uniform(seed, slot, step, draw):
+    return lib().ndo_uniform(seed, slot, step, draw)
+
+
+def rand_int(u, n):
+    return lib().ndo_rand_int(np.float32(u), n)
+
+
+def final_sample_size(desc):
+    return lib().ndo_final_sample_size(C.byref(desc))
+
+
+def sample_individual(graph, desc, seed, initial, first_sample=0, n_threads=8, want_stats=False):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    n_samples = len(initial) // desc.initial_size
+    F = final_sample_size(desc)
+    final = np.empty(n_samples * F, dtype=np.int32)
+    state = np.empty(n_samples, dtype=np.int32)
+    stats = Stats()
+    rc = lib().ndo_sample_individual(C.byref(graph.struct), C.byref(desc), seed, n_samples, first_sample,
+                                     _p(initial, C.c_int32), _p(final, C.c_int32), _p(state, C.c_int32),
+                                     C.byref(stats) if want_stats else None, n_threads)
+    assert rc == 0, rc
+    final = final.reshape(n_samples, F)
+    return (final, state, stats.as_dict()) if want_stats else (final, state)
+
+
+def sort_pairs(keys, vals):
+    keys = np.ascontiguousarray(keys, dtype=np.int32)
+    vals = np.ascontiguousarray(vals, dtype=np.int32)
+    ko, vo = np.empty_like(keys), np.empty_like(vals)
+    lib().ndo_sort_pairs(_p(keys, C.c_int32), _p(vals, C.c_int32), len(keys), _p(ko, C.c_int32), _p(vo, C.c_int32))
+    return ko, vo
+
+
+def unique_transits(sorted_keys, invalid):
+    k = np.ascontiguousarray(sorted_keys, dtype=np.int32)
+    n = len(k)
+    u, c, o = (np.empty(max(n, 1), np.int32) for _ in range(3))
+    nv = C.c_int64()
+    r = lib().ndo_unique_transits(_p(k, C.c_int32), n, invalid, _p(u, C.c_int32), _p(c, C.c_int32),
+                                  _p(o, C.c_int32), C.byref(nv))
+    return u[:r], c[:r], o[:r], nv.value
+
+
+def distinct(desc, final, invalid):
+    final = np.ascontiguousarray(final, dtype=np.int32).copy()
+    n_samples = final.shape[0]
+    counts = np.empty(n_samples * desc.steps, np.int32)
+    lib().ndo_distinct(C.byref(desc), n_samples, invalid, _p(final, C.c_int32), _p(counts, C.c_int32))
+    return final, counts.reshape(n_samples, desc.steps)
+
+
+def check_sampled_vertices(graph, desc, initial, final, invalid, n_threads=8):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    final = np.ascontiguousarray(final, dtype=np.int32)
+    return bool(lib().ndo_check_sampled_vertices(C.byref(graph.struct), C.byref(desc), final.shape[0],
+                                                 _p(initial, C.c_int32), _p(final, C.c_int32), invalid, n_threads))
+
+
+def check_exact_transits(graph, desc, initial, final, invalid):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    final = np.ascontiguousarray(final, dtype=np.int32)
+    return bool(lib().ndo_check_exact_transits(C.byref(graph.struct), C.byref(desc), final.shape[0],
+                                               _p(initial, C.c_int32), _p(final, C.c_int32), invalid))

@@ -1,0 +1,47 @@
+"""The C-ABI library loads and exports every symbol include/nextdoor_amd.h declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "nextdoor_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_reference_surface():
+    names = declared_symbols()
+    for needed in ("nd_graph_load", "nd_sampler_set_graph", "nd_sampler_alloc", "nd_sampler_do_transit_parallel",
+                   "nd_sampler_get_final_samples", "nd_sampler_final_sample_size", "nd_sampler_free_device",
+                   "nd_init_sampling", "nd_sample", "nd_final_sample_length", "nd_final_samples_array",
+                   "nd_free_device_memory"):
+        assert needed in names
+
+
+def test_library_exports_every_declared_symbol():
+    from nextdoor_amd import _capi
+    from nextdoor_amd.build import LIB_PATH
+    assert os.path.exists(LIB_PATH), "build the library first: python -m nextdoor_amd.build"
+    handle = ctypes.CDLL(LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(handle, name), name
+    # the Python binding covers the same set
+    assert sorted(_capi.SIGNATURES) == declared_symbols()
+
+
+def test_app_registry_lists_the_reference_apps():
+    import nextdoor_amd
+    names = nextdoor_amd.app_names()
+    for app in ("UniformRandomWalk", "DeepWalk", "PPR", "Node2Vec", "KHop", "WeightedNode2Vec"):
+        assert app in names
+
+
+def test_unknown_app_is_an_error_not_an_abort():
+    import nextdoor_amd
+    import pytest
+    g = nextdoor_amd.Graph.from_edges([0, 1], [1, 0])
+    with pytest.raises(nextdoor_amd.NextDoorError):
+        nextdoor_amd.Sampler("NoSuchApp", g)

@@ -1,0 +1,116 @@
+"""GPU parity of the transit-parallel engine against the CPU oracle: same graph, same
+roots, same seed -> byte-identical final samples, with load balancing on and off,
+for every IndividualNeighborhood app; plus the reference's check_results invariants."""
+import numpy as np
+import pytest
+
+import nextdoor_amd as nd
+from tests import graphs
+
+pytestmark = pytest.mark.gpu
+
+SEED = 42
+
+
+def desc_for(oracle, sampler, kind):
+    steps = sampler.steps
+    return oracle.app_desc(kind, steps, [sampler.step_size(k) for k in range(steps)],
+                           initial_size=sampler.initial_sample_size)
+
+
+def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)):
+    og = graphs.oracle_view(g)
+    s = nd.Sampler(app, g, seed=SEED)
+    try:
+        d = desc_for(oracle, s, kind)
+        roots = s.initial_contents
+        assert s.invalid_vertex == g.n_vertices
+        want, want_state = oracle.sample_individual(og, d, SEED, roots)
+        assert want.shape == (s.num_samples, s.final_sample_size)
+        for lb in modes:
+            print("app", app, "V", g.n_vertices, "E", g.n_edges, "lb", lb, flush=True)
+            s.do_transit_parallel(load_balancing=lb)
+            got = s.final_samples()
+            if not np.array_equal(got, want):
+                bad = np.argwhere(got != want)
+                raise AssertionError(f"{app} lb={lb}: {len(bad)} mismatches, first at {bad[0]}: "
+                                     f"got {got[tuple(bad[0])]} want {want[tuple(bad[0])]}")
+            if check_state:
+                st = s.sample_states().view(np.int32)
+                alive = want_state != -1
+                assert np.array_equal(st[alive], want_state[alive])
+        assert oracle.check_sampled_vertices(og, d, roots, got, s.invalid_vertex)
+        assert oracle.check_exact_transits(og, d, roots, got, s.invalid_vertex)
+        return got
+    finally:
+        s.close()
+
+
+GRAPHS = {
+    "sparse": dict(n=300, mean_degree=3, seed=1, isolated_every=7),
+    "dense_hub": dict(n=2000, mean_degree=12, seed=2, hub=5),
+}
+
+
+@pytest.mark.parametrize("gname", list(GRAPHS))
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("DeepWalkPerVertex", "DEEPWALK", False),
+    ("PPRPerVertex", "PPR", False),
+    ("Node2VecPerVertex", "NODE2VEC", True),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+    ("KHop", "KHOP", False),
+    ("KHop4x3x2", "KHOP", False),
+])
+def test_app_matches_oracle(oracle, app, kind_name, state, gname):
+    g = graphs.random_graph(**GRAPHS[gname])
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+
+
+def test_reference_sized_deepwalk_has_100_walks_per_vertex(oracle):
+    # RandomWalkApp::numSamples (randomWalks.cu:23-26)
+    g = graphs.random_graph(n=120, mean_degree=4, seed=3)
+    s = nd.Sampler("DeepWalk", g, seed=SEED)
+    assert s.num_samples == 100 * 120
+    assert np.array_equal(s.initial_contents, np.arange(100 * 120) % 120)
+    s.close()
+    run_and_compare(oracle, "DeepWalk", oracle.DEEPWALK, g)
+
+
+def test_walks_concentrated_on_one_transit(oracle):
+    # star: every walk alternates hub <-> leaf, so every other step has ONE transit carrying
+    # all samples (the grid-wide case) and the others have one sample per transit
+    n = 3000
+    leaves = np.arange(1, n)
+    g = nd.Graph.from_edges(np.concatenate([np.zeros(n - 1, int), leaves]),
+                            np.concatenate([leaves, np.zeros(n - 1, int)]),
+                            np.linspace(1, 4.9, 2 * (n - 1)).astype(np.float32))
+    for app, kind in [("UniformRandomWalk8", oracle.UNIFORM_WALK), ("WeightedNode2Vec8", oracle.WEIGHTED_NODE2VEC)]:
+        run_and_compare(oracle, app, kind, g)
+
+
+def test_graph_without_edges_gives_all_invalid(oracle):
+    g = nd.Graph.from_csr(np.zeros(65, np.int32), np.zeros(0, np.int32))
+    got = run_and_compare(oracle, "UniformRandomWalk8", oracle.UNIFORM_WALK, g)
+    assert np.all(got == 64)
+
+
+def test_single_vertex_self_loop(oracle):
+    g = nd.Graph.from_edges([0], [0])
+    got = run_and_compare(oracle, "KHop3x2", oracle.KHOP, g)
+    assert np.all(got == 0)
+
+
+def test_runs_are_reproducible_and_seed_matters(oracle):
+    g = graphs.random_graph(n=500, mean_degree=6, seed=9)
+    s = nd.Sampler("UniformRandomWalk8", g, seed=1)
+    s.do_transit_parallel(True)
+    a = s.final_samples()
+    s.do_transit_parallel(True)
+    b = s.final_samples()
+    s.close()
+    s2 = nd.Sampler("UniformRandomWalk8", g, seed=2)
+    s2.do_transit_parallel(True)
+    c = s2.final_samples()
+    s2.close()
+    assert np.array_equal(a, b) and not np.array_equal(a, c)
