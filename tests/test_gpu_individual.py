@@ -39,7 +39,11 @@ def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)
                 st = s.sample_states().view(np.int32)
                 alive = want_state != -1
                 assert np.array_equal(st[alive], want_state[alive])
-        assert oracle.check_sampled_vertices(og, d, roots, got, s.invalid_vertex)
+        # the reference's own validator; its "nothing sampled only if the previous step had no
+        # edges" clause does not hold for PPR, whose walks end at random (the reference runs
+        # PPR unchecked: src/tests/singleGPU/ppr.cu:12-30)
+        if kind != oracle.PPR:
+            assert oracle.check_sampled_vertices(og, d, roots, got, s.invalid_vertex)
         assert oracle.check_exact_transits(og, d, roots, got, s.invalid_vertex)
         return got
     finally:
