@@ -1,0 +1,178 @@
+"""Benchmark of the transit-parallel sampling path on one MI355X.
+
+One "step" is one full pass of the hot path over one batch: doTransitParallelSampling
+(load balanced) of the weighted node2vec walk (p=2, q=0.5, length 100, one walk per
+vertex) on the symmetrised R-MAT scale-22 graph, i.e. 419,430,400 sampled edges (output
+slots).  The graph and all per-run buffers are resident in HBM before the timed region;
+the timed region is the step loop only, as the reference's "End to end time"
+(src/nextdoor.cu:2363-2963).
+
+Prints one JSON line:  metric / value (sampled edges per second) / roofline (dominant
+kernel, algorithmic bytes over its measured launch time) / cpu_baseline (the CPU oracle on
+a bounded sample of the same walks, on this box's host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (app, graph factory kwargs)
+    "weighted_node2vec_rmat22": dict(app="WeightedNode2Vec", kind="WEIGHTED_NODE2VEC",
+                                     graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
+    "weighted_node2vec_rmat16": dict(app="WeightedNode2Vec", kind="WEIGHTED_NODE2VEC",
+                                     graph=("rmat", dict(scale=16, edge_factor=16, symmetrise=True))),
+    "uniform_walk_chunglu57k": dict(app="UniformRandomWalk", kind="UNIFORM_WALK",
+                                    graph=("chung_lu", dict(n_vertices=56944, n_edges=818000, exponent=2.1))),
+    "khop_rmat21": dict(app="KHop", kind="KHOP", graph=("rmat", dict(scale=21, edge_factor=32, symmetrise=False))),
+}
+
+
+def make_graph(nd, spec):
+    kind, kw = spec
+    if kind == "rmat":
+        return nd.Graph.rmat(kw["scale"], kw["edge_factor"], seed=42, symmetrise=kw["symmetrise"])
+    return nd.Graph.chung_lu(kw["n_vertices"], kw["n_edges"], kw["exponent"], seed=42)
+
+
+def cpu_baseline(graph, sampler, kind_name, budget_s, seed):
+    """Times the CPU oracle on a strided subset of the same samples (whole walks), all host
+    cores, growing the subset until it has run for about budget_s seconds."""
+    from tests import graphs, oracle_binding as ob
+    og = graphs.oracle_view(graph)
+    steps = sampler.steps
+    desc = ob.app_desc(getattr(ob, kind_name), steps, [sampler.step_size(k) for k in range(steps)],
+                       initial_size=sampler.initial_sample_size)
+    roots = sampler.initial_contents.reshape(sampler.num_samples, -1)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    outputs_per_sample = sampler.final_sample_size
+    stride = max(1, sampler.num_samples // 4096)
+    best = None
+    while True:
+        sub = np.ascontiguousarray(roots[::stride]).reshape(-1)
+        t0 = time.perf_counter()
+        _, _, stats = ob.sample_individual(og, desc, seed, sub, n_threads=cores, want_stats=True)
+        dt = time.perf_counter() - t0
+        n = len(sub) // desc.initial_size
+        best = dict(seconds=dt, samples=n, stats=stats, stride=stride)
+        if dt >= budget_s / 3 or stride == 1:
+            break
+        stride = max(1, int(stride / min(8.0, max(2.0, budget_s / max(dt, 1e-3) / 2))))
+    edges = best["samples"] * outputs_per_sample
+    return {
+        "value": edges / best["seconds"], "unit": "sampled edges/s", "cores": cores, "kind": "port",
+        "sample": f"CPU oracle, every {best['stride']}th walk ({best['samples']} of {sampler.num_samples} samples, "
+                  f"all {steps} steps), {best['seconds']:.1f} s",
+    }, best
+
+
+def algorithmic_bytes_per_pass(sampler, oracle_run, weighted, second_order):
+    """Minimal 4-byte-granular HBM traffic of one pass, split by kernel family, scaled from
+    the oracle's counters on the sampled walks to all walks.
+    Step kernel, per pair: (transit, slot) 8 + row extent 8 (+4 max weight); per candidate
+    edge: id 4 (+4 weight); second order: previous vertex read+write 8, its row extent 8 per
+    next() call and 4 per binary-search probe; per output: next-step transit 4 + final sample 4.
+    Inversion, per pair and 8-bit pass: histogram read 4 + scatter read 8 / write 8 (the
+    first pass generates the slot instead of reading it)."""
+    st = oracle_run["stats"]
+    scale = sampler.num_samples / oracle_run["samples"]
+    steps = sampler.steps
+    pairs = sampler.num_samples * steps  # walks: one pair per sample and step
+    passes = (sampler.max_bits + 7) // 8
+    step_bytes = pairs * (8 + 8 + (4 if weighted else 0)) + pairs * 8
+    step_bytes += scale * (st["edge_reads"] * 4 + st["weight_reads"] * 4)
+    if second_order:
+        step_bytes += scale * (st["next_calls"] * 16 + st["search_probes"] * 4)
+    sort_pairs_n = sampler.num_samples * (steps - 1)
+    sort_bytes = sort_pairs_n * (passes * (4 + 8 + 8) - 4)
+    return step_bytes, sort_bytes
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="weighted_node2vec_rmat22", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-load-balancing", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=42)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X; this build has no multi-GPU path (samples would shard "
+                 "by contiguous ranges with the graph replicated). Run with --gpus 1.")
+
+    import nextdoor_amd as nd
+    w = WORKLOADS[args.workload]
+    t0 = time.perf_counter()
+    graph = make_graph(nd, w["graph"])
+    t_graph = time.perf_counter() - t0
+    sampler = nd.Sampler(w["app"], graph, seed=args.seed)
+    lb = not args.no_load_balancing
+    edges_per_pass = sampler.num_samples * sampler.final_sample_size
+
+    for _ in range(args.warmup):
+        sampler.do_transit_parallel(lb)
+    wall0 = time.perf_counter()
+    gpu_ms = []
+    for _ in range(args.steps):
+        sampler.do_transit_parallel(lb)  # synchronises its stream before returning
+        gpu_ms.append(sampler.phase_times()["end_to_end_ms"])
+    wall = time.perf_counter() - wall0
+    ms_per_step = wall * 1000.0 / args.steps
+
+    # per-kernel-family durations: one extra pass with events around every launch group
+    sampler.set_profiling(True)
+    sampler.do_transit_parallel(lb)
+    prof = sampler.phase_times()
+    sampler.set_profiling(False)
+    final = sampler.final_samples()
+    valid = int((final != sampler.invalid_vertex).sum())
+    del final
+
+    result = {
+        "metric": "sampled edges/sec on 1 MI355X", "value": edges_per_pass / (ms_per_step / 1000.0),
+        "unit": "sampled edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int32 ids / f32 weights", "data": "synthetic",
+        "config": {"workload": args.workload, "app": w["app"], "vertices": graph.n_vertices, "edges": graph.n_edges,
+                   "samples": sampler.num_samples, "walk_steps": sampler.steps, "load_balancing": lb,
+                   "sampled_edges_per_step": edges_per_pass, "valid_outputs": valid,
+                   "graph_build_s": round(t_graph, 1), "gpu_event_ms_per_step": float(np.mean(gpu_ms))},
+        "phases_ms": {k: round(v, 3) for k, v in prof.items()},
+    }
+
+    if not args.skip_cpu_baseline:
+        base, run = cpu_baseline(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
+        result["cpu_baseline"] = base
+        weighted = w["kind"] in ("WEIGHTED_NODE2VEC", "DEEPWALK", "PPR")
+        second = w["kind"] in ("WEIGHTED_NODE2VEC", "NODE2VEC")
+        step_bytes, sort_bytes = algorithmic_bytes_per_pass(sampler, run, weighted, second)
+        step_ms = prof["flat_kernel_ms"] + prof["workgroup_kernel_ms"]
+        launches = prof["flat_launches"]
+        # dominant kernel family: the step kernels (flat + workgroup launched back to back per walk step)
+        achieved = step_bytes / (step_ms / 1000.0) / 1e9
+        result["roofline"] = {
+            "bound": "hbm", "kernel": "step_flat_kernel + step_workgroup_kernel", "achieved": achieved,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes_per_launch": step_bytes / max(launches, 1), "avg_launch_ms": step_ms / max(launches, 1),
+            "whole_pass": {"algorithmic_bytes": step_bytes + sort_bytes,
+                           "achieved_GBps": (step_bytes + sort_bytes) / (np.mean(gpu_ms) / 1000.0) / 1e9,
+                           "frac": (step_bytes + sort_bytes) / (np.mean(gpu_ms) / 1000.0) / 1e9 / HBM_PEAK_GBS},
+        }
+        result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
+    sampler.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -89,10 +89,10 @@ int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
 /* The per-phase wall-clock breakdown the reference prints (src/nextdoor.cu:2963-2966),
  * measured with events on the sampler's stream when profiling is on.
  * out[0] end to end, [1] inversion, [2] load balancing, [3] flat (identity / sub-wavefront)
- * kernel, [4] workgroup + grid-wide kernel, all in milliseconds; [5] flat launches,
- * [6] workgroup launches, [7] sort passes. */
+ * kernel, [4] workgroup + grid-wide kernel, [8] final-row assembly, all in milliseconds;
+ * [5] flat launches, [6] workgroup launches, [7] sort passes; [9..11] reserved (0). */
 int nd_sampler_set_profiling(nd_sampler* s, int on);
-int nd_sampler_phase_times(const nd_sampler* s, float out[8]);
+int nd_sampler_phase_times(const nd_sampler* s, float out[12]);
 /* freeDeviceData(data), src/nextdoor.cu:2088-2115. */
 void nd_sampler_free_device(nd_sampler* s);
 void nd_sampler_destroy(nd_sampler* s);

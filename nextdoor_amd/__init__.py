@@ -192,11 +192,11 @@ class Sampler:
         check(lib().nd_sampler_set_profiling(self._h, int(on)))
 
     def phase_times(self):
-        out = (C.c_float * 8)()
+        out = (C.c_float * 12)()
         check(lib().nd_sampler_phase_times(self._h, out))
         keys = ["end_to_end_ms", "inversion_ms", "load_balancing_ms", "flat_kernel_ms", "workgroup_kernel_ms",
-                "flat_launches", "workgroup_launches", "sort_passes"]
-        return dict(zip(keys, list(out)))
+                "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms"]
+        return dict(zip(keys, list(out)[:9]))
 
     def free_device(self):
         lib().nd_sampler_free_device(self._h)

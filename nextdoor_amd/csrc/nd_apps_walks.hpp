@@ -167,6 +167,7 @@ struct Node2VecAppT : Sizing {
 template <int kWalkLength>
 struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
   static constexpr bool kUsesEdgeWeights = true;
+  static constexpr bool kUsesEdgeLookup = true;
 
   template <typename SampleType, typename EdgeArray, typename WeightArray>
   __device__ inline VertexID next(int step, CSRPartition* csr, const VertexID* transits, const VertexID,

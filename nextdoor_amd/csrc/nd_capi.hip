@@ -235,12 +235,14 @@ int nd_sampler_set_profiling(nd_sampler* s, int on) {
   return 0;
 }
 
-int nd_sampler_phase_times(const nd_sampler* s, float out[8]) {
+int nd_sampler_phase_times(const nd_sampler* s, float out[12]) {
   if (!s || !out) return fail("null argument");
   const nd::PhaseTimes& t = s->engine->times;
   out[0] = t.end_to_end; out[1] = t.inversion; out[2] = t.load_balancing; out[3] = t.flat_kernel;
   out[4] = t.workgroup_kernel; out[5] = (float)t.flat_launches; out[6] = (float)t.workgroup_launches;
   out[7] = (float)t.sort_launches;
+  out[8] = t.assemble;
+  out[9] = out[10] = out[11] = 0.0f;
   return 0;
 }
 

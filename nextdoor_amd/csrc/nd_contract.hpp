@@ -87,8 +87,35 @@ class CSRPartition {
   __host__ __device__ __forceinline__ const CSR::Edge* get_edges(VertexID v) const { return edges + row_ptr[v]; }
   __host__ __device__ __forceinline__ const float* get_weights(VertexID v) const { return weights + row_ptr[v]; }
 
-  // src/csr.hpp:342-359: binary search of dst in the sorted adjacency of src
+  // Optional exact edge index: open-addressing table of (src << 32 | dst) keys over all
+  // edges, at most half full, empty slots all-ones.  Built by the engine for apps that
+  // declare kUsesEdgeLookup; nullptr otherwise.
+  const unsigned long long* edge_table;
+  uint32_t edge_table_mask;
+
+  __host__ __device__ __forceinline__ static uint32_t edge_hash(unsigned long long key) {
+    key ^= key >> 33;
+    key *= 0xff51afd7ed558ccdull;
+    key ^= key >> 33;
+    key *= 0xc4ceb9fe1a85ec53ull;
+    key ^= key >> 33;
+    return (uint32_t)key;
+  }
+
+  // Is dst in the adjacency of src?  The reference answers with a binary search of the
+  // sorted adjacency (src/csr.hpp:342-359); with the edge index present the same answer
+  // comes from one or two probes of the table instead of log2(degree) dependent loads.
   __host__ __device__ __forceinline__ bool has_edge_logn(VertexID src, VertexID dst) const {
+    if (edge_table != nullptr) {
+      const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)dst;
+      uint32_t h = edge_hash(key) & edge_table_mask;
+      for (;;) {
+        const unsigned long long k = edge_table[h];
+        if (k == key) return true;
+        if (k == ~0ull) return false;
+        h = (h + 1) & edge_table_mask;
+      }
+    }
     EdgePos_t l = row_ptr[src];
     EdgePos_t r = row_ptr[src + 1] - 1;
     while (l <= r) {
@@ -145,10 +172,49 @@ struct LdsBackedArray {
 };
 
 // Optional compile-time hints an App may carry; absent members mean `false`.
-//   static constexpr bool kUsesEdgeWeights = true;  -> stage weights in LDS as well
+//   static constexpr bool kUsesEdgeWeights = true;  -> next() reads transitEdgeWeights: the
+//        engine keeps an interleaved (destination, weight) copy of the edges so that one
+//        8-byte gather serves both arrays, and stages weights in LDS as well
+//   static constexpr bool kUsesEdgeLookup = true;   -> next() calls csr->has_edge_logn: the
+//        engine builds the exact edge index behind it
 template <typename App, typename = void>
 struct app_uses_weights { static constexpr bool value = false; };
 template <typename App>
 struct app_uses_weights<App, decltype((void)App::kUsesEdgeWeights)> { static constexpr bool value = App::kUsesEdgeWeights; };
+template <typename App, typename = void>
+struct app_uses_edge_lookup { static constexpr bool value = false; };
+template <typename App>
+struct app_uses_edge_lookup<App, decltype((void)App::kUsesEdgeLookup)> { static constexpr bool value = App::kUsesEdgeLookup; };
+
+// Interleaved edge record and the two array views over it.  Both views share a one-entry
+// cache, so transitEdges[x] and transitEdgeWeights[x] cost one 8-byte load whichever
+// comes first.
+struct EdgeRecord {
+  VertexID dst;
+  float weight;
+};
+
+struct EdgeRecordCursor {
+  const EdgeRecord* base;
+  EdgePos_t index;
+  EdgeRecord record;
+  __device__ __forceinline__ const EdgeRecord& at(EdgePos_t i) {
+    if (i != index) {
+      record = base[i];
+      index = i;
+    }
+    return record;
+  }
+};
+
+struct PairedEdgeIds {
+  EdgeRecordCursor* cursor;
+  __device__ __forceinline__ VertexID operator[](EdgePos_t i) const { return cursor->at(i).dst; }
+};
+
+struct PairedEdgeWeights {
+  EdgeRecordCursor* cursor;
+  __device__ __forceinline__ float operator[](EdgePos_t i) const { return cursor->at(i).weight; }
+};
 
 }  // namespace nd

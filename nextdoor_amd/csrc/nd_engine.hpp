@@ -45,7 +45,7 @@ namespace nd {
 enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1 };
 
 struct PhaseTimes {  // milliseconds, accumulated over one sample() call when profiling is on
-  float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0;
+  float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0, assemble = 0;
   int flat_launches = 0, workgroup_launches = 0, sort_launches = 0;
 };
 
@@ -104,9 +104,12 @@ struct StepParams {
   uint32_t n_pairs;              // S * T_k
   const uint32_t* pair_keys;     // transit of each pair (sorted, or the raw map at step 0)
   const uint32_t* pair_slots;    // slot of each pair; nullptr: slot == index
-  int32_t* next_transits;        // map for step k+1, indexed by output slot
-  int32_t* final_samples;
+  int32_t* step_out;             // outputs of this step, indexed by output slot; it is both
+                                 // the (sample -> transit) map of step k+1 and, regrouped
+                                 // per sample at the end, this step's segment of the result
   void* samples;                 // SampleType[S] or nullptr
+  const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
+  uint32_t blocks_per_xcd;       // flat kernel: workgroups each XCD handles (see flat_block_index)
 };
 
 constexpr int kStepThreads = 256;
@@ -136,9 +139,16 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
         (VertexID_t)nbr, &rng);
     neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
   }
-  if (!P.is_last) P.next_transits[out_slot] = neighbor;
-  const uint64_t within = out_slot - (uint64_t)sample * P.transits_per_sample * P.step_size;
-  P.final_samples[(size_t)sample * P.final_size + P.seg_base + within] = neighbor;
+  P.step_out[out_slot] = neighbor;
+}
+
+constexpr uint32_t kXcds = 8;
+
+// Workgroups are handed to the 8 XCDs round-robin (workgroup b runs on XCD b % 8), each XCD
+// with its own L2.  The pairs are sorted by transit, so giving every XCD one CONTIGUOUS
+// eighth of the pairs keeps the adjacency of a hot transit in one L2 instead of all eight.
+__device__ __forceinline__ uint32_t flat_block_index(uint32_t blocks_per_xcd) {
+  return (blockIdx.x % kXcds) * blocks_per_xcd + blockIdx.x / kXcds;
 }
 
 // One lane per output: lane i draws neighbour (i % m) for pair (i / m).  With the map
@@ -147,27 +157,33 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
 template <class SampleType, class App>
 __global__ __launch_bounds__(kStepThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
   const uint64_t total = (uint64_t)P.n_pairs * P.step_size;
-  const uint64_t i = (uint64_t)blockIdx.x * kStepThreads + threadIdx.x;
+  const uint64_t i = (uint64_t)flat_block_index(P.blocks_per_xcd) * kStepThreads + threadIdx.x;
   if (i >= total) return;
   CSRPartition csr = P.csr;
   const uint32_t pair = P.step_size == 1 ? (uint32_t)i : (uint32_t)(i / P.step_size);
   const uint32_t nbr = (uint32_t)(i - (uint64_t)pair * P.step_size);
   const VertexID transit = (VertexID)P.pair_keys[pair];
   const uint32_t slot = P.pair_slots ? P.pair_slots[pair] : pair;
-  EdgePos_t n_edges = 0;
+  EdgePos_t n_edges = 0, begin = 0;
   float max_weight = 0.0f;
-  const CSR::Edge* edges = nullptr;
-  const float* weights = nullptr;
   if (transit != P.invalid) {
     if (skip_flag && skip_flag[transit]) return;
-    const EdgePos_t begin = csr.row_ptr[transit];
+    begin = csr.row_ptr[transit];
     n_edges = csr.row_ptr[transit + 1] - begin;
-    edges = csr.edges + begin;
-    weights = csr.weights + begin;
     max_weight = csr.max_weights[transit];
   }
-  produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, slot, nbr, n_edges, max_weight,
-                                                                 edges, weights);
+  if (app_uses_weights<App>::value) {
+    EdgeRecordCursor cursor{P.paired_edges + begin, -1, {}};
+    PairedEdgeIds edges{&cursor};
+    PairedEdgeWeights weights{&cursor};
+    produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, slot, nbr, n_edges, max_weight,
+                                                                      edges, weights);
+  } else {
+    const CSR::Edge* edges = csr.edges + begin;
+    const float* weights = csr.weights + begin;
+    produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, slot, nbr, n_edges, max_weight,
+                                                                   edges, weights);
+  }
 }
 
 // One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
@@ -260,6 +276,88 @@ __global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
 }
 
 // ---------------------------------------------------------------------------------------
+// Graph-side helpers built once per graph
+// ---------------------------------------------------------------------------------------
+
+__device__ __forceinline__ VertexID source_of_edge(const EdgePos_t* row_ptr, VertexID n_vertices, EdgePos_t e) {
+  // largest v with row_ptr[v] <= e
+  VertexID lo = 0, hi = n_vertices;
+  while (hi - lo > 1) {
+    const VertexID mid = lo + (hi - lo) / 2;
+    if (row_ptr[mid] <= e) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ void build_edge_table(CSRPartition csr, unsigned long long* table, uint32_t mask) {
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (size_t)csr.n_edges) return;
+  const VertexID src = source_of_edge(csr.row_ptr, csr.n_vertices, (EdgePos_t)e);
+  const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)csr.edges[e];
+  uint32_t h = CSRPartition::edge_hash(key) & mask;
+  for (;;) {
+    const unsigned long long seen = atomicCAS(&table[h], ~0ull, key);
+    if (seen == ~0ull || seen == key) return;  // inserted, or a duplicate edge already there
+    h = (h + 1) & mask;
+  }
+}
+
+__global__ void build_paired_edges(const CSR::Edge* col, const float* weight, size_t n, EdgeRecord* out) {
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) out[e] = EdgeRecord{col[e], weight[e]};
+}
+
+// ---------------------------------------------------------------------------------------
+// Final-sample assembly
+// ---------------------------------------------------------------------------------------
+
+constexpr int kMaxSteps = 128;
+
+struct StepLayout {
+  int n_steps;
+  uint32_t seg_base[kMaxSteps];  // offset of the step's segment inside a final sample
+  uint32_t seg_len[kMaxSteps];   // outputs of the step per sample
+};
+
+// The step kernels leave step k's outputs in one array per step, grouped by sample
+// (step_out_k[s * len_k + j]).  The result layout is one row per sample
+// (final[s * F + base_k + j], getFinalSamples: src/nextdoor.cu:3211-3237).  A workgroup
+// stages the rows of a block of samples in LDS (row pitch padded to an odd word count) and
+// writes them out as whole contiguous lines, so HBM sees each result byte written once.
+__global__ __launch_bounds__(256) void assemble_final_rows(const int32_t* __restrict__ step_out,
+                                                           int32_t* __restrict__ final_samples, uint32_t n_samples,
+                                                           uint32_t final_size, uint32_t row_pitch,
+                                                           uint32_t samples_per_block, StepLayout layout) {
+  extern __shared__ int32_t s_rows[];
+  const uint32_t s0 = blockIdx.x * samples_per_block;
+  const uint32_t nb = n_samples - s0 < samples_per_block ? n_samples - s0 : samples_per_block;
+  for (int k = 0; k < layout.n_steps; ++k) {
+    const uint32_t len = layout.seg_len[k];
+    const int32_t* src = step_out + (size_t)n_samples * layout.seg_base[k] + (size_t)s0 * len;
+    for (uint32_t e = threadIdx.x; e < nb * len; e += 256) {
+      const uint32_t s = len == 1 ? e : e / len;
+      const uint32_t j = e - s * len;
+      s_rows[s * row_pitch + layout.seg_base[k] + j] = src[e];
+    }
+  }
+  __syncthreads();
+  int32_t* dst = final_samples + (size_t)s0 * final_size;
+  for (uint32_t e = threadIdx.x; e < nb * final_size; e += 256) {
+    const uint32_t s = e / final_size;
+    dst[e] = s_rows[s * row_pitch + (e - s * final_size)];
+  }
+}
+
+// Fallback for rows too long to stage: one launch per step, straight copy.
+__global__ void assemble_final_step(const int32_t* __restrict__ src, int32_t* __restrict__ final_samples,
+                                    size_t n_elems, uint32_t len, uint32_t final_size, uint32_t seg_base) {
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n_elems) return;
+  const size_t s = e / len;
+  final_samples[s * final_size + seg_base + (e - s * len)] = src[e];
+}
+
+// ---------------------------------------------------------------------------------------
 // Shape algebra (nextdoor.cu:126-197, 1913-1929)
 // ---------------------------------------------------------------------------------------
 
@@ -309,7 +407,8 @@ class Engine : public EngineBase {
     return std::is_empty<SampleType>::value ? 0 : sizeof(SampleType) * (size_t)n_samples_;
   }
 
-  // transferCSRToGPUs: the whole graph is resident on the device.
+  // transferCSRToGPUs: the whole graph is resident on the device, plus the derived
+  // structures the app asks for (interleaved edges, edge index).
   int set_graph(const CSR* graph) override {
     free_graph();
     graph_ = graph;
@@ -333,6 +432,25 @@ class Engine : public EngineBase {
     view_.max_weights = d_max_weight_;
     view_.n_vertices = (VertexID)V;
     view_.n_edges = (EdgePos_t)E;
+    view_.edge_table = nullptr;
+    view_.edge_table_mask = 0;
+    if (app_uses_weights<App>::value) {
+      ND_HIP_TRY(hipMalloc(&d_paired_, sizeof(EdgeRecord) * (E ? E : 1)));
+      if (E) build_paired_edges<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(d_col_, d_weight_, E, d_paired_);
+      ND_HIP_TRY(hipGetLastError());
+    }
+    if (app_uses_edge_lookup<App>::value) {
+      // power-of-two table at most half full
+      size_t slots = 16;
+      while (slots < 2 * E) slots <<= 1;
+      ND_HIP_TRY(hipMalloc(&d_edge_table_, sizeof(unsigned long long) * slots));
+      ND_HIP_TRY(hipMemset(d_edge_table_, 0xFF, sizeof(unsigned long long) * slots));
+      if (E) build_edge_table<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(view_, d_edge_table_, (uint32_t)(slots - 1));
+      ND_HIP_TRY(hipGetLastError());
+      view_.edge_table = d_edge_table_;
+      view_.edge_table_mask = (uint32_t)(slots - 1);
+    }
+    ND_HIP_TRY(hipDeviceSynchronize());
     return 0;
   }
 
@@ -347,6 +465,7 @@ class Engine : public EngineBase {
     if (app.hasExplicitTransits()) { last_error = "apps with explicit transits are not supported"; return -2; }
     if (is_collective<App>()) { last_error = "collective apps need the layer engine"; return -2; }
     const int n_steps = app.steps();
+    if (n_steps < 1 || n_steps > kMaxSteps) { last_error = "steps() must be in [1, 128]"; return -2; }
     for (int k = 0; k < n_steps; ++k)
       if (app.stepSize(k) <= 0) { last_error = "stepSize must be positive (ALL_NEIGHBORS is not supported)"; return -2; }
     n_samples_ = app.numSamples(csr);
@@ -370,20 +489,33 @@ class Engine : public EngineBase {
       initialContents.insert(initialContents.end(), roots.begin(), roots.end());
     }
 
-    // largest map: transits entering the last step
-    uint64_t max_pairs = (uint64_t)n_samples_ * init_size_;
-    uint64_t outputs = max_pairs;
-    uint64_t max_outputs = 0;
+    // shape of every step
+    layout_.n_steps = n_steps;
+    uint64_t pairs = (uint64_t)n_samples_ * init_size_, max_pairs = 0, max_outputs = 0, chunk_cap = 0;
+    uint64_t per_sample = (uint64_t)init_size_, base = 0;
     for (int k = 0; k < n_steps; ++k) {
-      outputs *= (uint64_t)app.stepSize(k);
-      if (outputs > max_outputs) max_outputs = outputs;
-      if (k < n_steps - 1) max_pairs = outputs;
+      const uint64_t mk = (uint64_t)app.stepSize(k);
+      if (k > 0 && pairs > max_pairs) max_pairs = pairs;  // step 0 is not sorted
+      // work-item list: a run of `count` pairs emits ceil(count / pairsPerChunk) items and at
+      // most outputs / kWorkgroupWork runs qualify, so this bound holds at every step
+      uint64_t per_chunk = kChunkOutputs / mk;
+      if (per_chunk == 0) per_chunk = 1;
+      const uint64_t need = pairs / per_chunk + pairs * mk / kWorkgroupWork + 2;
+      if (need > chunk_cap) chunk_cap = need;
+      pairs *= mk;
+      per_sample *= mk;
+      if (pairs > max_outputs) max_outputs = pairs;
+      layout_.seg_base[k] = (uint32_t)base;
+      layout_.seg_len[k] = (uint32_t)per_sample;
+      base += per_sample;
     }
     if (max_outputs >= (1ull << 32) || max_pairs >= (1ull << 31)) {
       last_error = "a step has 2^32 or more outputs; split the samples over several runs";
       return -2;
     }
+    if (max_pairs == 0) max_pairs = 1;
     max_pairs_ = (size_t)max_pairs;
+    chunk_capacity_ = (uint32_t)chunk_cap;
     const size_t F = (size_t)final_sample_size();
     hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
 
@@ -395,7 +527,7 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_samples_, sizeof(SampleType) * (size_t)n_samples_));
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
-    ND_HIP_TRY(hipMalloc(&d_map_, sizeof(int32_t) * max_pairs_));
+    ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * max_pairs_));
@@ -409,20 +541,6 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_run_start_, sizeof(uint32_t) * (max_pairs_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta)));
     ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta)));
-    // work-item list: a run of `count` pairs emits ceil(count / pairsPerChunk) items and at
-    // most outputs / kWorkgroupWork runs qualify, so this bound holds at every step
-    {
-      uint64_t cap = 0, pairs = (uint64_t)n_samples_ * init_size_;
-      for (int k = 0; k < n_steps; ++k) {
-        const uint64_t mk = (uint64_t)app.stepSize(k);
-        uint64_t per_chunk = kChunkOutputs / mk;
-        if (per_chunk == 0) per_chunk = 1;
-        const uint64_t need = pairs / per_chunk + pairs * mk / kWorkgroupWork + 2;
-        if (need > cap) cap = need;
-        pairs *= mk;
-      }
-      chunk_capacity_ = (uint32_t)cap;
-    }
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
     ND_HIP_TRY(hipMalloc(&d_skip_flag_, (size_t)invalid_ + 1));
     ND_HIP_TRY(hipMemset(d_skip_flag_, 0, (size_t)invalid_ + 1));
@@ -430,6 +548,15 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipEventCreate(&ev_b_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
     ND_HIP_TRY(hipEventCreate(&ev_end_));
+
+    // rows staged per workgroup by the final assembly: as many as fit 64 KiB of LDS
+    row_pitch_ = (uint32_t)(F | 1);
+    rows_per_block_ = (uint32_t)(65536 / (row_pitch_ * sizeof(int32_t)));
+    if (rows_per_block_ > 64) rows_per_block_ = 64;
+    if (rows_per_block_ > 0) {
+      ND_HIP_TRY(hipFuncSetAttribute((const void*)assemble_final_rows, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     65536));
+    }
     allocated_ = true;
     return 0;
   }
@@ -451,7 +578,7 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
 
     uint32_t transits_per_sample = (uint32_t)init_size_;
-    uint32_t seg_base = 0;
+    const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
     for (int step = 0; step < n_steps; ++step) {
       const uint32_t m = (uint32_t)app.stepSize(step);
       const uint32_t n_pairs = (uint32_t)((uint64_t)n_samples_ * transits_per_sample);
@@ -460,7 +587,7 @@ class Engine : public EngineBase {
       P.step = step;
       P.step_size = m;
       P.transits_per_sample = transits_per_sample;
-      P.seg_base = seg_base;
+      P.seg_base = layout_.seg_base[step];
       P.final_size = (uint32_t)F;
       P.invalid = invalid_;
       P.is_last = step == n_steps - 1;
@@ -468,16 +595,18 @@ class Engine : public EngineBase {
       P.first_slot = 0;
       P.first_sample = 0;
       P.n_pairs = n_pairs;
-      P.next_transits = d_map_;
-      P.final_samples = d_final_;
+      P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
       P.samples = d_samples_;
+      P.paired_edges = d_paired_;
       const uint64_t outputs = (uint64_t)n_pairs * m;
-      const unsigned flat_grid = (unsigned)((outputs + kStepThreads - 1) / kStepThreads);
+      const uint32_t flat_blocks = (uint32_t)((outputs + kStepThreads - 1) / kStepThreads);
+      P.blocks_per_xcd = (flat_blocks + kXcds - 1) / kXcds;
+      const unsigned flat_grid = P.blocks_per_xcd * kXcds;
 
       if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
         // when there is more than one step, nextdoor.cu:2400 and the FIXME at 2372)
-        P.pair_keys = (const uint32_t*)d_initial_;
+        P.pair_keys = (const uint32_t*)transits;
         P.pair_slots = nullptr;
         tick();
         step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, nullptr);
@@ -488,8 +617,8 @@ class Engine : public EngineBase {
         const SortPlan plan = make_sort_plan(n_pairs, max_bits_);
         uint32_t *sorted_keys = nullptr, *sorted_slots = nullptr;
         tick();
-        ND_HIP_TRY(radix_sort_pairs(plan, (const uint32_t*)d_map_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_,
-                                    d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots));
+        ND_HIP_TRY(radix_sort_pairs(plan, (const uint32_t*)transits, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
+                                    d_vals_b_, d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots));
         tock(&times.inversion);
         times.sort_launches += plan.passes;
         P.pair_keys = sorted_keys;
@@ -520,9 +649,27 @@ class Engine : public EngineBase {
         }
       }
       ND_HIP_TRY(hipGetLastError());
-      seg_base += transits_per_sample * m;
+      transits = P.step_out;
       transits_per_sample *= m;
     }
+
+    // regroup the per-step arrays into one row per sample
+    tick();
+    if (rows_per_block_ > 0) {
+      const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
+      const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
+      assemble_final_rows<<<dim3(blocks), dim3(256), lds, stream_>>>(d_step_out_, d_final_, (uint32_t)n_samples_,
+                                                                     (uint32_t)F, row_pitch_, rows_per_block_, layout_);
+    } else {
+      for (int k = 0; k < n_steps; ++k) {
+        const size_t n = (size_t)n_samples_ * layout_.seg_len[k];
+        assemble_final_step<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream_>>>(
+            d_step_out_ + (size_t)n_samples_ * layout_.seg_base[k], d_final_, n, layout_.seg_len[k], (uint32_t)F,
+            layout_.seg_base[k]);
+      }
+    }
+    tock(&times.assemble);
+    ND_HIP_TRY(hipGetLastError());
     ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
@@ -573,13 +720,15 @@ class Engine : public EngineBase {
     release(d_col_);
     release(d_weight_);
     release(d_max_weight_);
+    release(d_paired_);
+    release(d_edge_table_);
   }
 
   void free_run_buffers() {
     release(d_initial_);
     release(d_samples_);
     release(d_final_);
-    release(d_map_);
+    release(d_step_out_);
     release(d_keys_a_);
     release(d_vals_a_);
     release(d_keys_b_);
@@ -608,6 +757,8 @@ class Engine : public EngineBase {
   VertexID* d_col_ = nullptr;
   float* d_weight_ = nullptr;
   float* d_max_weight_ = nullptr;
+  EdgeRecord* d_paired_ = nullptr;
+  unsigned long long* d_edge_table_ = nullptr;
 
   std::vector<SampleType> samples_;
   int64_t n_samples_ = 0;
@@ -617,6 +768,8 @@ class Engine : public EngineBase {
   uint64_t seed_ = 0;
   size_t max_pairs_ = 0;
   uint32_t chunk_capacity_ = 0;
+  uint32_t row_pitch_ = 0, rows_per_block_ = 0;
+  StepLayout layout_{};
   bool allocated_ = false;
 
   hipStream_t stream_ = nullptr;
@@ -624,7 +777,7 @@ class Engine : public EngineBase {
   VertexID_t* d_initial_ = nullptr;
   SampleType* d_samples_ = nullptr;
   VertexID_t* d_final_ = nullptr;
-  int32_t* d_map_ = nullptr;
+  VertexID_t* d_step_out_ = nullptr;
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
