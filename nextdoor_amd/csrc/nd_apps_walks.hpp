@@ -180,19 +180,28 @@ struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
       return transitEdges[0];
     }
     const float p = 2.0f, q = 0.5f;
-    const float envelope = max_weight * fmaxf(fmaxf(p, 1 / q), 1.0f);
-    const VertexID prev = sample->t;
+    const float h_max = fmaxf(fmaxf(p, 1 / q), 1.0f), h_min = fminf(fminf(p, 1 / q), 1.0f);
+    const float envelope = max_weight * h_max;
+    VertexID prev = -1;  // read from the sample only when a decision depends on it
     for (;;) {
       const EdgePos_t x = RandNumGen::rand_int(state, numEdges);
       const VertexID v = transitEdges[x];
       const float wx = transitEdgeWeights[x];
       const float y = curand_uniform(state) * envelope;
-      float h = 1.0f;
-      if (step != 0) {
+      // h is one of {p, 1/q, 1}: when y is below h_min * w or not below h_max * w the
+      // outcome does not depend on which, and the adjacency test is skipped
+      bool accept;
+      if (step == 0) accept = y < wx;
+      else if (y < h_min * wx) accept = true;
+      else if (!(y < h_max * wx)) accept = false;
+      else {
+        if (prev < 0) prev = sample->t;
+        float h = 1.0f;
         if (v == prev) h = p;
         else if (csr->has_edge_logn(prev, v)) h = 1 / q;
+        accept = y < h * wx;
       }
-      if (y < h * wx) {
+      if (accept) {
         sample->t = *transits;
         return v;
       }

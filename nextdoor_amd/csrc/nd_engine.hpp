@@ -109,7 +109,6 @@ struct StepParams {
                                  // per sample at the end, this step's segment of the result
   void* samples;                 // SampleType[S] or nullptr
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
-  uint32_t blocks_per_xcd;       // flat kernel: workgroups each XCD handles (see flat_block_index)
 };
 
 constexpr int kStepThreads = 256;
@@ -143,12 +142,18 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
 }
 
 constexpr uint32_t kXcds = 8;
+// Consecutive workgroups (in sorted-pair order) one XCD handles before the next XCD takes over.
+constexpr uint32_t kXcdRun = 16;
 
 // Workgroups are handed to the 8 XCDs round-robin (workgroup b runs on XCD b % 8), each XCD
-// with its own L2.  The pairs are sorted by transit, so giving every XCD one CONTIGUOUS
-// eighth of the pairs keeps the adjacency of a hot transit in one L2 instead of all eight.
-__device__ __forceinline__ uint32_t flat_block_index(uint32_t blocks_per_xcd) {
-  return (blockIdx.x % kXcds) * blocks_per_xcd + blockIdx.x / kXcds;
+// with its own L2.  The pairs are sorted by transit, so an XCD is given runs of kXcdRun
+// CONSECUTIVE workgroups' worth of pairs: samples of one hot transit then mostly share one
+// L2, while the runs still interleave finely enough that all XCDs get equal shares of the
+// live prefix and of the INVALID tail of the sorted map.
+__device__ __forceinline__ uint32_t flat_block_index() {
+  const uint32_t xcd = blockIdx.x % kXcds;
+  const uint32_t turn = blockIdx.x / kXcds;  // how many workgroups this XCD has started before
+  return (turn / kXcdRun) * (kXcds * kXcdRun) + xcd * kXcdRun + turn % kXcdRun;
 }
 
 // One lane per output: lane i draws neighbour (i % m) for pair (i / m).  With the map
@@ -157,7 +162,7 @@ __device__ __forceinline__ uint32_t flat_block_index(uint32_t blocks_per_xcd) {
 template <class SampleType, class App>
 __global__ __launch_bounds__(kStepThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
   const uint64_t total = (uint64_t)P.n_pairs * P.step_size;
-  const uint64_t i = (uint64_t)flat_block_index(P.blocks_per_xcd) * kStepThreads + threadIdx.x;
+  const uint64_t i = (uint64_t)flat_block_index() * kStepThreads + threadIdx.x;
   if (i >= total) return;
   CSRPartition csr = P.csr;
   const uint32_t pair = P.step_size == 1 ? (uint32_t)i : (uint32_t)(i / P.step_size);
@@ -600,8 +605,8 @@ class Engine : public EngineBase {
       P.paired_edges = d_paired_;
       const uint64_t outputs = (uint64_t)n_pairs * m;
       const uint32_t flat_blocks = (uint32_t)((outputs + kStepThreads - 1) / kStepThreads);
-      P.blocks_per_xcd = (flat_blocks + kXcds - 1) / kXcds;
-      const unsigned flat_grid = P.blocks_per_xcd * kXcds;
+      // whole groups of kXcds * kXcdRun workgroups, so that flat_block_index is a bijection
+      const unsigned flat_grid = (flat_blocks + kXcds * kXcdRun - 1) / (kXcds * kXcdRun) * (kXcds * kXcdRun);
 
       if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
