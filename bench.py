@@ -24,6 +24,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes one launch of the dominant kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
+# this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
+# known size).  None where no such run has been recorded.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"weighted_node2vec_rmat22": 1.555e9}
+
 WORKLOADS = {
     # name: (app, graph factory kwargs)
     "weighted_node2vec_rmat22": dict(app="WeightedNode2Vec", kind="WEIGHTED_NODE2VEC",
@@ -163,7 +168,8 @@ def main():
         achieved = step_bytes / (step_ms / 1000.0) / 1e9
         result["roofline"] = {
             "bound": "hbm", "kernel": "step_flat_kernel + step_workgroup_kernel", "achieved": achieved,
-            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "algorithmic_bytes_per_launch": step_bytes / max(launches, 1), "avg_launch_ms": step_ms / max(launches, 1),
             "whole_pass": {"algorithmic_bytes": step_bytes + sort_bytes,
                            "achieved_GBps": (step_bytes + sort_bytes) / (np.mean(gpu_ms) / 1000.0) / 1e9,

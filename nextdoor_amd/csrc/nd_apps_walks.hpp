@@ -74,16 +74,21 @@ struct HundredWalksOnSmallGraphs : WalkCommon<kWalkLength> {
 
 // Rejection sampling of an edge proportionally to its weight, against the largest
 // weight of the transit (randomWalks.cu:81-88).  Returns the accepted edge index.
+// Candidate i consumes draws 2i (edge index) and 2i+1 (height), exactly as the loop in
+// the reference; two candidates are drawn and their weights gathered together so the two
+// memory accesses overlap, and the second is simply not used when the first is accepted.
 template <typename WeightArray>
 __device__ __forceinline__ EdgePos_t weighted_edge_by_rejection(const WeightArray& w, EdgePos_t n, float max_weight,
                                                                 curandState* state) {
-  EdgePos_t x = RandNumGen::rand_int(state, n);
-  float y = curand_uniform(state) * max_weight;
-  while (y > w[x]) {
-    x = RandNumGen::rand_int(state, n);
-    y = curand_uniform(state) * max_weight;
+  for (;;) {
+    const EdgePos_t x0 = RandNumGen::rand_int(state, n);
+    const float y0 = curand_uniform(state) * max_weight;
+    const EdgePos_t x1 = RandNumGen::rand_int(state, n);
+    const float y1 = curand_uniform(state) * max_weight;
+    const float w0 = w[x0], w1 = w[x1];
+    if (!(y0 > w0)) return x0;
+    if (!(y1 > w1)) return x1;
   }
-  return x;
 }
 
 }  // namespace apps
@@ -183,27 +188,35 @@ struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
     const float h_max = fmaxf(fmaxf(p, 1 / q), 1.0f), h_min = fminf(fminf(p, 1 / q), 1.0f);
     const float envelope = max_weight * h_max;
     VertexID prev = -1;  // read from the sample only when a decision depends on it
+    // h is one of {p, 1/q, 1}: a height below h_min * w is accepted and one not below
+    // h_max * w rejected whatever h is, so only the band in between needs the adjacency test
+    auto accepts = [&](VertexID v, float wx, float y) -> bool {
+      if (step == 0) return y < wx;  // no previous vertex yet: h = 1
+      if (y < h_min * wx) return true;
+      if (!(y < h_max * wx)) return false;
+      if (prev < 0) prev = sample->t;
+      float h = 1.0f;
+      if (v == prev) h = p;
+      else if (csr->has_edge_logn(prev, v)) h = 1 / q;
+      return y < h * wx;
+    };
+    // candidate i consumes draws 2i (edge index) and 2i+1 (height); two candidates are
+    // drawn and gathered together so their memory accesses overlap, and the second is not
+    // used when the first is accepted
     for (;;) {
-      const EdgePos_t x = RandNumGen::rand_int(state, numEdges);
-      const VertexID v = transitEdges[x];
-      const float wx = transitEdgeWeights[x];
-      const float y = curand_uniform(state) * envelope;
-      // h is one of {p, 1/q, 1}: when y is below h_min * w or not below h_max * w the
-      // outcome does not depend on which, and the adjacency test is skipped
-      bool accept;
-      if (step == 0) accept = y < wx;
-      else if (y < h_min * wx) accept = true;
-      else if (!(y < h_max * wx)) accept = false;
-      else {
-        if (prev < 0) prev = sample->t;
-        float h = 1.0f;
-        if (v == prev) h = p;
-        else if (csr->has_edge_logn(prev, v)) h = 1 / q;
-        accept = y < h * wx;
-      }
-      if (accept) {
+      const EdgePos_t x0 = RandNumGen::rand_int(state, numEdges);
+      const float y0 = curand_uniform(state) * envelope;
+      const EdgePos_t x1 = RandNumGen::rand_int(state, numEdges);
+      const float y1 = curand_uniform(state) * envelope;
+      const VertexID v0 = transitEdges[x0], v1 = transitEdges[x1];
+      const float w0 = transitEdgeWeights[x0], w1 = transitEdgeWeights[x1];
+      if (accepts(v0, w0, y0)) {
         sample->t = *transits;
-        return v;
+        return v0;
+      }
+      if (accepts(v1, w1, y1)) {
+        sample->t = *transits;
+        return v1;
       }
     }
   }

@@ -174,7 +174,7 @@ struct LdsBackedArray {
 // Optional compile-time hints an App may carry; absent members mean `false`.
 //   static constexpr bool kUsesEdgeWeights = true;  -> next() reads transitEdgeWeights: the
 //        engine keeps an interleaved (destination, weight) copy of the edges so that one
-//        8-byte gather serves both arrays, and stages weights in LDS as well
+//        8-byte record serves both arrays, and stages weights in LDS as well
 //   static constexpr bool kUsesEdgeLookup = true;   -> next() calls csr->has_edge_logn: the
 //        engine builds the exact edge index behind it
 template <typename App, typename = void>
@@ -186,35 +186,22 @@ struct app_uses_edge_lookup { static constexpr bool value = false; };
 template <typename App>
 struct app_uses_edge_lookup<App, decltype((void)App::kUsesEdgeLookup)> { static constexpr bool value = App::kUsesEdgeLookup; };
 
-// Interleaved edge record and the two array views over it.  Both views share a one-entry
-// cache, so transitEdges[x] and transitEdgeWeights[x] cost one 8-byte load whichever
-// comes first.
+// Interleaved edge record and the two array views over it: transitEdges[x] and
+// transitEdgeWeights[x] read the two halves of one 8-byte record, i.e. one memory line
+// instead of one line in each of two arrays.
 struct EdgeRecord {
   VertexID dst;
   float weight;
 };
 
-struct EdgeRecordCursor {
-  const EdgeRecord* base;
-  EdgePos_t index;
-  EdgeRecord record;
-  __device__ __forceinline__ const EdgeRecord& at(EdgePos_t i) {
-    if (i != index) {
-      record = base[i];
-      index = i;
-    }
-    return record;
-  }
-};
-
 struct PairedEdgeIds {
-  EdgeRecordCursor* cursor;
-  __device__ __forceinline__ VertexID operator[](EdgePos_t i) const { return cursor->at(i).dst; }
+  const EdgeRecord* base;
+  __device__ __forceinline__ VertexID operator[](EdgePos_t i) const { return base[i].dst; }
 };
 
 struct PairedEdgeWeights {
-  EdgeRecordCursor* cursor;
-  __device__ __forceinline__ float operator[](EdgePos_t i) const { return cursor->at(i).weight; }
+  const EdgeRecord* base;
+  __device__ __forceinline__ float operator[](EdgePos_t i) const { return base[i].weight; }
 };
 
 }  // namespace nd

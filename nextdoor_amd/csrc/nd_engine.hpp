@@ -178,9 +178,8 @@ __global__ __launch_bounds__(kStepThreads) void step_flat_kernel(StepParams P, c
     max_weight = csr.max_weights[transit];
   }
   if (app_uses_weights<App>::value) {
-    EdgeRecordCursor cursor{P.paired_edges + begin, -1, {}};
-    PairedEdgeIds edges{&cursor};
-    PairedEdgeWeights weights{&cursor};
+    PairedEdgeIds edges{P.paired_edges + begin};
+    PairedEdgeWeights weights{P.paired_edges + begin};
     produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, slot, nbr, n_edges, max_weight,
                                                                       edges, weights);
   } else {
