@@ -89,10 +89,18 @@ int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
 /* The per-phase wall-clock breakdown the reference prints (src/nextdoor.cu:2963-2966),
  * measured with events on the sampler's stream when profiling is on.
  * out[0] end to end, [1] inversion, [2] load balancing, [3] flat (identity / sub-wavefront)
- * kernel, [4] workgroup + grid-wide kernel, [8] final-row assembly, all in milliseconds;
- * [5] flat launches, [6] workgroup launches, [7] sort passes; [9..11] reserved (0). */
+ * kernel, [4] workgroup + grid-wide kernel, [8] final-row assembly, [9] the last distinct pass, all in
+ * milliseconds; [5] flat launches, [6] workgroup launches, [7] sort passes; [10..11] reserved (0). */
 int nd_sampler_set_profiling(nd_sampler* s, int on);
 int nd_sampler_phase_times(const nd_sampler* s, float out[12]);
+/* Distinct post-pass for SampledVertices results (GraphSAGE: draw with replacement, then
+ * distinct): every hop segment of every sample is replaced, on the device, by its ascending
+ * unique valid ids packed left and INVALID-padded; counts[sample * steps + hop] = ids kept.
+ * The reference's k-hop app does not deduplicate; the behaviour follows its unused helper
+ * remove_duplicates_in_hop_per_block, src/distinct.cuh:1-111.  Call after
+ * nd_sampler_do_transit_parallel; nd_sampler_get_final_samples then returns the packed rows. */
+int nd_sampler_distinct(nd_sampler* s);
+int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length);
 /* freeDeviceData(data), src/nextdoor.cu:2088-2115. */
 void nd_sampler_free_device(nd_sampler* s);
 void nd_sampler_destroy(nd_sampler* s);

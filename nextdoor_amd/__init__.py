@@ -180,6 +180,13 @@ class Sampler:
         flat = np.ctypeslib.as_array(p, shape=(n.value,)).copy()
         return flat.reshape(self.num_samples, self.final_sample_size)
 
+    def distinct(self):
+        """Distinct post-pass on the device rows; returns counts[num_samples, steps]."""
+        check(lib().nd_sampler_distinct(self._h))
+        p, n = C.POINTER(C.c_int32)(), C.c_int64()
+        check(lib().nd_sampler_get_distinct_counts(self._h, C.byref(p), C.byref(n)))
+        return np.ctypeslib.as_array(p, shape=(n.value,)).copy().reshape(self.num_samples, self.steps)
+
     def sample_states(self):
         nbytes = lib().nd_sampler_sample_state_bytes(self._h)
         if nbytes <= 0:
@@ -195,8 +202,8 @@ class Sampler:
         out = (C.c_float * 12)()
         check(lib().nd_sampler_phase_times(self._h, out))
         keys = ["end_to_end_ms", "inversion_ms", "load_balancing_ms", "flat_kernel_ms", "workgroup_kernel_ms",
-                "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms"]
-        return dict(zip(keys, list(out)[:9]))
+                "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms", "distinct_ms"]
+        return dict(zip(keys, list(out)[:10]))
 
     def free_device(self):
         lib().nd_sampler_free_device(self._h)

@@ -57,6 +57,8 @@ const AppEntry kApps[] = {
     {"WeightedNode2Vec8", make_engine<Node2VecSample, WeightedNode2VecAppT<8>>},
     {"KHop3x2", make_engine<KHopSample, KHopAppT<3, 2>>},
     {"KHop4x3x2", make_engine<KHopSample, KHopAppT<4, 3, 2>>},
+    {"KHop40x30", make_engine<KHopSample, KHopAppT<40, 30>>},
+    {"KHop10x10", make_engine<KHopSample, KHopAppT<10, 10>>},
 };
 constexpr int kNumApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
 
@@ -242,7 +244,21 @@ int nd_sampler_phase_times(const nd_sampler* s, float out[12]) {
   out[4] = t.workgroup_kernel; out[5] = (float)t.flat_launches; out[6] = (float)t.workgroup_launches;
   out[7] = (float)t.sort_launches;
   out[8] = t.assemble;
-  out[9] = out[10] = out[11] = 0.0f;
+  out[9] = t.distinct;
+  out[10] = out[11] = 0.0f;
+  return 0;
+}
+
+int nd_sampler_distinct(nd_sampler* s) {
+  if (!s) return fail("null sampler");
+  const int rc = s->engine->distinct();
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
+int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length) {
+  if (!s || !data || !length) return fail("null argument");
+  *data = s->engine->hDistinctCounts.data();
+  *length = (int64_t)s->engine->hDistinctCounts.size();
   return 0;
 }
 

@@ -33,6 +33,7 @@
 #include <vector>
 
 #include "nd_contract.hpp"
+#include "nd_distinct.hpp"
 #include "nd_radix_sort.hpp"
 #include "nd_transit_runs.hpp"
 
@@ -45,7 +46,7 @@ namespace nd {
 enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1 };
 
 struct PhaseTimes {  // milliseconds, accumulated over one sample() call when profiling is on
-  float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0, assemble = 0;
+  float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0, assemble = 0, distinct = 0;
   int flat_launches = 0, workgroup_launches = 0, sort_launches = 0;
 };
 
@@ -68,9 +69,11 @@ class EngineBase {
   virtual int max_bits() const = 0;
   virtual size_t sample_state_bytes() const = 0;
   virtual int fetch_sample_states(void* dst, size_t bytes) = 0;
+  virtual int distinct() = 0;
 
   std::vector<VertexID_t> hFinalSamples;       // as NextDoorData::hFinalSamples (libNextDoor.hpp:17)
   std::vector<VertexID_t> initialContents;     // as NextDoorData::initialContents (libNextDoor.hpp:18)
+  std::vector<int32_t> hDistinctCounts;        // [num_samples * steps] ids kept by distinct()
   std::string last_error;
   bool profiling = false;
   PhaseTimes times;
@@ -695,6 +698,36 @@ class Engine : public EngineBase {
     return 0;
   }
 
+  // Distinct post-pass over the device-resident result rows (see nd_distinct.hpp): every
+  // hop segment of every sample becomes its ascending unique valid ids, INVALID-padded.
+  int distinct() override {
+    if (!allocated_) { last_error = "distinct before alloc"; return -1; }
+    App app;
+    if (app.outputFormat() != SampledVertices) { last_error = "distinct needs SampledVertices output"; return -2; }
+    const int n_steps = app.steps();
+    if (!d_distinct_counts_) {
+      ND_HIP_TRY(hipMalloc(&d_distinct_counts_, sizeof(int32_t) * (size_t)n_samples_ * n_steps));
+    }
+    times.distinct = 0;
+    ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
+    for (int k = 0; k < n_steps; ++k) {
+      if (!launch_distinct_segment(d_final_, d_distinct_counts_, (uint32_t)n_samples_, (uint32_t)final_sample_size(),
+                                   layout_.seg_base[k], layout_.seg_len[k], invalid_, (uint32_t)n_steps, (uint32_t)k,
+                                   stream_)) {
+        last_error = "a hop segment is longer than 4096 ids";
+        return -2;
+      }
+    }
+    ND_HIP_TRY(hipGetLastError());
+    ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventElapsedTime(&times.distinct, ev_begin_, ev_end_));
+    hDistinctCounts.resize((size_t)n_samples_ * n_steps);
+    ND_HIP_TRY(hipMemcpy(hDistinctCounts.data(), d_distinct_counts_, sizeof(int32_t) * hDistinctCounts.size(),
+                         hipMemcpyDeviceToHost));
+    return 0;
+  }
+
   void free_device() override {
     free_run_buffers();
     free_graph();
@@ -744,6 +777,7 @@ class Engine : public EngineBase {
     release(d_meta_);
     release(d_chunks_);
     release(d_skip_flag_);
+    release(d_distinct_counts_);
     if (allocated_) {
       (void)hipEventDestroy(ev_a_);
       (void)hipEventDestroy(ev_b_);
@@ -790,6 +824,7 @@ class Engine : public EngineBase {
   RunsMeta* d_meta_ = nullptr;
   uint32_t* d_chunks_ = nullptr;
   uint8_t* d_skip_flag_ = nullptr;
+  int32_t* d_distinct_counts_ = nullptr;
 };
 
 }  // namespace nd

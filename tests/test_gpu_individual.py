@@ -118,3 +118,24 @@ def test_runs_are_reproducible_and_seed_matters(oracle):
     c = s2.final_samples()
     s2.close()
     assert np.array_equal(a, b) and not np.array_equal(a, c)
+
+
+@pytest.mark.parametrize("app,gname", [("KHop", "dense_hub"), ("KHop", "sparse"), ("KHop4x3x2", "dense_hub"),
+                                       ("KHop3x2", "sparse"), ("KHop40x30", "dense_hub"),
+                                       ("KHop10x10", "dense_hub")])
+def test_distinct_matches_oracle(oracle, app, gname):
+    g = graphs.random_graph(**GRAPHS[gname])
+    s = nd.Sampler(app, g, seed=SEED)
+    d = desc_for(oracle, s, oracle.KHOP)
+    s.do_transit_parallel(True)
+    raw = s.final_samples()
+    counts = s.distinct()
+    got = s.final_samples()
+    want, want_counts = oracle.distinct(d, raw, s.invalid_vertex)
+    assert np.array_equal(got, want) and np.array_equal(counts, want_counts)
+    # idempotent, and nothing but duplicates was dropped
+    counts2 = s.distinct()
+    assert np.array_equal(s.final_samples(), want) and np.array_equal(counts2, counts)
+    for row_raw, row in zip(raw[:50], got[:50]):
+        assert set(row_raw[row_raw != s.invalid_vertex]) == set(row[row != s.invalid_vertex])
+    s.close()
