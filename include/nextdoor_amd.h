@@ -137,6 +137,16 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
 int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
                        int32_t* offsets, int64_t* n_runs, int64_t* n_valid);
 
+/* collectiveNeighbrsSize + collectiveNeighborhood (src/nextdoor.cu:1206-1283) for n_samples
+ * samples of transits_per_sample transits each (transits[s * transits_per_sample + i]):
+ * sizes[s] = sum of the degrees of the valid transits, offsets = their exclusive scan
+ * (offsets[n_samples] = total), cols / weights = the adjacencies concatenated in transit
+ * order at offsets[s], row_offsets[s * transits_per_sample + i] = start of transit i inside
+ * its sample's concatenation.  Fails when the total exceeds capacity. */
+int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64_t n_samples,
+                               int32_t transits_per_sample, int32_t invalid, int32_t* sizes, int32_t* offsets,
+                               int32_t* cols, float* weights, int64_t capacity, int32_t* row_offsets);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,7 +22,7 @@ from . import _capi
 from ._capi import NextDoorError, check, lib
 
 __all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
-           "sort_pairs", "unique_transits"]
+           "sort_pairs", "unique_transits", "collective_neighborhood"]
 
 
 def app_names():
@@ -278,3 +278,18 @@ def unique_transits(sorted_keys, invalid):
                                    _ptr(offsets, C.c_int32), C.byref(n_runs), C.byref(n_valid)))
     r = n_runs.value
     return uniq[:r], counts[:r], offsets[:r], n_valid.value
+
+
+def collective_neighborhood(graph, transits, transits_per_sample, invalid, capacity):
+    """sizes, offsets, cols, weights, row_offsets of the collective neighbourhoods of the
+    samples whose transits are the rows of `transits`."""
+    t = _as(transits, np.int32).reshape(-1, transits_per_sample)
+    n = t.shape[0]
+    sizes, offsets = np.empty(n, np.int32), np.empty(n + 1, np.int32)
+    cols, weights = np.empty(capacity, np.int32), np.empty(capacity, np.float32)
+    rows = np.empty(n * transits_per_sample, np.int32)
+    check(lib().nd_collective_neighborhood(graph._h, _ptr(t, C.c_int32), n, transits_per_sample, invalid,
+                                           _ptr(sizes, C.c_int32), _ptr(offsets, C.c_int32), _ptr(cols, C.c_int32),
+                                           _ptr(weights, C.c_float), capacity, _ptr(rows, C.c_int32)))
+    total = int(offsets[n])
+    return sizes, offsets, cols[:total], weights[:total], rows.reshape(n, transits_per_sample)

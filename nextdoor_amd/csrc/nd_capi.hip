@@ -8,8 +8,10 @@
 #include <vector>
 
 #include "nd_apps_khop.hpp"
+#include "nd_apps_layer.hpp"
 #include "nd_apps_walks.hpp"
 #include "nd_engine.hpp"
+#include "nd_layer_engine.hpp"
 #include "nd_graph.hpp"
 
 struct nd_graph {
@@ -40,6 +42,11 @@ nd::EngineBase* make_engine(const char* name) {
   return new nd::Engine<SampleType, App>(name);
 }
 
+template <class SampleType, class App>
+nd::EngineBase* make_layer_engine(const char* name) {
+  return new nd::LayerEngine<SampleType, App>(name);
+}
+
 // name -> instantiation.  The first block carries the reference's app names and sizes.
 const AppEntry kApps[] = {
     {"UniformRandomWalk", make_engine<UniformRandomWalkSample, UniformRandomWalkApp>},
@@ -59,6 +66,15 @@ const AppEntry kApps[] = {
     {"KHop4x3x2", make_engine<KHopSample, KHopAppT<4, 3, 2>>},
     {"KHop40x30", make_engine<KHopSample, KHopAppT<40, 30>>},
     {"KHop10x10", make_engine<KHopSample, KHopAppT<10, 10>>},
+    // layer-wise apps: the reference's FastGCN / LADIES (5 layers of 64, 10000 samples) ...
+    {"FastGCN", make_layer_engine<FastGCNSample, FastGCNSamplingApp>},
+    {"LADIES", make_layer_engine<ImportanceSample, ImportanceSampleApp>},
+    {"LayerLiteral2x8", make_layer_engine<LayerSampleT<2, 8>, LayerSamplingAppT<2, 8, 50>>},
+    {"LayerLiteral3x16", make_layer_engine<LayerSampleT<3, 16>, LayerSamplingAppT<3, 16, 200>>},
+    // ... and importance sampling over the union neighbourhood
+    {"FastGCNImportance", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 64, 4096>>},
+    {"FastGCNImportance2x8", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 8, 100>>},
+    {"FastGCNImportance3x16", make_layer_engine<LayerNoState, FastGCNImportanceAppT<3, 16, 300>>},
 };
 constexpr int kNumApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
 
@@ -388,6 +404,45 @@ int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, i
     CAPI_HIP(hipMemcpy(counts, run_count.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
     CAPI_HIP(hipMemcpy(offsets, run_start.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
   }
+  return 0;
+}
+
+int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64_t n_samples,
+                               int32_t transits_per_sample, int32_t invalid, int32_t* sizes, int32_t* offsets,
+                               int32_t* cols, float* weights, int64_t capacity, int32_t* row_offsets) {
+  if (!g || !transits || n_samples < 1 || transits_per_sample < 1 || !sizes || !offsets || !cols || !weights ||
+      !row_offsets || (uint32_t)transits_per_sample > nd::kMaxLayerTransits || n_samples >= (1ll << 31))
+    return fail("bad argument");
+  nd::DeviceGraph dg;
+  std::string err;
+  if (!dg.upload(&g->csr, false, false, &err)) return fail(err);
+  const uint32_t S = (uint32_t)n_samples;
+  const size_t n_tr = (size_t)S * transits_per_sample;
+  DeviceBuffer d_tr, d_sizes, d_offsets, d_scratch, d_cols, d_weights, d_rows;
+  CAPI_HIP(d_tr.alloc(sizeof(int32_t) * n_tr));
+  CAPI_HIP(d_sizes.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+  CAPI_HIP(d_offsets.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+  CAPI_HIP(d_scratch.alloc(sizeof(uint32_t) * nd::scan_scratch_elems((size_t)S + 1)));
+  CAPI_HIP(d_rows.alloc(sizeof(uint32_t) * n_tr));
+  CAPI_HIP(hipMemcpy(d_tr.p, transits, sizeof(int32_t) * n_tr, hipMemcpyHostToDevice));
+  CAPI_HIP(hipMemset(d_sizes.p, 0, sizeof(uint32_t) * ((size_t)S + 1)));
+  nd::TransitView tv{d_tr.as<int32_t>(), (uint32_t)transits_per_sample, (uint32_t)transits_per_sample};
+  nd::collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, 0>>>(dg.view, tv, S, invalid, d_sizes.as<uint32_t>());
+  CAPI_HIP(nd::exclusive_scan_u32(d_sizes.as<uint32_t>(), d_offsets.as<uint32_t>(), (size_t)S + 1,
+                                  d_scratch.as<uint32_t>(), 0));
+  CAPI_HIP(hipMemcpy(sizes, d_sizes.p, sizeof(uint32_t) * S, hipMemcpyDeviceToHost));
+  CAPI_HIP(hipMemcpy(offsets, d_offsets.p, sizeof(uint32_t) * ((size_t)S + 1), hipMemcpyDeviceToHost));
+  const int64_t total = offsets[S];
+  if (total > capacity) return fail("collective neighbourhood larger than the capacity given");
+  CAPI_HIP(d_cols.alloc(sizeof(int32_t) * (size_t)total));
+  CAPI_HIP(d_weights.alloc(sizeof(float) * (size_t)total));
+  nd::collective_build<<<dim3(S), dim3(256), 0, 0>>>(dg.view, tv, invalid, d_offsets.as<uint32_t>(),
+                                                    d_cols.as<int32_t>(), d_weights.as<float>(), nullptr,
+                                                    d_rows.as<uint32_t>());
+  CAPI_HIP(hipGetLastError());
+  CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
+  CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));
+  CAPI_HIP(hipMemcpy(row_offsets, d_rows.p, sizeof(uint32_t) * n_tr, hipMemcpyDeviceToHost));
   return 0;
 }
 

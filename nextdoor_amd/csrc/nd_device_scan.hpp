@@ -100,7 +100,101 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply(const uint32_t* __res
   }
 }
 
+// ---- 64-bit inclusive prefix sum (same three-launch scheme) ----
+
+__device__ __forceinline__ uint64_t wave_inclusive_scan_u64(uint64_t v) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t lo = __shfl_up((uint32_t)v, d, kWave);
+    const uint32_t hi = __shfl_up((uint32_t)(v >> 32), d, kWave);
+    if (lane >= d) v += ((uint64_t)hi << 32) | lo;
+  }
+  return v;
+}
+
+// Exclusive scan of one uint64 per thread across a 256-thread workgroup (two barriers).
+__device__ __forceinline__ uint64_t block_exclusive_scan_256_u64(uint64_t v, uint64_t* s_wave_totals,
+                                                                 uint64_t* block_total) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const uint64_t incl = wave_inclusive_scan_u64(v);
+  if (lane == kWave - 1) s_wave_totals[wave] = incl;
+  __syncthreads();
+  uint64_t before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / kWave; ++w) {
+    const uint64_t t = s_wave_totals[w];
+    if (w < wave) before += t;
+    total += t;
+  }
+  __syncthreads();
+  *block_total = total;
+  return before + incl - v;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan64_tile_totals(const uint64_t* __restrict__ in, size_t n,
+                                                                   uint64_t* __restrict__ tile_totals) {
+  __shared__ uint64_t s_wave[kScanThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * kScanTile;
+  uint64_t sum = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    const size_t idx = base + (size_t)i * kScanThreads + threadIdx.x;
+    if (idx < n) sum += in[idx];
+  }
+  uint64_t total;
+  block_exclusive_scan_256_u64(sum, s_wave, &total);
+  if (threadIdx.x == 0) tile_totals[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan64_of_totals(uint64_t* __restrict__ tile_totals, size_t num_tiles) {
+  __shared__ uint64_t s_wave[kScanThreads / kWave];
+  uint64_t carry = 0;
+  for (size_t start = 0; start < num_tiles; start += kScanThreads) {
+    const size_t idx = start + threadIdx.x;
+    const uint64_t v = idx < num_tiles ? tile_totals[idx] : 0ull;
+    uint64_t total;
+    const uint64_t excl = block_exclusive_scan_256_u64(v, s_wave, &total);
+    if (idx < num_tiles) tile_totals[idx] = carry + excl;
+    carry += total;
+  }
+  if (threadIdx.x == 0) tile_totals[num_tiles] = carry;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan64_apply_inclusive(const uint64_t* __restrict__ in,
+                                                                       uint64_t* __restrict__ out, size_t n,
+                                                                       const uint64_t* __restrict__ tile_offsets) {
+  __shared__ uint64_t s_wave[kScanThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
+  uint64_t v[kScanItems];
+  uint64_t sum = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    v[i] = base + i < n ? in[base + i] : 0ull;
+    sum += v[i];
+  }
+  uint64_t total;
+  uint64_t running = block_exclusive_scan_256_u64(sum, s_wave, &total) + tile_offsets[blockIdx.x];
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    running += v[i];
+    if (base + i < n) out[base + i] = running;
+  }
+}
+
 inline size_t scan_num_tiles(size_t n) { return (n + kScanTile - 1) / kScanTile; }
+
+// out[i] = sum of in[0..i]; in and out may alias.  scratch needs scan_num_tiles(n) + 1 uint64.
+inline hipError_t inclusive_scan_u64(const uint64_t* in, uint64_t* out, size_t n, uint64_t* scratch,
+                                     hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  const size_t tiles = (n + kScanTile - 1) / kScanTile;
+  scan64_tile_totals<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, n, scratch);
+  scan64_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream>>>(scratch, tiles);
+  scan64_apply_inclusive<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, out, n, scratch);
+  return hipGetLastError();
+}
 
 // Scratch needed by exclusive_scan_u32 for n elements, in uint32 units.
 inline size_t scan_scratch_elems(size_t n) { return scan_num_tiles(n) + 1; }

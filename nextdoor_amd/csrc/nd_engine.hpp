@@ -33,6 +33,7 @@
 #include <vector>
 
 #include "nd_contract.hpp"
+#include "nd_device_graph.hpp"
 #include "nd_distinct.hpp"
 #include "nd_radix_sort.hpp"
 #include "nd_transit_runs.hpp"
@@ -283,38 +284,6 @@ __global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Graph-side helpers built once per graph
-// ---------------------------------------------------------------------------------------
-
-__device__ __forceinline__ VertexID source_of_edge(const EdgePos_t* row_ptr, VertexID n_vertices, EdgePos_t e) {
-  // largest v with row_ptr[v] <= e
-  VertexID lo = 0, hi = n_vertices;
-  while (hi - lo > 1) {
-    const VertexID mid = lo + (hi - lo) / 2;
-    if (row_ptr[mid] <= e) lo = mid; else hi = mid;
-  }
-  return lo;
-}
-
-__global__ void build_edge_table(CSRPartition csr, unsigned long long* table, uint32_t mask) {
-  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= (size_t)csr.n_edges) return;
-  const VertexID src = source_of_edge(csr.row_ptr, csr.n_vertices, (EdgePos_t)e);
-  const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)csr.edges[e];
-  uint32_t h = CSRPartition::edge_hash(key) & mask;
-  for (;;) {
-    const unsigned long long seen = atomicCAS(&table[h], ~0ull, key);
-    if (seen == ~0ull || seen == key) return;  // inserted, or a duplicate edge already there
-    h = (h + 1) & mask;
-  }
-}
-
-__global__ void build_paired_edges(const CSR::Edge* col, const float* weight, size_t n, EdgeRecord* out) {
-  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e < n) out[e] = EdgeRecord{col[e], weight[e]};
-}
-
-// ---------------------------------------------------------------------------------------
 // Final-sample assembly
 // ---------------------------------------------------------------------------------------
 
@@ -417,47 +386,10 @@ class Engine : public EngineBase {
   // transferCSRToGPUs: the whole graph is resident on the device, plus the derived
   // structures the app asks for (interleaved edges, edge index).
   int set_graph(const CSR* graph) override {
-    free_graph();
+    graph_ = nullptr;
+    if (!dgraph_.upload(graph, app_uses_weights<App>::value, app_uses_edge_lookup<App>::value, &last_error)) return -1;
     graph_ = graph;
-    const size_t V = (size_t)graph->get_n_vertices();
-    const size_t E = graph->col.size();
-    if (V == 0) { last_error = "graph has no vertices"; return -1; }
-    if (E >= (size_t)INT32_MAX) { last_error = "edge count does not fit int32 edge positions"; return -1; }
-    ND_HIP_TRY(hipMalloc(&d_row_ptr_, sizeof(EdgePos_t) * (V + 1)));
-    ND_HIP_TRY(hipMalloc(&d_col_, sizeof(VertexID) * (E ? E : 1)));
-    ND_HIP_TRY(hipMalloc(&d_weight_, sizeof(float) * (E ? E : 1)));
-    ND_HIP_TRY(hipMalloc(&d_max_weight_, sizeof(float) * V));
-    ND_HIP_TRY(hipMemcpy(d_row_ptr_, graph->row_ptr.data(), sizeof(EdgePos_t) * (V + 1), hipMemcpyHostToDevice));
-    if (E) {
-      ND_HIP_TRY(hipMemcpy(d_col_, graph->col.data(), sizeof(VertexID) * E, hipMemcpyHostToDevice));
-      ND_HIP_TRY(hipMemcpy(d_weight_, graph->weight.data(), sizeof(float) * E, hipMemcpyHostToDevice));
-    }
-    ND_HIP_TRY(hipMemcpy(d_max_weight_, graph->max_weight.data(), sizeof(float) * V, hipMemcpyHostToDevice));
-    view_.row_ptr = d_row_ptr_;
-    view_.edges = d_col_;
-    view_.weights = d_weight_;
-    view_.max_weights = d_max_weight_;
-    view_.n_vertices = (VertexID)V;
-    view_.n_edges = (EdgePos_t)E;
-    view_.edge_table = nullptr;
-    view_.edge_table_mask = 0;
-    if (app_uses_weights<App>::value) {
-      ND_HIP_TRY(hipMalloc(&d_paired_, sizeof(EdgeRecord) * (E ? E : 1)));
-      if (E) build_paired_edges<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(d_col_, d_weight_, E, d_paired_);
-      ND_HIP_TRY(hipGetLastError());
-    }
-    if (app_uses_edge_lookup<App>::value) {
-      // power-of-two table at most half full
-      size_t slots = 16;
-      while (slots < 2 * E) slots <<= 1;
-      ND_HIP_TRY(hipMalloc(&d_edge_table_, sizeof(unsigned long long) * slots));
-      ND_HIP_TRY(hipMemset(d_edge_table_, 0xFF, sizeof(unsigned long long) * slots));
-      if (E) build_edge_table<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(view_, d_edge_table_, (uint32_t)(slots - 1));
-      ND_HIP_TRY(hipGetLastError());
-      view_.edge_table = d_edge_table_;
-      view_.edge_table_mask = (uint32_t)(slots - 1);
-    }
-    ND_HIP_TRY(hipDeviceSynchronize());
+    view_ = dgraph_.view;
     return 0;
   }
 
@@ -531,7 +463,11 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipMemcpy(d_initial_, initialContents.data(), sizeof(VertexID_t) * initialContents.size(),
                          hipMemcpyHostToDevice));
     if (!std::is_empty<SampleType>::value) {
+      // the states initializeSample produced stay on the device; every run starts from a copy
       ND_HIP_TRY(hipMalloc(&d_samples_, sizeof(SampleType) * (size_t)n_samples_));
+      ND_HIP_TRY(hipMalloc(&d_samples_init_, sizeof(SampleType) * (size_t)n_samples_));
+      ND_HIP_TRY(hipMemcpy(d_samples_init_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
+                           hipMemcpyHostToDevice));
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
@@ -578,8 +514,8 @@ class Engine : public EngineBase {
     const size_t F = (size_t)final_sample_size();
     times = PhaseTimes();
     if (!std::is_empty<SampleType>::value) {
-      ND_HIP_TRY(hipMemcpyAsync(d_samples_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
-                                hipMemcpyHostToDevice, stream_));
+      ND_HIP_TRY(hipMemcpyAsync(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
+                                hipMemcpyDeviceToDevice, stream_));
     }
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
@@ -604,7 +540,7 @@ class Engine : public EngineBase {
       P.n_pairs = n_pairs;
       P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
       P.samples = d_samples_;
-      P.paired_edges = d_paired_;
+      P.paired_edges = dgraph_.paired;
       const uint64_t outputs = (uint64_t)n_pairs * m;
       const uint32_t flat_blocks = (uint32_t)((outputs + kStepThreads - 1) / kStepThreads);
       // whole groups of kXcds * kXcdRun workgroups, so that flat_block_index is a bijection
@@ -641,7 +577,7 @@ class Engine : public EngineBase {
                                        d_scratch_, stream_));
           const unsigned max_runs = n_pairs < (uint32_t)invalid_ ? n_pairs : (uint32_t)invalid_;
           classify_runs<<<dim3((max_runs + 255) / 256), dim3(256), 0, stream_>>>(
-              d_run_key_, d_run_start_, d_meta_, d_row_ptr_, m, d_chunks_, chunk_capacity_, d_skip_flag_);
+              d_run_key_, d_run_start_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_, d_skip_flag_);
           tock(&times.load_balancing);
           tick();
           step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, d_skip_flag_);
@@ -753,17 +689,14 @@ class Engine : public EngineBase {
   }
 
   void free_graph() {
-    release(d_row_ptr_);
-    release(d_col_);
-    release(d_weight_);
-    release(d_max_weight_);
-    release(d_paired_);
-    release(d_edge_table_);
+    dgraph_.release();
+    graph_ = nullptr;
   }
 
   void free_run_buffers() {
     release(d_initial_);
     release(d_samples_);
+    release(d_samples_init_);
     release(d_final_);
     release(d_step_out_);
     release(d_keys_a_);
@@ -791,12 +724,7 @@ class Engine : public EngineBase {
   const char* name_;
   const CSR* graph_ = nullptr;
   CSRPartition view_{};
-  EdgePos_t* d_row_ptr_ = nullptr;
-  VertexID* d_col_ = nullptr;
-  float* d_weight_ = nullptr;
-  float* d_max_weight_ = nullptr;
-  EdgeRecord* d_paired_ = nullptr;
-  unsigned long long* d_edge_table_ = nullptr;
+  DeviceGraph dgraph_;
 
   std::vector<SampleType> samples_;
   int64_t n_samples_ = 0;
@@ -814,6 +742,7 @@ class Engine : public EngineBase {
   hipEvent_t ev_a_ = nullptr, ev_b_ = nullptr, ev_begin_ = nullptr, ev_end_ = nullptr;
   VertexID_t* d_initial_ = nullptr;
   SampleType* d_samples_ = nullptr;
+  SampleType* d_samples_init_ = nullptr;
   VertexID_t* d_final_ = nullptr;
   VertexID_t* d_step_out_ = nullptr;
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;

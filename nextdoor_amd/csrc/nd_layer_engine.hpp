@@ -1,0 +1,565 @@
+// Layer-wise (CollectiveNeighborhood) sampling engine for one MI355X (gfx950, wave64).
+//
+// Reference behaviour this covers (file:line in the reference tree):
+//   collective branch of doTransitParallelSampling   src/nextdoor.cu:2402-2453, 2475-2496, 2900-2923
+//   collectiveNeighbrsSize                           src/nextdoor.cu:1206-1246  -> collective_sizes
+//   collectiveNeighborhood                           src/nextdoor.cu:1248-1283  -> collective_build
+//   sampleParallelKernel, Collective branch          src/nextdoor.cu:1394-1446, 1485-1487 -> layer_execute_kernel
+//
+// Per layer k, for every sample s: its transits are the initial vertices (k = 0) or the
+// layer k-1 segment of its result row; the collective neighbourhood is the concatenation
+// of the transits' adjacencies; next() runs once per (sample, nbr < stepSize(k)) and its
+// result goes to final[s * F + stepSizeAtStep(k-1) + nbr].
+//
+// Differences that are deliberate:
+//  * The reference sizes the neighbourhood with a global atomic (offsets in arrival order),
+//    cudaMallocs it inside the step loop and never hands it to next() (transitEdges is
+//    nullptr, nextdoor.cu:1441-1446).  Here offsets are an exclusive scan over samples
+//    (deterministic), the buffers are grown once and reused, and next() receives the
+//    neighbourhood in the form the app declares (nd::apps::NeighborhoodForm).
+//  * For kDistinctByDegreeSquared the concatenation is sorted by (sample, vertex) with two
+//    stable radix sorts, run heads give the distinct vertices, and a 64-bit inclusive scan
+//    of degree^2 gives the running sums the app inverts.
+//  * Random numbers: Philox keyed by the output slot s * stepSize(k) + nbr and the layer.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "nd_apps_layer.hpp"
+#include "nd_contract.hpp"
+#include "nd_device_graph.hpp"
+#include "nd_engine.hpp"
+#include "nd_radix_sort.hpp"
+
+namespace nd {
+
+constexpr uint32_t kMaxLayerTransits = 1024;  // transits of one sample the build kernel stages in LDS
+
+// transits of sample s: base[s * stride + i], i < count
+struct TransitView {
+  const int32_t* base;
+  uint32_t stride;
+  uint32_t count;
+};
+
+// One wave per sample: sum of the degrees of its valid transits.
+__global__ __launch_bounds__(256) void collective_sizes(CSRPartition csr, TransitView tv, uint32_t n_samples,
+                                                        int32_t invalid, uint32_t* __restrict__ sizes) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t s = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (s >= n_samples) return;
+  const int32_t* transits = tv.base + (size_t)s * tv.stride;
+  uint32_t sum = 0;
+  for (uint32_t i = lane; i < tv.count; i += 64u) {
+    const int32_t t = transits[i];
+    if (t != invalid && t != -1) sum += (uint32_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) sum += __shfl_down(sum, d, 64);
+  if (lane == 0) sizes[s] = sum;
+}
+
+// One workgroup per sample: copy the adjacencies of its transits, in transit order, to
+// cols[offsets[s] ...] (and weights, and the owning sample id when asked for).
+__global__ __launch_bounds__(256) void collective_build(CSRPartition csr, TransitView tv, int32_t invalid,
+                                                        const uint32_t* __restrict__ offsets,
+                                                        int32_t* __restrict__ cols, float* __restrict__ weights,
+                                                        uint32_t* __restrict__ sample_of,
+                                                        uint32_t* __restrict__ row_offsets) {
+  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
+  __shared__ uint32_t s_scan_tmp[4];
+  const uint32_t s = blockIdx.x;
+  const int32_t* transits = tv.base + (size_t)s * tv.stride;
+  uint32_t carry = 0;
+  for (uint32_t chunk = 0; chunk < tv.count; chunk += 256) {
+    const uint32_t i = chunk + threadIdx.x;
+    uint32_t deg = 0;
+    if (i < tv.count) {
+      const int32_t t = transits[i];
+      if (t != invalid && t != -1) deg = (uint32_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
+    }
+    uint32_t total;
+    const uint32_t excl = block_exclusive_scan_256(deg, s_scan_tmp, &total);
+    if (i < tv.count) s_start[i] = carry + excl;
+    carry += total;
+  }
+  if (threadIdx.x == 0) s_start[tv.count] = carry;
+  __syncthreads();
+  const uint32_t base = offsets[s];
+  const uint32_t size = s_start[tv.count];
+  if (row_offsets)
+    for (uint32_t i = threadIdx.x; i < tv.count; i += 256) row_offsets[(size_t)s * tv.count + i] = s_start[i];
+  for (uint32_t e = threadIdx.x; e < size; e += 256) {
+    // transit whose range holds e: last i with s_start[i] <= e
+    uint32_t lo = 0, hi = tv.count;
+    while (hi - lo > 1) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (s_start[mid] <= e) lo = mid; else hi = mid;
+    }
+    const int32_t t = transits[lo];
+    const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[lo]);
+    cols[base + e] = csr.edges[src];
+    if (weights) weights[base + e] = csr.weights[src];
+    if (sample_of) sample_of[base + e] = s;
+  }
+}
+
+__global__ void gather_u32(const uint32_t* __restrict__ table, const uint32_t* __restrict__ index, size_t n,
+                           uint32_t* __restrict__ out, uint32_t* __restrict__ index_copy) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t p = index[i];
+  out[i] = table[p];
+  if (index_copy) index_copy[i] = p;
+}
+
+__device__ __forceinline__ bool is_pair_head(const uint32_t* sample_key, const uint32_t* vertex, size_t i) {
+  return i == 0 || sample_key[i] != sample_key[i - 1] || vertex[i] != vertex[i - 1];
+}
+
+__global__ __launch_bounds__(kScanThreads) void count_pair_heads(const uint32_t* __restrict__ sample_key,
+                                                                 const uint32_t* __restrict__ vertex, size_t n,
+                                                                 uint32_t* __restrict__ tile_counts) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * kScanTile;
+  uint32_t heads = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    const size_t idx = base + (size_t)i * kScanThreads + threadIdx.x;
+    if (idx < n && is_pair_head(sample_key, vertex, idx)) heads++;
+  }
+  uint32_t total;
+  block_exclusive_scan_256(heads, s_wave, &total);
+  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+}
+
+// Distinct (sample, vertex) pairs in order: the vertex id, degree^2, and one count per sample.
+__global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_t* __restrict__ sample_key,
+                                                                   const uint32_t* __restrict__ vertex, size_t n,
+                                                                   const uint32_t* __restrict__ tile_offsets,
+                                                                   const EdgePos_t* __restrict__ row_ptr,
+                                                                   int32_t* __restrict__ distinct_ids,
+                                                                   uint64_t* __restrict__ degree_sq,
+                                                                   uint32_t* __restrict__ per_sample_count) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
+  bool head[kScanItems];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    head[i] = base + i < n && is_pair_head(sample_key, vertex, base + i);
+    mine += head[i] ? 1u : 0u;
+  }
+  uint32_t total;
+  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    if (head[i]) {
+      const uint32_t v = vertex[base + i];
+      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+      distinct_ids[r] = (int32_t)v;
+      degree_sq[r] = d * d;
+      atomicAdd(&per_sample_count[sample_key[base + i]], 1u);
+      ++r;
+    }
+  }
+}
+
+__global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
+// running sums of one sample's distinct ids, as the WeightArray handed to next()
+struct SegmentRunningSums {
+  const uint64_t* sums;  // global inclusive sums, already offset to the sample's first distinct id
+  uint64_t before;       // inclusive sum just before the sample's first distinct id
+  __device__ __forceinline__ uint64_t operator[](EdgePos_t i) const { return sums[i] - before; }
+};
+
+struct LayerParams {
+  CSRPartition csr;
+  TransitView transits;
+  int step;
+  uint32_t step_size;
+  uint32_t n_samples;
+  uint32_t final_size;
+  uint32_t out_base;  // stepSizeAtStep(step - 1)
+  int32_t invalid;
+  uint64_t seed;
+  uint64_t first_slot;
+  uint32_t first_sample;
+  int32_t* final_samples;
+  void* samples;
+  // kConcatenated
+  const uint32_t* offsets;
+  const int32_t* nbr_cols;
+  const float* nbr_weights;
+  // kDistinctByDegreeSquared
+  const uint32_t* distinct_start;
+  const int32_t* distinct_ids;
+  const uint64_t* running_sums;
+};
+
+template <class SampleType, class App>
+__global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
+  const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (uint64_t)P.n_samples * P.step_size) return;
+  const uint32_t s = (uint32_t)(i / P.step_size);
+  const uint32_t nbr = (uint32_t)(i - (uint64_t)s * P.step_size);
+  CSRPartition csr = P.csr;
+  const int32_t* transits = P.transits.base + (size_t)s * P.transits.stride;
+  SampleType local_state;
+  SampleType* state = std::is_empty<SampleType>::value ? &local_state : (SampleType*)P.samples + s;
+  curandState rng;
+  rng.reset(P.seed, P.first_slot + i, (uint32_t)P.step);
+  VertexID neighbor = P.invalid;
+  if constexpr (App::kNeighborhoodForm == apps::kConcatenated) {
+    // only the first transit decides whether next() runs (nextdoor.cu:1421)
+    if (transits[0] != P.invalid && transits[0] != -1) {
+      const uint32_t begin = P.offsets[s];
+      const CSR::Edge* edges = P.nbr_cols + begin;
+      const float* weights = P.nbr_weights + begin;
+      const VertexID r = App().template next<SampleType, const CSR::Edge*, const float*>(
+          P.step, &csr, transits, (VertexID)(P.first_sample + s), state, 0.0f, edges, weights,
+          (EdgePos_t)(P.offsets[s + 1] - begin), (VertexID_t)nbr, &rng);
+      neighbor = r == -1 ? P.invalid : r;
+    }
+  } else {
+    const uint32_t begin = P.distinct_start[s];
+    const CSR::Edge* ids = P.distinct_ids + begin;
+    SegmentRunningSums sums{P.running_sums + begin, begin ? P.running_sums[begin - 1] : 0ull};
+    const VertexID r = App().template next<SampleType, const CSR::Edge*, SegmentRunningSums>(
+        P.step, &csr, transits, (VertexID)(P.first_sample + s), state, 0.0f, ids, sums,
+        (EdgePos_t)(P.distinct_start[s + 1] - begin), (VertexID_t)nbr, &rng);
+    neighbor = r == -1 ? P.invalid : r;
+  }
+  P.final_samples[(size_t)s * P.final_size + P.out_base + nbr] = neighbor;
+}
+
+template <class SampleType, class App>
+class LayerEngine : public EngineBase {
+ public:
+  explicit LayerEngine(const char* name) : name_(name) {}
+  ~LayerEngine() override { free_device(); }
+
+  const char* app_name() const override { return name_; }
+  int64_t num_samples() const override { return n_samples_; }
+  int final_sample_size() const override { return nd::final_sample_size<App>(); }
+  int steps() const override { return App().steps(); }
+  int step_size(int k) const override { return App().stepSize(k); }
+  int initial_sample_size() const override { return App().initialSampleSize(nullptr); }
+  int sampling_type() const override { return App().samplingType(); }
+  int32_t invalid_vertex() const override { return invalid_; }
+  int max_bits() const override { return max_bits_; }
+  size_t sample_state_bytes() const override {
+    return std::is_empty<SampleType>::value ? 0 : sizeof(SampleType) * (size_t)n_samples_;
+  }
+
+  int set_graph(const CSR* graph) override {
+    graph_ = nullptr;
+    if (!dgraph_.upload(graph, false, app_uses_edge_lookup<App>::value, &last_error)) return -1;
+    graph_ = graph;
+    return 0;
+  }
+
+  int alloc(uint64_t seed) override {
+    if (!graph_) { last_error = "alloc before set_graph"; return -1; }
+    free_run_buffers();
+    seed_ = seed;
+    CSR* csr = const_cast<CSR*>(graph_);
+    App app;
+    if (!is_collective<App>()) { last_error = "not a CollectiveNeighborhood app"; return -2; }
+    if (app.hasExplicitTransits()) { last_error = "apps with explicit transits are not supported"; return -2; }
+    const int n_steps = app.steps();
+    if (n_steps < 1 || n_steps > kMaxSteps) { last_error = "steps() must be in [1, 128]"; return -2; }
+    n_samples_ = app.numSamples(csr);
+    init_size_ = app.initialSampleSize(csr);
+    if (n_samples_ <= 0 || init_size_ <= 0) { last_error = "app yields no samples"; return -2; }
+    uint32_t widest = (uint32_t)init_size_;
+    for (int k = 0; k < n_steps; ++k) {
+      if (app.stepSize(k) <= 0) { last_error = "stepSize must be positive"; return -2; }
+      if ((uint32_t)app.stepSize(k) > widest) widest = (uint32_t)app.stepSize(k);
+    }
+    if (widest > kMaxLayerTransits) { last_error = "more than 1024 transits per sample"; return -2; }
+    invalid_ = graph_->get_n_vertices();
+    max_bits_ = 0;
+    while ((invalid_ >> max_bits_) != 0) max_bits_++;
+    sample_bits_ = 1;
+    while (((uint64_t)n_samples_ >> sample_bits_) != 0) sample_bits_++;
+
+    samples_.clear();
+    initialContents.clear();
+    samples_.reserve((size_t)n_samples_);
+    for (int64_t s = 0; s < n_samples_; ++s) {
+      samples_.push_back(app.template initializeSample<SampleType>(csr, (VertexID_t)s));
+      std::vector<VertexID_t> roots = app.initialSample((int)s, csr, samples_.back());
+      if ((EdgePos_t)roots.size() != init_size_) {
+        last_error = "initialSample size differs from initialSampleSize";
+        return -2;
+      }
+      initialContents.insert(initialContents.end(), roots.begin(), roots.end());
+    }
+    const size_t F = (size_t)final_sample_size();
+    hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
+
+    ND_HIP_TRY(hipStreamCreate(&stream_));
+    ND_HIP_TRY(hipEventCreate(&ev_begin_));
+    ND_HIP_TRY(hipEventCreate(&ev_end_));
+    allocated_ = true;
+    ND_HIP_TRY(hipMalloc(&d_initial_, sizeof(VertexID_t) * initialContents.size()));
+    ND_HIP_TRY(hipMemcpy(d_initial_, initialContents.data(), sizeof(VertexID_t) * initialContents.size(),
+                         hipMemcpyHostToDevice));
+    if (!std::is_empty<SampleType>::value) {
+      ND_HIP_TRY(hipMalloc(&d_samples_, sizeof(SampleType) * (size_t)n_samples_));
+      ND_HIP_TRY(hipMalloc(&d_samples_init_, sizeof(SampleType) * (size_t)n_samples_));
+      ND_HIP_TRY(hipMemcpy(d_samples_init_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
+                           hipMemcpyHostToDevice));
+      std::vector<SampleType>().swap(samples_);  // the pristine copy now lives on the device
+    }
+    ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
+    ND_HIP_TRY(hipMalloc(&d_sizes_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_offsets_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_row_offsets_, sizeof(uint32_t) * (size_t)n_samples_ * widest));
+    ND_HIP_TRY(hipMalloc(&d_small_scratch_, sizeof(uint32_t) * scan_scratch_elems((size_t)n_samples_ + 1)));
+    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+      ND_HIP_TRY(hipMalloc(&d_distinct_count_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+      ND_HIP_TRY(hipMalloc(&d_distinct_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    }
+    return 0;
+  }
+
+  int sample(int) override {
+    if (!allocated_) { last_error = "sample before alloc"; return -1; }
+    App app;
+    const int n_steps = app.steps();
+    const size_t F = (size_t)final_sample_size();
+    times = PhaseTimes();
+    neighborhood_total_ = 0;
+    distinct_total_ = 0;
+    if (!std::is_empty<SampleType>::value) {
+      ND_HIP_TRY(hipMemcpyAsync(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
+                                hipMemcpyDeviceToDevice, stream_));
+    }
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
+    const uint32_t S = (uint32_t)n_samples_;
+    for (int step = 0; step < n_steps; ++step) {
+      TransitView tv;
+      if (step == 0) {
+        tv.base = d_initial_;
+        tv.stride = (uint32_t)init_size_;
+        tv.count = (uint32_t)init_size_;
+      } else {
+        tv.base = d_final_ + step_size_at_step<App>(step - 2);
+        tv.stride = (uint32_t)F;
+        tv.count = (uint32_t)app.stepSize(step - 1);
+      }
+      // collective neighbourhood: sizes -> offsets -> concatenation
+      collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, stream_>>>(dgraph_.view, tv, S, invalid_, d_sizes_);
+      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_sizes_ + S, 1, 0u);
+      ND_HIP_TRY(exclusive_scan_u32(d_sizes_, d_offsets_, (size_t)S + 1, d_small_scratch_, stream_));
+      uint32_t total = 0;
+      ND_HIP_TRY(hipMemcpyAsync(&total, d_offsets_ + S, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
+      ND_HIP_TRY(hipStreamSynchronize(stream_));
+      if (total >= (1u << 31)) { last_error = "collective neighbourhood of a layer exceeds 2^31 entries"; return -2; }
+      if (ensure_neighborhood_capacity(total) != 0) return -1;
+      neighborhood_total_ += total;
+      const bool distinct_form = App::kNeighborhoodForm == apps::kDistinctByDegreeSquared;
+      collective_build<<<dim3(S), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_offsets_, d_nbr_cols_,
+                                                           d_nbr_weights_, distinct_form ? d_sample_of_ : nullptr,
+                                                           d_row_offsets_);
+      ND_HIP_TRY(hipGetLastError());
+
+      LayerParams P{};
+      P.csr = dgraph_.view;
+      P.transits = tv;
+      P.step = step;
+      P.step_size = (uint32_t)app.stepSize(step);
+      P.n_samples = S;
+      P.final_size = (uint32_t)F;
+      P.out_base = (uint32_t)step_size_at_step<App>(step - 1);
+      P.invalid = invalid_;
+      P.seed = seed_;
+      P.first_slot = 0;
+      P.first_sample = 0;
+      P.final_samples = d_final_;
+      P.samples = d_samples_;
+      P.offsets = d_offsets_;
+      P.nbr_cols = d_nbr_cols_;
+      P.nbr_weights = d_nbr_weights_;
+      if (distinct_form) {
+        if (build_distinct(total) != 0) return -1;
+        P.distinct_start = d_distinct_start_;
+        P.distinct_ids = d_distinct_ids_;
+        P.running_sums = d_running_sums_;
+      }
+      const uint64_t outputs = (uint64_t)S * P.step_size;
+      layer_execute_kernel<SampleType, App><<<dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, stream_>>>(P);
+      ND_HIP_TRY(hipGetLastError());
+    }
+    ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
+    return 0;
+  }
+
+  int fetch_final_samples() override {
+    if (!allocated_) { last_error = "no device data"; return -1; }
+    ND_HIP_TRY(hipMemcpy(hFinalSamples.data(), d_final_, sizeof(VertexID_t) * hFinalSamples.size(),
+                         hipMemcpyDeviceToHost));
+    return 0;
+  }
+
+  int fetch_sample_states(void* dst, size_t bytes) override {
+    if (!allocated_ || std::is_empty<SampleType>::value) { last_error = "no sample state"; return -1; }
+    if (bytes != sample_state_bytes()) { last_error = "sample state size mismatch"; return -1; }
+    ND_HIP_TRY(hipMemcpy(dst, d_samples_, bytes, hipMemcpyDeviceToHost));
+    return 0;
+  }
+
+  int distinct() override {
+    last_error = "distinct applies to IndividualNeighborhood results";
+    return -2;
+  }
+
+  // sizes of the last run, for the algorithmic-bytes figure
+  uint64_t neighborhood_total() const { return neighborhood_total_; }
+  uint64_t distinct_total() const { return distinct_total_; }
+
+  void free_device() override {
+    free_run_buffers();
+    dgraph_.release();
+    graph_ = nullptr;
+  }
+
+ private:
+  template <class T>
+  static void release(T*& p) {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+  }
+
+  int ensure_neighborhood_capacity(uint32_t total) {
+    if (total <= capacity_ && capacity_ > 0) return 0;
+    size_t cap = (size_t)total + total / 8 + 1024;
+    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
+    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
+    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
+    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+    ND_HIP_TRY(hipMalloc(&d_nbr_cols_, sizeof(int32_t) * cap));
+    ND_HIP_TRY(hipMalloc(&d_nbr_weights_, sizeof(float) * cap));
+    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+      ND_HIP_TRY(hipMalloc(&d_sample_of_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_key2_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_pos_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_vertex_sorted_, sizeof(uint32_t) * cap));
+      const SortPlan plan = make_sort_plan(cap, 32);
+      ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * plan.hist_elems));
+      size_t scratch = plan.scratch_elems;
+      if (scan_scratch_elems(cap) > scratch) scratch = scan_scratch_elems(cap);
+      ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
+      ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
+    }
+    capacity_ = cap;
+    return 0;
+  }
+
+  // distinct (sample, vertex) pairs of the concatenation, their per-sample extents and
+  // the running sums of degree^2
+  int build_distinct(uint32_t total) {
+    const uint32_t S = (uint32_t)n_samples_;
+    fill_u32<<<dim3((S + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_count_, (size_t)S + 1, 0u);
+    if (total > 0) {
+      // sort by vertex, carrying the position in the concatenation ...
+      const SortPlan by_vertex = make_sort_plan(total, max_bits_);
+      uint32_t *k1 = nullptr, *p1 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_vertex, (const uint32_t*)d_nbr_cols_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
+                                  d_vals_b_, d_hist_, d_scratch_, stream_, &k1, &p1));
+      // ... then stably by owning sample: (sample, vertex) order
+      const unsigned blocks = (total + 255) / 256;
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_sample_of_, p1, total, d_key2_, d_pos_);
+      const SortPlan by_sample = make_sort_plan(total, sample_bits_);
+      uint32_t *k2 = nullptr, *p2 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_pos_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                  d_scratch_, stream_, &k2, &p2));
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_nbr_cols_, p2, total, d_vertex_sorted_,
+                                                          nullptr);
+      // run heads -> distinct ids, degree^2, per-sample counts
+      const size_t tiles = scan_num_tiles(total);
+      count_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(k2, d_vertex_sorted_, total,
+                                                                                  d_scratch_);
+      scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
+      compact_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(
+          k2, d_vertex_sorted_, total, d_scratch_, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
+          d_distinct_count_);
+      uint32_t n_distinct = 0;
+      ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
+      ND_HIP_TRY(hipStreamSynchronize(stream_));
+      distinct_total_ += n_distinct;
+      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
+    }
+    ND_HIP_TRY(exclusive_scan_u32(d_distinct_count_, d_distinct_start_, (size_t)S + 1, d_small_scratch_, stream_));
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
+
+  void free_run_buffers() {
+    release(d_initial_); release(d_samples_); release(d_samples_init_); release(d_final_);
+    release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
+    release(d_distinct_count_); release(d_distinct_start_);
+    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
+    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
+    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
+    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+    capacity_ = 0;
+    if (allocated_) {
+      (void)hipEventDestroy(ev_begin_);
+      (void)hipEventDestroy(ev_end_);
+      (void)hipStreamDestroy(stream_);
+    }
+    allocated_ = false;
+  }
+
+  const char* name_;
+  const CSR* graph_ = nullptr;
+  DeviceGraph dgraph_;
+  std::vector<SampleType> samples_;
+  int64_t n_samples_ = 0;
+  int init_size_ = 0;
+  int32_t invalid_ = 0;
+  int max_bits_ = 0, sample_bits_ = 0;
+  uint64_t seed_ = 0;
+  bool allocated_ = false;
+  size_t capacity_ = 0;
+  uint64_t neighborhood_total_ = 0, distinct_total_ = 0;
+
+  hipStream_t stream_ = nullptr;
+  hipEvent_t ev_begin_ = nullptr, ev_end_ = nullptr;
+  VertexID_t* d_initial_ = nullptr;
+  SampleType* d_samples_ = nullptr;
+  SampleType* d_samples_init_ = nullptr;
+  VertexID_t* d_final_ = nullptr;
+  uint32_t *d_sizes_ = nullptr, *d_offsets_ = nullptr, *d_row_offsets_ = nullptr, *d_small_scratch_ = nullptr;
+  uint32_t *d_distinct_count_ = nullptr, *d_distinct_start_ = nullptr;
+  int32_t* d_nbr_cols_ = nullptr;
+  float* d_nbr_weights_ = nullptr;
+  uint32_t* d_sample_of_ = nullptr;
+  uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
+  uint32_t *d_key2_ = nullptr, *d_pos_ = nullptr, *d_vertex_sorted_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
+  int32_t* d_distinct_ids_ = nullptr;
+  uint64_t *d_degree_sq_ = nullptr, *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
+};
+
+}  // namespace nd

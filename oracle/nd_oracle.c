@@ -501,3 +501,184 @@ int ndo_check_exact_transits(const ndo_graph* g, const ndo_app_desc* app,
   }
   return 1;
 }
+
+/* ------------------------------------------------------------------------- */
+/* CollectiveNeighborhood sampling                                            */
+/* ------------------------------------------------------------------------- */
+
+int64_t ndo_collective_neighborhood(const ndo_graph* g, const int32_t* transits, int n_transits,
+                                    int32_t invalid, int32_t* cols, float* weights, int32_t* row_offsets) {
+  int64_t size = 0;
+  for (int i = 0; i < n_transits; ++i) {
+    if (row_offsets) row_offsets[i] = (int32_t)size;
+    const int32_t t = transits[i];
+    if (t == invalid || t == -1) continue;
+    const int32_t b = g->row_ptr[t], e = g->row_ptr[t + 1];
+    for (int32_t x = b; x < e; ++x) {
+      if (cols) cols[size] = g->col[x];
+      if (weights) weights[size] = g->weight[x];
+      size++;
+    }
+  }
+  return size;
+}
+
+/* transits of sample-row `row` at step k, and how many there are */
+static const int32_t* layer_transits(const ndo_app_desc* app, int k, const int32_t* initial_of_sample,
+                                     const int32_t* row, int* count) {
+  if (k == 0) { *count = app->initial_size; return initial_of_sample; }
+  *count = app->step_size[k - 1];
+  return row + ndo_step_size_at_step(app, k - 2);
+}
+
+int ndo_sample_layer_literal(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                             int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                             int32_t* final_samples, int32_t* rows, int32_t* cols, int n_threads) {
+  if (!ndo_is_collective(app)) return -1;
+  const int32_t invalid = g->n_vertices;
+  const int64_t F = ndo_final_sample_size(app);
+  const int B = app->initial_size; /* VERTICES_PER_SAMPLE; the reference's apps use it for every layer */
+  if (n_threads < 1) n_threads = 1;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 4) num_threads(n_threads)
+#endif
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int32_t* row = final_samples + s * F;
+    for (int k = 0; k < app->steps; ++k) {
+      const int m = app->step_size[k];
+      int n_tr;
+      const int32_t* transits = layer_transits(app, k, initial + s * app->initial_size, row, &n_tr);
+      int32_t* out = row + ndo_step_size_at_step(app, k - 1);
+      for (int nbr = 0; nbr < m; ++nbr) {
+        int32_t neighbor = invalid;
+        /* nextdoor.cu:1421: only the first transit is looked at */
+        if (transits[0] != invalid && transits[0] != -1) {
+          rng_cursor rc;
+          rc.seed = seed; rc.slot = (uint64_t)((first_sample + s) * m + nbr); rc.step = (uint32_t)k;
+          rc.draw = 0; rc.st = 0;
+          const int32_t id = next_int(&rc, g->n_vertices);
+          for (int i = 0; i < B; ++i) {
+            const int has = ndo_has_edge(g, transits[i], id);
+            const int64_t len = (int64_t)i * B + nbr;
+            const int64_t at = (s * app->steps + k) * (int64_t)B * B + len;
+            rows[at] = has ? i : -1;
+            cols[at] = has ? nbr : -1;
+          }
+          neighbor = id;
+        }
+        out[nbr] = neighbor;
+      }
+    }
+  }
+  return 0;
+}
+
+int ndo_check_adjacency_matrix(const ndo_graph* g, const ndo_app_desc* app, int64_t n_samples,
+                               const int32_t* initial, const int32_t* final_samples,
+                               const int32_t* rows, const int32_t* cols, int32_t invalid) {
+  const int64_t F = ndo_final_sample_size(app);
+  const int B = app->initial_size;
+  const int max_steps = app->steps < 4 ? app->steps : 4; /* check_results.cu:57 */
+  int64_t sampled_before = 0; /* numNeighborsToSampleAtStep */
+  for (int step = 0; step < max_steps; ++step) {
+    const int64_t cur = step == 0 ? 0 : sampled_before + app->step_size[step]; /* check_results.cu:66 */
+    for (int64_t s = 0; s < n_samples; ++s) {
+      const int32_t* fs = final_samples + s * F;
+      const int32_t* r = rows + (s * app->steps + step) * (int64_t)B * B;
+      const int32_t* c = cols + (s * app->steps + step) * (int64_t)B * B;
+      const int64_t len = (int64_t)B * B; /* adjacencyMatrixLen stays 0 -> B*B (check_results.cu:76-79) */
+      /* 1: every recorded pair is an edge of the graph */
+      for (int64_t v = 0; v < len; ++v) {
+        if (c[v] == -1 && r[v] == -1) continue;
+        const int32_t to = fs[cur + c[v]];
+        const int32_t from = step == 0 ? initial[s * app->initial_size + r[v]] : fs[sampled_before + r[v]];
+        if (to != invalid && !ndo_has_edge(g, from, to)) return 0;
+      }
+      /* 2: every edge between the two layers is recorded */
+      const int prev_n = step == 0 ? app->initial_size : app->step_size[step - 1];
+      for (int v = 0; v < app->step_size[step]; ++v) {
+        const int32_t to = fs[cur + v];
+        for (int pi = 0; pi < prev_n; ++pi) {
+          const int32_t from = step == 0 ? initial[s * app->initial_size + pi] : fs[sampled_before + pi];
+          if (to == invalid || !ndo_has_edge(g, from, to)) continue;
+          int found = 0;
+          for (int64_t e = 0; e < len && !found; ++e) {
+            if (c[e] == -1 && r[e] == -1) continue;
+            const int32_t v1 = step == 0 ? initial[s * app->initial_size + r[e]] : fs[sampled_before + r[e]];
+            const int32_t v2 = fs[cur + c[e]];
+            if (v1 == from && v2 == to) found = 1;
+          }
+          if (!found) return 0;
+        }
+      }
+    }
+    if (step >= 1) sampled_before += app->step_size[step];
+  }
+  return 1;
+}
+
+int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                                  int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                                  int32_t* final_samples, ndo_stats* stats, int n_threads) {
+  if (!ndo_is_collective(app)) return -1;
+  const int32_t invalid = g->n_vertices;
+  const int64_t F = ndo_final_sample_size(app);
+  if (stats) memset(stats, 0, sizeof(*stats));
+  if (n_threads < 1) n_threads = 1;
+  int64_t total_edges = 0, total_distinct = 0, total_valid = 0;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 4) num_threads(n_threads) reduction(+ : total_edges, total_distinct, total_valid)
+#endif
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int32_t* row = final_samples + s * F;
+    for (int k = 0; k < app->steps; ++k) {
+      const int m = app->step_size[k];
+      int n_tr;
+      const int32_t* transits = layer_transits(app, k, initial + s * app->initial_size, row, &n_tr);
+      int32_t* out = row + ndo_step_size_at_step(app, k - 1);
+      const int64_t size = ndo_collective_neighborhood(g, transits, n_tr, invalid, 0, 0, 0);
+      int32_t* nb = (int32_t*)malloc(sizeof(int32_t) * (size_t)(size > 0 ? size : 1));
+      ndo_collective_neighborhood(g, transits, n_tr, invalid, nb, 0, 0);
+      qsort(nb, (size_t)size, sizeof(int32_t), cmp_i32);
+      int64_t distinct = 0;
+      for (int64_t i = 0; i < size; ++i)
+        if (distinct == 0 || nb[distinct - 1] != nb[i]) nb[distinct++] = nb[i];
+      uint64_t* prefix = (uint64_t*)malloc(sizeof(uint64_t) * (size_t)(distinct > 0 ? distinct : 1));
+      uint64_t total = 0;
+      for (int64_t i = 0; i < distinct; ++i) {
+        const uint64_t d = (uint64_t)degree_of(g, nb[i]);
+        total += d * d;
+        prefix[i] = total;
+      }
+      for (int nbr = 0; nbr < m; ++nbr) {
+        int32_t pick = invalid;
+        if (distinct > 0 && total > 0) {
+          uint32_t ctr[4] = {0, 0, (uint32_t)k, 0}, key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)}, w[4];
+          const uint64_t slot = (uint64_t)((first_sample + s) * m + nbr);
+          ctr[0] = (uint32_t)slot; ctr[1] = (uint32_t)(slot >> 32);
+          ndo_philox4x32_10(ctr, key, w);
+          const uint64_t r = w[0] >> 8;
+          const uint64_t target = (uint64_t)(((unsigned __int128)r * total) >> 24);
+          int64_t lo = 0, hi = distinct; /* first i with prefix[i] > target */
+          while (lo < hi) {
+            const int64_t mid = lo + (hi - lo) / 2;
+            if (prefix[mid] > target) hi = mid; else lo = mid + 1;
+          }
+          pick = nb[lo];
+          total_valid++;
+        }
+        out[nbr] = pick;
+      }
+      total_edges += size;
+      total_distinct += distinct;
+      free(prefix);
+      free(nb);
+    }
+  }
+  if (stats) {
+    stats->edge_reads = total_edges;      /* sum of collective-neighbourhood sizes */
+    stats->search_probes = total_distinct; /* sum of distinct counts */
+    stats->valid_outputs = total_valid;
+  }
+  return 0;
+}

@@ -151,6 +151,49 @@ int ndo_check_exact_transits(const ndo_graph* g, const ndo_app_desc* app,
 /* CSRPartition::has_edge_logn (csr.hpp:342-359). */
 int ndo_has_edge(const ndo_graph* g, int32_t src, int32_t dst);
 
+/* ---- CollectiveNeighborhood sampling (layer-wise: FastGCN, LADIES) ----
+ * Transits of sample s at step k (sampleParallelKernel, nextdoor.cu:1394-1411): the
+ * initial vertices for k = 0, else the step k-1 segment of its result row,
+ * final[s*F + stepSizeAtStep(k-2) ...].  Output nbr of step k goes to
+ * final[s*F + stepSizeAtStep(k-1) + nbr] (nextdoor.cu:1485-1487); its RNG slot is
+ * (first_sample + s) * m_k + nbr. */
+
+/* Collective neighbourhood of one sample (collectiveNeighbrsSize nextdoor.cu:1206-1246,
+ * collectiveNeighborhood 1248-1283): the adjacencies of its valid transits concatenated in
+ * transit order.  row_offsets[i] = start of transit i's adjacency inside the concatenation
+ * (INVALID transits contribute nothing).  cols / weights may be NULL (size only).
+ * pinned by a numpy concatenation in tests. */
+int64_t ndo_collective_neighborhood(const ndo_graph* g, const int32_t* transits, int n_transits,
+                                    int32_t invalid, int32_t* cols, float* weights, int32_t* row_offsets);
+
+/* The reference's FastGCN / LADIES apps as written (identical bodies,
+ * fastgcnSampling.cu:23-47, ladiessampling.cu:23-47): the vertex is drawn uniformly from
+ * ALL vertices, and for every transit i the pair (i, nbr) is recorded at
+ * [step][i*B + nbr] when the graph has the edge transit_i -> vertex, else (-1, -1).
+ * rows / cols: [n_samples][steps][B*B] (adjacencyMatrixRow / adjacencyMatrixCol).
+ * pinned by closed form (draw 0 of the slot) and brute-force adjacency on small graphs. */
+int ndo_sample_layer_literal(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                             int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                             int32_t* final_samples, int32_t* rows, int32_t* cols, int n_threads);
+
+/* checkAdjacencyMatrixResult (check_results.cu:46-160) as written: every recorded
+ * (row, col) is a graph edge, and every graph edge between consecutive layers is recorded. */
+int ndo_check_adjacency_matrix(const ndo_graph* g, const ndo_app_desc* app, int64_t n_samples,
+                               const int32_t* initial, const int32_t* final_samples,
+                               const int32_t* rows, const int32_t* cols, int32_t invalid);
+
+/* FastGCN-style importance sampling over the union neighbourhood (own definition; the
+ * reference's app ignores the neighbourhood, see above): D = ascending distinct vertices
+ * of the collective neighbourhood; weight(v) = degree(v)^2 (the squared degree normalised
+ * over D, up to the common factor); m_k independent draws WITH replacement by inverse CDF
+ * in exact integer arithmetic: r = top 24 bits of draw 0 of the slot,
+ * target = (r * total) >> 24, result = D[first i with prefix_i > target].
+ * Empty neighbourhood or total 0 -> INVALID.  parity unpinned by the reference; pinned by
+ * brute-force probability vectors and chi-square tests. */
+int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                                  int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                                  int32_t* final_samples, ndo_stats* stats, int n_threads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -71,6 +71,14 @@ def lib():
         L.ndo_check_exact_transits.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
                                                C.c_int32]
         L.ndo_has_edge.argtypes = [C.POINTER(GraphStruct), C.c_int32, C.c_int32]
+        L.ndo_collective_neighborhood.restype = C.c_int64
+        L.ndo_collective_neighborhood.argtypes = [C.POINTER(GraphStruct), i32p, C.c_int, C.c_int32, i32p, f32p, i32p]
+        L.ndo_sample_layer_literal.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64, C.c_int64,
+                                               C.c_int64, i32p, i32p, i32p, i32p, C.c_int]
+        L.ndo_check_adjacency_matrix.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
+                                                 i32p, i32p, C.c_int32]
+        L.ndo_sample_fastgcn_importance.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64,
+                                                    C.c_int64, C.c_int64, i32p, i32p, C.POINTER(Stats), C.c_int]
         _lib = L
     return _lib
 
@@ -196,3 +204,51 @@ def check_exact_transits(graph, desc, initial, final, invalid):
     final = np.ascontiguousarray(final, dtype=np.int32)
     return bool(lib().ndo_check_exact_transits(C.byref(graph.struct), C.byref(desc), final.shape[0],
                                                _p(initial, C.c_int32), _p(final, C.c_int32), invalid))
+
+
+def collective_neighborhood(graph, transits, invalid):
+    """(cols, weights, row_offsets) of one sample's collective neighbourhood."""
+    t = np.ascontiguousarray(transits, dtype=np.int32)
+    size = lib().ndo_collective_neighborhood(C.byref(graph.struct), _p(t, C.c_int32), len(t), invalid, None, None,
+                                             None)
+    cols, w, rows = np.empty(max(size, 1), np.int32), np.empty(max(size, 1), np.float32), np.empty(len(t), np.int32)
+    lib().ndo_collective_neighborhood(C.byref(graph.struct), _p(t, C.c_int32), len(t), invalid, _p(cols, C.c_int32),
+                                      _p(w, C.c_float), _p(rows, C.c_int32))
+    return cols[:size], w[:size], rows
+
+
+def sample_layer_literal(graph, desc, seed, initial, first_sample=0, n_threads=8):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    n = len(initial) // desc.initial_size
+    F, B = final_sample_size(desc), desc.initial_size
+    final = np.empty(n * F, np.int32)
+    rows = np.full(n * desc.steps * B * B, -1, np.int32)
+    cols = np.full(n * desc.steps * B * B, -1, np.int32)
+    rc = lib().ndo_sample_layer_literal(C.byref(graph.struct), C.byref(desc), seed, n, first_sample,
+                                        _p(initial, C.c_int32), _p(final, C.c_int32), _p(rows, C.c_int32),
+                                        _p(cols, C.c_int32), n_threads)
+    assert rc == 0
+    return final.reshape(n, F), rows.reshape(n, desc.steps, B * B), cols.reshape(n, desc.steps, B * B)
+
+
+def check_adjacency_matrix(graph, desc, initial, final, rows, cols, invalid):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    final = np.ascontiguousarray(final, dtype=np.int32)
+    rows = np.ascontiguousarray(rows, dtype=np.int32)
+    cols = np.ascontiguousarray(cols, dtype=np.int32)
+    return bool(lib().ndo_check_adjacency_matrix(C.byref(graph.struct), C.byref(desc), final.shape[0],
+                                                 _p(initial, C.c_int32), _p(final, C.c_int32), _p(rows, C.c_int32),
+                                                 _p(cols, C.c_int32), invalid))
+
+
+def sample_fastgcn_importance(graph, desc, seed, initial, first_sample=0, n_threads=8, want_stats=False):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    n = len(initial) // desc.initial_size
+    F = final_sample_size(desc)
+    final = np.empty(n * F, np.int32)
+    stats = Stats()
+    rc = lib().ndo_sample_fastgcn_importance(C.byref(graph.struct), C.byref(desc), seed, n, first_sample,
+                                             _p(initial, C.c_int32), _p(final, C.c_int32), C.byref(stats), n_threads)
+    assert rc == 0
+    final = final.reshape(n, F)
+    return (final, stats.as_dict()) if want_stats else final
