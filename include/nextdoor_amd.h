@@ -101,6 +101,10 @@ int nd_sampler_phase_times(const nd_sampler* s, float out[12]);
  * nd_sampler_do_transit_parallel; nd_sampler_get_final_samples then returns the packed rows. */
 int nd_sampler_distinct(nd_sampler* s);
 int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length);
+/* Sizes the last run worked on, for traffic accounting.  Layer-wise apps: which 0 = entries
+ * of all collective neighbourhoods built, 1 = distinct (sample, vertex) pairs found,
+ * 2 = chunks of samples processed; other apps return 0. */
+int64_t nd_sampler_counter(const nd_sampler* s, int which);
 /* freeDeviceData(data), src/nextdoor.cu:2088-2115. */
 void nd_sampler_free_device(nd_sampler* s);
 void nd_sampler_destroy(nd_sampler* s);

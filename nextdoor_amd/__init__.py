@@ -205,6 +205,9 @@ class Sampler:
                 "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms", "distinct_ms"]
         return dict(zip(keys, list(out)[:10]))
 
+    def counter(self, which):
+        return lib().nd_sampler_counter(self._h, which)
+
     def free_device(self):
         lib().nd_sampler_free_device(self._h)
 

@@ -48,6 +48,7 @@ SIGNATURES = {
     "nd_sampler_phase_times": (C.c_int, [C.c_void_p, c_f32p]),
     "nd_sampler_distinct": (C.c_int, [C.c_void_p]),
     "nd_sampler_get_distinct_counts": (C.c_int, [C.c_void_p, C.POINTER(c_i32p), c_i64p]),
+    "nd_sampler_counter": (C.c_int64, [C.c_void_p, C.c_int]),
     "nd_sampler_free_device": (None, [C.c_void_p]),
     "nd_sampler_destroy": (None, [C.c_void_p]),
     "nd_init_sampling": (C.c_int, [C.c_char_p, C.c_char_p, C.c_uint64]),

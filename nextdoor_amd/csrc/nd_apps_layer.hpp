@@ -32,7 +32,10 @@ namespace apps {
 //   kConcatenated  the adjacencies of the sample's transits, concatenated (ids, float weights)
 //   kDistinctByDegreeSquared  the ascending distinct ids of that neighbourhood and the
 //                  running sums (uint64) of degree(id)^2 over them
-enum NeighborhoodForm { kConcatenated = 0, kDistinctByDegreeSquared = 1 };
+//   kRankedByLadiesImportance  the distinct ids ordered by descending Efraimidis-Spirakis key
+//                  for the LADIES importance (squared column norm of the row-normalised
+//                  adjacency restricted to the transits); no weights
+enum NeighborhoodForm { kConcatenated = 0, kDistinctByDegreeSquared = 1, kRankedByLadiesImportance = 2 };
 
 template <int kLayers, int kBatch, int kNumSamples>
 struct LayerCommon {
@@ -133,6 +136,24 @@ struct FastGCNImportanceAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSample
   template <class SampleType>
   __host__ SampleType initializeSample(CSR*, const VertexID_t) {
     return SampleType();
+  }
+};
+
+// LADIES-style layer-dependent importance sampling WITHOUT replacement.  With U the
+// previous layer, importance(v) = sum over edges u -> v, u in U, of (w_uv / rowsum(u))^2.
+// The engine computes it over the collective neighbourhood, draws one Efraimidis-Spirakis
+// key log2(uniform) / importance per distinct vertex (uniform from Philox at slot
+// sample * |V| + v) and hands next() the vertices in descending key order: the first
+// stepSize(k) of them are a weighted sample without replacement, in selection order.
+template <int kLayers, int kBatch, int kNumSamples>
+struct LadiesImportanceAppT : FastGCNImportanceAppT<kLayers, kBatch, kNumSamples> {
+  static constexpr int kNeighborhoodForm = nd::apps::kRankedByLadiesImportance;
+
+  template <typename SampleType, typename EdgeArray, typename WeightArray>
+  __device__ inline VertexID next(int, CSRPartition*, const VertexID*, const VertexID, SampleType*, const float,
+                                  EdgeArray& rankedIds, WeightArray&, const EdgePos_t numDistinct,
+                                  const VertexID_t neighbrID, curandState*) {
+    return neighbrID < numDistinct ? rankedIds[neighbrID] : -1;
   }
 };
 

@@ -75,6 +75,9 @@ const AppEntry kApps[] = {
     {"FastGCNImportance", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 64, 4096>>},
     {"FastGCNImportance2x8", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 8, 100>>},
     {"FastGCNImportance3x16", make_layer_engine<LayerNoState, FastGCNImportanceAppT<3, 16, 300>>},
+    {"LADIESImportance", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 512, 1024>>},
+    {"LADIESImportance2x8", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 8, 100>>},
+    {"LADIESImportance3x16", make_layer_engine<LayerNoState, LadiesImportanceAppT<3, 16, 300>>},
 };
 constexpr int kNumApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
 
@@ -278,6 +281,8 @@ int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, in
   return 0;
 }
 
+int64_t nd_sampler_counter(const nd_sampler* s, int which) { return s ? s->engine->counter(which) : 0; }
+
 void nd_sampler_free_device(nd_sampler* s) {
   if (s) s->engine->free_device();
 }
@@ -438,7 +443,7 @@ int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64
   CAPI_HIP(d_weights.alloc(sizeof(float) * (size_t)total));
   nd::collective_build<<<dim3(S), dim3(256), 0, 0>>>(dg.view, tv, invalid, d_offsets.as<uint32_t>(),
                                                     d_cols.as<int32_t>(), d_weights.as<float>(), nullptr,
-                                                    d_rows.as<uint32_t>());
+                                                    d_rows.as<uint32_t>(), nullptr);
   CAPI_HIP(hipGetLastError());
   CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
   CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));

@@ -71,6 +71,9 @@ class EngineBase {
   virtual size_t sample_state_bytes() const = 0;
   virtual int fetch_sample_states(void* dst, size_t bytes) = 0;
   virtual int distinct() = 0;
+  // engine-specific sizes of the last run (layer engine: 0 = entries of all collective
+  // neighbourhoods, 1 = distinct (sample, vertex) pairs, 2 = chunks); 0 where not applicable
+  virtual int64_t counter(int) const { return 0; }
 
   std::vector<VertexID_t> hFinalSamples;       // as NextDoorData::hFinalSamples (libNextDoor.hpp:17)
   std::vector<VertexID_t> initialContents;     // as NextDoorData::initialContents (libNextDoor.hpp:18)

@@ -20,11 +20,18 @@
 //  * For kDistinctByDegreeSquared the concatenation is sorted by (sample, vertex) with two
 //    stable radix sorts, run heads give the distinct vertices, and a 64-bit inclusive scan
 //    of degree^2 gives the running sums the app inverts.
+//  * For kRankedByLadiesImportance each entry of the concatenation carries
+//    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed in concatenation
+//    order (the sorts are stable), Efraimidis-Spirakis keys are computed per distinct vertex
+//    and two more stable sorts order the distinct vertices of every sample by descending key.
+//  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
+//    of entries, so a layer whose frontier sits on hubs cannot outgrow memory.
 //  * Random numbers: Philox keyed by the output slot s * stepSize(k) + nbr and the layer.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <string>
 #include <type_traits>
@@ -66,11 +73,13 @@ __global__ __launch_bounds__(256) void collective_sizes(CSRPartition csr, Transi
 
 // One workgroup per sample: copy the adjacencies of its transits, in transit order, to
 // cols[offsets[s] ...] (and weights, and the owning sample id when asked for).
+// row_sums (nullable): when given, the weight slot receives (weight / row_sums[transit])^2.
 __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, TransitView tv, int32_t invalid,
                                                         const uint32_t* __restrict__ offsets,
                                                         int32_t* __restrict__ cols, float* __restrict__ weights,
                                                         uint32_t* __restrict__ sample_of,
-                                                        uint32_t* __restrict__ row_offsets) {
+                                                        uint32_t* __restrict__ row_offsets,
+                                                        const float* __restrict__ row_sums) {
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
   __shared__ uint32_t s_scan_tmp[4];
   const uint32_t s = blockIdx.x;
@@ -104,7 +113,14 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
     const int32_t t = transits[lo];
     const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[lo]);
     cols[base + e] = csr.edges[src];
-    if (weights) weights[base + e] = csr.weights[src];
+    if (weights) {
+      float w = csr.weights[src];
+      if (row_sums) {
+        const float p = w / row_sums[t];
+        w = p * p;
+      }
+      weights[base + e] = w;
+    }
     if (sample_of) sample_of[base + e] = s;
   }
 }
@@ -145,7 +161,9 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
                                                                    const EdgePos_t* __restrict__ row_ptr,
                                                                    int32_t* __restrict__ distinct_ids,
                                                                    uint64_t* __restrict__ degree_sq,
-                                                                   uint32_t* __restrict__ per_sample_count) {
+                                                                   uint32_t* __restrict__ per_sample_count,
+                                                                   uint32_t* __restrict__ run_begin,
+                                                                   uint32_t* __restrict__ distinct_sample) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
   bool head[kScanItems];
@@ -163,7 +181,9 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
       const uint32_t v = vertex[base + i];
       const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
       distinct_ids[r] = (int32_t)v;
-      degree_sq[r] = d * d;
+      if (degree_sq) degree_sq[r] = d * d;
+      if (run_begin) run_begin[r] = (uint32_t)(base + i);
+      if (distinct_sample) distinct_sample[r] = sample_key[base + i];
       atomicAdd(&per_sample_count[sample_key[base + i]], 1u);
       ++r;
     }
@@ -175,6 +195,63 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
   if (i < n) dst[i] = value;
 }
 
+// log2 of a positive normal float from exponent extraction and an atanh series; every step
+// is a single IEEE operation so that host and device agree bit for bit.
+__host__ __device__ __forceinline__ float det_log2(float x) {
+  uint32_t bits;
+#if defined(__HIP_DEVICE_COMPILE__)
+  bits = __float_as_uint(x);
+#else
+  memcpy(&bits, &x, sizeof(bits));
+#endif
+  int e = (int)(bits >> 23) - 127;
+  const uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
+  float m;
+#if defined(__HIP_DEVICE_COMPILE__)
+  m = __uint_as_float(mbits);
+#else
+  memcpy(&m, &mbits, sizeof(m));
+#endif
+  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
+  const float z = (m - 1.0f) / (m + 1.0f);
+  const float z2 = z * z;
+  float poly = z2 * 0.142857149f;
+  poly = poly + 0.2f;
+  poly = poly * z2;
+  poly = poly + 0.333333343f;
+  poly = poly * z2;
+  poly = poly + 1.0f;
+  float ln_m = z * poly;
+  ln_m = ln_m * 2.0f;
+  return (float)e + ln_m * 1.44269502f;
+}
+
+// One lane per distinct (sample, vertex): importance = its terms summed in concatenation
+// order; Efraimidis-Spirakis key log2(u) / importance with u from Philox at slot
+// sample * |V| + vertex; stored as sortable bits, inverted so that an ascending sort
+// yields descending keys.
+__global__ __launch_bounds__(256) void ladies_keys(const uint32_t* __restrict__ run_begin,
+                                                   const uint32_t* __restrict__ sorted_pos,
+                                                   const float* __restrict__ terms,
+                                                   const int32_t* __restrict__ distinct_ids,
+                                                   const uint32_t* __restrict__ distinct_sample, uint32_t n_distinct,
+                                                   uint64_t seed, uint64_t first_sample, uint32_t n_vertices,
+                                                   uint32_t step, uint32_t* __restrict__ key_bits) {
+  const uint32_t j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= n_distinct) return;
+  float importance = 0.0f;
+  for (uint32_t i = run_begin[j]; i < run_begin[j + 1]; ++i) importance = importance + terms[sorted_pos[i]];
+  const uint64_t slot = (first_sample + distinct_sample[j]) * (uint64_t)n_vertices + (uint32_t)distinct_ids[j];
+  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
+                                        (uint32_t)(seed >> 32));
+  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+  float key = -__builtin_inff();
+  if (importance > 0.0f) key = det_log2(u) / importance;
+  uint32_t b = __float_as_uint(key);
+  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  key_bits[j] = ~b;
+}
+
 // running sums of one sample's distinct ids, as the WeightArray handed to next()
 struct SegmentRunningSums {
   const uint64_t* sums;  // global inclusive sums, already offset to the sample's first distinct id
@@ -184,63 +261,77 @@ struct SegmentRunningSums {
 
 struct LayerParams {
   CSRPartition csr;
-  TransitView transits;
+  TransitView transits;   // base already points at the first sample of the chunk
   int step;
   uint32_t step_size;
-  uint32_t n_samples;
+  uint32_t chunk_samples; // samples in this launch
+  uint32_t sample_begin;  // index of the chunk's first sample
   uint32_t final_size;
-  uint32_t out_base;  // stepSizeAtStep(step - 1)
+  uint32_t out_base;      // stepSizeAtStep(step - 1)
   int32_t invalid;
   uint64_t seed;
-  uint64_t first_slot;
-  uint32_t first_sample;
+  uint64_t first_sample;  // index of the device's first sample (multi-device offset)
   int32_t* final_samples;
   void* samples;
-  // kConcatenated
+  // kConcatenated: offsets are relative to the chunk
   const uint32_t* offsets;
   const int32_t* nbr_cols;
   const float* nbr_weights;
-  // kDistinctByDegreeSquared
+  // kDistinctByDegreeSquared / kRankedByLadiesImportance
   const uint32_t* distinct_start;
-  const int32_t* distinct_ids;
+  const int32_t* distinct_ids;   // ascending ids, or ids in descending key order
   const uint64_t* running_sums;
 };
 
 template <class SampleType, class App>
 __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
   const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (uint64_t)P.n_samples * P.step_size) return;
-  const uint32_t s = (uint32_t)(i / P.step_size);
-  const uint32_t nbr = (uint32_t)(i - (uint64_t)s * P.step_size);
+  if (i >= (uint64_t)P.chunk_samples * P.step_size) return;
+  const uint32_t ls = (uint32_t)(i / P.step_size);  // sample inside the chunk
+  const uint32_t nbr = (uint32_t)(i - (uint64_t)ls * P.step_size);
+  const uint32_t s = P.sample_begin + ls;
   CSRPartition csr = P.csr;
-  const int32_t* transits = P.transits.base + (size_t)s * P.transits.stride;
+  const int32_t* transits = P.transits.base + (size_t)ls * P.transits.stride;
   SampleType local_state;
   SampleType* state = std::is_empty<SampleType>::value ? &local_state : (SampleType*)P.samples + s;
   curandState rng;
-  rng.reset(P.seed, P.first_slot + i, (uint32_t)P.step);
+  rng.reset(P.seed, (P.first_sample + s) * P.step_size + nbr, (uint32_t)P.step);
+  const VertexID sample_id = (VertexID)(P.first_sample + s);
   VertexID neighbor = P.invalid;
   if constexpr (App::kNeighborhoodForm == apps::kConcatenated) {
     // only the first transit decides whether next() runs (nextdoor.cu:1421)
     if (transits[0] != P.invalid && transits[0] != -1) {
-      const uint32_t begin = P.offsets[s];
+      const uint32_t begin = P.offsets[ls];
       const CSR::Edge* edges = P.nbr_cols + begin;
       const float* weights = P.nbr_weights + begin;
       const VertexID r = App().template next<SampleType, const CSR::Edge*, const float*>(
-          P.step, &csr, transits, (VertexID)(P.first_sample + s), state, 0.0f, edges, weights,
-          (EdgePos_t)(P.offsets[s + 1] - begin), (VertexID_t)nbr, &rng);
+          P.step, &csr, transits, sample_id, state, 0.0f, edges, weights, (EdgePos_t)(P.offsets[ls + 1] - begin),
+          (VertexID_t)nbr, &rng);
       neighbor = r == -1 ? P.invalid : r;
     }
-  } else {
-    const uint32_t begin = P.distinct_start[s];
+  } else if constexpr (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+    const uint32_t begin = P.distinct_start[ls];
     const CSR::Edge* ids = P.distinct_ids + begin;
     SegmentRunningSums sums{P.running_sums + begin, begin ? P.running_sums[begin - 1] : 0ull};
     const VertexID r = App().template next<SampleType, const CSR::Edge*, SegmentRunningSums>(
-        P.step, &csr, transits, (VertexID)(P.first_sample + s), state, 0.0f, ids, sums,
-        (EdgePos_t)(P.distinct_start[s + 1] - begin), (VertexID_t)nbr, &rng);
+        P.step, &csr, transits, sample_id, state, 0.0f, ids, sums, (EdgePos_t)(P.distinct_start[ls + 1] - begin),
+        (VertexID_t)nbr, &rng);
+    neighbor = r == -1 ? P.invalid : r;
+  } else {
+    const uint32_t begin = P.distinct_start[ls];
+    const CSR::Edge* ranked = P.distinct_ids + begin;
+    const float* no_weights = nullptr;
+    const VertexID r = App().template next<SampleType, const CSR::Edge*, const float*>(
+        P.step, &csr, transits, sample_id, state, 0.0f, ranked, no_weights,
+        (EdgePos_t)(P.distinct_start[ls + 1] - begin), (VertexID_t)nbr, &rng);
     neighbor = r == -1 ? P.invalid : r;
   }
   P.final_samples[(size_t)s * P.final_size + P.out_base + nbr] = neighbor;
 }
+
+// Entries of concatenated neighbourhood one chunk of samples may hold (about 70 bytes of
+// device memory per entry across all work arrays).
+constexpr uint64_t kLayerChunkEntries = 96ull << 20;
 
 template <class SampleType, class App>
 class LayerEngine : public EngineBase {
@@ -263,7 +354,20 @@ class LayerEngine : public EngineBase {
 
   int set_graph(const CSR* graph) override {
     graph_ = nullptr;
+    release(d_row_sums_);
     if (!dgraph_.upload(graph, false, app_uses_edge_lookup<App>::value, &last_error)) return -1;
+    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+      // weights of every vertex summed in edge order (sequential float adds)
+      const size_t V = (size_t)graph->get_n_vertices();
+      std::vector<float> sums(V);
+      for (size_t v = 0; v < V; ++v) {
+        float acc = 0.0f;
+        for (EdgePos_t x = graph->row_ptr[v]; x < graph->row_ptr[v + 1]; ++x) acc = acc + graph->weight[x];
+        sums[v] = acc;
+      }
+      ND_HIP_TRY(hipMalloc(&d_row_sums_, sizeof(float) * V));
+      ND_HIP_TRY(hipMemcpy(d_row_sums_, sums.data(), sizeof(float) * V, hipMemcpyHostToDevice));
+    }
     graph_ = graph;
     return 0;
   }
@@ -281,6 +385,7 @@ class LayerEngine : public EngineBase {
     n_samples_ = app.numSamples(csr);
     init_size_ = app.initialSampleSize(csr);
     if (n_samples_ <= 0 || init_size_ <= 0) { last_error = "app yields no samples"; return -2; }
+    if (n_samples_ >= (1ll << 31)) { last_error = "too many samples"; return -2; }
     uint32_t widest = (uint32_t)init_size_;
     for (int k = 0; k < n_steps; ++k) {
       if (app.stepSize(k) <= 0) { last_error = "stepSize must be positive"; return -2; }
@@ -290,8 +395,6 @@ class LayerEngine : public EngineBase {
     invalid_ = graph_->get_n_vertices();
     max_bits_ = 0;
     while ((invalid_ >> max_bits_) != 0) max_bits_++;
-    sample_bits_ = 1;
-    while (((uint64_t)n_samples_ >> sample_bits_) != 0) sample_bits_++;
 
     samples_.clear();
     initialContents.clear();
@@ -307,6 +410,12 @@ class LayerEngine : public EngineBase {
     }
     const size_t F = (size_t)final_sample_size();
     hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
+    h_sizes_.resize((size_t)n_samples_);
+    chunk_entries_ = kLayerChunkEntries;
+    if (const char* env = getenv("ND_LAYER_CHUNK_ENTRIES")) {  // smaller chunks, e.g. to exercise chunking
+      const long long v = atoll(env);
+      if (v > 0) chunk_entries_ = (uint64_t)v;
+    }
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
@@ -324,10 +433,11 @@ class LayerEngine : public EngineBase {
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     ND_HIP_TRY(hipMalloc(&d_sizes_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    ND_HIP_TRY(hipMemset(d_sizes_, 0, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_offsets_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_row_offsets_, sizeof(uint32_t) * (size_t)n_samples_ * widest));
     ND_HIP_TRY(hipMalloc(&d_small_scratch_, sizeof(uint32_t) * scan_scratch_elems((size_t)n_samples_ + 1)));
-    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+    if (App::kNeighborhoodForm != apps::kConcatenated) {
       ND_HIP_TRY(hipMalloc(&d_distinct_count_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
       ND_HIP_TRY(hipMalloc(&d_distinct_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     }
@@ -342,6 +452,7 @@ class LayerEngine : public EngineBase {
     times = PhaseTimes();
     neighborhood_total_ = 0;
     distinct_total_ = 0;
+    chunks_run_ = 0;
     if (!std::is_empty<SampleType>::value) {
       ND_HIP_TRY(hipMemcpyAsync(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
                                 hipMemcpyDeviceToDevice, stream_));
@@ -350,58 +461,31 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
     const uint32_t S = (uint32_t)n_samples_;
     for (int step = 0; step < n_steps; ++step) {
-      TransitView tv;
+      TransitView all;
       if (step == 0) {
-        tv.base = d_initial_;
-        tv.stride = (uint32_t)init_size_;
-        tv.count = (uint32_t)init_size_;
+        all.base = d_initial_;
+        all.stride = (uint32_t)init_size_;
+        all.count = (uint32_t)init_size_;
       } else {
-        tv.base = d_final_ + step_size_at_step<App>(step - 2);
-        tv.stride = (uint32_t)F;
-        tv.count = (uint32_t)app.stepSize(step - 1);
+        all.base = d_final_ + step_size_at_step<App>(step - 2);
+        all.stride = (uint32_t)F;
+        all.count = (uint32_t)app.stepSize(step - 1);
       }
-      // collective neighbourhood: sizes -> offsets -> concatenation
-      collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, stream_>>>(dgraph_.view, tv, S, invalid_, d_sizes_);
-      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_sizes_ + S, 1, 0u);
-      ND_HIP_TRY(exclusive_scan_u32(d_sizes_, d_offsets_, (size_t)S + 1, d_small_scratch_, stream_));
-      uint32_t total = 0;
-      ND_HIP_TRY(hipMemcpyAsync(&total, d_offsets_ + S, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
+      // size of every sample's collective neighbourhood, then chunks of samples that fit the budget
+      collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, stream_>>>(dgraph_.view, all, S, invalid_, d_sizes_);
+      ND_HIP_TRY(hipMemcpyAsync(h_sizes_.data(), d_sizes_, sizeof(uint32_t) * S, hipMemcpyDeviceToHost, stream_));
       ND_HIP_TRY(hipStreamSynchronize(stream_));
-      if (total >= (1u << 31)) { last_error = "collective neighbourhood of a layer exceeds 2^31 entries"; return -2; }
-      if (ensure_neighborhood_capacity(total) != 0) return -1;
-      neighborhood_total_ += total;
-      const bool distinct_form = App::kNeighborhoodForm == apps::kDistinctByDegreeSquared;
-      collective_build<<<dim3(S), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_offsets_, d_nbr_cols_,
-                                                           d_nbr_weights_, distinct_form ? d_sample_of_ : nullptr,
-                                                           d_row_offsets_);
-      ND_HIP_TRY(hipGetLastError());
-
-      LayerParams P{};
-      P.csr = dgraph_.view;
-      P.transits = tv;
-      P.step = step;
-      P.step_size = (uint32_t)app.stepSize(step);
-      P.n_samples = S;
-      P.final_size = (uint32_t)F;
-      P.out_base = (uint32_t)step_size_at_step<App>(step - 1);
-      P.invalid = invalid_;
-      P.seed = seed_;
-      P.first_slot = 0;
-      P.first_sample = 0;
-      P.final_samples = d_final_;
-      P.samples = d_samples_;
-      P.offsets = d_offsets_;
-      P.nbr_cols = d_nbr_cols_;
-      P.nbr_weights = d_nbr_weights_;
-      if (distinct_form) {
-        if (build_distinct(total) != 0) return -1;
-        P.distinct_start = d_distinct_start_;
-        P.distinct_ids = d_distinct_ids_;
-        P.running_sums = d_running_sums_;
+      uint32_t s0 = 0;
+      while (s0 < S) {
+        uint64_t total = h_sizes_[s0];
+        uint32_t s1 = s0 + 1;
+        while (s1 < S && total + h_sizes_[s1] <= chunk_entries_) total += h_sizes_[s1++];
+        if (total >= (1ull << 31)) { last_error = "collective neighbourhood of one sample exceeds 2^31 entries"; return -2; }
+        if (run_chunk(step, all, s0, s1, (uint32_t)total) != 0) return -1;
+        neighborhood_total_ += total;
+        chunks_run_++;
+        s0 = s1;
       }
-      const uint64_t outputs = (uint64_t)S * P.step_size;
-      layer_execute_kernel<SampleType, App><<<dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, stream_>>>(P);
-      ND_HIP_TRY(hipGetLastError());
     }
     ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
@@ -429,11 +513,13 @@ class LayerEngine : public EngineBase {
   }
 
   // sizes of the last run, for the algorithmic-bytes figure
-  uint64_t neighborhood_total() const { return neighborhood_total_; }
-  uint64_t distinct_total() const { return distinct_total_; }
+  int64_t counter(int which) const override {
+    return which == 0 ? (int64_t)neighborhood_total_ : which == 1 ? (int64_t)distinct_total_ : (int64_t)chunks_run_;
+  }
 
   void free_device() override {
     free_run_buffers();
+    release(d_row_sums_);
     dgraph_.release();
     graph_ = nullptr;
   }
@@ -445,16 +531,61 @@ class LayerEngine : public EngineBase {
     p = nullptr;
   }
 
+  // One chunk of samples [s0, s1) of one layer: concatenate, post-process in the form the
+  // app asks for, run next() for every (sample, nbr).
+  int run_chunk(int step, const TransitView& all, uint32_t s0, uint32_t s1, uint32_t total) {
+    App app;
+    const uint32_t n = s1 - s0;
+    const size_t F = (size_t)final_sample_size();
+    if (ensure_neighborhood_capacity(total) != 0) return -1;
+    TransitView tv = all;
+    tv.base = all.base + (size_t)s0 * all.stride;
+    // offsets of the chunk's samples, relative to the chunk (element n = total)
+    ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
+    constexpr int form = App::kNeighborhoodForm;
+    collective_build<<<dim3(n), dim3(256), 0, stream_>>>(
+        dgraph_.view, tv, invalid_, d_offsets_, d_nbr_cols_, d_nbr_weights_,
+        form != apps::kConcatenated ? d_sample_of_ : nullptr, d_row_offsets_ + (size_t)s0 * all.count,
+        form == apps::kRankedByLadiesImportance ? d_row_sums_ : nullptr);
+    ND_HIP_TRY(hipGetLastError());
+
+    LayerParams P{};
+    P.csr = dgraph_.view;
+    P.transits = tv;
+    P.step = step;
+    P.step_size = (uint32_t)app.stepSize(step);
+    P.chunk_samples = n;
+    P.sample_begin = s0;
+    P.final_size = (uint32_t)F;
+    P.out_base = (uint32_t)step_size_at_step<App>(step - 1);
+    P.invalid = invalid_;
+    P.seed = seed_;
+    P.first_sample = 0;
+    P.final_samples = d_final_;
+    P.samples = d_samples_;
+    P.offsets = d_offsets_;
+    P.nbr_cols = d_nbr_cols_;
+    P.nbr_weights = d_nbr_weights_;
+    if (form != apps::kConcatenated) {
+      if (build_distinct(step, s0, n, total) != 0) return -1;
+      P.distinct_start = d_distinct_start_;
+      P.distinct_ids = form == apps::kRankedByLadiesImportance ? d_ranked_ids_ : d_distinct_ids_;
+      P.running_sums = d_running_sums_;
+    }
+    const uint64_t outputs = (uint64_t)n * P.step_size;
+    layer_execute_kernel<SampleType, App><<<dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, stream_>>>(P);
+    ND_HIP_TRY(hipGetLastError());
+    return 0;
+  }
+
   int ensure_neighborhood_capacity(uint32_t total) {
     if (total <= capacity_ && capacity_ > 0) return 0;
-    size_t cap = (size_t)total + total / 8 + 1024;
-    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
-    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
-    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
-    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+    const size_t cap = (size_t)total + total / 8 + 1024;
+    release_neighborhood_buffers();
     ND_HIP_TRY(hipMalloc(&d_nbr_cols_, sizeof(int32_t) * cap));
     ND_HIP_TRY(hipMalloc(&d_nbr_weights_, sizeof(float) * cap));
-    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+    constexpr int form = App::kNeighborhoodForm;
+    if (form != apps::kConcatenated) {
       ND_HIP_TRY(hipMalloc(&d_sample_of_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * cap));
@@ -469,61 +600,100 @@ class LayerEngine : public EngineBase {
       if (scan_scratch_elems(cap) > scratch) scratch = scan_scratch_elems(cap);
       ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
       ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
+    }
+    if (form == apps::kDistinctByDegreeSquared) {
       ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
+    }
+    if (form == apps::kRankedByLadiesImportance) {
+      ND_HIP_TRY(hipMalloc(&d_run_begin_, sizeof(uint32_t) * (cap + 1)));
+      ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
     }
     capacity_ = cap;
     return 0;
   }
 
-  // distinct (sample, vertex) pairs of the concatenation, their per-sample extents and
-  // the running sums of degree^2
-  int build_distinct(uint32_t total) {
-    const uint32_t S = (uint32_t)n_samples_;
-    fill_u32<<<dim3((S + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_count_, (size_t)S + 1, 0u);
+  // Distinct (sample, vertex) pairs of the chunk's concatenation and their per-sample
+  // extents; then running sums of degree^2, or the ranking by Efraimidis-Spirakis key.
+  int build_distinct(int step, uint32_t s0, uint32_t n, uint32_t total) {
+    constexpr int form = App::kNeighborhoodForm;
+    int chunk_bits = 1;
+    while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
+    fill_u32<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_count_, (size_t)n + 1, 0u);
+    uint32_t n_distinct = 0;
+    uint32_t* sorted_pos = nullptr;
     if (total > 0) {
       // sort by vertex, carrying the position in the concatenation ...
       const SortPlan by_vertex = make_sort_plan(total, max_bits_);
       uint32_t *k1 = nullptr, *p1 = nullptr;
       ND_HIP_TRY(radix_sort_pairs(by_vertex, (const uint32_t*)d_nbr_cols_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
                                   d_vals_b_, d_hist_, d_scratch_, stream_, &k1, &p1));
-      // ... then stably by owning sample: (sample, vertex) order
+      // ... then stably by owning sample: (sample, vertex) order, duplicates in concatenation order
       const unsigned blocks = (total + 255) / 256;
       gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_sample_of_, p1, total, d_key2_, d_pos_);
-      const SortPlan by_sample = make_sort_plan(total, sample_bits_);
+      const SortPlan by_sample = make_sort_plan(total, chunk_bits);
       uint32_t *k2 = nullptr, *p2 = nullptr;
       ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_pos_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
                                   d_scratch_, stream_, &k2, &p2));
       gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_nbr_cols_, p2, total, d_vertex_sorted_,
-                                                          nullptr);
-      // run heads -> distinct ids, degree^2, per-sample counts
+                                                          form == apps::kRankedByLadiesImportance ? d_pos_ : nullptr);
+      sorted_pos = d_pos_;  // (LADIES) positions in (sample, vertex) order, safe from the later sorts
+      // run heads -> distinct ids, per-sample counts (+ degree^2, or run extents)
       const size_t tiles = scan_num_tiles(total);
       count_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(k2, d_vertex_sorted_, total,
                                                                                   d_scratch_);
       scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
       compact_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(
           k2, d_vertex_sorted_, total, d_scratch_, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
-          d_distinct_count_);
-      uint32_t n_distinct = 0;
+          d_distinct_count_, d_run_begin_, d_distinct_sample_);
       ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
       ND_HIP_TRY(hipStreamSynchronize(stream_));
       distinct_total_ += n_distinct;
-      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
     }
-    ND_HIP_TRY(exclusive_scan_u32(d_distinct_count_, d_distinct_start_, (size_t)S + 1, d_small_scratch_, stream_));
+    ND_HIP_TRY(exclusive_scan_u32(d_distinct_count_, d_distinct_start_, (size_t)n + 1, d_small_scratch_, stream_));
+    if (form == apps::kDistinctByDegreeSquared) {
+      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
+    } else if (n_distinct > 0) {
+      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_run_begin_ + n_distinct, 1, total);
+      ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
+          d_run_begin_, sorted_pos, d_nbr_weights_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_,
+          (uint64_t)s0, (uint32_t)invalid_, (uint32_t)step, d_key_bits_);
+      // order the distinct vertices of every sample by descending key: the list is in
+      // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
+      // ascending vertex id among equal keys
+      const SortPlan by_key = make_sort_plan(n_distinct, 32);
+      uint32_t *k3 = nullptr, *j3 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_key, d_key_bits_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                  d_scratch_, stream_, &k3, &j3));
+      const unsigned blocks = (n_distinct + 255) / 256;
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_distinct_sample_, j3, n_distinct, d_key2_, d_vertex_sorted_);
+      const SortPlan by_sample = make_sort_plan(n_distinct, chunk_bits);
+      uint32_t *k4 = nullptr, *j4 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_vertex_sorted_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_,
+                                  d_hist_, d_scratch_, stream_, &k4, &j4));
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_distinct_ids_, j4, n_distinct,
+                                                          (uint32_t*)d_ranked_ids_, nullptr);
+    }
     return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
+
+  void release_neighborhood_buffers() {
+    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
+    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
+    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
+    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+    release(d_run_begin_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
+    capacity_ = 0;
   }
 
   void free_run_buffers() {
     release(d_initial_); release(d_samples_); release(d_samples_init_); release(d_final_);
     release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
     release(d_distinct_count_); release(d_distinct_start_);
-    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
-    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
-    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
-    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
-    capacity_ = 0;
+    release_neighborhood_buffers();
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
       (void)hipEventDestroy(ev_end_);
@@ -535,15 +705,18 @@ class LayerEngine : public EngineBase {
   const char* name_;
   const CSR* graph_ = nullptr;
   DeviceGraph dgraph_;
+  float* d_row_sums_ = nullptr;
   std::vector<SampleType> samples_;
+  std::vector<uint32_t> h_sizes_;
   int64_t n_samples_ = 0;
   int init_size_ = 0;
   int32_t invalid_ = 0;
-  int max_bits_ = 0, sample_bits_ = 0;
+  int max_bits_ = 0;
   uint64_t seed_ = 0;
   bool allocated_ = false;
   size_t capacity_ = 0;
-  uint64_t neighborhood_total_ = 0, distinct_total_ = 0;
+  uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
+  uint64_t chunk_entries_ = kLayerChunkEntries;
 
   hipStream_t stream_ = nullptr;
   hipEvent_t ev_begin_ = nullptr, ev_end_ = nullptr;
@@ -560,6 +733,8 @@ class LayerEngine : public EngineBase {
   uint32_t *d_key2_ = nullptr, *d_pos_ = nullptr, *d_vertex_sorted_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
   uint64_t *d_degree_sq_ = nullptr, *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
+  uint32_t *d_run_begin_ = nullptr, *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
+  int32_t* d_ranked_ids_ = nullptr;
 };
 
 }  // namespace nd

@@ -682,3 +682,130 @@ int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, u
   }
   return 0;
 }
+
+/* ------------------------------------------------------------------------- */
+/* LADIES importance sampling                                                 */
+/* ------------------------------------------------------------------------- */
+
+float ndo_det_log2(float x) {
+  uint32_t bits;
+  memcpy(&bits, &x, sizeof(bits));
+  int e = (int)(bits >> 23) - 127;
+  uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
+  float m;
+  memcpy(&m, &mbits, sizeof(m));
+  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
+  const float z = (m - 1.0f) / (m + 1.0f);
+  const float z2 = z * z;
+  float poly = z2 * 0.142857149f; /* 1 + z^2/3 + z^4/5 + z^6/7 by Horner */
+  poly = poly + 0.2f;
+  poly = poly * z2;
+  poly = poly + 0.333333343f;
+  poly = poly * z2;
+  poly = poly + 1.0f;
+  float ln_m = z * poly;
+  ln_m = ln_m * 2.0f;
+  return (float)e + ln_m * 1.44269502f;
+}
+
+static uint32_t descending_key_bits(float key) {
+  /* monotone float -> uint32, then inverted so that an ascending sort gives descending keys */
+  uint32_t b;
+  memcpy(&b, &key, sizeof(b));
+  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  return ~b;
+}
+
+typedef struct { int32_t vertex; int64_t pos; } occ_t;
+static int cmp_occ(const void* a, const void* b) {
+  const occ_t* x = (const occ_t*)a; const occ_t* y = (const occ_t*)b;
+  if (x->vertex != y->vertex) return (x->vertex > y->vertex) - (x->vertex < y->vertex);
+  return (x->pos > y->pos) - (x->pos < y->pos);
+}
+typedef struct { uint32_t key; int32_t vertex; } ranked_t;
+static int cmp_ranked(const void* a, const void* b) {
+  const ranked_t* x = (const ranked_t*)a; const ranked_t* y = (const ranked_t*)b;
+  if (x->key != y->key) return (x->key > y->key) - (x->key < y->key);
+  return (x->vertex > y->vertex) - (x->vertex < y->vertex);
+}
+
+int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                                 int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                                 int32_t* final_samples, ndo_stats* stats, int n_threads) {
+  if (!ndo_is_collective(app)) return -1;
+  const int32_t invalid = g->n_vertices;
+  const int64_t F = ndo_final_sample_size(app);
+  if (stats) memset(stats, 0, sizeof(*stats));
+  if (n_threads < 1) n_threads = 1;
+  /* row sums in edge order */
+  float* rowsum = (float*)malloc(sizeof(float) * (size_t)g->n_vertices);
+  for (int32_t v = 0; v < g->n_vertices; ++v) {
+    float acc = 0.0f;
+    for (int32_t x = g->row_ptr[v]; x < g->row_ptr[v + 1]; ++x) acc = acc + g->weight[x];
+    rowsum[v] = acc;
+  }
+  int64_t total_edges = 0, total_distinct = 0, total_valid = 0;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 1) num_threads(n_threads) reduction(+ : total_edges, total_distinct, total_valid)
+#endif
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int32_t* row = final_samples + s * F;
+    for (int k = 0; k < app->steps; ++k) {
+      const int m = app->step_size[k];
+      int n_tr;
+      const int32_t* transits = layer_transits(app, k, initial + s * app->initial_size, row, &n_tr);
+      int32_t* out = row + ndo_step_size_at_step(app, k - 1);
+      const int64_t size = ndo_collective_neighborhood(g, transits, n_tr, invalid, 0, 0, 0);
+      occ_t* occ = (occ_t*)malloc(sizeof(occ_t) * (size_t)(size > 0 ? size : 1));
+      float* term = (float*)malloc(sizeof(float) * (size_t)(size > 0 ? size : 1));
+      int64_t at = 0;
+      for (int i = 0; i < n_tr; ++i) {
+        const int32_t u = transits[i];
+        if (u == invalid || u == -1) continue;
+        for (int32_t x = g->row_ptr[u]; x < g->row_ptr[u + 1]; ++x) {
+          const float p = g->weight[x] / rowsum[u];
+          term[at] = p * p;
+          occ[at].vertex = g->col[x];
+          occ[at].pos = at;
+          at++;
+        }
+      }
+      qsort(occ, (size_t)size, sizeof(occ_t), cmp_occ);
+      ranked_t* ranked = (ranked_t*)malloc(sizeof(ranked_t) * (size_t)(size > 0 ? size : 1));
+      int64_t distinct = 0;
+      for (int64_t i = 0; i < size;) {
+        int64_t j = i;
+        float imp = 0.0f;
+        while (j < size && occ[j].vertex == occ[i].vertex) { imp = imp + term[occ[j].pos]; j++; }
+        const int32_t v = occ[i].vertex;
+        uint32_t ctr[4], key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)}, w[4];
+        const uint64_t slot = (uint64_t)(first_sample + s) * (uint64_t)g->n_vertices + (uint64_t)v;
+        ctr[0] = (uint32_t)slot; ctr[1] = (uint32_t)(slot >> 32); ctr[2] = (uint32_t)k; ctr[3] = 0;
+        ndo_philox4x32_10(ctr, key, w);
+        const float u01 = ((float)(w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+        float keyf;
+        if (imp > 0.0f) keyf = ndo_det_log2(u01) / imp;
+        else keyf = -__builtin_inff();
+        ranked[distinct].key = descending_key_bits(keyf);
+        ranked[distinct].vertex = v;
+        distinct++;
+        i = j;
+      }
+      qsort(ranked, (size_t)distinct, sizeof(ranked_t), cmp_ranked);
+      for (int nbr = 0; nbr < m; ++nbr) {
+        out[nbr] = nbr < distinct ? ranked[nbr].vertex : invalid;
+        if (nbr < distinct) total_valid++;
+      }
+      total_edges += size;
+      total_distinct += distinct;
+      free(ranked); free(term); free(occ);
+    }
+  }
+  free(rowsum);
+  if (stats) {
+    stats->edge_reads = total_edges;
+    stats->search_probes = total_distinct;
+    stats->valid_outputs = total_valid;
+  }
+  return 0;
+}

@@ -194,6 +194,27 @@ int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, u
                                   int64_t n_samples, int64_t first_sample, const int32_t* initial,
                                   int32_t* final_samples, ndo_stats* stats, int n_threads);
 
+/* LADIES-style layer-dependent importance sampling (own definition; parity unpinned by
+ * the reference, whose LADIES app is the literal one above).  For a layer with frontier
+ * (transits) U: every occurrence (u, x) of an edge u -> v = col[x], u a valid transit, in
+ * concatenation order, contributes term = (w_x / rowsum_u)^2, rowsum_u = the weights of u
+ * summed in edge order (float, sequential).  importance(v) = the terms of v's occurrences
+ * summed in concatenation order: the squared column norm of the row-normalised adjacency
+ * restricted to the frontier.  m_k vertices are drawn WITHOUT replacement with probability
+ * proportional to importance by Efraimidis-Spirakis keys: key(v) = log2(u_v) / importance(v),
+ * u_v = ((word >> 8) + 0.5) * 2^-24 from Philox at slot (first_sample + s) * |V| + v, layer k;
+ * log2 is ndo_det_log2 (single IEEE operations only, so the GPU reproduces it bit for bit).
+ * The result is the m_k largest keys in descending key order, ties by ascending vertex id;
+ * fewer than m_k distinct vertices leave INVALID.  pinned by brute-force probability
+ * vectors on tiny graphs and inclusion-frequency tests. */
+int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
+                                 int64_t n_samples, int64_t first_sample, const int32_t* initial,
+                                 int32_t* final_samples, ndo_stats* stats, int n_threads);
+
+/* log2 of a positive normal float from exponent extraction and an atanh series; every step
+ * is one IEEE single-precision operation.  pinned against libm (absolute error < 2e-6). */
+float ndo_det_log2(float x);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,10 @@ def lib():
                                                C.c_int64, i32p, i32p, i32p, i32p, C.c_int]
         L.ndo_check_adjacency_matrix.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
                                                  i32p, i32p, C.c_int32]
+        L.ndo_det_log2.restype = C.c_float
+        L.ndo_det_log2.argtypes = [C.c_float]
+        L.ndo_sample_ladies_importance.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64,
+                                                   C.c_int64, C.c_int64, i32p, i32p, C.POINTER(Stats), C.c_int]
         L.ndo_sample_fastgcn_importance.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64,
                                                     C.c_int64, C.c_int64, i32p, i32p, C.POINTER(Stats), C.c_int]
         _lib = L
@@ -249,6 +253,19 @@ def sample_fastgcn_importance(graph, desc, seed, initial, first_sample=0, n_thre
     stats = Stats()
     rc = lib().ndo_sample_fastgcn_importance(C.byref(graph.struct), C.byref(desc), seed, n, first_sample,
                                              _p(initial, C.c_int32), _p(final, C.c_int32), C.byref(stats), n_threads)
+    assert rc == 0
+    final = final.reshape(n, F)
+    return (final, stats.as_dict()) if want_stats else final
+
+
+def sample_ladies_importance(graph, desc, seed, initial, first_sample=0, n_threads=8, want_stats=False):
+    initial = np.ascontiguousarray(initial, dtype=np.int32)
+    n = len(initial) // desc.initial_size
+    F = final_sample_size(desc)
+    final = np.empty(n * F, np.int32)
+    stats = Stats()
+    rc = lib().ndo_sample_ladies_importance(C.byref(graph.struct), C.byref(desc), seed, n, first_sample,
+                                            _p(initial, C.c_int32), _p(final, C.c_int32), C.byref(stats), n_threads)
     assert rc == 0
     final = final.reshape(n, F)
     return (final, stats.as_dict()) if want_stats else final

@@ -98,3 +98,45 @@ def test_distinct_is_refused_for_layer_apps():
     with pytest.raises(nd.NextDoorError):
         s.distinct()
     s.close()
+
+
+@pytest.mark.parametrize("app", ["LADIESImportance2x8", "LADIESImportance3x16"])
+@pytest.mark.parametrize("gname", ["sparse", "hub"])
+def test_ladies_importance_matches_oracle(oracle, app, gname):
+    g = (graphs.random_graph(n=300, mean_degree=3, seed=1, isolated_every=4) if gname == "sparse"
+         else graphs.random_graph(n=2000, mean_degree=12, seed=2, hub=5))
+    og = graphs.oracle_view(g)
+    s = nd.Sampler(app, g, seed=SEED)
+    d = layer_desc(oracle, s, oracle.LADIES_IMPORTANCE)
+    roots = s.initial_contents
+    want = oracle.sample_ladies_importance(og, d, SEED, roots)
+    print("app", app, "graph", gname, flush=True)
+    s.do_transit_parallel(True)
+    got = s.final_samples()
+    assert np.array_equal(got, want)
+    # without replacement: no vertex twice inside a layer segment
+    B = s.step_size(0)
+    for row in got[:100]:
+        for k in range(s.steps):
+            seg = row[k * B:(k + 1) * B]
+            seg = seg[seg != s.invalid_vertex]
+            assert len(set(seg.tolist())) == len(seg)
+    s.close()
+
+
+@pytest.mark.parametrize("app,kind_name", [("FastGCNImportance3x16", "FASTGCN_IMPORTANCE"),
+                                           ("LADIESImportance3x16", "LADIES_IMPORTANCE"),
+                                           ("LayerLiteral3x16", "LAYER_LITERAL")])
+def test_chunked_processing_gives_the_same_samples(oracle, app, kind_name, monkeypatch):
+    g = graphs.random_graph(n=2000, mean_degree=12, seed=2, hub=5)
+    s = nd.Sampler(app, g, seed=SEED)
+    s.do_transit_parallel(True)
+    whole = s.final_samples()
+    assert s.counter(2) == s.steps  # one chunk per layer
+    s.close()
+    monkeypatch.setenv("ND_LAYER_CHUNK_ENTRIES", "3000")  # a few samples per chunk
+    s = nd.Sampler(app, g, seed=SEED)
+    s.do_transit_parallel(True)
+    assert s.counter(2) > 3 * s.steps
+    assert np.array_equal(s.final_samples(), whole)
+    s.close()

@@ -109,3 +109,55 @@ def test_fastgcn_importance_follows_squared_degree(oracle):
     counts = np.array([(final == v).sum() for v in (1, 2, 3, 4)], dtype=float)
     expected = S * B * np.array([1, 4, 9, 16]) / 30.0
     assert (((counts - expected) ** 2) / expected).sum() < 17.7
+
+
+def test_det_log2_against_libm(oracle):
+    xs = np.concatenate([np.float32(2.0) ** -np.arange(0, 26), np.random.default_rng(0).random(2000).astype(np.float32),
+                         np.array([1.0, 0.70710678, 0.70710683, 1.4142135 / 2, 2.0 ** -24 * 0.5], np.float32)])
+    xs = xs[xs > 0]
+    got = np.array([oracle.lib().ndo_det_log2(float(x)) for x in xs], dtype=np.float64)
+    assert np.max(np.abs(got - np.log2(xs.astype(np.float64)))) < 2e-6
+    assert oracle.lib().ndo_det_log2(1.0) == 0.0 and oracle.lib().ndo_det_log2(0.25) == -2.0
+
+
+def test_ladies_importance_definition_on_a_tiny_graph(oracle):
+    # frontier {0, 1}; 0 -> {2 (w 1), 3 (w 3)}, 1 -> {3 (w 2), 4 (w 2)}
+    adj = [[2, 3], [3, 4], [], [], []]
+    w = [[1.0, 3.0], [2.0, 2.0], [], [], []]
+    g = oracle.Graph.from_adjacency(adj, w)
+    n = 5
+    # importance: 2 -> (1/4)^2, 3 -> (3/4)^2 + (2/4)^2, 4 -> (2/4)^2
+    imp = {2: np.float32(0.0625), 3: np.float32(0.5625) + np.float32(0.25), 4: np.float32(0.25)}
+    d = oracle.app_desc(oracle.LADIES_IMPORTANCE, 1, 2, initial_size=2)
+    S = 20000
+    final = oracle.sample_ladies_importance(g, d, SEED, np.tile([0, 1], S).astype(np.int32))
+    assert np.all(final[:, 0] != final[:, 1])  # without replacement
+    # exact keys for a few samples
+    for s in range(50):
+        keys = {}
+        for v in (2, 3, 4):
+            word = oracle.philox(((s * n + v) & 0xffffffff, (s * n + v) >> 32, 0, 0), (SEED, 0))[0]
+            u = np.float32((np.float32(word >> 8) + np.float32(0.5)) * np.float32(2.0 ** -24))
+            keys[v] = np.float32(oracle.lib().ndo_det_log2(float(u))) / imp[v]
+        order = sorted(keys, key=lambda v: (-keys[v], v))
+        assert list(final[s]) == order[:2]
+    # first pick is proportional to importance (Efraimidis-Spirakis)
+    total = float(sum(imp.values()))
+    counts = np.array([(final[:, 0] == v).sum() for v in (2, 3, 4)], dtype=float)
+    expected = S * np.array([float(imp[v]) for v in (2, 3, 4)]) / total
+    assert (((counts - expected) ** 2) / expected).sum() < 15.2  # 2 dof
+    # inclusion in a sample of 2: P(v in sample) = p_v + sum_{u != v} p_u p_v / (1 - p_u)
+    p = {v: float(imp[v]) / total for v in imp}
+    for v in imp:
+        incl = p[v] + sum(p[u] * p[v] / (1 - p[u]) for u in imp if u != v)
+        freq = ((final == v).any(axis=1)).mean()
+        assert abs(freq - incl) < 0.012
+
+
+def test_ladies_importance_short_neighbourhood_leaves_invalid(oracle):
+    adj = [[1], [0], []]
+    g = oracle.Graph.from_adjacency(adj)
+    d = oracle.app_desc(oracle.LADIES_IMPORTANCE, 2, 3, initial_size=1)
+    final = oracle.sample_ladies_importance(g, d, SEED, np.array([0, 2], np.int32))
+    assert list(final[0]) == [1, 3, 3, 0, 3, 3]   # one neighbour per layer, then INVALID (= 3)
+    assert np.all(final[1] == 3)
