@@ -76,6 +76,9 @@ const AppEntry kApps[] = {
     {"FastGCNImportance2x8", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 8, 100>>},
     {"FastGCNImportance3x16", make_layer_engine<LayerNoState, FastGCNImportanceAppT<3, 16, 300>>},
     {"LADIESImportance", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 512, 1024>>},
+    // the same samplers with fewer batches per launch (quick checks on the full-size graphs)
+    {"FastGCNImportanceB128", make_layer_engine<LayerNoState, FastGCNImportanceAppT<2, 64, 128>>},
+    {"LADIESImportanceB8", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 512, 8>>},
     {"LADIESImportance2x8", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 8, 100>>},
     {"LADIESImportance3x16", make_layer_engine<LayerNoState, LadiesImportanceAppT<3, 16, 300>>},
 };

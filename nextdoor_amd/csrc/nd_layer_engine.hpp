@@ -31,6 +31,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 #include <stdlib.h>
 
 #include <string>
@@ -412,6 +413,7 @@ class LayerEngine : public EngineBase {
     hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
     h_sizes_.resize((size_t)n_samples_);
     chunk_entries_ = kLayerChunkEntries;
+    progress_ = getenv("ND_PROGRESS") != nullptr;  // long layers report on stderr every 16 chunks
     if (const char* env = getenv("ND_LAYER_CHUNK_ENTRIES")) {  // smaller chunks, e.g. to exercise chunking
       const long long v = atoll(env);
       if (v > 0) chunk_entries_ = (uint64_t)v;
@@ -484,6 +486,12 @@ class LayerEngine : public EngineBase {
         if (run_chunk(step, all, s0, s1, (uint32_t)total) != 0) return -1;
         neighborhood_total_ += total;
         chunks_run_++;
+        if (progress_ && chunks_run_ % 16 == 0) {
+          ND_HIP_TRY(hipStreamSynchronize(stream_));
+          fprintf(stderr, "[nextdoor] layer %d: samples %u of %u done, %llu neighbourhood entries so far\n", step, s1,
+                  S, (unsigned long long)neighborhood_total_);
+          fflush(stderr);
+        }
         s0 = s1;
       }
     }
@@ -717,6 +725,7 @@ class LayerEngine : public EngineBase {
   size_t capacity_ = 0;
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
   uint64_t chunk_entries_ = kLayerChunkEntries;
+  bool progress_ = false;
 
   hipStream_t stream_ = nullptr;
   hipEvent_t ev_begin_ = nullptr, ev_end_ = nullptr;
