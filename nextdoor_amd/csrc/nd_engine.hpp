@@ -109,6 +109,7 @@ struct StepParams {
   uint64_t first_slot;           // RNG slot of local output 0 (first sample of this device)
   uint32_t first_sample;
   uint32_t n_pairs;              // S * T_k
+  const uint32_t* live_pairs;    // device count of pairs in pair_keys (sorted map: pairs with a real transit); nullptr: n_pairs
   const uint32_t* pair_keys;     // transit of each pair (sorted, or the raw map at step 0)
   const uint32_t* pair_slots;    // slot of each pair; nullptr: slot == index
   int32_t* step_out;             // outputs of this step, indexed by output slot; it is both
@@ -168,7 +169,7 @@ __device__ __forceinline__ uint32_t flat_block_index() {
 // skip_flag (nullable): per-vertex marker of transits the workgroup kernel handles.
 template <class SampleType, class App>
 __global__ __launch_bounds__(kStepThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
-  const uint64_t total = (uint64_t)P.n_pairs * P.step_size;
+  const uint64_t total = (uint64_t)(P.live_pairs ? *P.live_pairs : P.n_pairs) * P.step_size;
   const uint64_t i = (uint64_t)flat_block_index() * kStepThreads + threadIdx.x;
   if (i >= total) return;
   CSRPartition csr = P.csr;
@@ -239,7 +240,14 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
   }
 }
 
-// One lane per unique transit: decide which kernel class serves it and emit work items.
+// Load balancing without a scan: the pairs are sorted by transit, so the first pair of a
+// run knows where the run starts (the exclusive scan of the run lengths IS that position)
+// and the last pair of a run knows where it ends.  mark_run_heads records the start per
+// transit vertex; classify_run_tails, one lane per pair, lets the last pair of each run
+// decide which kernel class serves the transit and emit work items.  Two launches where the
+// reference has a boundary search, a run-length encode, a scan, a partition kernel and
+// three blocking copies (src/nextdoor.cu:2498-2636).
+//
 // Classes by neighbour-work (outputs drawn from the transit = count * stepSize):
 //   work <  kWorkgroupWork                      -> flat kernel (sub-wavefront: the lanes of a
 //                                                  wave that share the transit share its lines)
@@ -247,16 +255,35 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
 //   work >  kChunkOutputs, several work items   -> grid-wide: the transit is split over workgroups
 // A transit whose adjacency does not fit the LDS cache, or is much longer than the number
 // of draws taken from it, is cheaper to gather directly and stays with the flat kernel.
-__global__ __launch_bounds__(256) void classify_runs(const uint32_t* __restrict__ run_key,
-                                                     const uint32_t* __restrict__ run_start, RunsMeta* meta,
-                                                     const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
-                                                     uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
-                                                     uint8_t* __restrict__ skip_flag) {
-  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
-  if (r >= meta->n_runs) return;
-  const uint32_t start = run_start[r];
-  const uint32_t count = run_start[r + 1] - start;
-  const uint32_t transit = run_key[r];
+__global__ __launch_bounds__(256) void mark_run_heads(const uint32_t* __restrict__ keys,
+                                                      const uint32_t* __restrict__ n_dev,
+                                                      uint32_t* __restrict__ start_of, RunsMeta* meta) {
+  const uint32_t n = *n_dev;
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i == 0) {
+    meta->n_valid = n;
+    meta->n_runs = 0;
+    meta->n_chunks = 0;
+    meta->n_big_pairs = 0;
+  }
+  if (i >= n) return;
+  const uint32_t k = keys[i];
+  if (i == 0 || keys[i - 1] != k) start_of[k] = i;
+}
+
+__global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __restrict__ keys,
+                                                          const uint32_t* __restrict__ n_dev,
+                                                          const uint32_t* __restrict__ start_of, RunsMeta* meta,
+                                                          const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
+                                                          uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
+                                                          uint8_t* __restrict__ skip_flag) {
+  const uint32_t n = *n_dev;
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t transit = keys[i];
+  if (i + 1 != n && keys[i + 1] == transit) return;  // not the last pair of its run
+  const uint32_t start = start_of[transit];
+  const uint32_t count = i + 1 - start;
   const uint64_t work = (uint64_t)count * step_size;
   if (work < kWorkgroupWork) return;
   const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
@@ -480,11 +507,9 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * max_pairs_));
     const SortPlan plan = make_sort_plan(max_pairs_, max_bits_);
     ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * plan.hist_elems));
-    size_t scratch = plan.scratch_elems;
-    if (runs_scratch_elems(max_pairs_) > scratch) scratch = runs_scratch_elems(max_pairs_);
-    ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
-    ND_HIP_TRY(hipMalloc(&d_run_key_, sizeof(uint32_t) * max_pairs_));
-    ND_HIP_TRY(hipMalloc(&d_run_start_, sizeof(uint32_t) * (max_pairs_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * plan.scratch_elems));
+    ND_HIP_TRY(hipMalloc(&d_run_start_of_, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_live_, sizeof(uint32_t)));
     ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta)));
     ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta)));
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
@@ -523,6 +548,13 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
 
+    // pairs whose transit is INVALID are dropped by the inversion and never reach a step
+    // kernel: their outputs keep this fill
+    {
+      const size_t n_out = (size_t)n_samples_ * F;
+      fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(d_step_out_, n_out, invalid_);
+    }
+
     uint32_t transits_per_sample = (uint32_t)init_size_;
     const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
     for (int step = 0; step < n_steps; ++step) {
@@ -541,6 +573,7 @@ class Engine : public EngineBase {
       P.first_slot = 0;
       P.first_sample = 0;
       P.n_pairs = n_pairs;
+      P.live_pairs = nullptr;
       P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
       P.samples = d_samples_;
       P.paired_edges = dgraph_.paired;
@@ -564,11 +597,13 @@ class Engine : public EngineBase {
         uint32_t *sorted_keys = nullptr, *sorted_slots = nullptr;
         tick();
         ND_HIP_TRY(radix_sort_pairs(plan, (const uint32_t*)transits, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
-                                    d_vals_b_, d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots));
+                                    d_vals_b_, d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots,
+                                    (uint32_t)invalid_, d_live_));
         tock(&times.inversion);
         times.sort_launches += plan.passes;
         P.pair_keys = sorted_keys;
         P.pair_slots = sorted_slots;
+        P.live_pairs = d_live_;
         if (!balance) {
           tick();
           step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, nullptr);
@@ -576,11 +611,11 @@ class Engine : public EngineBase {
           times.flat_launches++;
         } else {
           tick();
-          ND_HIP_TRY(find_transit_runs(sorted_keys, n_pairs, (uint32_t)invalid_, d_run_key_, d_run_start_, d_meta_,
-                                       d_scratch_, stream_));
-          const unsigned max_runs = n_pairs < (uint32_t)invalid_ ? n_pairs : (uint32_t)invalid_;
-          classify_runs<<<dim3((max_runs + 255) / 256), dim3(256), 0, stream_>>>(
-              d_run_key_, d_run_start_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_, d_skip_flag_);
+          const unsigned pair_blocks = (n_pairs + 255) / 256;
+          mark_run_heads<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(sorted_keys, d_live_, d_run_start_of_, d_meta_);
+          classify_run_tails<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
+              sorted_keys, d_live_, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+              d_skip_flag_);
           tock(&times.load_balancing);
           tick();
           step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kStepThreads), 0, stream_>>>(P, d_skip_flag_);
@@ -708,8 +743,8 @@ class Engine : public EngineBase {
     release(d_vals_b_);
     release(d_hist_);
     release(d_scratch_);
-    release(d_run_key_);
-    release(d_run_start_);
+    release(d_run_start_of_);
+    release(d_live_);
     release(d_meta_);
     release(d_chunks_);
     release(d_skip_flag_);
@@ -751,8 +786,8 @@ class Engine : public EngineBase {
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
-  uint32_t* d_run_key_ = nullptr;
-  uint32_t* d_run_start_ = nullptr;
+  uint32_t* d_run_start_of_ = nullptr;  // per transit vertex: first position of its run in the sorted map
+  uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits)
   RunsMeta* d_meta_ = nullptr;
   uint32_t* d_chunks_ = nullptr;
   uint8_t* d_skip_flag_ = nullptr;

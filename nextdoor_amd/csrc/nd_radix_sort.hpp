@@ -36,17 +36,24 @@ __device__ __forceinline__ int tile_offset(int wave, int it, int lane) {
   return wave * (kWave * kSortItems) + it * kWave + lane;
 }
 
-__global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* __restrict__ keys, size_t n, int shift,
-                                                                uint32_t mask, uint32_t* __restrict__ hist,
-                                                                uint32_t num_tiles) {
+// n_dev (nullable): element count kept in device memory; overrides n when given.
+// drop_key: keys equal to it are left out of the sort (kPadKey: nothing is left out).
+__global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* __restrict__ keys, size_t n,
+                                                                const uint32_t* __restrict__ n_dev, int shift,
+                                                                uint32_t mask, uint32_t drop_key,
+                                                                uint32_t* __restrict__ hist, uint32_t num_tiles) {
   __shared__ uint32_t s_hist[kRadix];
   s_hist[threadIdx.x] = 0;
   __syncthreads();
+  if (n_dev) n = *n_dev;
   const size_t tile_start = (size_t)blockIdx.x * kSortTile;
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
     const size_t idx = tile_start + (size_t)it * kSortThreads + threadIdx.x;
-    if (idx < n) atomicAdd(&s_hist[(keys[idx] >> shift) & mask], 1u);
+    if (idx < n) {
+      const uint32_t k = keys[idx];
+      if (k != drop_key) atomicAdd(&s_hist[(k >> shift) & mask], 1u);
+    }
   }
   __syncthreads();
   if (threadIdx.x <= mask) hist[(size_t)threadIdx.x * num_tiles + blockIdx.x] = s_hist[threadIdx.x];
@@ -56,10 +63,11 @@ template <bool kIotaValues>
 __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __restrict__ keys_in,
                                                               const uint32_t* __restrict__ vals_in,
                                                               uint32_t* __restrict__ keys_out,
-                                                              uint32_t* __restrict__ vals_out, size_t n, int shift,
-                                                              uint32_t mask, int digit_bits,
+                                                              uint32_t* __restrict__ vals_out, size_t n,
+                                                              const uint32_t* __restrict__ n_dev, int shift,
+                                                              uint32_t mask, int digit_bits, uint32_t drop_key,
                                                               const uint32_t* __restrict__ scanned_hist,
-                                                              uint32_t num_tiles) {
+                                                              uint32_t num_tiles, uint32_t* __restrict__ kept_out) {
   __shared__ uint32_t s_keys[kSortTile];
   __shared__ uint32_t s_vals[kSortTile];
   __shared__ uint32_t s_wave_count[kSortWaves][kRadix];
@@ -70,7 +78,11 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
+  if (n_dev) n = *n_dev;
   const size_t tile_start = (size_t)blockIdx.x * kSortTile;
+  // number of keys the whole sort keeps = total of the scanned digit table; published once
+  if (kept_out && blockIdx.x == 0 && tid == 0) kept_out[0] = scanned_hist[(size_t)(mask + 1) * num_tiles];
+  if (tile_start >= n) return;
   const uint32_t in_tile = (uint32_t)((n - tile_start) < (size_t)kSortTile ? (n - tile_start) : (size_t)kSortTile);
 
 #pragma unroll
@@ -78,29 +90,31 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   __syncthreads();
 
   uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
+  bool live[kSortItems];
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
     const uint32_t off = (uint32_t)tile_offset(wave, it, lane);
-    const bool live = off < in_tile;
-    key[it] = live ? keys_in[tile_start + off] : kPadKey;
+    const bool inside = off < in_tile;
+    key[it] = inside ? keys_in[tile_start + off] : kPadKey;
+    live[it] = inside && key[it] != drop_key;
     if (kIotaValues) val[it] = (uint32_t)(tile_start + off);
-    else val[it] = live ? vals_in[tile_start + off] : 0u;
+    else val[it] = inside ? vals_in[tile_start + off] : 0u;
   }
 
   const uint64_t lanes_below = (1ull << lane) - 1ull;
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
     const uint32_t digit = (key[it] >> shift) & mask;
-    // peers = lanes of this wave holding the same digit
-    uint64_t peers = ~0ull;
+    // peers = live lanes of this wave holding the same digit
+    uint64_t peers = __ballot(live[it]);
     for (int b = 0; b < digit_bits; ++b) {
       const bool bit = (digit >> b) & 1u;
       const uint64_t vote = __ballot(bit);
       peers &= bit ? vote : ~vote;
     }
-    const int leader = __ffsll((unsigned long long)peers) - 1;
     uint32_t before = 0;
-    if (lane == leader) before = atomicAdd(&s_wave_count[wave][digit], (uint32_t)__popcll(peers));
+    const int leader = peers ? __ffsll((unsigned long long)peers) - 1 : 0;
+    if (live[it] && lane == leader) before = atomicAdd(&s_wave_count[wave][digit], (uint32_t)__popcll(peers));
     before = __shfl(before, leader, kWave);
     rank[it] = before + (uint32_t)__popcll(peers & lanes_below);
   }
@@ -115,24 +129,24 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
     s_wave_count[w][tid] = digit_total;
     digit_total += c;
   }
-  uint32_t tile_total;
-  const uint32_t digit_base = block_exclusive_scan_256(digit_total, s_scan_tmp, &tile_total);
+  uint32_t live_in_tile;
+  const uint32_t digit_base = block_exclusive_scan_256(digit_total, s_scan_tmp, &live_in_tile);
   s_digit_base[tid] = digit_base;
   if ((uint32_t)tid <= mask) s_global_base[tid] = scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
   __syncthreads();
 
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
-    const uint32_t digit = (key[it] >> shift) & mask;
-    const uint32_t pos = s_digit_base[digit] + s_wave_count[wave][digit] + rank[it];
-    s_keys[pos] = key[it];
-    s_vals[pos] = val[it];
+    if (live[it]) {
+      const uint32_t digit = (key[it] >> shift) & mask;
+      const uint32_t pos = s_digit_base[digit] + s_wave_count[wave][digit] + rank[it];
+      s_keys[pos] = key[it];
+      s_vals[pos] = val[it];
+    }
   }
   __syncthreads();
 
-  // pad keys carry the largest digit and come last in input order, so the live keys
-  // occupy positions [0, in_tile)
-  for (uint32_t p = tid; p < in_tile; p += kSortThreads) {
+  for (uint32_t p = tid; p < live_in_tile; p += kSortThreads) {
     const uint32_t k = s_keys[p];
     const uint32_t out = s_global_base[(k >> shift) & mask] + p;
     keys_out[out] = k;
@@ -155,7 +169,7 @@ inline SortPlan make_sort_plan(size_t n, int key_bits) {
   p.key_bits = key_bits < 1 ? 1 : key_bits;
   p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
   p.num_tiles = (uint32_t)((n + kSortTile - 1) / kSortTile);
-  p.hist_elems = (size_t)kRadix * p.num_tiles;
+  p.hist_elems = (size_t)kRadix * p.num_tiles + 1;  // + the grand total the scan appends
   p.scratch_elems = scan_scratch_elems(p.hist_elems);
   return p;
 }
@@ -164,10 +178,15 @@ inline SortPlan make_sort_plan(size_t n, int key_bits) {
 // vals_in == nullptr means "value = index".  Two ping-pong buffer pairs (a, b) of n
 // elements each; the result lands in *keys_sorted / *vals_sorted (one of a / b).
 // hist needs plan.hist_elems and scratch plan.scratch_elems uint32.
+// drop_key / kept_dev: pairs whose key equals drop_key are left out by the first pass and
+// the number of pairs kept is stored in kept_dev[0] (device memory); later passes and the
+// caller's kernels read the count from there, no host round trip.  Pass kPadKey and
+// nullptr to sort everything.
 inline hipError_t radix_sort_pairs(const SortPlan& plan, const uint32_t* keys_in, const uint32_t* vals_in,
                                    uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b, uint32_t* vals_b,
                                    uint32_t* hist, uint32_t* scratch, hipStream_t stream,
-                                   uint32_t** keys_sorted, uint32_t** vals_sorted) {
+                                   uint32_t** keys_sorted, uint32_t** vals_sorted, uint32_t drop_key = kPadKey,
+                                   uint32_t* kept_dev = nullptr) {
   *keys_sorted = keys_a;
   *vals_sorted = vals_a;
   if (plan.n == 0) return hipSuccess;
@@ -183,16 +202,20 @@ inline hipError_t radix_sort_pairs(const SortPlan& plan, const uint32_t* keys_in
     const int bits = (remaining + passes_left - 1) / passes_left;
     const uint32_t mask = (1u << bits) - 1u;
     const size_t table = ((size_t)mask + 1) * plan.num_tiles;
-    radix_histogram<<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(src_k, plan.n, shift, mask, hist,
-                                                                            plan.num_tiles);
-    hipError_t e = exclusive_scan_u32(hist, hist, table, scratch, stream);
+    const uint32_t* n_dev = pass > 0 ? kept_dev : nullptr;
+    const uint32_t drop = pass == 0 ? drop_key : kPadKey;
+    radix_histogram<<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(src_k, plan.n, n_dev, shift, mask, drop,
+                                                                            hist, plan.num_tiles);
+    // one element more than the table: the scan leaves the grand total there
+    hipError_t e = exclusive_scan_u32(hist, hist, table + 1, scratch, stream);
     if (e != hipSuccess) return e;
+    uint32_t* kept_out = pass == 0 ? kept_dev : nullptr;
     if (pass == 0 && src_v == nullptr)
       radix_scatter<true><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
-          src_k, nullptr, dst_k, dst_v, plan.n, shift, mask, bits, hist, plan.num_tiles);
+          src_k, nullptr, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, plan.num_tiles, kept_out);
     else
       radix_scatter<false><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
-          src_k, src_v, dst_k, dst_v, plan.n, shift, mask, bits, hist, plan.num_tiles);
+          src_k, src_v, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, plan.num_tiles, kept_out);
     *keys_sorted = dst_k;
     *vals_sorted = dst_v;
     src_k = dst_k;
