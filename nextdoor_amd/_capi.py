@@ -73,10 +73,11 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("NEXTDOOR_AMD_LIB", LIB_PATH)  # an explicitly chosen build of the library
+    if path == LIB_PATH and not os.path.exists(LIB_PATH):
         from .build import build
         build()
-    handle = C.CDLL(LIB_PATH)
+    handle = C.CDLL(path)
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(handle, name)  # AttributeError here = the library lacks a declared symbol
         fn.restype = restype

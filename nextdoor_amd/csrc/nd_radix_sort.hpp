@@ -7,8 +7,9 @@
 // not the sample id, so the step kernels can place outputs without atomics; on the first
 // pass the values are generated from the index instead of being read.
 //
-// Per 8-bit digit pass: (1) per-tile digit histogram, (2) exclusive scan of the
-// digit-major histogram table, (3) scatter.  The scatter ranks keys inside a tile with
+// Per 8-bit digit pass: (1) per-tile digit histogram into a digit-major table, (2) one
+// workgroup per digit turns its row into exclusive prefixes over tiles and leaves the row
+// total, (3) scatter (every workgroup scans the 256 row totals itself).  The scatter ranks keys inside a tile with
 // wave64 ballots (match-any on the digit), keeps one running counter per wave and digit in
 // LDS, stages the tile digit-sorted in LDS and writes runs of equal digits to HBM.
 // No spinning, no inter-workgroup waiting.
@@ -59,6 +60,28 @@ __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* 
   if (threadIdx.x <= mask) hist[(size_t)threadIdx.x * num_tiles + blockIdx.x] = s_hist[threadIdx.x];
 }
 
+// One workgroup per digit: exclusive scan of the digit's row of the table (over tiles) in
+// place, and the row total.
+__global__ __launch_bounds__(kSortThreads) void radix_row_scan(uint32_t* __restrict__ hist, uint32_t num_tiles,
+                                                               uint32_t* __restrict__ row_totals) {
+  __shared__ uint32_t s_scan_tmp[kSortWaves];
+  uint32_t* row = hist + (size_t)blockIdx.x * num_tiles;
+  // thread t owns a contiguous stretch of the row
+  const uint32_t per_thread = (num_tiles + kSortThreads - 1) / kSortThreads;
+  const uint32_t begin = threadIdx.x * per_thread;
+  const uint32_t end = begin + per_thread < num_tiles ? begin + per_thread : num_tiles;
+  uint32_t sum = 0;
+  for (uint32_t i = begin; i < end; ++i) sum += row[i];
+  uint32_t total;
+  uint32_t running = block_exclusive_scan_256(sum, s_scan_tmp, &total);
+  for (uint32_t i = begin; i < end; ++i) {
+    const uint32_t c = row[i];
+    row[i] = running;
+    running += c;
+  }
+  if (threadIdx.x == 0) row_totals[blockIdx.x] = total;
+}
+
 template <bool kIotaValues>
 __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __restrict__ keys_in,
                                                               const uint32_t* __restrict__ vals_in,
@@ -67,6 +90,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
                                                               const uint32_t* __restrict__ n_dev, int shift,
                                                               uint32_t mask, int digit_bits, uint32_t drop_key,
                                                               const uint32_t* __restrict__ scanned_hist,
+                                                              const uint32_t* __restrict__ row_totals,
                                                               uint32_t num_tiles, uint32_t* __restrict__ kept_out) {
   __shared__ uint32_t s_keys[kSortTile];
   __shared__ uint32_t s_vals[kSortTile];
@@ -80,8 +104,13 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   const int wave = tid >> 6;
   if (n_dev) n = *n_dev;
   const size_t tile_start = (size_t)blockIdx.x * kSortTile;
-  // number of keys the whole sort keeps = total of the scanned digit table; published once
-  if (kept_out && blockIdx.x == 0 && tid == 0) kept_out[0] = scanned_hist[(size_t)(mask + 1) * num_tiles];
+  if (tile_start >= n && !(kept_out && blockIdx.x == 0)) return;
+  // first position of every digit in the output: exclusive scan of the row totals
+  uint32_t kept_total;
+  const uint32_t digit_first = block_exclusive_scan_256((uint32_t)tid <= mask ? row_totals[tid] : 0u, s_scan_tmp,
+                                                        &kept_total);
+  // number of keys the whole sort keeps; published once
+  if (kept_out && blockIdx.x == 0 && tid == 0) kept_out[0] = kept_total;
   if (tile_start >= n) return;
   const uint32_t in_tile = (uint32_t)((n - tile_start) < (size_t)kSortTile ? (n - tile_start) : (size_t)kSortTile);
 
@@ -132,7 +161,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   uint32_t live_in_tile;
   const uint32_t digit_base = block_exclusive_scan_256(digit_total, s_scan_tmp, &live_in_tile);
   s_digit_base[tid] = digit_base;
-  if ((uint32_t)tid <= mask) s_global_base[tid] = scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
+  if ((uint32_t)tid <= mask)
+    s_global_base[tid] = digit_first + scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
   __syncthreads();
 
 #pragma unroll
@@ -160,7 +190,7 @@ struct SortPlan {
   int passes = 0;
   uint32_t num_tiles = 0;
   size_t hist_elems = 0;     // kRadix * num_tiles
-  size_t scratch_elems = 0;  // scan scratch
+  size_t scratch_elems = 0;  // digit row totals
 };
 
 inline SortPlan make_sort_plan(size_t n, int key_bits) {
@@ -169,8 +199,8 @@ inline SortPlan make_sort_plan(size_t n, int key_bits) {
   p.key_bits = key_bits < 1 ? 1 : key_bits;
   p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
   p.num_tiles = (uint32_t)((n + kSortTile - 1) / kSortTile);
-  p.hist_elems = (size_t)kRadix * p.num_tiles + 1;  // + the grand total the scan appends
-  p.scratch_elems = scan_scratch_elems(p.hist_elems);
+  p.hist_elems = (size_t)kRadix * p.num_tiles;
+  p.scratch_elems = kRadix;  // row totals
   return p;
 }
 
@@ -201,21 +231,18 @@ inline hipError_t radix_sort_pairs(const SortPlan& plan, const uint32_t* keys_in
     const int passes_left = plan.passes - pass;
     const int bits = (remaining + passes_left - 1) / passes_left;
     const uint32_t mask = (1u << bits) - 1u;
-    const size_t table = ((size_t)mask + 1) * plan.num_tiles;
     const uint32_t* n_dev = pass > 0 ? kept_dev : nullptr;
     const uint32_t drop = pass == 0 ? drop_key : kPadKey;
     radix_histogram<<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(src_k, plan.n, n_dev, shift, mask, drop,
                                                                             hist, plan.num_tiles);
-    // one element more than the table: the scan leaves the grand total there
-    hipError_t e = exclusive_scan_u32(hist, hist, table + 1, scratch, stream);
-    if (e != hipSuccess) return e;
+    radix_row_scan<<<dim3(mask + 1), dim3(kSortThreads), 0, stream>>>(hist, plan.num_tiles, scratch);
     uint32_t* kept_out = pass == 0 ? kept_dev : nullptr;
     if (pass == 0 && src_v == nullptr)
       radix_scatter<true><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
-          src_k, nullptr, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, plan.num_tiles, kept_out);
+          src_k, nullptr, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, scratch, plan.num_tiles, kept_out);
     else
       radix_scatter<false><<<dim3(plan.num_tiles), dim3(kSortThreads), 0, stream>>>(
-          src_k, src_v, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, plan.num_tiles, kept_out);
+          src_k, src_v, dst_k, dst_v, plan.n, n_dev, shift, mask, bits, drop, hist, scratch, plan.num_tiles, kept_out);
     *keys_sorted = dst_k;
     *vals_sorted = dst_v;
     src_k = dst_k;
