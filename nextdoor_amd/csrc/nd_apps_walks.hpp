@@ -74,21 +74,17 @@ struct HundredWalksOnSmallGraphs : WalkCommon<kWalkLength> {
 
 // Rejection sampling of an edge proportionally to its weight, against the largest
 // weight of the transit (randomWalks.cu:81-88).  Returns the accepted edge index.
-// Candidate i consumes draws 2i (edge index) and 2i+1 (height), exactly as the loop in
-// the reference; two candidates are drawn and their weights gathered together so the two
-// memory accesses overlap, and the second is simply not used when the first is accepted.
+// Candidate i consumes draws 2i (edge index) and 2i+1 (height).
 template <typename WeightArray>
 __device__ __forceinline__ EdgePos_t weighted_edge_by_rejection(const WeightArray& w, EdgePos_t n, float max_weight,
                                                                 curandState* state) {
-  for (;;) {
-    const EdgePos_t x0 = RandNumGen::rand_int(state, n);
-    const float y0 = curand_uniform(state) * max_weight;
-    const EdgePos_t x1 = RandNumGen::rand_int(state, n);
-    const float y1 = curand_uniform(state) * max_weight;
-    const float w0 = w[x0], w1 = w[x1];
-    if (!(y0 > w0)) return x0;
-    if (!(y1 > w1)) return x1;
+  EdgePos_t x = RandNumGen::rand_int(state, n);
+  float y = curand_uniform(state) * max_weight;
+  while (y > w[x]) {
+    x = RandNumGen::rand_int(state, n);
+    y = curand_uniform(state) * max_weight;
   }
+  return x;
 }
 
 }  // namespace apps
@@ -200,23 +196,15 @@ struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
       else if (csr->has_edge_logn(prev, v)) h = 1 / q;
       return y < h * wx;
     };
-    // candidate i consumes draws 2i (edge index) and 2i+1 (height); two candidates are
-    // drawn and gathered together so their memory accesses overlap, and the second is not
-    // used when the first is accepted
+    // candidate i consumes draws 2i (edge index) and 2i+1 (height)
     for (;;) {
-      const EdgePos_t x0 = RandNumGen::rand_int(state, numEdges);
-      const float y0 = curand_uniform(state) * envelope;
-      const EdgePos_t x1 = RandNumGen::rand_int(state, numEdges);
-      const float y1 = curand_uniform(state) * envelope;
-      const VertexID v0 = transitEdges[x0], v1 = transitEdges[x1];
-      const float w0 = transitEdgeWeights[x0], w1 = transitEdgeWeights[x1];
-      if (accepts(v0, w0, y0)) {
+      const EdgePos_t x = RandNumGen::rand_int(state, numEdges);
+      const float y = curand_uniform(state) * envelope;
+      const VertexID v = transitEdges[x];
+      const float wx = transitEdgeWeights[x];
+      if (accepts(v, wx, y)) {
         sample->t = *transits;
-        return v0;
-      }
-      if (accepts(v1, w1, y1)) {
-        sample->t = *transits;
-        return v1;
+        return v;
       }
     }
   }
