@@ -190,10 +190,12 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
   EdgePos_t n_edges = 0, begin = 0;
   float max_weight = 0.0f;
   if (transit != P.invalid) {
-    if (skip_flag && skip_flag[transit]) return;
+    // the marker, the row extent and the largest weight are fetched together
+    const uint8_t taken = skip_flag ? skip_flag[transit] : (uint8_t)0;
     begin = csr.row_ptr[transit];
     n_edges = csr.row_ptr[transit + 1] - begin;
     max_weight = csr.max_weights[transit];
+    if (taken) return;
   }
   if (app_uses_weights<App>::value) {
     PairedEdgeIds edges{P.paired_edges + begin};
@@ -347,14 +349,26 @@ __global__ __launch_bounds__(256) void assemble_final_rows(const int32_t* __rest
   extern __shared__ int32_t s_rows[];
   const uint32_t s0 = blockIdx.x * samples_per_block;
   const uint32_t nb = n_samples - s0 < samples_per_block ? n_samples - s0 : samples_per_block;
-  for (int k = 0; k < layout.n_steps; ++k) {
+  // Steps whose slice of this block is narrower than the workgroup (walks: one entry per
+  // sample and step) are read several steps at a time, so that all lanes have a load in
+  // flight; wider slices one step at a time.
+  int k = 0;
+  while (k < layout.n_steps) {
     const uint32_t len = layout.seg_len[k];
-    const int32_t* src = step_out + (size_t)n_samples * layout.seg_base[k] + (size_t)s0 * len;
-    for (uint32_t e = threadIdx.x; e < nb * len; e += 256) {
-      const uint32_t s = len == 1 ? e : e / len;
-      const uint32_t j = e - s * len;
-      s_rows[s * row_pitch + layout.seg_base[k] + j] = src[e];
+    const uint32_t slice = nb * len;
+    uint32_t group = slice >= 256 ? 1u : 256u / slice;
+    uint32_t same = 1;  // consecutive steps with the same segment length
+    while (same < group && k + (int)same < layout.n_steps && layout.seg_len[k + same] == len) ++same;
+    group = same;
+    for (uint32_t e = threadIdx.x; e < slice * group; e += 256) {
+      const uint32_t g = e / slice;
+      const uint32_t within = e - g * slice;
+      const uint32_t s = len == 1 ? within : within / len;
+      const uint32_t j = within - s * len;
+      const uint32_t base = layout.seg_base[k + g];
+      s_rows[s * row_pitch + base + j] = step_out[(size_t)n_samples * base + (size_t)s0 * len + within];
     }
+    k += (int)group;
   }
   __syncthreads();
   int32_t* dst = final_samples + (size_t)s0 * final_size;
