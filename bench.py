@@ -40,6 +40,15 @@ WORKLOADS = {
     "uniform_walk_chunglu57k": dict(app="UniformRandomWalk", kind="UNIFORM_WALK",
                                     graph=("chung_lu", dict(n_vertices=56944, n_edges=818000, exponent=2.1))),
     "khop_rmat21": dict(app="KHop", kind="KHOP", graph=("rmat", dict(scale=21, edge_factor=32, symmetrise=False))),
+    "fastgcn_importance_rmat22": dict(app="FastGCNImportance", kind="FASTGCN_IMPORTANCE",
+                                      graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
+    "fastgcn_importance_rmat22_b128": dict(app="FastGCNImportanceB128", kind="FASTGCN_IMPORTANCE",
+                                           graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
+    "ladies_importance_chunglu3m": dict(app="LADIESImportance", kind="LADIES_IMPORTANCE",
+                                        graph=("chung_lu", dict(n_vertices=3072441, n_edges=117000000, exponent=2.0))),
+    "ladies_importance_chunglu3m_b8": dict(app="LADIESImportanceB8", kind="LADIES_IMPORTANCE",
+                                           graph=("chung_lu", dict(n_vertices=3072441, n_edges=117000000,
+                                                                   exponent=2.0))),
 }
 
 
@@ -158,6 +167,15 @@ def main():
         "phases_ms": {k: round(v, 3) for k, v in prof.items()},
     }
 
+    if w["kind"] in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE", "LAYER_LITERAL"):
+        result["config"]["neighbourhood_entries"] = sampler.counter(0)
+        result["config"]["distinct_pairs"] = sampler.counter(1)
+        result["config"]["chunks"] = sampler.counter(2)
+        args.skip_cpu_baseline = True  # the walk/k-hop accounting below does not apply to layer-wise apps
+    if w["kind"] == "KHOP":
+        counts = sampler.distinct()
+        result["config"]["distinct_ms"] = sampler.phase_times()["distinct_ms"]
+        result["config"]["distinct_kept"] = int(counts.sum())
     if not args.skip_cpu_baseline:
         base, run = cpu_baseline(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
         result["cpu_baseline"] = base

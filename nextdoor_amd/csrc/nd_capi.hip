@@ -444,9 +444,21 @@ int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64
   if (total > capacity) return fail("collective neighbourhood larger than the capacity given");
   CAPI_HIP(d_cols.alloc(sizeof(int32_t) * (size_t)total));
   CAPI_HIP(d_weights.alloc(sizeof(float) * (size_t)total));
-  nd::collective_build<<<dim3(S), dim3(256), 0, 0>>>(dg.view, tv, invalid, d_offsets.as<uint32_t>(),
-                                                    d_cols.as<int32_t>(), d_weights.as<float>(), nullptr,
-                                                    d_rows.as<uint32_t>(), nullptr);
+  DeviceBuffer d_item_count, d_item_start;
+  CAPI_HIP(d_item_count.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+  CAPI_HIP(d_item_start.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+  uint64_t n_items = 0;
+  for (uint32_t i = 0; i < S; ++i) {
+    const uint64_t items = ((uint64_t)(uint32_t)sizes[i] + nd::kBuildItemEntries - 1) / nd::kBuildItemEntries;
+    n_items += items ? items : 1;
+  }
+  nd::build_item_counts<<<dim3((S + 1 + 255) / 256), dim3(256), 0, 0>>>(d_sizes.as<uint32_t>(), S,
+                                                                       d_item_count.as<uint32_t>());
+  CAPI_HIP(nd::exclusive_scan_u32(d_item_count.as<uint32_t>(), d_item_start.as<uint32_t>(), (size_t)S + 1,
+                                  d_scratch.as<uint32_t>(), 0));
+  nd::collective_build<<<dim3((unsigned)n_items), dim3(256), 0, 0>>>(
+      dg.view, tv, invalid, d_offsets.as<uint32_t>(), d_item_start.as<uint32_t>(), S, d_cols.as<int32_t>(),
+      d_weights.as<float>(), nullptr, d_rows.as<uint32_t>(), nullptr);
   CAPI_HIP(hipGetLastError());
   CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
   CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));

@@ -21,8 +21,8 @@
 //    stable radix sorts, run heads give the distinct vertices, and a 64-bit inclusive scan
 //    of degree^2 gives the running sums the app inverts.
 //  * For kRankedByLadiesImportance each entry of the concatenation carries
-//    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed in concatenation
-//    order (the sorts are stable), Efraimidis-Spirakis keys are computed per distinct vertex
+//    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed as 2^53
+//    fixed-point integers, Efraimidis-Spirakis keys are computed per distinct vertex
 //    and two more stable sorts order the distinct vertices of every sample by descending key.
 //  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
 //    of entries, so a layer whose frontier sits on hubs cannot outgrow memory.
@@ -72,18 +72,33 @@ __global__ __launch_bounds__(256) void collective_sizes(CSRPartition csr, Transi
   if (lane == 0) sizes[s] = sum;
 }
 
-// One workgroup per sample: copy the adjacencies of its transits, in transit order, to
+// Entries of a sample's concatenation one workgroup of collective_build copies; samples
+// with longer neighbourhoods are spread over several workgroups.
+constexpr uint32_t kBuildItemEntries = 8192;
+
+// Copies the adjacencies of every sample's transits, in transit order, to
 // cols[offsets[s] ...] (and weights, and the owning sample id when asked for).
+// Work items: item_start[s] = number of items of the samples before s (exclusive scan of
+// ceil(size_s / kBuildItemEntries), with the total at [n_samples]); workgroup b serves the
+// sample whose item range holds b and the b - item_start[s]-th stretch of its entries.
 // row_sums (nullable): when given, the weight slot receives (weight / row_sums[transit])^2.
 __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, TransitView tv, int32_t invalid,
                                                         const uint32_t* __restrict__ offsets,
+                                                        const uint32_t* __restrict__ item_start, uint32_t n_samples,
                                                         int32_t* __restrict__ cols, float* __restrict__ weights,
                                                         uint32_t* __restrict__ sample_of,
                                                         uint32_t* __restrict__ row_offsets,
                                                         const float* __restrict__ row_sums) {
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
   __shared__ uint32_t s_scan_tmp[4];
-  const uint32_t s = blockIdx.x;
+  // sample of this work item: last s with item_start[s] <= blockIdx.x
+  uint32_t lo_s = 0, hi_s = n_samples;
+  while (hi_s - lo_s > 1) {
+    const uint32_t mid = lo_s + (hi_s - lo_s) / 2;
+    if (item_start[mid] <= blockIdx.x) lo_s = mid; else hi_s = mid;
+  }
+  const uint32_t s = lo_s;
+  const uint32_t item = blockIdx.x - item_start[s];
   const int32_t* transits = tv.base + (size_t)s * tv.stride;
   uint32_t carry = 0;
   for (uint32_t chunk = 0; chunk < tv.count; chunk += 256) {
@@ -102,17 +117,23 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
   __syncthreads();
   const uint32_t base = offsets[s];
   const uint32_t size = s_start[tv.count];
-  if (row_offsets)
+  if (row_offsets && item == 0)
     for (uint32_t i = threadIdx.x; i < tv.count; i += 256) row_offsets[(size_t)s * tv.count + i] = s_start[i];
-  for (uint32_t e = threadIdx.x; e < size; e += 256) {
-    // transit whose range holds e: last i with s_start[i] <= e
-    uint32_t lo = 0, hi = tv.count;
-    while (hi - lo > 1) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      if (s_start[mid] <= e) lo = mid; else hi = mid;
+  const uint32_t first = item * kBuildItemEntries;
+  const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
+  uint32_t cur = 0;  // transit of the previous entry this lane copied: the next one is usually the same
+  for (uint32_t e = first + threadIdx.x; e < last; e += 256) {
+    if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
+      // transit whose range holds e: last i with s_start[i] <= e
+      uint32_t lo = 0, hi = tv.count;
+      while (hi - lo > 1) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        if (s_start[mid] <= e) lo = mid; else hi = mid;
+      }
+      cur = lo;
     }
-    const int32_t t = transits[lo];
-    const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[lo]);
+    const int32_t t = transits[cur];
+    const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur]);
     cols[base + e] = csr.edges[src];
     if (weights) {
       float w = csr.weights[src];
@@ -123,6 +144,17 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
       weights[base + e] = w;
     }
     if (sample_of) sample_of[base + e] = s;
+  }
+}
+
+// item_count[s] = work items of sample s (at least one, so that row offsets get written)
+__global__ void build_item_counts(const uint32_t* __restrict__ sizes, uint32_t n, uint32_t* __restrict__ item_count) {
+  const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s < n) {
+    const uint32_t items = (sizes[s] + kBuildItemEntries - 1) / kBuildItemEntries;
+    item_count[s] = items ? items : 1u;
+  } else if (s == n) {
+    item_count[s] = 0;
   }
 }
 
@@ -155,16 +187,31 @@ __global__ __launch_bounds__(kScanThreads) void count_pair_heads(const uint32_t*
   if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
-// Distinct (sample, vertex) pairs in order: the vertex id, degree^2, and one count per sample.
+// (weight / rowsum)^2 as a 2^53 fixed-point integer: sums of up to 1024 of them fit 64 bits
+// and, unlike float sums, do not depend on the order of the additions.
+__host__ __device__ __forceinline__ unsigned long long importance_term_fixed(float term) {
+  if (!(term > 0.0f)) return 0ull;
+  if (term >= 1.0f) return 1ull << 53;
+  return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
+}
+
+// Distinct (sample, vertex) pairs in order.  Every head writes its vertex id (and degree^2,
+// or the extent bookkeeping of the LADIES form); the first head of a sample writes the
+// sample's start in the distinct list.  terms (nullable, LADIES form): the fixed-point terms
+// of every run are summed into importance[run] - a lane adds up the stretch it owns and
+// flushes with one atomic per run it touches, so a vertex reached over very many
+// (duplicate) edges costs many lanes one atomic each instead of one lane a long loop.
 __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_t* __restrict__ sample_key,
                                                                    const uint32_t* __restrict__ vertex, size_t n,
                                                                    const uint32_t* __restrict__ tile_offsets,
                                                                    const EdgePos_t* __restrict__ row_ptr,
                                                                    int32_t* __restrict__ distinct_ids,
                                                                    uint64_t* __restrict__ degree_sq,
-                                                                   uint32_t* __restrict__ per_sample_count,
-                                                                   uint32_t* __restrict__ run_begin,
-                                                                   uint32_t* __restrict__ distinct_sample) {
+                                                                   uint32_t* __restrict__ distinct_start,
+                                                                   uint32_t* __restrict__ distinct_sample,
+                                                                   const uint32_t* __restrict__ sorted_pos,
+                                                                   const float* __restrict__ terms,
+                                                                   unsigned long long* __restrict__ importance) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
   bool head[kScanItems];
@@ -176,18 +223,40 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
   }
   uint32_t total;
   uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
+  unsigned long long partial = 0;  // terms of run r - 1 seen by this lane so far
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
+    if (base + i >= n) break;
     if (head[i]) {
+      if (terms && partial) atomicAdd(&importance[r - 1], partial);
+      partial = 0;
       const uint32_t v = vertex[base + i];
-      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+      const uint32_t s = sample_key[base + i];
       distinct_ids[r] = (int32_t)v;
-      if (degree_sq) degree_sq[r] = d * d;
-      if (run_begin) run_begin[r] = (uint32_t)(base + i);
-      if (distinct_sample) distinct_sample[r] = sample_key[base + i];
-      atomicAdd(&per_sample_count[sample_key[base + i]], 1u);
+      if (degree_sq) {
+        const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+        degree_sq[r] = d * d;
+      }
+      if (distinct_sample) distinct_sample[r] = s;
+      if (base + i == 0 || sample_key[base + i - 1] != s) distinct_start[s] = r;
       ++r;
     }
+    if (terms) partial += importance_term_fixed(terms[sorted_pos[base + i]]);
+  }
+  if (terms && partial) atomicAdd(&importance[r - 1], partial);
+}
+
+// distinct_start[s] was written for samples that have distinct vertices; the others take
+// the start of the next sample that has (the list holds nothing of theirs).  One lane: the
+// number of samples per chunk is small.
+__global__ void fill_empty_sample_starts(uint32_t* distinct_start, uint32_t n_samples, uint32_t n_distinct,
+                                         uint32_t unset) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  uint32_t next = n_distinct;
+  distinct_start[n_samples] = n_distinct;
+  for (uint32_t s = n_samples; s-- > 0;) {
+    if (distinct_start[s] == unset) distinct_start[s] = next;
+    else next = distinct_start[s];
   }
 }
 
@@ -227,21 +296,18 @@ __host__ __device__ __forceinline__ float det_log2(float x) {
   return (float)e + ln_m * 1.44269502f;
 }
 
-// One lane per distinct (sample, vertex): importance = its terms summed in concatenation
-// order; Efraimidis-Spirakis key log2(u) / importance with u from Philox at slot
-// sample * |V| + vertex; stored as sortable bits, inverted so that an ascending sort
-// yields descending keys.
-__global__ __launch_bounds__(256) void ladies_keys(const uint32_t* __restrict__ run_begin,
-                                                   const uint32_t* __restrict__ sorted_pos,
-                                                   const float* __restrict__ terms,
+// One lane per distinct (sample, vertex): Efraimidis-Spirakis key log2(u) / importance with u
+// from Philox at slot sample * |V| + vertex and importance the fixed-point sum of the
+// vertex's terms (the common 2^53 scale does not change the order of the keys); stored as
+// sortable bits, inverted so that an ascending sort yields descending keys.
+__global__ __launch_bounds__(256) void ladies_keys(const unsigned long long* __restrict__ importance_fixed,
                                                    const int32_t* __restrict__ distinct_ids,
                                                    const uint32_t* __restrict__ distinct_sample, uint32_t n_distinct,
                                                    uint64_t seed, uint64_t first_sample, uint32_t n_vertices,
                                                    uint32_t step, uint32_t* __restrict__ key_bits) {
   const uint32_t j = blockIdx.x * 256 + threadIdx.x;
   if (j >= n_distinct) return;
-  float importance = 0.0f;
-  for (uint32_t i = run_begin[j]; i < run_begin[j + 1]; ++i) importance = importance + terms[sorted_pos[i]];
+  const float importance = (float)importance_fixed[j];
   const uint64_t slot = (first_sample + distinct_sample[j]) * (uint64_t)n_vertices + (uint32_t)distinct_ids[j];
   const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
                                         (uint32_t)(seed >> 32));
@@ -437,10 +503,11 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_sizes_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMemset(d_sizes_, 0, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_offsets_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_item_count_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
+    ND_HIP_TRY(hipMalloc(&d_item_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_row_offsets_, sizeof(uint32_t) * (size_t)n_samples_ * widest));
     ND_HIP_TRY(hipMalloc(&d_small_scratch_, sizeof(uint32_t) * scan_scratch_elems((size_t)n_samples_ + 1)));
     if (App::kNeighborhoodForm != apps::kConcatenated) {
-      ND_HIP_TRY(hipMalloc(&d_distinct_count_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
       ND_HIP_TRY(hipMalloc(&d_distinct_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     }
     return 0;
@@ -551,8 +618,16 @@ class LayerEngine : public EngineBase {
     // offsets of the chunk's samples, relative to the chunk (element n = total)
     ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
     constexpr int form = App::kNeighborhoodForm;
-    collective_build<<<dim3(n), dim3(256), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, d_offsets_, d_nbr_cols_, d_nbr_weights_,
+    // work items of the build: long neighbourhoods are spread over several workgroups
+    uint64_t n_items = 0;
+    for (uint32_t s = s0; s < s1; ++s) {
+      const uint64_t items = ((uint64_t)h_sizes_[s] + kBuildItemEntries - 1) / kBuildItemEntries;
+      n_items += items ? items : 1;
+    }
+    build_item_counts<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_sizes_ + s0, n, d_item_count_);
+    ND_HIP_TRY(exclusive_scan_u32(d_item_count_, d_item_start_, (size_t)n + 1, d_small_scratch_, stream_));
+    collective_build<<<dim3((unsigned)n_items), dim3(256), 0, stream_>>>(
+        dgraph_.view, tv, invalid_, d_offsets_, d_item_start_, n, d_nbr_cols_, d_nbr_weights_,
         form != apps::kConcatenated ? d_sample_of_ : nullptr, d_row_offsets_ + (size_t)s0 * all.count,
         form == apps::kRankedByLadiesImportance ? d_row_sums_ : nullptr);
     ND_HIP_TRY(hipGetLastError());
@@ -615,7 +690,7 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
     }
     if (form == apps::kRankedByLadiesImportance) {
-      ND_HIP_TRY(hipMalloc(&d_run_begin_, sizeof(uint32_t) * (cap + 1)));
+      ND_HIP_TRY(hipMalloc(&d_importance_, sizeof(unsigned long long) * cap));
       ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
@@ -630,7 +705,8 @@ class LayerEngine : public EngineBase {
     constexpr int form = App::kNeighborhoodForm;
     int chunk_bits = 1;
     while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
-    fill_u32<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_count_, (size_t)n + 1, 0u);
+    constexpr uint32_t kUnset = 0xFFFFFFFFu;
+    fill_u32<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_start_, (size_t)n + 1, kUnset);
     uint32_t n_distinct = 0;
     uint32_t* sorted_pos = nullptr;
     if (total > 0) {
@@ -654,21 +730,24 @@ class LayerEngine : public EngineBase {
       count_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(k2, d_vertex_sorted_, total,
                                                                                   d_scratch_);
       scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
+      if (form == apps::kRankedByLadiesImportance) {
+        ND_HIP_TRY(hipMemsetAsync(d_importance_, 0, sizeof(unsigned long long) * (size_t)total, stream_));
+      }
       compact_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(
           k2, d_vertex_sorted_, total, d_scratch_, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
-          d_distinct_count_, d_run_begin_, d_distinct_sample_);
+          d_distinct_start_, d_distinct_sample_, sorted_pos,
+          form == apps::kRankedByLadiesImportance ? d_nbr_weights_ : nullptr, d_importance_);
       ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
       ND_HIP_TRY(hipStreamSynchronize(stream_));
       distinct_total_ += n_distinct;
     }
-    ND_HIP_TRY(exclusive_scan_u32(d_distinct_count_, d_distinct_start_, (size_t)n + 1, d_small_scratch_, stream_));
+    fill_empty_sample_starts<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_, n, n_distinct, kUnset);
     if (form == apps::kDistinctByDegreeSquared) {
       ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
     } else if (n_distinct > 0) {
-      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_run_begin_ + n_distinct, 1, total);
       ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
-          d_run_begin_, sorted_pos, d_nbr_weights_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_,
-          (uint64_t)s0, (uint32_t)invalid_, (uint32_t)step, d_key_bits_);
+          d_importance_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_, (uint64_t)s0, (uint32_t)invalid_,
+          (uint32_t)step, d_key_bits_);
       // order the distinct vertices of every sample by descending key: the list is in
       // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
       // ascending vertex id among equal keys
@@ -693,14 +772,15 @@ class LayerEngine : public EngineBase {
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
     release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
-    release(d_run_begin_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
+    release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
     capacity_ = 0;
   }
 
   void free_run_buffers() {
     release(d_initial_); release(d_samples_); release(d_samples_init_); release(d_final_);
     release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
-    release(d_distinct_count_); release(d_distinct_start_);
+    release(d_item_count_); release(d_item_start_);
+    release(d_distinct_start_);
     release_neighborhood_buffers();
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
@@ -734,7 +814,8 @@ class LayerEngine : public EngineBase {
   SampleType* d_samples_init_ = nullptr;
   VertexID_t* d_final_ = nullptr;
   uint32_t *d_sizes_ = nullptr, *d_offsets_ = nullptr, *d_row_offsets_ = nullptr, *d_small_scratch_ = nullptr;
-  uint32_t *d_distinct_count_ = nullptr, *d_distinct_start_ = nullptr;
+  uint32_t *d_item_count_ = nullptr, *d_item_start_ = nullptr;
+  uint32_t* d_distinct_start_ = nullptr;
   int32_t* d_nbr_cols_ = nullptr;
   float* d_nbr_weights_ = nullptr;
   uint32_t* d_sample_of_ = nullptr;
@@ -742,7 +823,8 @@ class LayerEngine : public EngineBase {
   uint32_t *d_key2_ = nullptr, *d_pos_ = nullptr, *d_vertex_sorted_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
   uint64_t *d_degree_sq_ = nullptr, *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
-  uint32_t *d_run_begin_ = nullptr, *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
+  unsigned long long* d_importance_ = nullptr;
+  uint32_t *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
   int32_t* d_ranked_ids_ = nullptr;
 };
 

@@ -716,6 +716,13 @@ static uint32_t descending_key_bits(float key) {
   return ~b;
 }
 
+/* (weight / rowsum)^2 as a 2^53 fixed-point integer (exact scaling, truncation) */
+static uint64_t term_fixed(float term) {
+  if (!(term > 0.0f)) return 0;
+  if (term >= 1.0f) return (uint64_t)1 << 53;
+  return (uint64_t)(term * 9007199254740992.0f);
+}
+
 typedef struct { int32_t vertex; int64_t pos; } occ_t;
 static int cmp_occ(const void* a, const void* b) {
   const occ_t* x = (const occ_t*)a; const occ_t* y = (const occ_t*)b;
@@ -775,8 +782,9 @@ int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, ui
       int64_t distinct = 0;
       for (int64_t i = 0; i < size;) {
         int64_t j = i;
-        float imp = 0.0f;
-        while (j < size && occ[j].vertex == occ[i].vertex) { imp = imp + term[occ[j].pos]; j++; }
+        uint64_t imp_fixed = 0;
+        while (j < size && occ[j].vertex == occ[i].vertex) { imp_fixed += term_fixed(term[occ[j].pos]); j++; }
+        const float imp = (float)imp_fixed;
         const int32_t v = occ[i].vertex;
         uint32_t ctr[4], key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)}, w[4];
         const uint64_t slot = (uint64_t)(first_sample + s) * (uint64_t)g->n_vertices + (uint64_t)v;

@@ -127,7 +127,8 @@ def test_ladies_importance_definition_on_a_tiny_graph(oracle):
     g = oracle.Graph.from_adjacency(adj, w)
     n = 5
     # importance: 2 -> (1/4)^2, 3 -> (3/4)^2 + (2/4)^2, 4 -> (2/4)^2
-    imp = {2: np.float32(0.0625), 3: np.float32(0.5625) + np.float32(0.25), 4: np.float32(0.25)}
+    # (as 2^53 fixed point; these terms are exact binary fractions)
+    imp = {2: np.float32(0.0625 * 2.0 ** 53), 3: np.float32((0.5625 + 0.25) * 2.0 ** 53), 4: np.float32(0.25 * 2.0 ** 53)}
     d = oracle.app_desc(oracle.LADIES_IMPORTANCE, 1, 2, initial_size=2)
     S = 20000
     final = oracle.sample_ladies_importance(g, d, SEED, np.tile([0, 1], S).astype(np.int32))
