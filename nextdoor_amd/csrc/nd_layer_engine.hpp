@@ -198,9 +198,7 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
 // Distinct (sample, vertex) pairs in order.  Every head writes its vertex id (and degree^2,
 // or the extent bookkeeping of the LADIES form); the first head of a sample writes the
 // sample's start in the distinct list.  terms (nullable, LADIES form): the fixed-point terms
-// of every run are summed into importance[run] - a lane adds up the stretch it owns and
-// flushes with one atomic per run it touches, so a vertex reached over very many
-// (duplicate) edges costs many lanes one atomic each instead of one lane a long loop.
+// of every run are summed into importance[run], which the caller has zeroed.
 __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_t* __restrict__ sample_key,
                                                                    const uint32_t* __restrict__ vertex, size_t n,
                                                                    const uint32_t* __restrict__ tile_offsets,
@@ -223,12 +221,22 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
   }
   uint32_t total;
   uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
-  unsigned long long partial = 0;  // terms of run r - 1 seen by this lane so far
+  // Terms: a lane sums the stretch it owns.  What precedes its first head belongs to the run
+  // that was open when the stretch began (first_partial); what follows its last head stays
+  // open (partial); runs that begin and end inside the stretch are flushed on the spot.
+  const uint32_t r_begin = r;
+  unsigned long long first_partial = 0, partial = 0;
+  bool seen_head = false;
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
     if (base + i >= n) break;
     if (head[i]) {
-      if (terms && partial) atomicAdd(&importance[r - 1], partial);
+      if (!seen_head) {
+        first_partial = partial;
+        seen_head = true;
+      } else if (partial) {
+        atomicAdd(&importance[r - 1], partial);
+      }
       partial = 0;
       const uint32_t v = vertex[base + i];
       const uint32_t s = sample_key[base + i];
@@ -243,7 +251,31 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
     }
     if (terms) partial += importance_term_fixed(terms[sorted_pos[base + i]]);
   }
-  if (terms && partial) atomicAdd(&importance[r - 1], partial);
+  if (!terms) return;
+  // Open partials are combined along the wave before they reach memory (a segmented scan in
+  // which a lane with a head starts a new segment): a vertex reached over very many
+  // (duplicate) edges then costs one atomic per wave instead of a long loop in one lane.
+  const int lane = threadIdx.x & (kWave - 1);
+  unsigned long long open = partial;
+  bool closed = seen_head;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t lo = __shfl_up((uint32_t)open, d, kWave);
+    const uint32_t hi = __shfl_up((uint32_t)(open >> 32), d, kWave);
+    const int up_closed = __shfl_up((int)closed, d, kWave);
+    if (lane >= d) {
+      if (!closed) open += ((unsigned long long)hi << 32) | lo;
+      closed = closed || up_closed;
+    }
+  }
+  const uint32_t in_lo = __shfl_up((uint32_t)open, 1, kWave);
+  const uint32_t in_hi = __shfl_up((uint32_t)(open >> 32), 1, kWave);
+  const unsigned long long carry_in = lane == 0 ? 0ull : ((unsigned long long)in_hi << 32) | in_lo;
+  if (seen_head) {
+    const unsigned long long before = first_partial + carry_in;
+    if (before) atomicAdd(&importance[r_begin - 1], before);
+  }
+  if (lane == kWave - 1 && open) atomicAdd(&importance[r - 1], open);
 }
 
 // distinct_start[s] was written for samples that have distinct vertices; the others take
