@@ -8,7 +8,7 @@
 //   freeDeviceData             src/nextdoor.cu:2088-2115   -> Engine::free_device
 //   samplingKernel / identityKernel / gridKernel  212-336 / 338-504 / 976-1204
 //                                                      -> step_flat_kernel / step_workgroup_kernel
-//   partitionTransitsInKernels 1520-1802               -> classify_runs
+//   partitionTransitsInKernels 1520-1802               -> mark_run_heads / classify_run_tails
 //
 // Differences that are deliberate:
 //  * The (sample -> transit) map stores only the transit; the map index IS the slot
