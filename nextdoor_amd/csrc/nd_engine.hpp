@@ -117,6 +117,23 @@ struct StepParams {
                                  // per sample at the end, this step's segment of the result
   void* samples;                 // SampleType[S] or nullptr
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
+  // Walks (one transit per sample, stepSize 1 everywhere): the step kernels also emit the
+  // next step's pairs in THIS step's pair order - coalesced, and without the pairs the
+  // inversion dropped - and a 4-byte SampleType travels with its pair instead of being
+  // gathered from samples[] by every next() (nullptr: not in use).
+  int state_travels;             // the state is read from pair_state (samples[] at step 0) and
+                                 // goes back to samples[] only when its walk ends
+  const uint32_t* pair_state;    // state of each pair entering the step; nullptr: samples[sample]
+  uint32_t* emit_keys;           // next transit of each pair; nullptr: nothing is emitted
+  uint32_t* emit_slots;          // its slot
+  uint32_t* emit_state;          // its state after next()
+};
+
+// A SampleType small enough to travel with its pair through the inversion.
+template <class SampleType>
+struct state_fits_pair {
+  static constexpr bool value = !std::is_empty<SampleType>::value && sizeof(SampleType) == sizeof(uint32_t) &&
+                                std::is_trivially_copyable<SampleType>::value;
 };
 
 constexpr int kStepThreads = 256;
@@ -135,17 +152,35 @@ constexpr uint32_t kWorkgroupWork = 256;
 // over several workgroups (the grid-wide case).
 constexpr uint32_t kChunkOutputs = 2048;
 
+// pair: index of the pair in the order the step kernels walk them (sorted by transit, or
+// the raw map at step 0).
 template <class SampleType, class App, class EdgeArray, class WeightArray>
-__device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit,
+__device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
                                                uint32_t pair_slot, uint32_t nbr, EdgePos_t n_edges, float max_weight,
                                                EdgeArray& edges, WeightArray& weights) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
   VertexID neighbor = P.invalid;
-  // next() only runs for a real transit that has edges (nextdoor.cu:250-262)
-  if (transit != P.invalid && n_edges != 0) {
-    curandState rng;
-    rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  const bool runs = transit != P.invalid && n_edges != 0;  // next() only runs for a real transit
+                                                           // that has edges (nextdoor.cu:250-262)
+  curandState rng;
+  if (runs) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  if (state_fits_pair<SampleType>::value && P.state_travels) {
+    // the state travels with the pair
+    SampleType state;
+    uint32_t bits = P.pair_state ? P.pair_state[pair] : ((const uint32_t*)P.samples)[sample];
+    __builtin_memcpy(&state, &bits, sizeof(uint32_t));
+    if (runs) {
+      const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
+          P.step, &csr, &transit, (VertexID)(P.first_sample + sample), &state, max_weight, edges, weights, n_edges,
+          (VertexID_t)nbr, &rng);
+      neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
+    }
+    __builtin_memcpy(&bits, &state, sizeof(uint32_t));
+    if (P.emit_state) P.emit_state[pair] = bits;
+    // a walk that ends here leaves the stream of pairs: its state goes home
+    if (P.is_last || neighbor == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
+  } else if (runs) {
     SampleType local_state;
     SampleType* state = std::is_empty<SampleType>::value ? &local_state : (SampleType*)P.samples + sample;
     const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
@@ -154,6 +189,10 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
     neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
   }
   P.step_out[out_slot] = neighbor;
+  if (P.emit_keys) {
+    P.emit_keys[pair] = (uint32_t)neighbor;
+    P.emit_slots[pair] = pair_slot;
+  }
 }
 
 constexpr uint32_t kXcds = 8;
@@ -200,13 +239,13 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
   if (app_uses_weights<App>::value) {
     PairedEdgeIds edges{P.paired_edges + begin};
     PairedEdgeWeights weights{P.paired_edges + begin};
-    produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, slot, nbr, n_edges, max_weight,
-                                                                      edges, weights);
+    produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, nbr, n_edges,
+                                                                      max_weight, edges, weights);
   } else {
     const CSR::Edge* edges = csr.edges + begin;
     const float* weights = csr.weights + begin;
-    produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, slot, nbr, n_edges, max_weight,
-                                                                   edges, weights);
+    produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, nbr, n_edges,
+                                                                   max_weight, edges, weights);
   }
 }
 
@@ -247,7 +286,7 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
       const uint32_t nbr = o - p * P.step_size;
       const uint32_t slot = P.pair_slots[first_pair + p];
       produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
-          P, csr, transit, slot, nbr, n_edges, max_weight, edges, lds_weights);
+          P, csr, transit, first_pair + p, slot, nbr, n_edges, max_weight, edges, lds_weights);
     }
   }
 }
@@ -530,10 +569,23 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * max_pairs_));
     const SortPlan plan = make_sort_plan(max_pairs_, max_bits_);
-    ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * plan.hist_elems));
+    ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(max_pairs_)));
     ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * plan.scratch_elems));
     ND_HIP_TRY(hipMalloc(&d_run_start_of_, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
-    ND_HIP_TRY(hipMalloc(&d_live_, sizeof(uint32_t)));
+    ND_HIP_TRY(hipMalloc(&d_live_, sizeof(uint32_t) * 2));
+    // walks: every step has one pair per sample and one output per pair
+    walk_mode_ = init_size_ == 1 && n_steps > 1;
+    for (int k = 0; k < n_steps; ++k) walk_mode_ = walk_mode_ && app.stepSize(k) == 1;
+    state_travels_ = walk_mode_ && state_fits_pair<SampleType>::value;
+    if (walk_mode_) {
+      ND_HIP_TRY(hipMalloc(&d_emit_keys_, sizeof(uint32_t) * max_pairs_));
+      ND_HIP_TRY(hipMalloc(&d_emit_slots_, sizeof(uint32_t) * max_pairs_));
+    }
+    if (state_travels_) {
+      ND_HIP_TRY(hipMalloc(&d_emit_state_, sizeof(uint32_t) * max_pairs_));
+      ND_HIP_TRY(hipMalloc(&d_aux_a_, sizeof(uint32_t) * max_pairs_));
+      ND_HIP_TRY(hipMalloc(&d_aux_b_, sizeof(uint32_t) * max_pairs_));
+    }
     ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta)));
     ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta)));
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
@@ -601,10 +653,15 @@ class Engine : public EngineBase {
       P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
       P.samples = d_samples_;
       P.paired_edges = dgraph_.paired;
+      const bool emits = walk_mode_ && step + 1 < n_steps;
+      P.state_travels = state_travels_;
+      P.pair_state = nullptr;
+      P.emit_keys = emits ? d_emit_keys_ : nullptr;
+      P.emit_slots = emits ? d_emit_slots_ : nullptr;
+      P.emit_state = emits && state_travels_ ? d_emit_state_ : nullptr;
+      uint32_t* live_now = d_live_ + (step & 1);  // pairs the inversion of this step keeps
       const uint64_t outputs = (uint64_t)n_pairs * m;
-      const uint32_t flat_blocks = (uint32_t)((outputs + kFlatThreads - 1) / kFlatThreads);
-      // whole groups of kXcds * kXcdRun workgroups, so that flat_block_index is a bijection
-      const unsigned flat_grid = (flat_blocks + kXcds * kXcdRun - 1) / (kXcds * kXcdRun) * (kXcds * kXcdRun);
+      const unsigned flat_grid = flat_grid_for(outputs);
 
       if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
@@ -616,18 +673,38 @@ class Engine : public EngineBase {
         tock(&times.flat_kernel);
         times.flat_launches++;
       } else {
-        // inversion: sort (transit, slot) by transit
+        // inversion: sort (transit, slot) by transit.  Walks sort the pairs the previous
+        // step emitted (only those still alive); other apps sort the previous step's
+        // output array, whose index is the slot.
         const SortPlan plan = make_sort_plan(n_pairs, max_bits_);
-        uint32_t *sorted_keys = nullptr, *sorted_slots = nullptr;
+        SortJob job;
+        if (walk_mode_) {
+          job.keys_in = d_emit_keys_;
+          job.vals_in = d_emit_slots_;
+          job.aux_in = state_travels_ ? d_emit_state_ : nullptr;
+          job.n_in_dev = step == 1 ? nullptr : d_live_ + ((step - 1) & 1);
+        } else {
+          job.keys_in = (const uint32_t*)transits;
+        }
+        job.keys_a = d_keys_a_;
+        job.vals_a = d_vals_a_;
+        job.aux_a = d_aux_a_;
+        job.keys_b = d_keys_b_;
+        job.vals_b = d_vals_b_;
+        job.aux_b = d_aux_b_;
+        job.hist = d_hist_;
+        job.scratch = d_scratch_;
+        job.drop_key = (uint32_t)invalid_;
+        job.kept_dev = live_now;
         tick();
-        ND_HIP_TRY(radix_sort_pairs(plan, (const uint32_t*)transits, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
-                                    d_vals_b_, d_hist_, d_scratch_, stream_, &sorted_keys, &sorted_slots,
-                                    (uint32_t)invalid_, d_live_));
+        ND_HIP_TRY(radix_sort(plan, job, stream_));
         tock(&times.inversion);
         times.sort_launches += plan.passes;
+        uint32_t* sorted_keys = job.keys_sorted;
         P.pair_keys = sorted_keys;
-        P.pair_slots = sorted_slots;
-        P.live_pairs = d_live_;
+        P.pair_slots = job.vals_sorted;
+        P.pair_state = state_travels_ ? job.aux_sorted : nullptr;
+        P.live_pairs = live_now;
         if (!balance) {
           tick();
           step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, nullptr);
@@ -636,9 +713,9 @@ class Engine : public EngineBase {
         } else {
           tick();
           const unsigned pair_blocks = (n_pairs + 255) / 256;
-          mark_run_heads<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(sorted_keys, d_live_, d_run_start_of_, d_meta_);
+          mark_run_heads<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(sorted_keys, live_now, d_run_start_of_, d_meta_);
           classify_run_tails<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
-              sorted_keys, d_live_, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+              sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
               d_skip_flag_);
           tock(&times.load_balancing);
           tick();
@@ -732,6 +809,13 @@ class Engine : public EngineBase {
   }
 
  private:
+  // workgroups of the flat kernel for this many outputs: whole groups of kXcds * kXcdRun, so
+  // that flat_block_index is a bijection
+  static unsigned flat_grid_for(uint64_t outputs) {
+    const uint64_t blocks = (outputs + kFlatThreads - 1) / kFlatThreads;
+    return (unsigned)((blocks + kXcds * kXcdRun - 1) / (kXcds * kXcdRun) * (kXcds * kXcdRun));
+  }
+
   void tick() {
     if (profiling) (void)hipEventRecord(ev_a_, stream_);
   }
@@ -769,6 +853,11 @@ class Engine : public EngineBase {
     release(d_scratch_);
     release(d_run_start_of_);
     release(d_live_);
+    release(d_emit_keys_);
+    release(d_emit_slots_);
+    release(d_emit_state_);
+    release(d_aux_a_);
+    release(d_aux_b_);
     release(d_meta_);
     release(d_chunks_);
     release(d_skip_flag_);
@@ -811,7 +900,10 @@ class Engine : public EngineBase {
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
   uint32_t* d_run_start_of_ = nullptr;  // per transit vertex: first position of its run in the sorted map
-  uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits)
+  uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
+  bool walk_mode_ = false, state_travels_ = false;
+  uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
+  uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;
   uint32_t* d_chunks_ = nullptr;
   uint8_t* d_skip_flag_ = nullptr;

@@ -710,7 +710,7 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_pos_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_vertex_sorted_, sizeof(uint32_t) * cap));
       const SortPlan plan = make_sort_plan(cap, 32);
-      ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * plan.hist_elems));
+      ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(cap)));
       size_t scratch = plan.scratch_elems;
       if (scan_scratch_elems(cap) > scratch) scratch = scan_scratch_elems(cap);
       ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
