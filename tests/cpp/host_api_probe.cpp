@@ -1,0 +1,35 @@
+// Compiles the C++ host API header against the library and exercises what runs without a
+// GPU: the app registry, graph ingest through loadGraph, and the error path of a sampler
+// whose app does not exist.  With "gpu" as the third argument it also runs the whole
+// nextdoor<>() sequence and checks the shape of the result.
+#include <string.h>
+
+#include <libNextDoor_amd.hpp>
+
+int main(int argc, char** argv) {
+  if (argc < 2) return 2;
+  const char* graph_file = argv[1];
+  const bool gpu = argc > 2 && strcmp(argv[2], "gpu") == 0;
+  if (nd_num_apps() < 5) return 3;
+  CSR* csr = loadGraph(graph_file, "edge-list", "text");
+  if (!csr) return 4;
+  printf("vertices %d edges %lld\n", nd_graph_num_vertices(csr), (long long)nd_graph_num_edges(csr));
+  {
+    NextDoorData bogus("NoSuchApp");
+    if (transferCSRToGPUs(bogus, csr)) return 5;  // unknown app: false, message, no abort
+    printf("error %s\n", nd_last_error());
+  }
+  if (loadGraph("/nonexistent/graph", "edge-list", "text") != nullptr) return 6;
+  nd_graph_free(csr);
+  if (!gpu) return 0;
+  int final_size = 0;
+  size_t n_values = 0;
+  const bool ok = nextdoor("UniformRandomWalk8", graph_file, "edge-list", "text", 2, true, false, "TransitParallel", true,
+                           [&](NextDoorData& data) {
+                             final_size = getFinalSampleSize(data);
+                             n_values = data.hFinalSamples.size();
+                             return final_size == 8 && n_values == data.initialContents.size() * 8;
+                           });
+  printf("final_size %d values %zu\n", final_size, n_values);
+  return ok ? 0 : 7;
+}
