@@ -112,9 +112,13 @@ struct StepParams {
   const uint32_t* live_pairs;    // device count of pairs in pair_keys (sorted map: pairs with a real transit); nullptr: n_pairs
   const uint32_t* pair_keys;     // transit of each pair (sorted, or the raw map at step 0)
   const uint32_t* pair_slots;    // slot of each pair; nullptr: slot == index
-  int32_t* step_out;             // outputs of this step, indexed by output slot; it is both
-                                 // the (sample -> transit) map of step k+1 and, regrouped
-                                 // per sample at the end, this step's segment of the result
+  int32_t* step_out;             // outputs of this step: output slot o of sample s sits at
+                                 // step_out[s * out_pitch + (o - s * T_k * m_k)].  Either an
+                                 // array of its own (out_pitch = T_k * m_k: indexed by o),
+                                 // regrouped per sample at the end, or the step's segment
+                                 // inside the rows of the result (out_pitch = F).  It is also
+                                 // the (sample -> transit) map of step k+1.
+  uint32_t out_pitch;
   void* samples;                 // SampleType[S] or nullptr
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
   // Walks (one transit per sample, stepSize 1 everywhere): the step kernels also emit the
@@ -188,7 +192,8 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
         (VertexID_t)nbr, &rng);
     neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
   }
-  P.step_out[out_slot] = neighbor;
+  const uint32_t per_sample = P.transits_per_sample * P.step_size;
+  P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
   if (P.emit_keys) {
     P.emit_keys[pair] = (uint32_t)neighbor;
     P.emit_slots[pair] = pair_slot;
@@ -322,40 +327,95 @@ __global__ __launch_bounds__(256) void mark_run_heads(const uint32_t* __restrict
   if (i == 0 || keys[i - 1] != k) start_of[k] = i;
 }
 
+constexpr uint32_t kDirectSegment = 16;  // ids: segments this long are written straight into the result rows
+// Consecutive pairs per lane of classify_run_tails: many for large maps (fewer atomics),
+// one for small ones (the launch is latency bound: 3.4 vs 1.8 ms over the 99 steps of 4.2 M walks).
+constexpr int kClassifyItemsLarge = 16;
+constexpr uint32_t kClassifyLargeFrom = 16u << 20;  // pairs
+
+// Is pair i the last of a run that the workgroup kernel should take?  Gives the run and the
+// number of work items it needs.
+__device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict__ keys, uint32_t i, uint32_t n,
+                                                      const uint32_t* __restrict__ start_of,
+                                                      const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
+                                                      uint32_t* transit_out, uint32_t* start_out, uint32_t* count_out,
+                                                      uint32_t* n_items_out) {
+  const uint32_t transit = keys[i];
+  if (i + 1 != n && keys[i + 1] == transit) return false;  // not the last pair of its run
+  const uint32_t start = start_of[transit];
+  const uint32_t count = i + 1 - start;
+  const uint64_t work = (uint64_t)count * step_size;
+  if (work < kWorkgroupWork) return false;
+  const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
+  if (degree == 0 || degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) return false;
+  uint32_t pairs_per_chunk = kChunkOutputs / step_size;
+  if (pairs_per_chunk == 0) pairs_per_chunk = 1;
+  *transit_out = transit;
+  *start_out = start;
+  *count_out = count;
+  *n_items_out = (count + pairs_per_chunk - 1) / pairs_per_chunk;
+  return true;
+}
+
+// Every lane looks at kClassifyItems consecutive pairs.  The work items of a workgroup's
+// runs are claimed with ONE atomic per workgroup or wavefront (atomics on a single counter are served
+// one after the other, ~10 ns each: one per run cost 3 ms on 1.5e5 qualifying runs); their
+// order in the list is irrelevant to the results.  The list is sized so that every claim
+// fits (see Engine::alloc); should one not fit, the transit is left to the flat kernel and
+// the entries that did fit are processed twice with identical results.
+template <int kClassifyItems>
 __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __restrict__ keys,
                                                           const uint32_t* __restrict__ n_dev,
                                                           const uint32_t* __restrict__ start_of, RunsMeta* meta,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                           uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
                                                           uint8_t* __restrict__ skip_flag) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  __shared__ uint32_t s_base;
   const uint32_t n = *n_dev;
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t transit = keys[i];
-  if (i + 1 != n && keys[i + 1] == transit) return;  // not the last pair of its run
-  const uint32_t start = start_of[transit];
-  const uint32_t count = i + 1 - start;
-  const uint64_t work = (uint64_t)count * step_size;
-  if (work < kWorkgroupWork) return;
-  const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
-  if (degree == 0 || degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) return;
+  const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
+  uint32_t transit, start, count, n_items;
+  uint32_t mine = 0;
+  for (int k = 0; k < kClassifyItems; ++k) {
+    const uint64_t i = first + k;
+    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, start_of, row_ptr, step_size, &transit, &start, &count,
+                                       &n_items))
+      mine += n_items;
+  }
+  uint32_t base;
+  if (kClassifyItems == 1) {
+    // small maps: one atomic per wavefront, no barrier
+    const uint32_t incl = wave_inclusive_scan(mine);
+    const uint32_t wave_total = __shfl(incl, kWave - 1, kWave);
+    if (wave_total == 0) return;  // the same for every lane of the wavefront
+    uint32_t wave_base = 0;
+    if ((threadIdx.x & (kWave - 1)) == kWave - 1) wave_base = atomicAdd(&meta->n_chunks, wave_total);
+    base = __shfl(wave_base, kWave - 1, kWave) + incl - mine;
+  } else {
+    uint32_t block_total;
+    base = block_exclusive_scan_256(mine, s_wave, &block_total);
+    if (block_total == 0) return;  // the same for every lane of the workgroup
+    if (threadIdx.x == 0) s_base = atomicAdd(&meta->n_chunks, block_total);
+    __syncthreads();
+    base += s_base;
+  }
+  if (mine == 0) return;
   uint32_t pairs_per_chunk = kChunkOutputs / step_size;
   if (pairs_per_chunk == 0) pairs_per_chunk = 1;
-  const uint32_t n_items = (count + pairs_per_chunk - 1) / pairs_per_chunk;
-  // Work items are claimed with one atomic; their order in the list is irrelevant to the
-  // results.  The list is sized so that every claim fits (see Engine::alloc); should one
-  // not fit, the transit is left to the flat kernel and the entries that did fit are
-  // processed twice with identical results.
-  const uint32_t base = atomicAdd(&meta->n_chunks, n_items);
-  const bool fits = base + n_items <= chunk_capacity;
-  for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
-    const uint32_t off = g * pairs_per_chunk;
-    chunks[2 * (base + g)] = start + off;
-    chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
-  }
-  if (fits) {
-    skip_flag[transit] = 1;
-    atomicAdd(&meta->n_big_pairs, count);
+  for (int k = 0; k < kClassifyItems; ++k) {
+    const uint64_t i = first + k;
+    // one pair per lane: the run found above is still in the registers
+    if (kClassifyItems > 1 && !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, start_of, row_ptr, step_size,
+                                                               &transit, &start, &count, &n_items)))
+      continue;
+    const bool fits = base + n_items <= chunk_capacity;
+    for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
+      const uint32_t off = g * pairs_per_chunk;
+      chunks[2 * (base + g)] = start + off;
+      chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+    }
+    if (fits) skip_flag[transit] = 1;
+    base += n_items;
   }
 }
 
@@ -563,7 +623,12 @@ class Engine : public EngineBase {
                            hipMemcpyHostToDevice));
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
-    ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
+    // Steps whose segment of a result row is at least a memory line long write straight
+    // into the rows; short segments (walks: one id per step) would touch a separate line of
+    // the result per output, so they go to one array per step and are regrouped at the end.
+    rows_direct_ = true;
+    for (int k = 0; k < n_steps; ++k) rows_direct_ = rows_direct_ && layout_.seg_len[k] >= kDirectSegment;
+    if (!rows_direct_) ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * max_pairs_));
@@ -628,11 +693,13 @@ class Engine : public EngineBase {
     // kernel: their outputs keep this fill
     {
       const size_t n_out = (size_t)n_samples_ * F;
-      fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(d_step_out_, n_out, invalid_);
+      fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(
+          rows_direct_ ? d_final_ : d_step_out_, n_out, invalid_);
     }
 
     uint32_t transits_per_sample = (uint32_t)init_size_;
     const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
+    KeyLayout transits_layout;             // and how it is laid out
     for (int step = 0; step < n_steps; ++step) {
       const uint32_t m = (uint32_t)app.stepSize(step);
       const uint32_t n_pairs = (uint32_t)((uint64_t)n_samples_ * transits_per_sample);
@@ -650,7 +717,13 @@ class Engine : public EngineBase {
       P.first_sample = 0;
       P.n_pairs = n_pairs;
       P.live_pairs = nullptr;
-      P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
+      if (rows_direct_) {
+        P.step_out = d_final_ + layout_.seg_base[step];
+        P.out_pitch = (uint32_t)F;
+      } else {
+        P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
+        P.out_pitch = layout_.seg_len[step];
+      }
       P.samples = d_samples_;
       P.paired_edges = dgraph_.paired;
       const bool emits = walk_mode_ && step + 1 < n_steps;
@@ -685,6 +758,7 @@ class Engine : public EngineBase {
           job.n_in_dev = step == 1 ? nullptr : d_live_ + ((step - 1) & 1);
         } else {
           job.keys_in = (const uint32_t*)transits;
+          job.keys_in_layout = transits_layout;
         }
         job.keys_a = d_keys_a_;
         job.vals_a = d_vals_a_;
@@ -714,9 +788,16 @@ class Engine : public EngineBase {
           tick();
           const unsigned pair_blocks = (n_pairs + 255) / 256;
           mark_run_heads<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(sorted_keys, live_now, d_run_start_of_, d_meta_);
-          classify_run_tails<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
-              sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
-              d_skip_flag_);
+          if (n_pairs >= kClassifyLargeFrom) {
+            const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
+            classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
+                sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                d_skip_flag_);
+          } else {
+            classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
+                sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                d_skip_flag_);
+          }
           tock(&times.load_balancing);
           tick();
           step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, d_skip_flag_);
@@ -732,12 +813,18 @@ class Engine : public EngineBase {
       }
       ND_HIP_TRY(hipGetLastError());
       transits = P.step_out;
+      if (rows_direct_) {
+        transits_layout.seg_len = layout_.seg_len[step];
+        transits_layout.pitch = (uint32_t)F;
+      }
       transits_per_sample *= m;
     }
 
     // regroup the per-step arrays into one row per sample
     tick();
-    if (rows_per_block_ > 0) {
+    if (rows_direct_) {
+      // the step kernels wrote the rows themselves
+    } else if (rows_per_block_ > 0) {
       const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
       assemble_final_rows<<<dim3(blocks), dim3(256), lds, stream_>>>(d_step_out_, d_final_, (uint32_t)n_samples_,
@@ -901,7 +988,7 @@ class Engine : public EngineBase {
   uint32_t* d_scratch_ = nullptr;
   uint32_t* d_run_start_of_ = nullptr;  // per transit vertex: first position of its run in the sorted map
   uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
-  bool walk_mode_ = false, state_travels_ = false;
+  bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false;
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;

@@ -44,13 +44,25 @@ __device__ __forceinline__ int tile_offset(int wave, int it, int lane) {
   return wave * (kWave * kSortItems) + it * kWave + lane;
 }
 
+// Where key i of the input sits: keys[i], or, when the keys are segments of rows of a wider
+// table (seg_len keys at the start of every row of `pitch` words), keys[(i / seg_len) * pitch
+// + i % seg_len].  Only the first pass of a sort reads such an input.
+struct KeyLayout {
+  uint32_t seg_len = 0;  // 0: contiguous
+  uint32_t pitch = 0;
+  __host__ __device__ size_t at(size_t i) const {
+    return seg_len ? (i / seg_len) * (size_t)pitch + i % seg_len : i;
+  }
+};
+
 // n_dev (nullable): element count kept in device memory; overrides n when given.
 // drop_key: keys equal to it are left out of the sort (kPadKey: nothing is left out).
 template <int kSortItems>
 __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* __restrict__ keys, size_t n,
                                                                 const uint32_t* __restrict__ n_dev, int shift,
                                                                 uint32_t mask, uint32_t drop_key,
-                                                                uint32_t* __restrict__ hist, uint32_t num_tiles) {
+                                                                uint32_t* __restrict__ hist, uint32_t num_tiles,
+                                                                KeyLayout layout) {
   constexpr int kSortTile = kSortThreads * kSortItems;
   __shared__ uint32_t s_hist[kRadix];
   s_hist[threadIdx.x] = 0;
@@ -61,7 +73,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* 
   for (int it = 0; it < kSortItems; ++it) {
     const size_t idx = tile_start + (size_t)it * kSortThreads + threadIdx.x;
     if (idx < n) {
-      const uint32_t k = keys[idx];
+      const uint32_t k = keys[layout.at(idx)];
       if (k != drop_key) atomicAdd(&s_hist[(k >> shift) & mask], 1u);
     }
   }
@@ -105,7 +117,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
                                                               uint32_t mask, int digit_bits, uint32_t drop_key,
                                                               const uint32_t* __restrict__ scanned_hist,
                                                               const uint32_t* __restrict__ row_totals,
-                                                              uint32_t num_tiles, uint32_t* __restrict__ kept_out) {
+                                                              uint32_t num_tiles, uint32_t* __restrict__ kept_out,
+                                                              KeyLayout layout) {
   constexpr int kSortTile = kSortThreads * kSortItems;
   __shared__ uint32_t s_keys[kSortTile];
   __shared__ uint32_t s_vals[kSortTile];
@@ -139,7 +152,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   for (int it = 0; it < kSortItems; ++it) {
     const uint32_t off = (uint32_t)tile_offset<kSortItems>(wave, it, lane);
     const bool inside = off < in_tile;
-    key[it] = inside ? keys_in[tile_start + off] : kPadKey;
+    key[it] = inside ? keys_in[layout.at(tile_start + off)] : kPadKey;
     live[it] = inside && key[it] != drop_key;
     if (kIotaValues) val[it] = (uint32_t)(tile_start + off);
     else val[it] = inside ? vals_in[tile_start + off] : 0u;
@@ -262,6 +275,7 @@ struct SortJob {
   uint32_t* hist = nullptr;
   uint32_t* scratch = nullptr;
   const uint32_t* n_in_dev = nullptr;
+  KeyLayout keys_in_layout;  // how keys_in is laid out (values are then the key's index i)
   uint32_t drop_key = kPadKey;
   uint32_t* kept_dev = nullptr;
   // results
@@ -272,23 +286,24 @@ struct SortJob {
 template <int kSortItems>
 inline void sort_pass(const SortPlan& plan, const SortJob& job, const uint32_t* src_k, const uint32_t* src_v,
                       const uint32_t* src_x, uint32_t* dst_k, uint32_t* dst_v, uint32_t* dst_x, const uint32_t* n_dev,
-                      int shift, uint32_t mask, int bits, uint32_t drop, uint32_t* kept_out, hipStream_t stream) {
+                      int shift, uint32_t mask, int bits, uint32_t drop, uint32_t* kept_out, KeyLayout layout,
+                      hipStream_t stream) {
   const dim3 grid(plan.num_tiles), block(kSortThreads);
   radix_histogram<kSortItems><<<grid, block, 0, stream>>>(src_k, plan.n, n_dev, shift, mask, drop, job.hist,
-                                                          plan.num_tiles);
+                                                          plan.num_tiles, layout);
   radix_row_scan<<<dim3(mask + 1), block, 0, stream>>>(job.hist, plan.num_tiles, job.scratch);
   if (src_v == nullptr)
     radix_scatter<kSortItems, true, false><<<grid, block, 0, stream>>>(src_k, nullptr, nullptr, dst_k, dst_v, nullptr,
                                                                        plan.n, n_dev, shift, mask, bits, drop, job.hist,
-                                                                       job.scratch, plan.num_tiles, kept_out);
+                                                                       job.scratch, plan.num_tiles, kept_out, layout);
   else if (src_x == nullptr)
     radix_scatter<kSortItems, false, false><<<grid, block, 0, stream>>>(src_k, src_v, nullptr, dst_k, dst_v, nullptr,
                                                                         plan.n, n_dev, shift, mask, bits, drop,
-                                                                        job.hist, job.scratch, plan.num_tiles, kept_out);
+                                                                        job.hist, job.scratch, plan.num_tiles, kept_out, layout);
   else
     radix_scatter<kSortItems, false, true><<<grid, block, 0, stream>>>(src_k, src_v, src_x, dst_k, dst_v, dst_x, plan.n,
                                                                        n_dev, shift, mask, bits, drop, job.hist,
-                                                                       job.scratch, plan.num_tiles, kept_out);
+                                                                       job.scratch, plan.num_tiles, kept_out, layout);
 }
 
 inline hipError_t radix_sort(const SortPlan& plan, SortJob& job, hipStream_t stream) {
@@ -314,12 +329,13 @@ inline hipError_t radix_sort(const SortPlan& plan, SortJob& job, hipStream_t str
     const uint32_t* n_dev = pass > 0 ? job.kept_dev : job.n_in_dev;
     const uint32_t drop = pass == 0 ? job.drop_key : kPadKey;
     uint32_t* kept_out = pass == 0 ? job.kept_dev : nullptr;
+    const KeyLayout layout = pass == 0 ? job.keys_in_layout : KeyLayout();
     if (plan.items == kSortItemsLarge)
       sort_pass<kSortItemsLarge>(plan, job, src_k, src_v, src_x, dst_k, dst_v, dst_x, n_dev, shift, mask, bits, drop,
-                                 kept_out, stream);
+                                 kept_out, layout, stream);
     else
       sort_pass<kSortItemsSmall>(plan, job, src_k, src_v, src_x, dst_k, dst_v, dst_x, n_dev, shift, mask, bits, drop,
-                                 kept_out, stream);
+                                 kept_out, layout, stream);
     job.keys_sorted = dst_k;
     job.vals_sorted = dst_v;
     job.aux_sorted = dst_x;
