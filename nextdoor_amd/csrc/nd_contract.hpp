@@ -163,11 +163,16 @@ namespace nd {
 // the rest from HBM.  One of the two EdgeArray / WeightArray types an App::next is
 // instantiated with (the other is a plain pointer); only operator[] is required
 // (the reference's CachedArray, src/nextdoor.cu:76-124, plays this role).
+// The LDS half is held as a pointer in the LDS address space, so reads of it are plain LDS
+// loads and no generic-pointer test is generated.
 template <typename T>
 struct LdsBackedArray {
-  const T* lds;
+  typedef const __attribute__((address_space(3))) T* LdsPointer;
+  LdsPointer lds;
   const T* global;
   EdgePos_t cached;
+  __device__ __forceinline__ LdsBackedArray(const T* lds_array, const T* global_array, EdgePos_t n_cached)
+      : lds((LdsPointer)lds_array), global(global_array), cached(n_cached) {}
   __device__ __forceinline__ T operator[](EdgePos_t i) const { return i < cached ? lds[i] : global[i]; }
 };
 

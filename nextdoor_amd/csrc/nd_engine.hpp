@@ -100,6 +100,7 @@ struct StepParams {
   CSRPartition csr;
   int step;
   uint32_t step_size;            // m_k
+  uint32_t lanes_shift;          // flat kernel: 2^lanes_shift lanes share the outputs of a pair
   uint32_t transits_per_sample;  // T_k
   uint32_t seg_base;             // offset of this step's segment inside a final sample
   uint32_t final_size;           // F
@@ -144,6 +145,9 @@ constexpr int kStepThreads = 256;
 // Workgroup size of the flat kernel: one wavefront.  A workgroup keeps its slot until its
 // slowest wave is done and rejection loops make wave run times very uneven, so single-wave
 // workgroups keep more waves in flight (256 -> 64 threads: 34.6 -> 32.8 ms per pass).
+#ifndef ND_CHUNK_OUTPUTS
+#define ND_CHUNK_OUTPUTS 2048
+#endif
 #ifndef ND_FLAT_THREADS
 #define ND_FLAT_THREADS 64
 #endif
@@ -154,7 +158,7 @@ constexpr int kCacheEdges = 8192;
 constexpr uint32_t kWorkgroupWork = 256;
 // Outputs one work item of the workgroup kernel covers at most; larger runs are split
 // over several workgroups (the grid-wide case).
-constexpr uint32_t kChunkOutputs = 2048;
+constexpr uint32_t kChunkOutputs = ND_CHUNK_OUTPUTS;
 
 // pair: index of the pair in the order the step kernels walk them (sorted by transit, or
 // the raw map at step 0).
@@ -200,6 +204,9 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
   }
 }
 
+// Lanes the flat kernel wants before it gives a lane all the outputs of a pair.
+constexpr uint64_t kFlatLanesWanted = 1ull << 20;
+
 constexpr uint32_t kXcds = 8;
 // Consecutive workgroups (in sorted-pair order) one XCD handles before the next XCD takes over.
 #ifndef ND_XCD_RUN
@@ -218,17 +225,27 @@ __device__ __forceinline__ uint32_t flat_block_index() {
   return (turn / kXcdRun) * (kXcds * kXcdRun) + xcd * kXcdRun + turn % kXcdRun;
 }
 
-// One lane per output: lane i draws neighbour (i % m) for pair (i / m).  With the map
-// sorted by transit, neighbouring lanes share row extents and adjacency lines.
+// 2^lanes_shift lanes per pair: lane i serves pair i >> lanes_shift and draws the
+// neighbours sub, sub + L, ... (sub = i mod L, L = 2^lanes_shift) of it.  One lane per pair
+// (L = 1) when there are enough pairs to fill the machine: the pair, its row extent and the
+// marker are then fetched once for all stepSize draws, whose gathers are independent and
+// overlap; several lanes per pair when pairs are few.  With the map sorted by transit,
+// neighbouring lanes share row extents and adjacency lines.
 // skip_flag (nullable): per-vertex marker of transits the workgroup kernel handles.
-template <class SampleType, class App>
+// kSingleOutput: stepSize is 1 (walks); the loop over neighbours is compiled away.
+template <class SampleType, class App, bool kSingleOutput>
 __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
-  const uint64_t total = (uint64_t)(P.live_pairs ? *P.live_pairs : P.n_pairs) * P.step_size;
+  if (kSingleOutput) {
+    P.lanes_shift = 0;
+    P.step_size = 1;
+  }
+  const uint64_t total = (uint64_t)(P.live_pairs ? *P.live_pairs : P.n_pairs) << P.lanes_shift;
   const uint64_t i = (uint64_t)flat_block_index() * kFlatThreads + threadIdx.x;
   if (i >= total) return;
   CSRPartition csr = P.csr;
-  const uint32_t pair = P.step_size == 1 ? (uint32_t)i : (uint32_t)(i / P.step_size);
-  const uint32_t nbr = (uint32_t)(i - (uint64_t)pair * P.step_size);
+  const uint32_t pair = (uint32_t)(i >> P.lanes_shift);
+  const uint32_t first_nbr = (uint32_t)i & ((1u << P.lanes_shift) - 1u);
+  const uint32_t nbr_stride = 1u << P.lanes_shift;
   const VertexID transit = (VertexID)P.pair_keys[pair];
   const uint32_t slot = P.pair_slots ? P.pair_slots[pair] : pair;
   EdgePos_t n_edges = 0, begin = 0;
@@ -244,13 +261,15 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
   if (app_uses_weights<App>::value) {
     PairedEdgeIds edges{P.paired_edges + begin};
     PairedEdgeWeights weights{P.paired_edges + begin};
-    produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, nbr, n_edges,
-                                                                      max_weight, edges, weights);
+    for (uint32_t nbr = first_nbr; nbr < P.step_size; nbr += nbr_stride)
+      produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, nbr, n_edges,
+                                                                        max_weight, edges, weights);
   } else {
     const CSR::Edge* edges = csr.edges + begin;
     const float* weights = csr.weights + begin;
-    produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, nbr, n_edges,
-                                                                   max_weight, edges, weights);
+    for (uint32_t nbr = first_nbr; nbr < P.step_size; nbr += nbr_stride)
+      produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, nbr, n_edges,
+                                                                     max_weight, edges, weights);
   }
 }
 
@@ -733,8 +752,11 @@ class Engine : public EngineBase {
       P.emit_slots = emits ? d_emit_slots_ : nullptr;
       P.emit_state = emits && state_travels_ ? d_emit_state_ : nullptr;
       uint32_t* live_now = d_live_ + (step & 1);  // pairs the inversion of this step keeps
-      const uint64_t outputs = (uint64_t)n_pairs * m;
-      const unsigned flat_grid = flat_grid_for(outputs);
+      // lanes of the flat kernel per pair: one when the pairs alone fill the machine, else
+      // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
+      P.lanes_shift = 0;
+      while ((1u << P.lanes_shift) < m && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted) P.lanes_shift++;
+      const unsigned flat_grid = flat_grid_for((uint64_t)n_pairs << P.lanes_shift);
 
       if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
@@ -742,7 +764,7 @@ class Engine : public EngineBase {
         P.pair_keys = (const uint32_t*)transits;
         P.pair_slots = nullptr;
         tick();
-        step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, nullptr);
+        launch_flat(P, flat_grid, nullptr);
         tock(&times.flat_kernel);
         times.flat_launches++;
       } else {
@@ -781,7 +803,7 @@ class Engine : public EngineBase {
         P.live_pairs = live_now;
         if (!balance) {
           tick();
-          step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, nullptr);
+          launch_flat(P, flat_grid, nullptr);
           tock(&times.flat_kernel);
           times.flat_launches++;
         } else {
@@ -800,7 +822,7 @@ class Engine : public EngineBase {
           }
           tock(&times.load_balancing);
           tick();
-          step_flat_kernel<SampleType, App><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, d_skip_flag_);
+          launch_flat(P, flat_grid, d_skip_flag_);
           tock(&times.flat_kernel);
           times.flat_launches++;
           tick();
@@ -896,6 +918,13 @@ class Engine : public EngineBase {
   }
 
  private:
+  void launch_flat(const StepParams& P, unsigned flat_grid, const uint8_t* skip_flag) {
+    if (P.step_size == 1)
+      step_flat_kernel<SampleType, App, true><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
+    else
+      step_flat_kernel<SampleType, App, false><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
+  }
+
   // workgroups of the flat kernel for this many outputs: whole groups of kXcds * kXcdRun, so
   // that flat_block_index is a bijection
   static unsigned flat_grid_for(uint64_t outputs) {
