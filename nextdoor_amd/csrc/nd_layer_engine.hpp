@@ -17,13 +17,16 @@
 //    nullptr, nextdoor.cu:1441-1446).  Here offsets are an exclusive scan over samples
 //    (deterministic), the buffers are grown once and reused, and next() receives the
 //    neighbourhood in the form the app declares (nd::apps::NeighborhoodForm).
-//  * For kDistinctByDegreeSquared the concatenation is sorted by (sample, vertex) with two
-//    stable radix sorts, run heads give the distinct vertices, and a 64-bit inclusive scan
-//    of degree^2 gives the running sums the app inverts.
+//  * For kDistinctByDegreeSquared the concatenation is never stored: every entry sets a bit
+//    in a per-sample bitmap over the vertices, the set bits in ascending order are the
+//    distinct vertices, and a 64-bit inclusive scan of degree^2 gives the running sums the
+//    app inverts.
 //  * For kRankedByLadiesImportance each entry of the concatenation carries
 //    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed as 2^53
 //    fixed-point integers, Efraimidis-Spirakis keys are computed per distinct vertex
 //    and two more stable sorts order the distinct vertices of every sample by descending key.
+//    (The concatenation is sorted by (sample, vertex) with two stable radix sorts; run heads
+//    give the distinct vertices.)
 //  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
 //    of entries, so a layer whose frontier sits on hubs cannot outgrow memory.
 //  * Random numbers: Philox keyed by the output slot s * stepSize(k) + nbr and the layer.
@@ -147,6 +150,116 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
   }
 }
 
+// ---- distinct vertices of a collective neighbourhood through a bitmap ----
+//
+// One bitmap of |V| bits per sample of the chunk (words_per_sample words, a multiple of the
+// tile below).  collective_mark walks the neighbourhood exactly as collective_build does,
+// but instead of copying an entry it sets the entry's bit; nothing of the concatenation is
+// stored.  A neighbourhood that sits on hubs repeats its vertices many times over (3.8e10
+// entries hold 2.0e9 distinct pairs at FastGCN's full size), so the bit is tested with a
+// plain load first and the atomic is issued only when the bit reads clear.  A stale read
+// costs one redundant atomic, never a wrong bit.
+constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words
+
+__global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, TransitView tv, int32_t invalid,
+                                                       const uint32_t* __restrict__ item_start, uint32_t n_samples,
+                                                       uint32_t* __restrict__ bitmap, uint32_t words_per_sample) {
+  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
+  __shared__ uint32_t s_scan_tmp[4];
+  uint32_t lo_s = 0, hi_s = n_samples;
+  while (hi_s - lo_s > 1) {
+    const uint32_t mid = lo_s + (hi_s - lo_s) / 2;
+    if (item_start[mid] <= blockIdx.x) lo_s = mid; else hi_s = mid;
+  }
+  const uint32_t s = lo_s;
+  const uint32_t item = blockIdx.x - item_start[s];
+  const int32_t* transits = tv.base + (size_t)s * tv.stride;
+  uint32_t carry = 0;
+  for (uint32_t chunk = 0; chunk < tv.count; chunk += 256) {
+    const uint32_t i = chunk + threadIdx.x;
+    uint32_t deg = 0;
+    if (i < tv.count) {
+      const int32_t t = transits[i];
+      if (t != invalid && t != -1) deg = (uint32_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
+    }
+    uint32_t total;
+    const uint32_t excl = block_exclusive_scan_256(deg, s_scan_tmp, &total);
+    if (i < tv.count) s_start[i] = carry + excl;
+    carry += total;
+  }
+  if (threadIdx.x == 0) s_start[tv.count] = carry;
+  __syncthreads();
+  const uint32_t size = s_start[tv.count];
+  uint32_t* bits = bitmap + (size_t)s * words_per_sample;
+  const uint32_t first = item * kBuildItemEntries;
+  const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
+  uint32_t cur = 0;
+  for (uint32_t e = first + threadIdx.x; e < last; e += 256) {
+    if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
+      uint32_t lo = 0, hi = tv.count;
+      while (hi - lo > 1) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        if (s_start[mid] <= e) lo = mid; else hi = mid;
+      }
+      cur = lo;
+    }
+    const int32_t t = transits[cur];
+    const uint32_t v = (uint32_t)csr.edges[csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur])];
+    const uint32_t bit = 1u << (v & 31u);
+    uint32_t* word = bits + (v >> 5);
+    if ((*word & bit) == 0) atomicOr(word, bit);
+  }
+}
+
+// tile_counts[s * tiles_per_sample + t] = bits set in tile t of sample s's bitmap
+__global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __restrict__ bitmap,
+                                                          uint32_t* __restrict__ tile_counts) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const uint4* words = (const uint4*)(bitmap + (size_t)blockIdx.x * kBitmapTileWords) + threadIdx.x * 2;
+  const uint4 a = words[0], b = words[1];
+  const uint32_t mine = __popc(a.x) + __popc(a.y) + __popc(a.z) + __popc(a.w) + __popc(b.x) + __popc(b.y) +
+                        __popc(b.z) + __popc(b.w);
+  uint32_t total;
+  block_exclusive_scan_256(mine, s_wave, &total);
+  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+}
+
+// The set bits of every sample's bitmap, in ascending order, become the sample's distinct
+// vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
+// tile of a sample is where the sample's list starts).
+__global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
+                                                      const uint32_t* __restrict__ tile_offsets,
+                                                      uint32_t tiles_per_sample, const EdgePos_t* __restrict__ row_ptr,
+                                                      int32_t* __restrict__ distinct_ids,
+                                                      uint64_t* __restrict__ degree_sq,
+                                                      uint32_t* __restrict__ distinct_start) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const uint32_t sample = blockIdx.x / tiles_per_sample;
+  const uint32_t tile = blockIdx.x - sample * tiles_per_sample;
+  const uint4* words = (const uint4*)(bitmap + (size_t)blockIdx.x * kBitmapTileWords) + threadIdx.x * 2;
+  const uint4 a = words[0], b = words[1];
+  const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  uint32_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) mine += __popc(w[k]);
+  uint32_t total;
+  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
+  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = tile_offsets[blockIdx.x];
+  const uint32_t first_vertex = (tile * kBitmapTileWords + threadIdx.x * 8u) * 32u;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    uint32_t bits = w[k];
+    while (bits) {
+      const uint32_t v = first_vertex + k * 32u + (uint32_t)__ffs((int)bits) - 1u;
+      bits &= bits - 1u;
+      distinct_ids[r] = (int32_t)v;
+      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+      degree_sq[r] = d * d;
+      ++r;
+    }
+  }
+}
+
 // item_count[s] = work items of sample s (at least one, so that row offsets get written)
 __global__ void build_item_counts(const uint32_t* __restrict__ sizes, uint32_t n, uint32_t* __restrict__ item_count) {
   const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
@@ -195,16 +308,14 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
   return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
 }
 
-// Distinct (sample, vertex) pairs in order.  Every head writes its vertex id (and degree^2,
-// or the extent bookkeeping of the LADIES form); the first head of a sample writes the
-// sample's start in the distinct list.  terms (nullable, LADIES form): the fixed-point terms
-// of every run are summed into importance[run], which the caller has zeroed.
+// Distinct (sample, vertex) pairs in order (LADIES form).  Every head writes its vertex id
+// and sample; the first head of a sample writes the sample's start in the distinct list.
+// terms (nullable): the fixed-point terms of every run are summed into importance[run],
+// which the caller has zeroed.
 __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_t* __restrict__ sample_key,
                                                                    const uint32_t* __restrict__ vertex, size_t n,
                                                                    const uint32_t* __restrict__ tile_offsets,
-                                                                   const EdgePos_t* __restrict__ row_ptr,
                                                                    int32_t* __restrict__ distinct_ids,
-                                                                   uint64_t* __restrict__ degree_sq,
                                                                    uint32_t* __restrict__ distinct_start,
                                                                    uint32_t* __restrict__ distinct_sample,
                                                                    const uint32_t* __restrict__ sorted_pos,
@@ -241,10 +352,6 @@ __global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_
       const uint32_t v = vertex[base + i];
       const uint32_t s = sample_key[base + i];
       distinct_ids[r] = (int32_t)v;
-      if (degree_sq) {
-        const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-        degree_sq[r] = d * d;
-      }
       if (distinct_sample) distinct_sample[r] = s;
       if (base + i == 0 || sample_key[base + i - 1] != s) distinct_start[s] = r;
       ++r;
@@ -431,6 +538,10 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
 // Entries of concatenated neighbourhood one chunk of samples may hold (about 70 bytes of
 // device memory per entry across all work arrays).
 constexpr uint64_t kLayerChunkEntries = 96ull << 20;
+// Bitmap form: nothing is stored per entry, so a chunk is bounded by the memory of its
+// bitmaps and by the number of marking work items (entries / kBuildItemEntries) of one launch.
+constexpr uint64_t kBitmapBudgetBytes = 4ull << 30;
+constexpr uint64_t kBitmapChunkEntries = 1ull << 40;
 
 template <class SampleType, class App>
 class LayerEngine : public EngineBase {
@@ -511,11 +622,15 @@ class LayerEngine : public EngineBase {
     hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
     h_sizes_.resize((size_t)n_samples_);
     chunk_entries_ = kLayerChunkEntries;
+    bitmap_chunk_entries_ = kBitmapChunkEntries;
     progress_ = getenv("ND_PROGRESS") != nullptr;  // long layers report on stderr every 16 chunks
     if (const char* env = getenv("ND_LAYER_CHUNK_ENTRIES")) {  // smaller chunks, e.g. to exercise chunking
       const long long v = atoll(env);
-      if (v > 0) chunk_entries_ = (uint64_t)v;
+      if (v > 0) chunk_entries_ = bitmap_chunk_entries_ = (uint64_t)v;
     }
+    bitmap_words_ = (((uint32_t)invalid_ + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
+    const uint64_t fit = kBitmapBudgetBytes / ((uint64_t)bitmap_words_ * sizeof(uint32_t));
+    bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
@@ -576,13 +691,21 @@ class LayerEngine : public EngineBase {
       collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, stream_>>>(dgraph_.view, all, S, invalid_, d_sizes_);
       ND_HIP_TRY(hipMemcpyAsync(h_sizes_.data(), d_sizes_, sizeof(uint32_t) * S, hipMemcpyDeviceToHost, stream_));
       ND_HIP_TRY(hipStreamSynchronize(stream_));
+      // chunk limits: entries of concatenation the work arrays hold, or (bitmap form) bitmaps
+      // that fit the budget and a grid of marking work items that fits 31 bits
+      constexpr bool by_bitmap = App::kNeighborhoodForm == apps::kDistinctByDegreeSquared;
+      const uint64_t entry_budget = by_bitmap ? bitmap_chunk_entries_ : chunk_entries_;
+      const uint32_t sample_budget = by_bitmap ? bitmap_chunk_samples_ : S;
       uint32_t s0 = 0;
       while (s0 < S) {
         uint64_t total = h_sizes_[s0];
         uint32_t s1 = s0 + 1;
-        while (s1 < S && total + h_sizes_[s1] <= chunk_entries_) total += h_sizes_[s1++];
-        if (total >= (1ull << 31)) { last_error = "collective neighbourhood of one sample exceeds 2^31 entries"; return -2; }
-        if (run_chunk(step, all, s0, s1, (uint32_t)total) != 0) return -1;
+        while (s1 < S && s1 - s0 < sample_budget && total + h_sizes_[s1] <= entry_budget) total += h_sizes_[s1++];
+        if (total >= (1ull << 31) && !by_bitmap) {
+          last_error = "collective neighbourhood of one sample exceeds 2^31 entries";
+          return -2;
+        }
+        if (run_chunk(step, all, s0, s1, total) != 0) return -1;
         neighborhood_total_ += total;
         chunks_run_++;
         if (progress_ && chunks_run_ % 16 == 0) {
@@ -640,29 +763,34 @@ class LayerEngine : public EngineBase {
 
   // One chunk of samples [s0, s1) of one layer: concatenate, post-process in the form the
   // app asks for, run next() for every (sample, nbr).
-  int run_chunk(int step, const TransitView& all, uint32_t s0, uint32_t s1, uint32_t total) {
+  int run_chunk(int step, const TransitView& all, uint32_t s0, uint32_t s1, uint64_t total) {
     App app;
     const uint32_t n = s1 - s0;
     const size_t F = (size_t)final_sample_size();
-    if (ensure_neighborhood_capacity(total) != 0) return -1;
+    constexpr int form = App::kNeighborhoodForm;
     TransitView tv = all;
     tv.base = all.base + (size_t)s0 * all.stride;
-    // offsets of the chunk's samples, relative to the chunk (element n = total)
-    ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
-    constexpr int form = App::kNeighborhoodForm;
     // work items of the build: long neighbourhoods are spread over several workgroups
     uint64_t n_items = 0;
     for (uint32_t s = s0; s < s1; ++s) {
       const uint64_t items = ((uint64_t)h_sizes_[s] + kBuildItemEntries - 1) / kBuildItemEntries;
       n_items += items ? items : 1;
     }
+    if (n_items >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more work items"; return -2; }
     build_item_counts<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_sizes_ + s0, n, d_item_count_);
     ND_HIP_TRY(exclusive_scan_u32(d_item_count_, d_item_start_, (size_t)n + 1, d_small_scratch_, stream_));
-    collective_build<<<dim3((unsigned)n_items), dim3(256), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, d_offsets_, d_item_start_, n, d_nbr_cols_, d_nbr_weights_,
-        form != apps::kConcatenated ? d_sample_of_ : nullptr, d_row_offsets_ + (size_t)s0 * all.count,
-        form == apps::kRankedByLadiesImportance ? d_row_sums_ : nullptr);
-    ND_HIP_TRY(hipGetLastError());
+    if (form == apps::kDistinctByDegreeSquared) {
+      if (build_distinct_by_bitmap(tv, n, (unsigned)n_items) != 0) return -1;
+    } else {
+      if (ensure_neighborhood_capacity((uint32_t)total) != 0) return -1;
+      // offsets of the chunk's samples, relative to the chunk (element n = total)
+      ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
+      collective_build<<<dim3((unsigned)n_items), dim3(256), 0, stream_>>>(
+          dgraph_.view, tv, invalid_, d_offsets_, d_item_start_, n, d_nbr_cols_, d_nbr_weights_,
+          form != apps::kConcatenated ? d_sample_of_ : nullptr, d_row_offsets_ + (size_t)s0 * all.count,
+          form == apps::kRankedByLadiesImportance ? d_row_sums_ : nullptr);
+      ND_HIP_TRY(hipGetLastError());
+    }
 
     LayerParams P{};
     P.csr = dgraph_.view;
@@ -682,7 +810,7 @@ class LayerEngine : public EngineBase {
     P.nbr_cols = d_nbr_cols_;
     P.nbr_weights = d_nbr_weights_;
     if (form != apps::kConcatenated) {
-      if (build_distinct(step, s0, n, total) != 0) return -1;
+      if (form == apps::kRankedByLadiesImportance && build_distinct(step, s0, n, (uint32_t)total) != 0) return -1;
       P.distinct_start = d_distinct_start_;
       P.distinct_ids = form == apps::kRankedByLadiesImportance ? d_ranked_ids_ : d_distinct_ids_;
       P.running_sums = d_running_sums_;
@@ -691,6 +819,45 @@ class LayerEngine : public EngineBase {
     layer_execute_kernel<SampleType, App><<<dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, stream_>>>(P);
     ND_HIP_TRY(hipGetLastError());
     return 0;
+  }
+
+  // Distinct vertices of every sample of the chunk, ascending, with running sums of
+  // degree^2: mark bits, count them per tile, scan, write the ids out.
+  int build_distinct_by_bitmap(const TransitView& tv, uint32_t n, unsigned n_items) {
+    const uint32_t tiles_per_sample = bitmap_words_ / kBitmapTileWords;
+    const size_t n_tiles = (size_t)n * tiles_per_sample;
+    if (n > bitmap_samples_) {
+      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
+      ND_HIP_TRY(hipMalloc(&d_bitmap_, sizeof(uint32_t) * (size_t)n * bitmap_words_));
+      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
+      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
+      bitmap_samples_ = n;
+    }
+    ND_HIP_TRY(hipMemsetAsync(d_bitmap_, 0, sizeof(uint32_t) * (size_t)n * bitmap_words_, stream_));
+    collective_mark<<<dim3(n_items), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_item_start_, n, d_bitmap_,
+                                                              bitmap_words_);
+    bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
+    ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
+    uint32_t n_distinct = 0;
+    ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_tile_scratch_ + scan_num_tiles(n_tiles), sizeof(uint32_t),
+                              hipMemcpyDeviceToHost, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    distinct_total_ += n_distinct;
+    if (n_distinct > distinct_capacity_) {
+      const size_t cap = (size_t)n_distinct + n_distinct / 8 + 1024;
+      release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+      ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
+      distinct_capacity_ = cap;
+    }
+    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_, tiles_per_sample,
+                                                                      dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
+                                                                      d_distinct_start_);
+    fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
+    ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
+    return hipGetLastError() == hipSuccess ? 0 : -1;
   }
 
   int ensure_neighborhood_capacity(uint32_t total) {
@@ -716,11 +883,6 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
       ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
     }
-    if (form == apps::kDistinctByDegreeSquared) {
-      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
-    }
     if (form == apps::kRankedByLadiesImportance) {
       ND_HIP_TRY(hipMalloc(&d_importance_, sizeof(unsigned long long) * cap));
       ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
@@ -731,8 +893,8 @@ class LayerEngine : public EngineBase {
     return 0;
   }
 
-  // Distinct (sample, vertex) pairs of the chunk's concatenation and their per-sample
-  // extents; then running sums of degree^2, or the ranking by Efraimidis-Spirakis key.
+  // LADIES form: distinct (sample, vertex) pairs of the chunk's concatenation with their
+  // summed importance and per-sample extents; then the ranking by Efraimidis-Spirakis key.
   int build_distinct(int step, uint32_t s0, uint32_t n, uint32_t total) {
     constexpr int form = App::kNeighborhoodForm;
     int chunk_bits = 1;
@@ -755,28 +917,23 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_pos_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
                                   d_scratch_, stream_, &k2, &p2));
       gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_nbr_cols_, p2, total, d_vertex_sorted_,
-                                                          form == apps::kRankedByLadiesImportance ? d_pos_ : nullptr);
+                                                          d_pos_);
       sorted_pos = d_pos_;  // (LADIES) positions in (sample, vertex) order, safe from the later sorts
       // run heads -> distinct ids, per-sample counts (+ degree^2, or run extents)
       const size_t tiles = scan_num_tiles(total);
       count_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(k2, d_vertex_sorted_, total,
                                                                                   d_scratch_);
       scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
-      if (form == apps::kRankedByLadiesImportance) {
-        ND_HIP_TRY(hipMemsetAsync(d_importance_, 0, sizeof(unsigned long long) * (size_t)total, stream_));
-      }
+      ND_HIP_TRY(hipMemsetAsync(d_importance_, 0, sizeof(unsigned long long) * (size_t)total, stream_));
       compact_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(
-          k2, d_vertex_sorted_, total, d_scratch_, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
-          d_distinct_start_, d_distinct_sample_, sorted_pos,
-          form == apps::kRankedByLadiesImportance ? d_nbr_weights_ : nullptr, d_importance_);
+          k2, d_vertex_sorted_, total, d_scratch_, d_distinct_ids_, d_distinct_start_, d_distinct_sample_, sorted_pos,
+          d_nbr_weights_, d_importance_);
       ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
       ND_HIP_TRY(hipStreamSynchronize(stream_));
       distinct_total_ += n_distinct;
     }
     fill_empty_sample_starts<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_, n, n_distinct, kUnset);
-    if (form == apps::kDistinctByDegreeSquared) {
-      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
-    } else if (n_distinct > 0) {
+    if (n_distinct > 0) {
       ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
           d_importance_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_, (uint64_t)s0, (uint32_t)invalid_,
           (uint32_t)step, d_key_bits_);
@@ -805,7 +962,10 @@ class LayerEngine : public EngineBase {
     release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
     release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
     release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
+    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
     capacity_ = 0;
+    bitmap_samples_ = 0;
+    distinct_capacity_ = 0;
   }
 
   void free_run_buffers() {
@@ -835,6 +995,12 @@ class LayerEngine : public EngineBase {
   uint64_t seed_ = 0;
   bool allocated_ = false;
   size_t capacity_ = 0;
+  uint32_t bitmap_words_ = 0;          // words of one sample's bitmap (a multiple of kBitmapTileWords)
+  uint32_t bitmap_chunk_samples_ = 0;  // samples whose bitmaps fit the budget
+  uint64_t bitmap_chunk_entries_ = 0;
+  uint32_t bitmap_samples_ = 0;        // samples the allocated bitmaps hold
+  size_t distinct_capacity_ = 0;
+  uint32_t *d_bitmap_ = nullptr, *d_tile_offsets_ = nullptr, *d_tile_scratch_ = nullptr;
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
   uint64_t chunk_entries_ = kLayerChunkEntries;
   bool progress_ = false;
