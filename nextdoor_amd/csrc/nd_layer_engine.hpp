@@ -190,24 +190,43 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   if (threadIdx.x == 0) s_start[tv.count] = carry;
   __syncthreads();
   const uint32_t size = s_start[tv.count];
-  uint32_t* bits = bitmap + (size_t)s * words_per_sample;
+  uint32_t* sample_bits = bitmap + (size_t)s * words_per_sample;
   const uint32_t first = item * kBuildItemEntries;
   const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
   uint32_t cur = 0;
-  for (uint32_t e = first + threadIdx.x; e < last; e += 256) {
-    if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
-      uint32_t lo = 0, hi = tv.count;
-      while (hi - lo > 1) {
-        const uint32_t mid = lo + (hi - lo) / 2;
-        if (s_start[mid] <= e) lo = mid; else hi = mid;
+  const uint32_t lane = threadIdx.x & 63u;
+  for (uint32_t e0 = first; e0 < last; e0 += 256) {  // the same trip count for every lane
+    const uint32_t e = e0 + threadIdx.x;
+    uint32_t word_index = 0xFFFFFFFFu, bits = 0;
+    if (e < last) {
+      if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
+        uint32_t lo = 0, hi = tv.count;
+        while (hi - lo > 1) {
+          const uint32_t mid = lo + (hi - lo) / 2;
+          if (s_start[mid] <= e) lo = mid; else hi = mid;
+        }
+        cur = lo;
       }
-      cur = lo;
+      const int32_t t = transits[cur];
+      const uint32_t v = (uint32_t)csr.edges[csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur])];
+      word_index = v >> 5;
+      bits = 1u << (v & 31u);
     }
-    const int32_t t = transits[cur];
-    const uint32_t v = (uint32_t)csr.edges[csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur])];
-    const uint32_t bit = 1u << (v & 31u);
-    uint32_t* word = bits + (v >> 5);
-    if ((*word & bit) == 0) atomicOr(word, bit);
+    // Adjacencies are sorted, so neighbouring lanes mostly hit the same word: OR the bits
+    // of equal words along the wave and let the last lane of each stretch do the memory
+    // work (a dense hub row then costs 8 words per wavefront instead of 64).
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint32_t up_index = __shfl_up(word_index, d, kWave);
+      const uint32_t up_bits = __shfl_up(bits, d, kWave);
+      if (lane >= (uint32_t)d && up_index == word_index) bits |= up_bits;
+    }
+    const uint32_t next_index = __shfl_down(word_index, 1, kWave);
+    const bool last_of_stretch = lane == 63u || next_index != word_index;
+    if (bits != 0 && last_of_stretch) {
+      uint32_t* word = sample_bits + word_index;
+      if ((*word & bits) != bits) atomicOr(word, bits);
+    }
   }
 }
 
@@ -236,21 +255,20 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   const uint32_t sample = blockIdx.x / tiles_per_sample;
   const uint32_t tile = blockIdx.x - sample * tiles_per_sample;
-  const uint4* words = (const uint4*)(bitmap + (size_t)blockIdx.x * kBitmapTileWords) + threadIdx.x * 2;
-  const uint4 a = words[0], b = words[1];
-  const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-  uint32_t mine = 0;
-#pragma unroll
-  for (int k = 0; k < 8; ++k) mine += __popc(w[k]);
-  uint32_t total;
-  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
-  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = tile_offsets[blockIdx.x];
-  const uint32_t first_vertex = (tile * kBitmapTileWords + threadIdx.x * 8u) * 32u;
-#pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    uint32_t bits = w[k];
+  const uint32_t* words = bitmap + (size_t)blockIdx.x * kBitmapTileWords;
+  uint32_t running = tile_offsets[blockIdx.x];
+  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = running;
+  // 256 consecutive words per round, one per lane: the ids a wavefront writes in a round
+  // are one contiguous stretch of the output
+  for (uint32_t round = 0; round < kBitmapTileWords / 256; ++round) {
+    const uint32_t w = round * 256 + threadIdx.x;
+    uint32_t bits = words[w];
+    uint32_t total;
+    uint32_t r = running + block_exclusive_scan_256((uint32_t)__popc(bits), s_wave, &total);
+    running += total;
+    const uint32_t first_vertex = (tile * kBitmapTileWords + w) * 32u;
     while (bits) {
-      const uint32_t v = first_vertex + k * 32u + (uint32_t)__ffs((int)bits) - 1u;
+      const uint32_t v = first_vertex + (uint32_t)__ffs((int)bits) - 1u;
       bits &= bits - 1u;
       distinct_ids[r] = (int32_t)v;
       const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
