@@ -458,7 +458,7 @@ int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64
                                   d_scratch.as<uint32_t>(), 0));
   nd::collective_build<<<dim3((unsigned)n_items), dim3(256), 0, 0>>>(
       dg.view, tv, invalid, d_offsets.as<uint32_t>(), d_item_start.as<uint32_t>(), S, d_cols.as<int32_t>(),
-      d_weights.as<float>(), nullptr, d_rows.as<uint32_t>(), nullptr);
+      d_weights.as<float>(), d_rows.as<uint32_t>());
   CAPI_HIP(hipGetLastError());
   CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
   CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));

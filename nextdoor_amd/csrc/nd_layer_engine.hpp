@@ -80,18 +80,15 @@ __global__ __launch_bounds__(256) void collective_sizes(CSRPartition csr, Transi
 constexpr uint32_t kBuildItemEntries = 8192;
 
 // Copies the adjacencies of every sample's transits, in transit order, to
-// cols[offsets[s] ...] (and weights, and the owning sample id when asked for).
+// cols[offsets[s] ...] (and weights).
 // Work items: item_start[s] = number of items of the samples before s (exclusive scan of
 // ceil(size_s / kBuildItemEntries), with the total at [n_samples]); workgroup b serves the
 // sample whose item range holds b and the b - item_start[s]-th stretch of its entries.
-// row_sums (nullable): when given, the weight slot receives (weight / row_sums[transit])^2.
 __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, TransitView tv, int32_t invalid,
                                                         const uint32_t* __restrict__ offsets,
                                                         const uint32_t* __restrict__ item_start, uint32_t n_samples,
                                                         int32_t* __restrict__ cols, float* __restrict__ weights,
-                                                        uint32_t* __restrict__ sample_of,
-                                                        uint32_t* __restrict__ row_offsets,
-                                                        const float* __restrict__ row_sums) {
+                                                        uint32_t* __restrict__ row_offsets) {
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
   __shared__ uint32_t s_scan_tmp[4];
   // sample of this work item: last s with item_start[s] <= blockIdx.x
@@ -138,16 +135,16 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
     const int32_t t = transits[cur];
     const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur]);
     cols[base + e] = csr.edges[src];
-    if (weights) {
-      float w = csr.weights[src];
-      if (row_sums) {
-        const float p = w / row_sums[t];
-        w = p * p;
-      }
-      weights[base + e] = w;
-    }
-    if (sample_of) sample_of[base + e] = s;
+    if (weights) weights[base + e] = csr.weights[src];
   }
+}
+
+// (weight / rowsum)^2 as a 2^53 fixed-point integer: sums of up to 1024 of them fit 64 bits
+// and, unlike float sums, do not depend on the order of the additions.
+__host__ __device__ __forceinline__ unsigned long long importance_term_fixed(float term) {
+  if (!(term > 0.0f)) return 0ull;
+  if (term >= 1.0f) return 1ull << 53;
+  return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
 }
 
 // ---- distinct vertices of a collective neighbourhood through a bitmap ----
@@ -161,9 +158,18 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
 // costs one redundant atomic, never a wrong bit.
 constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words
 
+// kWithImportance (LADIES form): every entry also adds (weight / row_sums[transit])^2, as a
+// fixed-point integer, to sums[sample * sums_per_sample + vertex].  Parallel edges make a
+// vertex repeat in neighbouring lanes; their terms are added up along the wavefront first
+// (a segmented scan in which a lane whose vertex differs from its left neighbour's starts a
+// new segment) and the last lane of each segment issues the one atomic.
+template <bool kWithImportance>
 __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, TransitView tv, int32_t invalid,
                                                        const uint32_t* __restrict__ item_start, uint32_t n_samples,
-                                                       uint32_t* __restrict__ bitmap, uint32_t words_per_sample) {
+                                                       uint32_t* __restrict__ bitmap, uint32_t words_per_sample,
+                                                       const float* __restrict__ row_sums,
+                                                       unsigned long long* __restrict__ sums,
+                                                       uint32_t sums_per_sample) {
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
   __shared__ uint32_t s_scan_tmp[4];
   uint32_t lo_s = 0, hi_s = n_samples;
@@ -197,7 +203,8 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   const uint32_t lane = threadIdx.x & 63u;
   for (uint32_t e0 = first; e0 < last; e0 += 256) {  // the same trip count for every lane
     const uint32_t e = e0 + threadIdx.x;
-    uint32_t word_index = 0xFFFFFFFFu, bits = 0;
+    uint32_t word_index = 0xFFFFFFFFu, bits = 0, vertex = 0xFFFFFFFFu;
+    unsigned long long term = 0;
     if (e < last) {
       if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
         uint32_t lo = 0, hi = tv.count;
@@ -208,9 +215,31 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
         cur = lo;
       }
       const int32_t t = transits[cur];
-      const uint32_t v = (uint32_t)csr.edges[csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur])];
-      word_index = v >> 5;
-      bits = 1u << (v & 31u);
+      const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur]);
+      vertex = (uint32_t)csr.edges[src];
+      word_index = vertex >> 5;
+      bits = 1u << (vertex & 31u);
+      if (kWithImportance) {
+        const float p = csr.weights[src] / row_sums[t];
+        term = importance_term_fixed(p * p);
+      }
+    }
+    if (kWithImportance) {
+      const uint32_t left = __shfl_up(vertex, 1, kWave);
+      bool closed = lane == 0 || left != vertex;  // this lane starts a segment
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t lo = __shfl_up((uint32_t)term, d, kWave);
+        const uint32_t hi = __shfl_up((uint32_t)(term >> 32), d, kWave);
+        const int up_closed = __shfl_up((int)closed, d, kWave);
+        if (lane >= (uint32_t)d) {
+          if (!closed) term += ((unsigned long long)hi << 32) | lo;
+          closed = closed || up_closed;
+        }
+      }
+      const uint32_t right = __shfl_down(vertex, 1, kWave);
+      if (vertex != 0xFFFFFFFFu && term != 0 && (lane == 63u || right != vertex))
+        atomicAdd(sums + (size_t)s * sums_per_sample + vertex, term);
     }
     // Adjacencies are sorted, so neighbouring lanes mostly hit the same word: OR the bits
     // of equal words along the wave and let the last lane of each stretch do the memory
@@ -245,13 +274,17 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
 
 // The set bits of every sample's bitmap, in ascending order, become the sample's distinct
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
-// tile of a sample is where the sample's list starts).
+// tile of a sample is where the sample's list starts).  Per distinct vertex either
+// degree^2 (degree_sq given) or the importance accumulated in sums (sums given).
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t tiles_per_sample, const EdgePos_t* __restrict__ row_ptr,
                                                       int32_t* __restrict__ distinct_ids,
                                                       uint64_t* __restrict__ degree_sq,
-                                                      uint32_t* __restrict__ distinct_start) {
+                                                      uint32_t* __restrict__ distinct_start,
+                                                      unsigned long long* __restrict__ sums, uint32_t sums_per_sample,
+                                                      unsigned long long* __restrict__ importance,
+                                                      uint32_t* __restrict__ distinct_sample) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   const uint32_t sample = blockIdx.x / tiles_per_sample;
   const uint32_t tile = blockIdx.x - sample * tiles_per_sample;
@@ -271,8 +304,17 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
       const uint32_t v = first_vertex + (uint32_t)__ffs((int)bits) - 1u;
       bits &= bits - 1u;
       distinct_ids[r] = (int32_t)v;
-      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-      degree_sq[r] = d * d;
+      if (degree_sq) {
+        const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+        degree_sq[r] = d * d;
+      }
+      if (sums) {
+        // collect the vertex's importance and leave the accumulator clear for the next chunk
+        unsigned long long* acc = sums + (size_t)sample * sums_per_sample + v;
+        importance[r] = *acc;
+        *acc = 0;
+        distinct_sample[r] = sample;
+      }
       ++r;
     }
   }
@@ -296,125 +338,6 @@ __global__ void gather_u32(const uint32_t* __restrict__ table, const uint32_t* _
   const uint32_t p = index[i];
   out[i] = table[p];
   if (index_copy) index_copy[i] = p;
-}
-
-__device__ __forceinline__ bool is_pair_head(const uint32_t* sample_key, const uint32_t* vertex, size_t i) {
-  return i == 0 || sample_key[i] != sample_key[i - 1] || vertex[i] != vertex[i - 1];
-}
-
-__global__ __launch_bounds__(kScanThreads) void count_pair_heads(const uint32_t* __restrict__ sample_key,
-                                                                 const uint32_t* __restrict__ vertex, size_t n,
-                                                                 uint32_t* __restrict__ tile_counts) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
-  const size_t base = (size_t)blockIdx.x * kScanTile;
-  uint32_t heads = 0;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    const size_t idx = base + (size_t)i * kScanThreads + threadIdx.x;
-    if (idx < n && is_pair_head(sample_key, vertex, idx)) heads++;
-  }
-  uint32_t total;
-  block_exclusive_scan_256(heads, s_wave, &total);
-  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
-}
-
-// (weight / rowsum)^2 as a 2^53 fixed-point integer: sums of up to 1024 of them fit 64 bits
-// and, unlike float sums, do not depend on the order of the additions.
-__host__ __device__ __forceinline__ unsigned long long importance_term_fixed(float term) {
-  if (!(term > 0.0f)) return 0ull;
-  if (term >= 1.0f) return 1ull << 53;
-  return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
-}
-
-// Distinct (sample, vertex) pairs in order (LADIES form).  Every head writes its vertex id
-// and sample; the first head of a sample writes the sample's start in the distinct list.
-// terms (nullable): the fixed-point terms of every run are summed into importance[run],
-// which the caller has zeroed.
-__global__ __launch_bounds__(kScanThreads) void compact_pair_heads(const uint32_t* __restrict__ sample_key,
-                                                                   const uint32_t* __restrict__ vertex, size_t n,
-                                                                   const uint32_t* __restrict__ tile_offsets,
-                                                                   int32_t* __restrict__ distinct_ids,
-                                                                   uint32_t* __restrict__ distinct_start,
-                                                                   uint32_t* __restrict__ distinct_sample,
-                                                                   const uint32_t* __restrict__ sorted_pos,
-                                                                   const float* __restrict__ terms,
-                                                                   unsigned long long* __restrict__ importance) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
-  const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
-  bool head[kScanItems];
-  uint32_t mine = 0;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    head[i] = base + i < n && is_pair_head(sample_key, vertex, base + i);
-    mine += head[i] ? 1u : 0u;
-  }
-  uint32_t total;
-  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
-  // Terms: a lane sums the stretch it owns.  What precedes its first head belongs to the run
-  // that was open when the stretch began (first_partial); what follows its last head stays
-  // open (partial); runs that begin and end inside the stretch are flushed on the spot.
-  const uint32_t r_begin = r;
-  unsigned long long first_partial = 0, partial = 0;
-  bool seen_head = false;
-#pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    if (base + i >= n) break;
-    if (head[i]) {
-      if (!seen_head) {
-        first_partial = partial;
-        seen_head = true;
-      } else if (partial) {
-        atomicAdd(&importance[r - 1], partial);
-      }
-      partial = 0;
-      const uint32_t v = vertex[base + i];
-      const uint32_t s = sample_key[base + i];
-      distinct_ids[r] = (int32_t)v;
-      if (distinct_sample) distinct_sample[r] = s;
-      if (base + i == 0 || sample_key[base + i - 1] != s) distinct_start[s] = r;
-      ++r;
-    }
-    if (terms) partial += importance_term_fixed(terms[sorted_pos[base + i]]);
-  }
-  if (!terms) return;
-  // Open partials are combined along the wave before they reach memory (a segmented scan in
-  // which a lane with a head starts a new segment): a vertex reached over very many
-  // (duplicate) edges then costs one atomic per wave instead of a long loop in one lane.
-  const int lane = threadIdx.x & (kWave - 1);
-  unsigned long long open = partial;
-  bool closed = seen_head;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const uint32_t lo = __shfl_up((uint32_t)open, d, kWave);
-    const uint32_t hi = __shfl_up((uint32_t)(open >> 32), d, kWave);
-    const int up_closed = __shfl_up((int)closed, d, kWave);
-    if (lane >= d) {
-      if (!closed) open += ((unsigned long long)hi << 32) | lo;
-      closed = closed || up_closed;
-    }
-  }
-  const uint32_t in_lo = __shfl_up((uint32_t)open, 1, kWave);
-  const uint32_t in_hi = __shfl_up((uint32_t)(open >> 32), 1, kWave);
-  const unsigned long long carry_in = lane == 0 ? 0ull : ((unsigned long long)in_hi << 32) | in_lo;
-  if (seen_head) {
-    const unsigned long long before = first_partial + carry_in;
-    if (before) atomicAdd(&importance[r_begin - 1], before);
-  }
-  if (lane == kWave - 1 && open) atomicAdd(&importance[r - 1], open);
-}
-
-// distinct_start[s] was written for samples that have distinct vertices; the others take
-// the start of the next sample that has (the list holds nothing of theirs).  One lane: the
-// number of samples per chunk is small.
-__global__ void fill_empty_sample_starts(uint32_t* distinct_start, uint32_t n_samples, uint32_t n_distinct,
-                                         uint32_t unset) {
-  if (blockIdx.x != 0 || threadIdx.x != 0) return;
-  uint32_t next = n_distinct;
-  distinct_start[n_samples] = n_distinct;
-  for (uint32_t s = n_samples; s-- > 0;) {
-    if (distinct_start[s] == unset) distinct_start[s] = next;
-    else next = distinct_start[s];
-  }
 }
 
 __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
@@ -647,7 +570,10 @@ class LayerEngine : public EngineBase {
       if (v > 0) chunk_entries_ = bitmap_chunk_entries_ = (uint64_t)v;
     }
     bitmap_words_ = (((uint32_t)invalid_ + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
-    const uint64_t fit = kBitmapBudgetBytes / ((uint64_t)bitmap_words_ * sizeof(uint32_t));
+    // LADIES form: one 64-bit importance accumulator per vertex next to the bitmap
+    sums_per_sample_ = App::kNeighborhoodForm == apps::kRankedByLadiesImportance ? (uint32_t)invalid_ : 0u;
+    const uint64_t fit = kBitmapBudgetBytes / ((uint64_t)bitmap_words_ * sizeof(uint32_t) +
+                                               (uint64_t)sums_per_sample_ * sizeof(unsigned long long));
     bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
@@ -711,7 +637,7 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipStreamSynchronize(stream_));
       // chunk limits: entries of concatenation the work arrays hold, or (bitmap form) bitmaps
       // that fit the budget and a grid of marking work items that fits 31 bits
-      constexpr bool by_bitmap = App::kNeighborhoodForm == apps::kDistinctByDegreeSquared;
+      constexpr bool by_bitmap = App::kNeighborhoodForm != apps::kConcatenated;
       const uint64_t entry_budget = by_bitmap ? bitmap_chunk_entries_ : chunk_entries_;
       const uint32_t sample_budget = by_bitmap ? bitmap_chunk_samples_ : S;
       uint32_t s0 = 0;
@@ -797,16 +723,15 @@ class LayerEngine : public EngineBase {
     if (n_items >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more work items"; return -2; }
     build_item_counts<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_sizes_ + s0, n, d_item_count_);
     ND_HIP_TRY(exclusive_scan_u32(d_item_count_, d_item_start_, (size_t)n + 1, d_small_scratch_, stream_));
-    if (form == apps::kDistinctByDegreeSquared) {
-      if (build_distinct_by_bitmap(tv, n, (unsigned)n_items) != 0) return -1;
+    if (form != apps::kConcatenated) {
+      if (build_distinct_by_bitmap(step, s0, tv, n, (unsigned)n_items) != 0) return -1;
     } else {
       if (ensure_neighborhood_capacity((uint32_t)total) != 0) return -1;
       // offsets of the chunk's samples, relative to the chunk (element n = total)
       ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
       collective_build<<<dim3((unsigned)n_items), dim3(256), 0, stream_>>>(
           dgraph_.view, tv, invalid_, d_offsets_, d_item_start_, n, d_nbr_cols_, d_nbr_weights_,
-          form != apps::kConcatenated ? d_sample_of_ : nullptr, d_row_offsets_ + (size_t)s0 * all.count,
-          form == apps::kRankedByLadiesImportance ? d_row_sums_ : nullptr);
+          d_row_offsets_ + (size_t)s0 * all.count);
       ND_HIP_TRY(hipGetLastError());
     }
 
@@ -828,7 +753,6 @@ class LayerEngine : public EngineBase {
     P.nbr_cols = d_nbr_cols_;
     P.nbr_weights = d_nbr_weights_;
     if (form != apps::kConcatenated) {
-      if (form == apps::kRankedByLadiesImportance && build_distinct(step, s0, n, (uint32_t)total) != 0) return -1;
       P.distinct_start = d_distinct_start_;
       P.distinct_ids = form == apps::kRankedByLadiesImportance ? d_ranked_ids_ : d_distinct_ids_;
       P.running_sums = d_running_sums_;
@@ -839,21 +763,30 @@ class LayerEngine : public EngineBase {
     return 0;
   }
 
-  // Distinct vertices of every sample of the chunk, ascending, with running sums of
-  // degree^2: mark bits, count them per tile, scan, write the ids out.
-  int build_distinct_by_bitmap(const TransitView& tv, uint32_t n, unsigned n_items) {
+  // Distinct vertices of every sample of the chunk, ascending: mark bits (and add up
+  // importance), count the bits per tile, scan, write the ids out.  Then running sums of
+  // degree^2, or the ranking by Efraimidis-Spirakis key.
+  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n, unsigned n_items) {
+    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
     const uint32_t tiles_per_sample = bitmap_words_ / kBitmapTileWords;
     const size_t n_tiles = (size_t)n * tiles_per_sample;
     if (n > bitmap_samples_) {
-      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
+      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_sums_);
       ND_HIP_TRY(hipMalloc(&d_bitmap_, sizeof(uint32_t) * (size_t)n * bitmap_words_));
       ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
       ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
+      if (ladies) {
+        // cleared once: the compaction leaves every accumulator it reads at zero again
+        const size_t bytes = sizeof(unsigned long long) * (size_t)n * sums_per_sample_;
+        ND_HIP_TRY(hipMalloc(&d_sums_, bytes));
+        ND_HIP_TRY(hipMemsetAsync(d_sums_, 0, bytes, stream_));
+      }
       bitmap_samples_ = n;
     }
     ND_HIP_TRY(hipMemsetAsync(d_bitmap_, 0, sizeof(uint32_t) * (size_t)n * bitmap_words_, stream_));
-    collective_mark<<<dim3(n_items), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_item_start_, n, d_bitmap_,
-                                                              bitmap_words_);
+    collective_mark<ladies><<<dim3(n_items), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_item_start_, n,
+                                                                      d_bitmap_, bitmap_words_, d_row_sums_, d_sums_,
+                                                                      sums_per_sample_);
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
     ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
     uint32_t n_distinct = 0;
@@ -861,97 +794,16 @@ class LayerEngine : public EngineBase {
                               hipMemcpyDeviceToHost, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     distinct_total_ += n_distinct;
-    if (n_distinct > distinct_capacity_) {
-      const size_t cap = (size_t)n_distinct + n_distinct / 8 + 1024;
-      release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
-      ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
-      distinct_capacity_ = cap;
-    }
-    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_, tiles_per_sample,
-                                                                      dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
-                                                                      d_distinct_start_);
+    if (ensure_distinct_capacity(n_distinct) != 0) return -1;
+    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
+        d_bitmap_, d_tile_offsets_, tiles_per_sample, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
+        d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
-    ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
-    return hipGetLastError() == hipSuccess ? 0 : -1;
-  }
-
-  int ensure_neighborhood_capacity(uint32_t total) {
-    if (total <= capacity_ && capacity_ > 0) return 0;
-    const size_t cap = (size_t)total + total / 8 + 1024;
-    release_neighborhood_buffers();
-    ND_HIP_TRY(hipMalloc(&d_nbr_cols_, sizeof(int32_t) * cap));
-    ND_HIP_TRY(hipMalloc(&d_nbr_weights_, sizeof(float) * cap));
-    constexpr int form = App::kNeighborhoodForm;
-    if (form != apps::kConcatenated) {
-      ND_HIP_TRY(hipMalloc(&d_sample_of_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_key2_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_pos_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_vertex_sorted_, sizeof(uint32_t) * cap));
-      const SortPlan plan = make_sort_plan(cap, 32);
-      ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(cap)));
-      size_t scratch = plan.scratch_elems;
-      if (scan_scratch_elems(cap) > scratch) scratch = scan_scratch_elems(cap);
-      ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
-      ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
-    }
-    if (form == apps::kRankedByLadiesImportance) {
-      ND_HIP_TRY(hipMalloc(&d_importance_, sizeof(unsigned long long) * cap));
-      ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
-    }
-    capacity_ = cap;
-    return 0;
-  }
-
-  // LADIES form: distinct (sample, vertex) pairs of the chunk's concatenation with their
-  // summed importance and per-sample extents; then the ranking by Efraimidis-Spirakis key.
-  int build_distinct(int step, uint32_t s0, uint32_t n, uint32_t total) {
-    constexpr int form = App::kNeighborhoodForm;
-    int chunk_bits = 1;
-    while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
-    constexpr uint32_t kUnset = 0xFFFFFFFFu;
-    fill_u32<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_distinct_start_, (size_t)n + 1, kUnset);
-    uint32_t n_distinct = 0;
-    uint32_t* sorted_pos = nullptr;
-    if (total > 0) {
-      // sort by vertex, carrying the position in the concatenation ...
-      const SortPlan by_vertex = make_sort_plan(total, max_bits_);
-      uint32_t *k1 = nullptr, *p1 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_vertex, (const uint32_t*)d_nbr_cols_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
-                                  d_vals_b_, d_hist_, d_scratch_, stream_, &k1, &p1));
-      // ... then stably by owning sample: (sample, vertex) order, duplicates in concatenation order
-      const unsigned blocks = (total + 255) / 256;
-      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_sample_of_, p1, total, d_key2_, d_pos_);
-      const SortPlan by_sample = make_sort_plan(total, chunk_bits);
-      uint32_t *k2 = nullptr, *p2 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_pos_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
-                                  d_scratch_, stream_, &k2, &p2));
-      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_nbr_cols_, p2, total, d_vertex_sorted_,
-                                                          d_pos_);
-      sorted_pos = d_pos_;  // (LADIES) positions in (sample, vertex) order, safe from the later sorts
-      // run heads -> distinct ids, per-sample counts (+ degree^2, or run extents)
-      const size_t tiles = scan_num_tiles(total);
-      count_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(k2, d_vertex_sorted_, total,
-                                                                                  d_scratch_);
-      scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
-      ND_HIP_TRY(hipMemsetAsync(d_importance_, 0, sizeof(unsigned long long) * (size_t)total, stream_));
-      compact_pair_heads<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream_>>>(
-          k2, d_vertex_sorted_, total, d_scratch_, d_distinct_ids_, d_distinct_start_, d_distinct_sample_, sorted_pos,
-          d_nbr_weights_, d_importance_);
-      ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
-      ND_HIP_TRY(hipStreamSynchronize(stream_));
-      distinct_total_ += n_distinct;
-    }
-    fill_empty_sample_starts<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_, n, n_distinct, kUnset);
-    if (n_distinct > 0) {
+    if (!ladies) {
+      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
+    } else if (n_distinct > 0) {
+      int chunk_bits = 1;
+      while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
       ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
           d_importance_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_, (uint64_t)s0, (uint32_t)invalid_,
           (uint32_t)step, d_key_bits_);
@@ -963,27 +815,72 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(radix_sort_pairs(by_key, d_key_bits_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
                                   d_scratch_, stream_, &k3, &j3));
       const unsigned blocks = (n_distinct + 255) / 256;
-      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_distinct_sample_, j3, n_distinct, d_key2_, d_vertex_sorted_);
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_distinct_sample_, j3, n_distinct, d_key2_, d_index2_);
       const SortPlan by_sample = make_sort_plan(n_distinct, chunk_bits);
       uint32_t *k4 = nullptr, *j4 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_vertex_sorted_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_,
-                                  d_hist_, d_scratch_, stream_, &k4, &j4));
+      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                  d_scratch_, stream_, &k4, &j4));
       gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_distinct_ids_, j4, n_distinct,
                                                           (uint32_t*)d_ranked_ids_, nullptr);
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
   }
 
-  void release_neighborhood_buffers() {
-    release(d_nbr_cols_); release(d_nbr_weights_); release(d_sample_of_);
-    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
-    release(d_key2_); release(d_pos_); release(d_vertex_sorted_); release(d_hist_); release(d_scratch_);
+  // Arrays with one entry per distinct (sample, vertex) pair of a chunk.
+  int ensure_distinct_capacity(uint32_t n_distinct) {
+    if (n_distinct <= distinct_capacity_ && distinct_capacity_ > 0) return 0;
+    constexpr int form = App::kNeighborhoodForm;
+    const size_t cap = (size_t)n_distinct + n_distinct / 8 + 1024;
+    release_distinct_buffers();
+    ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
+    if (form == apps::kDistinctByDegreeSquared) {
+      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
+    }
+    if (form == apps::kRankedByLadiesImportance) {
+      ND_HIP_TRY(hipMalloc(&d_importance_, sizeof(unsigned long long) * cap));
+      ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_vals_b_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_key2_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_index2_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(cap)));
+      ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * make_sort_plan(cap, 32).scratch_elems));
+    }
+    distinct_capacity_ = cap;
+    return 0;
+  }
+
+  // The concatenated neighbourhood itself (kConcatenated form).
+  int ensure_neighborhood_capacity(uint32_t total) {
+    if (total <= capacity_ && capacity_ > 0) return 0;
+    const size_t cap = (size_t)total + total / 8 + 1024;
+    release(d_nbr_cols_); release(d_nbr_weights_);
+    ND_HIP_TRY(hipMalloc(&d_nbr_cols_, sizeof(int32_t) * cap));
+    ND_HIP_TRY(hipMalloc(&d_nbr_weights_, sizeof(float) * cap));
+    capacity_ = cap;
+    return 0;
+  }
+
+  void release_distinct_buffers() {
     release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
     release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
-    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
+    release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
+    release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
+    distinct_capacity_ = 0;
+  }
+
+  void release_neighborhood_buffers() {
+    release(d_nbr_cols_); release(d_nbr_weights_);
+    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_sums_);
+    release_distinct_buffers();
     capacity_ = 0;
     bitmap_samples_ = 0;
-    distinct_capacity_ = 0;
   }
 
   void free_run_buffers() {
@@ -1019,6 +916,8 @@ class LayerEngine : public EngineBase {
   uint32_t bitmap_samples_ = 0;        // samples the allocated bitmaps hold
   size_t distinct_capacity_ = 0;
   uint32_t *d_bitmap_ = nullptr, *d_tile_offsets_ = nullptr, *d_tile_scratch_ = nullptr;
+  unsigned long long* d_sums_ = nullptr;  // LADIES form: importance accumulators, [sample][vertex]
+  uint32_t sums_per_sample_ = 0;
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
   uint64_t chunk_entries_ = kLayerChunkEntries;
   bool progress_ = false;
@@ -1034,9 +933,8 @@ class LayerEngine : public EngineBase {
   uint32_t* d_distinct_start_ = nullptr;
   int32_t* d_nbr_cols_ = nullptr;
   float* d_nbr_weights_ = nullptr;
-  uint32_t* d_sample_of_ = nullptr;
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
-  uint32_t *d_key2_ = nullptr, *d_pos_ = nullptr, *d_vertex_sorted_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
+  uint32_t *d_key2_ = nullptr, *d_index2_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
   uint64_t *d_degree_sq_ = nullptr, *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
   unsigned long long* d_importance_ = nullptr;
