@@ -27,9 +27,18 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the dominant kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
 # this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
 # known size).  None where no such run has been recorded.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"weighted_node2vec_rmat22": 1.469e9}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    "weighted_node2vec_rmat22": 1.245e9,     # step_flat_kernel
+    "uniform_walk_chunglu57k": 4.27e6,       # step_flat_kernel
+    "khop_rmat21": 1.94e9,                   # step kernels of one hop (2 x flat 0.688e9 + workgroup 2.495e9, over 2 hops)
+    "fastgcn_importance_rmat22": 8.101e10,   # collective_mark, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 5.242e10,  # collective_mark, average over its 12 launches per pass
+}
 # HBM bytes of all kernels of one pass, same source.
-MEASURED_TRAFFIC_BYTES_PER_PASS = {"weighted_node2vec_rmat22": 176.6e9}
+MEASURED_TRAFFIC_BYTES_PER_PASS = {
+    "weighted_node2vec_rmat22": 165.4e9, "uniform_walk_chunglu57k": 0.98e9, "khop_rmat21": 14.8e9,
+    "fastgcn_importance_rmat22": 270.2e9, "ladies_importance_chunglu3m": 2128.9e9,
+}
 
 WORKLOADS = {
     # name: (app, graph factory kwargs)
@@ -88,6 +97,32 @@ def cpu_baseline(graph, sampler, kind_name, budget_s, seed):
         "sample": f"CPU oracle, every {best['stride']}th walk ({best['samples']} of {sampler.num_samples} samples, "
                   f"all {steps} steps), {best['seconds']:.1f} s",
     }, best
+
+
+def cpu_baseline_layers(graph, sampler, kind_name, budget_s, seed):
+    """Layer-wise apps: times the CPU oracle on the first batches of the same launch, all
+    host cores (one batch per thread), doubling the number of batches until it has run for
+    about a third of budget_s."""
+    from tests import graphs, oracle_binding as ob
+    og = graphs.oracle_view(graph)
+    steps = sampler.steps
+    desc = ob.app_desc(getattr(ob, kind_name), steps, [sampler.step_size(k) for k in range(steps)],
+                       initial_size=sampler.initial_sample_size)
+    roots = sampler.initial_contents.reshape(sampler.num_samples, -1)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    fn = ob.sample_fastgcn_importance if kind_name == "FASTGCN_IMPORTANCE" else ob.sample_ladies_importance
+    n = min(sampler.num_samples, cores)
+    while True:
+        t0 = time.perf_counter()
+        fn(og, desc, seed, roots[:n].reshape(-1), first_sample=0, n_threads=cores)
+        dt = time.perf_counter() - t0
+        if dt >= budget_s / 3 or n == sampler.num_samples:
+            break
+        n = min(sampler.num_samples, n * 2)
+    return {
+        "value": n * sampler.final_sample_size / dt, "unit": "sampled edges/s", "cores": cores, "kind": "port",
+        "sample": f"CPU oracle, the first {n} of {sampler.num_samples} batches (all layers), {dt:.1f} s",
+    }
 
 
 def algorithmic_bytes_per_pass(sampler, oracle_run, weighted, second_order):
@@ -167,10 +202,28 @@ def main():
         "phases_ms": {k: round(v, 3) for k, v in prof.items()},
     }
 
-    if w["kind"] in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE", "LAYER_LITERAL"):
-        result["config"]["neighbourhood_entries"] = sampler.counter(0)
-        result["config"]["distinct_pairs"] = sampler.counter(1)
+    if w["kind"] in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE"):
+        entries, distinct = sampler.counter(0), sampler.counter(1)
+        result["config"]["neighbourhood_entries"] = entries
+        result["config"]["distinct_pairs"] = distinct
         result["config"]["chunks"] = sampler.counter(2)
+        result["config"]["neighbourhood_entries_per_s"] = entries / (ms_per_step / 1000.0)
+        # dominant kernel: collective_mark walks every entry of every collective neighbourhood
+        # once.  Minimal traffic: the entry's vertex id (4 B; + 4 B weight for LADIES) and one
+        # bit (FastGCN) or one bit + a 64-bit accumulator (LADIES) per distinct pair.
+        ladies = w["kind"] == "LADIES_IMPORTANCE"
+        mark_bytes = entries * (8 if ladies else 4) + distinct * (8.125 if ladies else 0.125)
+        launches = max(prof["neighbourhood_launches"], 1)
+        achieved = mark_bytes / (prof["neighbourhood_ms"] / 1000.0) / 1e9
+        result["roofline"] = {
+            "bound": "hbm", "kernel": "collective_mark", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "algorithmic_bytes_per_launch": mark_bytes / launches,
+            "avg_launch_ms": prof["neighbourhood_ms"] / launches,
+            "whole_pass": {"measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
+        }
+        if not args.skip_cpu_baseline:
+            result["cpu_baseline"] = cpu_baseline_layers(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
         args.skip_cpu_baseline = True  # the walk/k-hop accounting below does not apply to layer-wise apps
     if w["kind"] == "KHOP":
         counts = sampler.distinct()

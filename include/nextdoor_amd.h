@@ -90,7 +90,8 @@ int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
  * measured with events on the sampler's stream when profiling is on.
  * out[0] end to end, [1] inversion, [2] load balancing, [3] flat (identity / sub-wavefront)
  * kernel, [4] workgroup + grid-wide kernel, [8] final-row assembly, [9] the last distinct pass, all in
- * milliseconds; [5] flat launches, [6] workgroup launches, [7] sort passes; [10..11] reserved (0). */
+ * milliseconds; [5] flat launches, [6] workgroup launches, [7] sort passes; layer-wise apps:
+ * [10] milliseconds in the kernel that walks the collective neighbourhoods, [11] its launches. */
 int nd_sampler_set_profiling(nd_sampler* s, int on);
 int nd_sampler_phase_times(const nd_sampler* s, float out[12]);
 /* Distinct post-pass for SampledVertices results (GraphSAGE: draw with replacement, then

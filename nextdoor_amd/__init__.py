@@ -202,8 +202,9 @@ class Sampler:
         out = (C.c_float * 12)()
         check(lib().nd_sampler_phase_times(self._h, out))
         keys = ["end_to_end_ms", "inversion_ms", "load_balancing_ms", "flat_kernel_ms", "workgroup_kernel_ms",
-                "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms", "distinct_ms"]
-        return dict(zip(keys, list(out)[:10]))
+                "flat_launches", "workgroup_launches", "sort_passes", "assemble_ms", "distinct_ms",
+                "neighbourhood_ms", "neighbourhood_launches"]
+        return dict(zip(keys, list(out)))
 
     def counter(self, which):
         return lib().nd_sampler_counter(self._h, which)

@@ -267,7 +267,8 @@ int nd_sampler_phase_times(const nd_sampler* s, float out[12]) {
   out[7] = (float)t.sort_launches;
   out[8] = t.assemble;
   out[9] = t.distinct;
-  out[10] = out[11] = 0.0f;
+  out[10] = t.neighborhood;
+  out[11] = (float)t.neighborhood_launches;
   return 0;
 }
 

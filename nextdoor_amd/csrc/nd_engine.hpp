@@ -49,6 +49,9 @@ enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1 };
 struct PhaseTimes {  // milliseconds, accumulated over one sample() call when profiling is on
   float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0, assemble = 0, distinct = 0;
   int flat_launches = 0, workgroup_launches = 0, sort_launches = 0;
+  // layer-wise apps: the kernel that walks the collective neighbourhoods (marking / building)
+  float neighborhood = 0;
+  int neighborhood_launches = 0;
 };
 
 class EngineBase {

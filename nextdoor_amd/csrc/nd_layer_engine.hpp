@@ -579,6 +579,8 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipStreamCreate(&stream_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
     ND_HIP_TRY(hipEventCreate(&ev_end_));
+    ND_HIP_TRY(hipEventCreate(&ev_a_));
+    ND_HIP_TRY(hipEventCreate(&ev_b_));
     allocated_ = true;
     ND_HIP_TRY(hipMalloc(&d_initial_, sizeof(VertexID_t) * initialContents.size()));
     ND_HIP_TRY(hipMemcpy(d_initial_, initialContents.data(), sizeof(VertexID_t) * initialContents.size(),
@@ -705,6 +707,20 @@ class LayerEngine : public EngineBase {
     p = nullptr;
   }
 
+  // events around the neighbourhood kernel when profiling is on
+  void tick() {
+    if (profiling) (void)hipEventRecord(ev_a_, stream_);
+  }
+  void tock() {
+    if (!profiling) return;
+    (void)hipEventRecord(ev_b_, stream_);
+    (void)hipEventSynchronize(ev_b_);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, ev_a_, ev_b_);
+    times.neighborhood += ms;
+    times.neighborhood_launches++;
+  }
+
   // One chunk of samples [s0, s1) of one layer: concatenate, post-process in the form the
   // app asks for, run next() for every (sample, nbr).
   int run_chunk(int step, const TransitView& all, uint32_t s0, uint32_t s1, uint64_t total) {
@@ -729,9 +745,11 @@ class LayerEngine : public EngineBase {
       if (ensure_neighborhood_capacity((uint32_t)total) != 0) return -1;
       // offsets of the chunk's samples, relative to the chunk (element n = total)
       ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
+      tick();
       collective_build<<<dim3((unsigned)n_items), dim3(256), 0, stream_>>>(
           dgraph_.view, tv, invalid_, d_offsets_, d_item_start_, n, d_nbr_cols_, d_nbr_weights_,
           d_row_offsets_ + (size_t)s0 * all.count);
+      tock();
       ND_HIP_TRY(hipGetLastError());
     }
 
@@ -784,9 +802,11 @@ class LayerEngine : public EngineBase {
       bitmap_samples_ = n;
     }
     ND_HIP_TRY(hipMemsetAsync(d_bitmap_, 0, sizeof(uint32_t) * (size_t)n * bitmap_words_, stream_));
+    tick();
     collective_mark<ladies><<<dim3(n_items), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_item_start_, n,
                                                                       d_bitmap_, bitmap_words_, d_row_sums_, d_sums_,
                                                                       sums_per_sample_);
+    tock();
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
     ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
     uint32_t n_distinct = 0;
@@ -892,6 +912,8 @@ class LayerEngine : public EngineBase {
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
       (void)hipEventDestroy(ev_end_);
+      (void)hipEventDestroy(ev_a_);
+      (void)hipEventDestroy(ev_b_);
       (void)hipStreamDestroy(stream_);
     }
     allocated_ = false;
@@ -923,7 +945,7 @@ class LayerEngine : public EngineBase {
   bool progress_ = false;
 
   hipStream_t stream_ = nullptr;
-  hipEvent_t ev_begin_ = nullptr, ev_end_ = nullptr;
+  hipEvent_t ev_begin_ = nullptr, ev_end_ = nullptr, ev_a_ = nullptr, ev_b_ = nullptr;
   VertexID_t* d_initial_ = nullptr;
   SampleType* d_samples_ = nullptr;
   SampleType* d_samples_init_ = nullptr;
