@@ -46,6 +46,9 @@ WORKLOADS = {
                                      graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
     "weighted_node2vec_rmat16": dict(app="WeightedNode2Vec", kind="WEIGHTED_NODE2VEC",
                                      graph=("rmat", dict(scale=16, edge_factor=16, symmetrise=True))),
+    # the reference's literal node2vec (unweighted acceptance, src/apps/randomwalks/randomWalks.cu:132-178)
+    "node2vec_rmat22": dict(app="Node2VecPerVertex", kind="NODE2VEC",
+                            graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
     "uniform_walk_chunglu57k": dict(app="UniformRandomWalk", kind="UNIFORM_WALK",
                                     graph=("chung_lu", dict(n_vertices=56944, n_edges=818000, exponent=2.1))),
     "khop_rmat21": dict(app="KHop", kind="KHOP", graph=("rmat", dict(scale=21, edge_factor=32, symmetrise=False))),

@@ -65,14 +65,19 @@ __global__ __launch_bounds__(256) void collective_sizes(CSRPartition csr, Transi
   const uint32_t s = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (s >= n_samples) return;
   const int32_t* transits = tv.base + (size_t)s * tv.stride;
-  uint32_t sum = 0;
+  uint64_t sum = 0;
   for (uint32_t i = lane; i < tv.count; i += 64u) {
     const int32_t t = transits[i];
-    if (t != invalid && t != -1) sum += (uint32_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
+    if (t != invalid && t != -1) sum += (uint64_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
   }
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) sum += __shfl_down(sum, d, 64);
-  if (lane == 0) sizes[s] = sum;
+  for (int d = 32; d > 0; d >>= 1) {
+    const uint32_t lo = __shfl_down((uint32_t)sum, d, 64);
+    const uint32_t hi = __shfl_down((uint32_t)(sum >> 32), d, 64);
+    sum += ((uint64_t)hi << 32) | lo;
+  }
+  // sizes are 32-bit; a neighbourhood that does not fit saturates and the host refuses it
+  if (lane == 0) sizes[s] = sum > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)sum;
 }
 
 // Entries of a sample's concatenation one workgroup of collective_build copies; samples
@@ -642,15 +647,13 @@ class LayerEngine : public EngineBase {
       constexpr bool by_bitmap = App::kNeighborhoodForm != apps::kConcatenated;
       const uint64_t entry_budget = by_bitmap ? bitmap_chunk_entries_ : chunk_entries_;
       const uint32_t sample_budget = by_bitmap ? bitmap_chunk_samples_ : S;
+      for (uint32_t s = 0; s < S; ++s)
+        if (h_sizes_[s] >= (1u << 31)) { last_error = "collective neighbourhood of one sample has 2^31 or more entries"; return -2; }
       uint32_t s0 = 0;
       while (s0 < S) {
         uint64_t total = h_sizes_[s0];
         uint32_t s1 = s0 + 1;
         while (s1 < S && s1 - s0 < sample_budget && total + h_sizes_[s1] <= entry_budget) total += h_sizes_[s1++];
-        if (total >= (1ull << 31) && !by_bitmap) {
-          last_error = "collective neighbourhood of one sample exceeds 2^31 entries";
-          return -2;
-        }
         if (run_chunk(step, all, s0, s1, total) != 0) return -1;
         neighborhood_total_ += total;
         chunks_run_++;
