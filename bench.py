@@ -159,6 +159,9 @@ def main():
     ap.add_argument("--no-load-balancing", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--inversion-period", type=int, default=1,
+                    help="walks: invert the sample->transit map before every p-th step (1: every step, as the "
+                         "reference; 0: the engine decides); the samples do not depend on it")
     ap.add_argument("--seed", type=int, default=42)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -171,6 +174,7 @@ def main():
     graph = make_graph(nd, w["graph"])
     t_graph = time.perf_counter() - t0
     sampler = nd.Sampler(w["app"], graph, seed=args.seed)
+    sampler.set_inversion_period(args.inversion_period)
     lb = not args.no_load_balancing
     edges_per_pass = sampler.num_samples * sampler.final_sample_size
 
@@ -191,6 +195,20 @@ def main():
     sampler.set_profiling(False)
     final = sampler.final_samples()
     valid = int((final != sampler.invalid_vertex).sum())
+
+    # walks, for information only (not the headline): the same pass when the engine chooses how
+    # often to invert; the samples must come out the same
+    adaptive = None
+    if sampler.step_size(0) == 1 and sampler.steps > 1 and args.inversion_period == 1:
+        sampler.set_inversion_period(0)
+        sampler.do_transit_parallel(lb)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            sampler.do_transit_parallel(lb)
+        ms = (time.perf_counter() - t0) * 1000.0 / args.steps
+        same = bool(np.array_equal(sampler.final_samples(), final))
+        adaptive = {"ms_per_step": ms, "sampled_edges_per_s": edges_per_pass / (ms / 1000.0), "same_samples": same}
+        sampler.set_inversion_period(1)
     del final
 
     result = {
@@ -204,6 +222,9 @@ def main():
                    "graph_build_s": round(t_graph, 1), "gpu_event_ms_per_step": float(np.mean(gpu_ms))},
         "phases_ms": {k: round(v, 3) for k, v in prof.items()},
     }
+    result["config"]["inversion_period"] = args.inversion_period
+    if adaptive:
+        result["config"]["engine_chosen_inversion_period"] = adaptive
 
     if w["kind"] in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE"):
         entries, distinct = sampler.counter(0), sampler.counter(1)

@@ -195,6 +195,11 @@ class Sampler:
         check(lib().nd_sampler_get_sample_states(self._h, buf.ctypes.data_as(C.c_void_p), nbytes))
         return buf
 
+    def set_inversion_period(self, period):
+        """Walks: 1 inverts before every step (the reference's behaviour, default), p > 1
+        every p-th step, 0 lets the engine decide.  The samples do not depend on it."""
+        check(lib().nd_sampler_set_inversion_period(self._h, int(period)))
+
     def set_profiling(self, on):
         check(lib().nd_sampler_set_profiling(self._h, int(on)))
 

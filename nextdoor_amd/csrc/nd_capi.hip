@@ -253,6 +253,13 @@ int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes) {
   return rc == 0 ? 0 : fail(s->engine->last_error, rc);
 }
 
+int nd_sampler_set_inversion_period(nd_sampler* s, int period) {
+  if (!s) return fail("null sampler");
+  if (period < 0) return fail("the inversion period is 0 (engine decides) or positive");
+  s->engine->inversion_period = period;
+  return 0;
+}
+
 int nd_sampler_set_profiling(nd_sampler* s, int on) {
   if (!s) return fail("null sampler");
   s->engine->profiling = on != 0;

@@ -61,6 +61,12 @@ class EngineBase {
   virtual int set_graph(const CSR* graph) = 0;
   virtual int alloc(uint64_t seed) = 0;
   virtual int sample(int mode) = 0;
+  // Walks: how often the (sample -> transit) map is inverted.  1: before every step, as the
+  // reference does.  p > 1: before step 1 (which also drops the walks that cannot start) and
+  // then every p-th step; the steps between walk in the order of the last inversion, without
+  // load balancing.  0: the engine decides from the walks-per-vertex ratio.  Results do not
+  // depend on it.  Other apps always invert.
+  int inversion_period = 1;
   virtual int fetch_final_samples() = 0;
   virtual void free_device() = 0;
   virtual int64_t num_samples() const = 0;
@@ -206,6 +212,13 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
     P.emit_slots[pair] = pair_slot;
   }
 }
+
+// inversion_period == 0: walks are inverted before every step when there are at least this
+// many walks per vertex, else every kSparseInversionPeriod steps (measured on 4.2 M weighted
+// node2vec walks over 4.2 M vertices: 45.3 ms per 100 steps inverting every step, 38.0 every
+// 4th, 35.5 only once; the sorted order saves 3.4 ms in the step kernels and costs 13.7).
+constexpr double kWalksPerVertexForInversion = 4.0;
+constexpr int kSparseInversionPeriod = 32;
 
 // Lanes the flat kernel wants before it gives a lane all the outputs of a pair.
 constexpr uint64_t kFlatLanesWanted = 1ull << 20;
@@ -720,6 +733,13 @@ class Engine : public EngineBase {
     }
 
     uint32_t transits_per_sample = (uint32_t)init_size_;
+    const uint32_t* live_last = nullptr;  // pairs the last inversion kept (device count)
+    int sorts_done = 0;
+    // With few walks per vertex hardly any two walks share a transit: the sorted order then
+    // saves less in the step kernels (shared lines) than the inversion costs.
+    int sort_period = inversion_period;
+    if (sort_period <= 0)
+      sort_period = (double)n_samples_ < kWalksPerVertexForInversion * (double)invalid_ ? kSparseInversionPeriod : 1;
     const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
     KeyLayout transits_layout;             // and how it is laid out
     for (int step = 0; step < n_steps; ++step) {
@@ -754,14 +774,26 @@ class Engine : public EngineBase {
       P.emit_keys = emits ? d_emit_keys_ : nullptr;
       P.emit_slots = emits ? d_emit_slots_ : nullptr;
       P.emit_state = emits && state_travels_ ? d_emit_state_ : nullptr;
-      uint32_t* live_now = d_live_ + (step & 1);  // pairs the inversion of this step keeps
+      uint32_t* live_now = d_live_ + (sorts_done & 1);  // pairs the inversion of this step keeps
       // lanes of the flat kernel per pair: one when the pairs alone fill the machine, else
       // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
       P.lanes_shift = 0;
       while ((1u << P.lanes_shift) < m && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted) P.lanes_shift++;
       const unsigned flat_grid = flat_grid_for((uint64_t)n_pairs << P.lanes_shift);
 
-      if (step == 0) {
+      const bool skip_inversion = walk_mode_ && step > 0 && sort_period > 1 && (step - 1) % sort_period != 0;
+      if (skip_inversion) {
+        // walk in the order of the last inversion: the step kernel reads the pairs it
+        // emitted itself, in place
+        P.pair_keys = d_emit_keys_;
+        P.pair_slots = d_emit_slots_;
+        P.pair_state = state_travels_ ? d_emit_state_ : nullptr;
+        P.live_pairs = live_last;
+        tick();
+        launch_flat(P, flat_grid, nullptr);
+        tock(&times.flat_kernel);
+        times.flat_launches++;
+      } else if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
         // when there is more than one step, nextdoor.cu:2400 and the FIXME at 2372)
         P.pair_keys = (const uint32_t*)transits;
@@ -780,7 +812,7 @@ class Engine : public EngineBase {
           job.keys_in = d_emit_keys_;
           job.vals_in = d_emit_slots_;
           job.aux_in = state_travels_ ? d_emit_state_ : nullptr;
-          job.n_in_dev = step == 1 ? nullptr : d_live_ + ((step - 1) & 1);
+          job.n_in_dev = live_last;
         } else {
           job.keys_in = (const uint32_t*)transits;
           job.keys_in_layout = transits_layout;
@@ -804,6 +836,8 @@ class Engine : public EngineBase {
         P.pair_slots = job.vals_sorted;
         P.pair_state = state_travels_ ? job.aux_sorted : nullptr;
         P.live_pairs = live_now;
+        live_last = live_now;
+        sorts_done++;
         if (!balance) {
           tick();
           launch_flat(P, flat_grid, nullptr);

@@ -18,9 +18,10 @@ def desc_for(oracle, sampler, kind):
                            initial_size=sampler.initial_sample_size)
 
 
-def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)):
+def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True), inversion_period=1):
     og = graphs.oracle_view(g)
     s = nd.Sampler(app, g, seed=SEED)
+    s.set_inversion_period(inversion_period)
     try:
         d = desc_for(oracle, s, kind)
         roots = s.initial_contents
@@ -48,6 +49,21 @@ def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)
         return got
     finally:
         s.close()
+
+
+@pytest.mark.parametrize("period", [0, 3, 1000])
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("PPRPerVertex", "PPR", False),
+    ("Node2VecPerVertex", "NODE2VEC", True),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+    ("KHop", "KHOP", False),
+])
+def test_samples_do_not_depend_on_the_inversion_period(oracle, app, kind_name, state, period):
+    # walks that re-invert the sample -> transit map only now and then (or when the engine
+    # sees fit) give the bytes of the oracle too; for other apps the setting changes nothing
+    g = graphs.random_graph(n=1500, mean_degree=6, seed=9, hub=4, isolated_every=11)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, inversion_period=period)
 
 
 GRAPHS = {
