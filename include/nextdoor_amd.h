@@ -66,9 +66,10 @@ int nd_sampler_alloc(nd_sampler* s, uint64_t seed);
 /* doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006. */
 int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing);
 /* How often walks re-invert the (sample -> transit) map.  The reference inverts before every
- * step (src/nextdoor.cu:2924-2939), which is period 1 and the default.  period p > 1: before
- * step 1 and then every p-th step, the steps between walk in the order of the last inversion
- * (no load balancing there).  period 0: the engine decides from the walks-per-vertex ratio.
+ * step (src/nextdoor.cu:2924-2939), which is period 1 and the default.  period p > 1: the walks
+ * are not brought into transit order (no load balancing); before step 1 and then every p-th
+ * step the walks that have ended are dropped from the list, in between the list is walked as
+ * it stands.  period 0: the engine decides from the walks-per-vertex ratio.
  * The samples do not depend on the period.  Apps other than walks always invert. */
 int nd_sampler_set_inversion_period(nd_sampler* s, int period);
 /* getFinalSamples(data), src/nextdoor.cu:3211-3237: copies device -> host and returns the

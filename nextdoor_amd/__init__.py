@@ -196,8 +196,9 @@ class Sampler:
         return buf
 
     def set_inversion_period(self, period):
-        """Walks: 1 inverts before every step (the reference's behaviour, default), p > 1
-        every p-th step, 0 lets the engine decide.  The samples do not depend on it."""
+        """Walks: 1 inverts before every step (the reference's behaviour, default); p > 1 keeps
+        the walks out of transit order and only drops ended walks every p-th step; 0 lets the
+        engine decide.  The samples do not depend on it."""
         check(lib().nd_sampler_set_inversion_period(self._h, int(period)))
 
     def set_profiling(self, on):

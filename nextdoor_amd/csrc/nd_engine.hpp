@@ -62,10 +62,10 @@ class EngineBase {
   virtual int alloc(uint64_t seed) = 0;
   virtual int sample(int mode) = 0;
   // Walks: how often the (sample -> transit) map is inverted.  1: before every step, as the
-  // reference does.  p > 1: before step 1 (which also drops the walks that cannot start) and
-  // then every p-th step; the steps between walk in the order of the last inversion, without
-  // load balancing.  0: the engine decides from the walks-per-vertex ratio.  Results do not
-  // depend on it.  Other apps always invert.
+  // reference does.  p > 1: the walks are not brought into transit order at all; before step
+  // 1 and then every p-th step the walks that have ended are dropped from the list (a stable
+  // compaction in slot order), and there is no load balancing.  0: the engine decides from
+  // the walks-per-vertex ratio.  Results do not depend on it.  Other apps always invert.
   int inversion_period = 1;
   virtual int fetch_final_samples() = 0;
   virtual void free_device() = 0;
@@ -806,7 +806,11 @@ class Engine : public EngineBase {
         // inversion: sort (transit, slot) by transit.  Walks sort the pairs the previous
         // step emitted (only those still alive); other apps sort the previous step's
         // output array, whose index is the slot.
-        const SortPlan plan = make_sort_plan(n_pairs, max_bits_);
+        // Walks that invert only now and then gain nothing from the transit order (few of them
+        // share a transit, and the order is stale one step later): they only drop the walks
+        // that have ended, keeping slot order, in which the writes of a step's results coalesce.
+        const bool compact_only = walk_mode_ && sort_period > 1;
+        const SortPlan plan = make_sort_plan(n_pairs, compact_only ? 0 : max_bits_);
         SortJob job;
         if (walk_mode_) {
           job.keys_in = d_emit_keys_;
@@ -838,7 +842,7 @@ class Engine : public EngineBase {
         P.live_pairs = live_now;
         live_last = live_now;
         sorts_done++;
-        if (!balance) {
+        if (!balance || compact_only) {
           tick();
           launch_flat(P, flat_grid, nullptr);
           tock(&times.flat_kernel);

@@ -238,8 +238,10 @@ struct SortPlan {
 inline SortPlan make_sort_plan(size_t n, int key_bits) {
   SortPlan p;
   p.n = n;
-  p.key_bits = key_bits < 1 ? 1 : key_bits;
-  p.passes = (p.key_bits + kRadixBits - 1) / kRadixBits;
+  // key_bits == 0: one pass in which every key has digit 0, i.e. a stable compaction of the
+  // pairs the sort keeps (see SortJob::drop_key)
+  p.key_bits = key_bits < 0 ? 0 : key_bits;
+  p.passes = p.key_bits == 0 ? 1 : (p.key_bits + kRadixBits - 1) / kRadixBits;
   p.items = n >= kSortLargeFrom ? kSortItemsLarge : kSortItemsSmall;
   const size_t tile = (size_t)kSortThreads * p.items;
   p.num_tiles = (uint32_t)((n + tile - 1) / tile);
