@@ -289,6 +289,69 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
   }
 }
 
+// Walks that are not re-inverted for a while: one lane keeps its walk for a whole stretch of
+// steps, with the current vertex and the sample state in registers.  Besides saving the
+// reads and writes of the pair list between steps, this evens out the rejection loops: a
+// wavefront waits for the SUM of its lanes' rounds over the stretch, not for the slowest
+// lane of every single step.  Step k of the stretch writes step_out[k * out_stride + slot].
+template <class SampleType, class App>
+__global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P, int stretch_steps, int last_step,
+                                                                    size_t out_stride) {
+  const uint32_t total = P.live_pairs ? *P.live_pairs : P.n_pairs;
+  const uint32_t i = blockIdx.x * kFlatThreads + threadIdx.x;
+  if (i >= total) return;
+  CSRPartition csr = P.csr;
+  VertexID transit = (VertexID)P.pair_keys[i];
+  const uint32_t slot = P.pair_slots ? P.pair_slots[i] : i;  // == the sample: one transit per sample
+  constexpr bool kTravels = state_fits_pair<SampleType>::value;
+  SampleType local_state;
+  SampleType* state = &local_state;
+  if (kTravels) {
+    const uint32_t bits = P.pair_state ? P.pair_state[i] : ((const uint32_t*)P.samples)[slot];
+    __builtin_memcpy(&local_state, &bits, sizeof(uint32_t));
+  } else if (!std::is_empty<SampleType>::value) {
+    state = (SampleType*)P.samples + slot;
+  }
+  int step = P.step;
+  for (int k = 0; k < stretch_steps && transit != P.invalid; ++k, ++step) {
+    const EdgePos_t begin = csr.row_ptr[transit];
+    const EdgePos_t n_edges = csr.row_ptr[transit + 1] - begin;
+    VertexID neighbor = P.invalid;
+    if (n_edges != 0) {  // next() only runs for a transit that has edges (nextdoor.cu:250-262)
+      const float max_weight = csr.max_weights[transit];
+      curandState rng;
+      rng.reset(P.seed, P.first_slot + slot, (uint32_t)step);
+      VertexID r;
+      if (app_uses_weights<App>::value) {
+        PairedEdgeIds edges{P.paired_edges + begin};
+        PairedEdgeWeights weights{P.paired_edges + begin};
+        r = App().template next<SampleType, PairedEdgeIds, PairedEdgeWeights>(
+            step, &csr, &transit, (VertexID)(P.first_sample + slot), state, max_weight, edges, weights, n_edges, 0, &rng);
+      } else {
+        const CSR::Edge* edges = csr.edges + begin;
+        const float* weights = csr.weights + begin;
+        r = App().template next<SampleType, const CSR::Edge*, const float*>(
+            step, &csr, &transit, (VertexID)(P.first_sample + slot), state, max_weight, edges, weights, n_edges, 0, &rng);
+      }
+      neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
+    }
+    P.step_out[(size_t)k * out_stride + slot] = neighbor;
+    transit = neighbor;
+  }
+  // the walk as it stands after the stretch (INVALID: it has ended and the next compaction drops it)
+  const bool pass_over = step > last_step;
+  if (P.emit_keys && !pass_over) {
+    P.emit_keys[i] = (uint32_t)transit;
+    P.emit_slots[i] = slot;
+  }
+  if (kTravels) {
+    uint32_t bits;
+    __builtin_memcpy(&bits, &local_state, sizeof(uint32_t));
+    if (P.emit_state && !pass_over) P.emit_state[i] = bits;
+    if (pass_over || transit == P.invalid) ((uint32_t*)P.samples)[slot] = bits;  // the state goes home
+  }
+}
+
 // One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
 // transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
 // with coalesced reads and every draw of the stretch gathers from LDS.
@@ -781,19 +844,7 @@ class Engine : public EngineBase {
       while ((1u << P.lanes_shift) < m && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted) P.lanes_shift++;
       const unsigned flat_grid = flat_grid_for((uint64_t)n_pairs << P.lanes_shift);
 
-      const bool skip_inversion = walk_mode_ && step > 0 && sort_period > 1 && (step - 1) % sort_period != 0;
-      if (skip_inversion) {
-        // walk in the order of the last inversion: the step kernel reads the pairs it
-        // emitted itself, in place
-        P.pair_keys = d_emit_keys_;
-        P.pair_slots = d_emit_slots_;
-        P.pair_state = state_travels_ ? d_emit_state_ : nullptr;
-        P.live_pairs = live_last;
-        tick();
-        launch_flat(P, flat_grid, nullptr);
-        tock(&times.flat_kernel);
-        times.flat_launches++;
-      } else if (step == 0) {
+      if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
         // when there is more than one step, nextdoor.cu:2400 and the FIXME at 2372)
         P.pair_keys = (const uint32_t*)transits;
@@ -842,7 +893,19 @@ class Engine : public EngineBase {
         P.live_pairs = live_now;
         live_last = live_now;
         sorts_done++;
-        if (!balance || compact_only) {
+        if (compact_only) {
+          // the walks keep their lanes until the next compaction
+          const int stretch = n_steps - step < sort_period ? n_steps - step : sort_period;
+          P.emit_keys = d_emit_keys_;
+          P.emit_slots = d_emit_slots_;
+          P.emit_state = state_travels_ ? d_emit_state_ : nullptr;
+          tick();
+          walk_stretch_kernel<SampleType, App><<<dim3((n_pairs + kFlatThreads - 1) / kFlatThreads), dim3(kFlatThreads), 0,
+                                                 stream_>>>(P, stretch, n_steps - 1, (size_t)n_samples_);
+          tock(&times.flat_kernel);
+          times.flat_launches++;
+          step += stretch - 1;
+        } else if (!balance) {
           tick();
           launch_flat(P, flat_grid, nullptr);
           tock(&times.flat_kernel);
