@@ -74,16 +74,20 @@ inline bool allocNextDoorDataOnGPU(CSR* csr, NextDoorData& data) {
   return true;
 }
 
-// doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006.
+// doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006: the
+// sample -> transit map is inverted before every step.
 inline bool doTransitParallelSampling(CSR*, NextDoorData& data, bool enableLoadBalancing) {
-  return data.sampler && nd_sampler_do_transit_parallel(data.sampler, enableLoadBalancing ? 1 : 0) == 0;
+  return data.sampler && nd_sampler_set_inversion_period(data.sampler, 1) == 0 &&
+         nd_sampler_do_transit_parallel(data.sampler, enableLoadBalancing ? 1 : 0) == 0;
 }
 
 // doSampleParallelSampling(csr, data), src/nextdoor.cu:3009-3209: the reference's baseline
-// mode.  Results do not depend on the mode here (randomness is keyed by output slot), so
-// this runs the same engine without load balancing.
-inline bool doSampleParallelSampling(CSR* csr, NextDoorData& data) {
-  return doTransitParallelSampling(csr, data, false);
+// mode, every sample on its own lane.  For walks the engine then never brings the samples
+// into transit order (it only drops ended walks now and then); other apps have no such mode
+// here and run as above without load balancing.  The samples are the same bytes either way.
+inline bool doSampleParallelSampling(CSR*, NextDoorData& data) {
+  return data.sampler && nd_sampler_set_inversion_period(data.sampler, 32) == 0 &&
+         nd_sampler_do_transit_parallel(data.sampler, 0) == 0;
 }
 
 // getFinalSamples(data), src/nextdoor.cu:3211-3237.

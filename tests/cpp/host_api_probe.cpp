@@ -31,5 +31,19 @@ int main(int argc, char** argv) {
                              return final_size == 8 && n_values == data.initialContents.size() * 8;
                            });
   printf("final_size %d values %zu\n", final_size, n_values);
-  return ok ? 0 : 7;
+  if (!ok) return 7;
+  // the reference's other kernel type gives the same samples
+  std::vector<VertexID_t> transit_parallel, sample_parallel;
+  for (int mode = 0; mode < 2; ++mode) {
+    CSR* g = loadGraph(graph_file, "edge-list", "text");
+    NextDoorData data("UniformRandomWalk8");
+    if (!g || !allocNextDoorDataOnGPU(g, data)) return 8;
+    if (!(mode == 0 ? doTransitParallelSampling(g, data, true) : doSampleParallelSampling(g, data))) return 9;
+    (mode == 0 ? transit_parallel : sample_parallel) = getFinalSamples(data);
+    freeDeviceData(data);
+    nd_graph_free(g);
+  }
+  if (transit_parallel.empty() || transit_parallel != sample_parallel) return 10;
+  printf("kernel types agree\n");
+  return 0;
 }

@@ -45,3 +45,4 @@ def test_nextdoor_entry_runs_on_the_gpu(tmp_path):
     assert out.returncode == 0, out.stdout + out.stderr
     assert "totalSampledVertices 96" in out.stdout  # 12 walks x 8 steps, no dead ends
     assert "final_size 8 values 96" in out.stdout
+    assert "kernel types agree" in out.stdout
