@@ -47,3 +47,6 @@ struct KHopAppT {
 };
 
 typedef KHopAppT<25, 10> KHopApp;
+// src/apps/layer/layerSampling.cu:1-81: the same sampler with fan-outs 10 and 25
+class LayerSample {};
+typedef KHopAppT<10, 25> LayerSamplingApp;

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "nd_apps_khop.hpp"
+#include "nd_apps_multirw.hpp"
 #include "nd_apps_layer.hpp"
 #include "nd_apps_walks.hpp"
 #include "nd_engine.hpp"
@@ -66,6 +67,11 @@ const AppEntry kApps[] = {
     {"KHop4x3x2", make_engine<KHopSample, KHopAppT<4, 3, 2>>},
     {"KHop40x30", make_engine<KHopSample, KHopAppT<40, 30>>},
     {"KHop10x10", make_engine<KHopSample, KHopAppT<10, 10>>},
+    // the reference's LayerSamplingApp (src/apps/layer/layerSampling.cu: k-hop with fan-outs 10, 25)
+    // and its multi-dimensional random walk (explicit transits), with a short variant
+    {"Layer", make_engine<LayerSample, LayerSamplingApp>},
+    {"MultiRW", make_engine<MultiRWSample, MultiRWApp>},
+    {"MultiRW4x6", make_engine<MultiRWSampleT<4>, MultiRWAppT<4, 6>>},
     // layer-wise apps: the reference's FastGCN / LADIES (5 layers of 64, 10000 samples) ...
     {"FastGCN", make_layer_engine<FastGCNSample, FastGCNSamplingApp>},
     {"LADIES", make_layer_engine<ImportanceSample, ImportanceSampleApp>},

@@ -169,6 +169,34 @@ constexpr uint32_t kWorkgroupWork = 256;
 // over several workgroups (the grid-wide case).
 constexpr uint32_t kChunkOutputs = ND_CHUNK_OUTPUTS;
 
+// next() for one output and, for apps with explicit transits, stepTransits() for the step
+// after it (nextdoor.cu:279-289: the random state is the one next() used).  Returns the
+// sampled vertex; *next_transit is the transit the pair has at the next step.
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t sample,
+                                            uint32_t transit_index, uint64_t out_slot, uint32_t nbr,
+                                            EdgePos_t n_edges, float max_weight, EdgeArray& edges,
+                                            WeightArray& weights, SampleType* state, VertexID* next_transit) {
+  const VertexID sample_id = (VertexID)(P.first_sample + sample);
+  const bool runs = transit != P.invalid && n_edges != 0;  // next() only runs for a real transit
+                                                           // that has edges (nextdoor.cu:250-262)
+  const bool explicit_transits = App().hasExplicitTransits();
+  curandState rng;
+  if (runs || explicit_transits) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  VertexID neighbor = P.invalid;
+  if (runs) {
+    const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
+        P.step, &csr, &transit, sample_id, state, max_weight, edges, weights, n_edges, (VertexID_t)nbr, &rng);
+    neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
+  }
+  *next_transit = neighbor;
+  if (explicit_transits && !P.is_last) {
+    const VertexID_t t = App().stepTransits(P.step + 1, sample_id, *state, (int)transit_index, &rng);
+    *next_transit = t == -1 ? P.invalid : t;
+  }
+  return neighbor;
+}
+
 // pair: index of the pair in the order the step kernels walk them (sorted by transit, or
 // the raw map at step 0).
 template <class SampleType, class App, class EdgeArray, class WeightArray>
@@ -177,38 +205,31 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
                                                EdgeArray& edges, WeightArray& weights) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
-  VertexID neighbor = P.invalid;
-  const bool runs = transit != P.invalid && n_edges != 0;  // next() only runs for a real transit
-                                                           // that has edges (nextdoor.cu:250-262)
-  curandState rng;
-  if (runs) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  const uint32_t transit_index = pair_slot - sample * P.transits_per_sample;
+  VertexID neighbor, next_transit;
   if (state_fits_pair<SampleType>::value && P.state_travels) {
-    // the state travels with the pair
+    // the state travels with the pair: a register copy
     SampleType state;
     uint32_t bits = P.pair_state ? P.pair_state[pair] : ((const uint32_t*)P.samples)[sample];
     __builtin_memcpy(&state, &bits, sizeof(uint32_t));
-    if (runs) {
-      const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
-          P.step, &csr, &transit, (VertexID)(P.first_sample + sample), &state, max_weight, edges, weights, n_edges,
-          (VertexID_t)nbr, &rng);
-      neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
-    }
+    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                        edges, weights, &state, &next_transit);
     __builtin_memcpy(&bits, &state, sizeof(uint32_t));
     if (P.emit_state) P.emit_state[pair] = bits;
     // a walk that ends here leaves the stream of pairs: its state goes home
-    if (P.is_last || neighbor == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
-  } else if (runs) {
-    SampleType local_state;
-    SampleType* state = std::is_empty<SampleType>::value ? &local_state : (SampleType*)P.samples + sample;
-    const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
-        P.step, &csr, &transit, (VertexID)(P.first_sample + sample), state, max_weight, edges, weights, n_edges,
-        (VertexID_t)nbr, &rng);
-    neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
+    if (P.is_last || next_transit == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
+  } else if (std::is_empty<SampleType>::value) {
+    SampleType no_state;
+    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                        edges, weights, &no_state, &next_transit);
+  } else {
+    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                        edges, weights, (SampleType*)P.samples + sample, &next_transit);
   }
   const uint32_t per_sample = P.transits_per_sample * P.step_size;
   P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
   if (P.emit_keys) {
-    P.emit_keys[pair] = (uint32_t)neighbor;
+    P.emit_keys[pair] = (uint32_t)next_transit;
     P.emit_slots[pair] = pair_slot;
   }
 }
@@ -312,14 +333,15 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
   } else if (!std::is_empty<SampleType>::value) {
     state = (SampleType*)P.samples + slot;
   }
+  const bool explicit_transits = App().hasExplicitTransits();
   int step = P.step;
   for (int k = 0; k < stretch_steps && transit != P.invalid; ++k, ++step) {
     const EdgePos_t begin = csr.row_ptr[transit];
     const EdgePos_t n_edges = csr.row_ptr[transit + 1] - begin;
     VertexID neighbor = P.invalid;
+    curandState rng;
     if (n_edges != 0) {  // next() only runs for a transit that has edges (nextdoor.cu:250-262)
       const float max_weight = csr.max_weights[transit];
-      curandState rng;
       rng.reset(P.seed, P.first_slot + slot, (uint32_t)step);
       VertexID r;
       if (app_uses_weights<App>::value) {
@@ -337,6 +359,11 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
     }
     P.step_out[(size_t)k * out_stride + slot] = neighbor;
     transit = neighbor;
+    if (explicit_transits && step != last_step) {
+      if (n_edges == 0) rng.reset(P.seed, P.first_slot + slot, (uint32_t)step);
+      const VertexID_t t = App().stepTransits(step + 1, (VertexID)(P.first_sample + slot), *state, 0, &rng);
+      transit = t == -1 ? P.invalid : t;
+    }
   }
   // the walk as it stands after the stretch (INVALID: it has ended and the next compaction drops it)
   const bool pass_over = step > last_step;
@@ -652,7 +679,6 @@ class Engine : public EngineBase {
     seed_ = seed;
     CSR* csr = const_cast<CSR*>(graph_);
     App app;
-    if (app.hasExplicitTransits()) { last_error = "apps with explicit transits are not supported"; return -2; }
     if (is_collective<App>()) { last_error = "collective apps need the layer engine"; return -2; }
     const int n_steps = app.steps();
     if (n_steps < 1 || n_steps > kMaxSteps) { last_error = "steps() must be in [1, 128]"; return -2; }
@@ -740,6 +766,10 @@ class Engine : public EngineBase {
     walk_mode_ = init_size_ == 1 && n_steps > 1;
     for (int k = 0; k < n_steps; ++k) walk_mode_ = walk_mode_ && app.stepSize(k) == 1;
     state_travels_ = walk_mode_ && state_fits_pair<SampleType>::value;
+    if (app.hasExplicitTransits() && !walk_mode_) {
+      last_error = "explicit transits are supported for walks (one transit per sample, stepSize 1)";
+      return -2;
+    }
     if (walk_mode_) {
       ND_HIP_TRY(hipMalloc(&d_emit_keys_, sizeof(uint32_t) * max_pairs_));
       ND_HIP_TRY(hipMalloc(&d_emit_slots_, sizeof(uint32_t) * max_pairs_));

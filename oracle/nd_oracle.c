@@ -317,6 +317,52 @@ int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t 
 }
 
 /* ------------------------------------------------------------------------- */
+/* Multi-dimensional random walk                                              */
+/* ------------------------------------------------------------------------- */
+
+/* start vertex of walker root_index of a sample: a fixed Philox stream ("MRWR") */
+int32_t ndo_multirw_root(int64_t sample, int root_index, int32_t n_vertices) {
+  const float u = ndo_uniform(0x4D525752ull, (uint64_t)sample, 0x524F4F54u, (uint32_t)root_index);
+  return ndo_rand_int(u, n_vertices);
+}
+
+int ndo_sample_multirw(const ndo_graph* g, uint64_t seed, int64_t n_samples, int64_t first_sample, int n_roots,
+                       int steps, int32_t* roots, int32_t* last_root_idx, int32_t* final_samples,
+                       int32_t* transits_out) {
+  if (steps <= 0 || steps > NDO_MAX_STEPS || n_roots <= 0) return -1;
+  const int32_t invalid = g->n_vertices;
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int32_t* walkers = roots + s * n_roots;
+    int32_t last_idx = 0;
+    int32_t transit = walkers[0];  /* multiRW.cu:68-73: the initial sample is walker 0 */
+    for (int k = 0; k < steps; ++k) {
+      if (transits_out) transits_out[s * steps + k] = transit;
+      rng_cursor rc;
+      rc.seed = seed;
+      rc.slot = (uint64_t)(first_sample + s);
+      rc.step = (uint32_t)k;
+      rc.draw = 0;
+      rc.st = 0;
+      int32_t neighbor = invalid;
+      if (transit != invalid && degree_of(g, transit) != 0) {
+        const int32_t n = degree_of(g, transit);
+        const int32_t* edges = g->col + g->row_ptr[transit];
+        int32_t v = n == 1 ? edges[0] : edges[next_int(&rc, n)];  /* multiRW.cu:31-43 */
+        if (k > 0) walkers[last_idx] = v;                          /* multiRW.cu:34-36, 45-47 */
+        neighbor = v;
+      }
+      final_samples[s * steps + k] = neighbor;
+      if (k != steps - 1) {                                        /* nextdoor.cu:282-286 */
+        last_idx = next_int(&rc, n_roots);                         /* multiRW.cu:88-91 */
+        transit = walkers[last_idx];
+      }
+    }
+    if (last_root_idx) last_root_idx[s] = last_idx;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
 /* Inversion / RLE / scan / binning                                           */
 /* ------------------------------------------------------------------------- */
 

@@ -106,6 +106,26 @@ int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t 
                           const int32_t* initial, int32_t* final_samples,
                           int32_t* state_t, ndo_stats* stats, int n_threads);
 
+/* ---- multi-dimensional random walk (src/apps/multiRW/multiRW.cu:13-106) ----
+ * A sample owns n_roots walkers.  Step k: the transit is one of the walkers (step 0: walker
+ * 0); next() moves it to a uniformly drawn neighbour v, which is the step's output, and for
+ * k > 0 stores v in the walker's place (multiRW.cu:27-49; a walker without edges yields
+ * INVALID and stays).  Then, unless k is the last step, stepTransits(k + 1) draws the walker
+ * of the next step uniformly (multiRW.cu:84-92) from the SAME random state next() used, as
+ * the reference's step kernel does (nextdoor.cu:279-289): the draw after next()'s, i.e. draw
+ * 1 if next() drew (degree > 1), else draw 0, of the stream of output slot
+ * (first_sample + s) at step k.
+ * Walker start vertices: ndo_multirw_root.  The reference fills them with rand()
+ * (multiRW.cu:95-106); here they are Philox draws, so they are reproducible.
+ * roots[n_samples * n_roots] in/out (the walkers after the last step), last_root_idx[n_samples]
+ * out (0 if never drawn).  Pinned by a hand trace on a small graph and by the invariant that
+ * every output is adjacent to the walker that was the transit (tests); the sampled values
+ * themselves are parity unpinned by the reference, whose random numbers differ. */
+int32_t ndo_multirw_root(int64_t sample, int root_index, int32_t n_vertices);
+int ndo_sample_multirw(const ndo_graph* g, uint64_t seed, int64_t n_samples, int64_t first_sample, int n_roots,
+                       int steps, int32_t* roots, int32_t* last_root_idx, int32_t* final_samples,
+                       int32_t* transits_out);
+
 /* ---- inversion, run-length encode, scan, binning (nextdoor.cu:2924-2939, 2529-2572,
  *      1520-1802; utils.hpp:491-497) ---- */
 

@@ -269,3 +269,30 @@ def sample_ladies_importance(graph, desc, seed, initial, first_sample=0, n_threa
     assert rc == 0
     final = final.reshape(n, F)
     return (final, stats.as_dict()) if want_stats else final
+
+
+def multirw_roots(n_samples, n_roots, n_vertices, first_sample=0):
+    """Start vertices of every sample's walkers (ndo_multirw_root)."""
+    L = lib()
+    L.ndo_multirw_root.restype = C.c_int32
+    L.ndo_multirw_root.argtypes = [C.c_int64, C.c_int, C.c_int32]
+    return np.array([[L.ndo_multirw_root(first_sample + s, i, n_vertices) for i in range(n_roots)]
+                     for s in range(n_samples)], dtype=np.int32)
+
+
+def sample_multirw(graph, seed, roots, steps, first_sample=0):
+    """Returns (final [n, steps], walkers after the last step [n, n_roots], lastRootIdx [n],
+    transit of every step [n, steps])."""
+    L = lib()
+    L.ndo_sample_multirw.restype = C.c_int
+    L.ndo_sample_multirw.argtypes = [C.POINTER(GraphStruct), C.c_uint64, C.c_int64, C.c_int64, C.c_int, C.c_int,
+                                     i32p, i32p, i32p, i32p]
+    walkers = np.ascontiguousarray(roots, dtype=np.int32).copy()
+    n, n_roots = walkers.shape
+    final = np.empty((n, steps), np.int32)
+    last = np.empty(n, np.int32)
+    transits = np.empty((n, steps), np.int32)
+    rc = L.ndo_sample_multirw(C.byref(graph.struct), seed, n, first_sample, n_roots, steps, _p(walkers, C.c_int32),
+                              _p(last, C.c_int32), _p(final, C.c_int32), _p(transits, C.c_int32))
+    assert rc == 0
+    return final, walkers, last, transits

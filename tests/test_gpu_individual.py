@@ -155,3 +155,35 @@ def test_distinct_matches_oracle(oracle, app, gname):
     for row_raw, row in zip(raw[:50], got[:50]):
         assert set(row_raw[row_raw != s.invalid_vertex]) == set(row[row != s.invalid_vertex])
     s.close()
+
+
+@pytest.mark.parametrize("period", [1, 0, 3])
+@pytest.mark.parametrize("app,n_roots,steps", [("MultiRW4x6", 4, 6), ("MultiRW", 100, 100)])
+def test_multirw_matches_oracle(oracle, app, n_roots, steps, period):
+    # the app with explicit transits (src/apps/multiRW/multiRW.cu): stepTransits picks the
+    # walker of the next step; samples AND the walkers left in the sample state must agree
+    g = graphs.random_graph(n=700, mean_degree=4, seed=13, hub=2, isolated_every=9)
+    og = graphs.oracle_view(g)
+    s = nd.Sampler(app, g, seed=SEED)
+    try:
+        s.set_inversion_period(period)
+        assert (s.steps, s.final_sample_size, s.num_samples) == (steps, steps, g.n_vertices)
+        roots = oracle.multirw_roots(s.num_samples, n_roots, g.n_vertices)
+        assert np.array_equal(s.initial_contents, roots[:, 0])
+        want, want_walkers, want_last, _ = oracle.sample_multirw(og, SEED, roots, steps)
+        for lb in (False, True):
+            print("app", app, "period", period, "lb", lb, flush=True)
+            s.do_transit_parallel(load_balancing=lb)
+            assert np.array_equal(s.final_samples(), want)
+            state = s.sample_states().view(np.int32).reshape(s.num_samples, n_roots + 1)
+            assert np.array_equal(state[:, :n_roots], want_walkers)
+            assert np.array_equal(state[:, n_roots], want_last)
+    finally:
+        s.close()
+
+
+def test_layer_sampling_app_is_khop_10_25(oracle):
+    # src/apps/layer/layerSampling.cu: two hops with fan-outs 10 and 25
+    g = graphs.random_graph(n=400, mean_degree=5, seed=21)
+    got = run_and_compare(oracle, "Layer", oracle.KHOP, g)
+    assert got.shape == (400, 10 + 250)
