@@ -8,7 +8,7 @@
 //   freeDeviceData             src/nextdoor.cu:2088-2115   -> Engine::free_device
 //   samplingKernel / identityKernel / gridKernel  212-336 / 338-504 / 976-1204
 //                                                      -> step_flat_kernel / step_workgroup_kernel
-//   partitionTransitsInKernels 1520-1802               -> mark_run_heads / classify_run_tails
+//   partitionTransitsInKernels 1520-1802               -> classify_run_tails
 //
 // Differences that are deliberate:
 //  * The (sample -> transit) map stores only the transit; the map index IS the slot
@@ -421,13 +421,12 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
   }
 }
 
-// Load balancing without a scan: the pairs are sorted by transit, so the first pair of a
-// run knows where the run starts (the exclusive scan of the run lengths IS that position)
-// and the last pair of a run knows where it ends.  mark_run_heads records the start per
-// transit vertex; classify_run_tails, one lane per pair, lets the last pair of each run
-// decide which kernel class serves the transit and emit work items.  Two launches where the
-// reference has a boundary search, a run-length encode, a scan, a partition kernel and
-// three blocking copies (src/nextdoor.cu:2498-2636).
+// Load balancing without a scan or a run-length encode: the pairs are sorted by transit, so
+// the last pair of a run finds the run's start by looking back.  Only runs long enough for
+// the workgroup kernel matter, so the tail first looks one threshold back (a single read
+// that rules out nearly every run) and only then gallops to the start.  One launch,
+// classify_run_tails, where the reference has a boundary search, a run-length encode, a
+// scan, a partition kernel and three blocking copies (src/nextdoor.cu:2498-2636).
 //
 // Classes by neighbour-work (outputs drawn from the transit = count * stepSize):
 //   work <  kWorkgroupWork                      -> flat kernel (sub-wavefront: the lanes of a
@@ -436,20 +435,22 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
 //   work >  kChunkOutputs, several work items   -> grid-wide: the transit is split over workgroups
 // A transit whose adjacency does not fit the LDS cache, or is much longer than the number
 // of draws taken from it, is cheaper to gather directly and stays with the flat kernel.
-__global__ __launch_bounds__(256) void mark_run_heads(const uint32_t* __restrict__ keys,
-                                                      const uint32_t* __restrict__ n_dev,
-                                                      uint32_t* __restrict__ start_of, RunsMeta* meta) {
-  const uint32_t n = *n_dev;
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i == 0) {
-    meta->n_valid = n;
-    meta->n_runs = 0;
-    meta->n_chunks = 0;
-    meta->n_big_pairs = 0;
+
+// First index of the run of `transit` that ends at i (keys sorted, keys[i] == transit).
+__device__ __forceinline__ uint32_t run_start(const uint32_t* __restrict__ keys, uint32_t i, uint32_t transit) {
+  // gallop back while the key still matches ...
+  uint32_t hi = i, step = 1;
+  while (hi >= step && keys[hi - step] == transit) {
+    hi -= step;
+    step <<= 1;
   }
-  if (i >= n) return;
-  const uint32_t k = keys[i];
-  if (i == 0 || keys[i - 1] != k) start_of[k] = i;
+  // ... the start is in (hi - step, hi] (or [0, hi] when the gallop ran off the front)
+  uint32_t lo = hi >= step ? hi - step + 1 : 0;
+  while (lo < hi) {
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (keys[mid] == transit) hi = mid; else lo = mid + 1;
+  }
+  return lo;
 }
 
 constexpr uint32_t kDirectSegment = 16;  // ids: segments this long are written straight into the result rows
@@ -461,13 +462,15 @@ constexpr uint32_t kClassifyLargeFrom = 16u << 20;  // pairs
 // Is pair i the last of a run that the workgroup kernel should take?  Gives the run and the
 // number of work items it needs.
 __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict__ keys, uint32_t i, uint32_t n,
-                                                      const uint32_t* __restrict__ start_of,
                                                       const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                       uint32_t* transit_out, uint32_t* start_out, uint32_t* count_out,
                                                       uint32_t* n_items_out) {
   const uint32_t transit = keys[i];
   if (i + 1 != n && keys[i + 1] == transit) return false;  // not the last pair of its run
-  const uint32_t start = start_of[transit];
+  // pairs a run needs for the workgroup kernel; a shorter run is ruled out with one read
+  const uint32_t needed = (kWorkgroupWork + step_size - 1) / step_size;
+  if (i + 1 < needed || keys[i + 1 - needed] != transit) return false;
+  const uint32_t start = run_start(keys, i + 1 - needed, transit);
   const uint32_t count = i + 1 - start;
   const uint64_t work = (uint64_t)count * step_size;
   if (work < kWorkgroupWork) return false;
@@ -490,20 +493,23 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
 // the entries that did fit are processed twice with identical results.
 template <int kClassifyItems>
 __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __restrict__ keys,
-                                                          const uint32_t* __restrict__ n_dev,
-                                                          const uint32_t* __restrict__ start_of, RunsMeta* meta,
+                                                          const uint32_t* __restrict__ n_dev, RunsMeta* meta,
+                                                          RunsMeta* meta_of_next_step,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                           uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
                                                           uint8_t* __restrict__ skip_flag) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t s_base;
   const uint32_t n = *n_dev;
+  // the work-item counters alternate between steps: this launch clears the one the next
+  // step will count into (its last reader, the previous step's workgroup kernel, is done)
+  if (blockIdx.x == 0 && threadIdx.x == 0) meta_of_next_step->n_chunks = 0;
   const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
   uint32_t transit, start, count, n_items;
   uint32_t mine = 0;
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
-    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, start_of, row_ptr, step_size, &transit, &start, &count,
+    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count,
                                        &n_items))
       mine += n_items;
   }
@@ -530,7 +536,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
     // one pair per lane: the run found above is still in the registers
-    if (kClassifyItems > 1 && !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, start_of, row_ptr, step_size,
+    if (kClassifyItems > 1 && !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size,
                                                                &transit, &start, &count, &n_items)))
       continue;
     const bool fits = base + n_items <= chunk_capacity;
@@ -760,7 +766,6 @@ class Engine : public EngineBase {
     const SortPlan plan = make_sort_plan(max_pairs_, max_bits_);
     ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(max_pairs_)));
     ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * plan.scratch_elems));
-    ND_HIP_TRY(hipMalloc(&d_run_start_of_, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_live_, sizeof(uint32_t) * 2));
     // walks: every step has one pair per sample and one output per pair
     walk_mode_ = init_size_ == 1 && n_steps > 1;
@@ -779,8 +784,9 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_aux_a_, sizeof(uint32_t) * max_pairs_));
       ND_HIP_TRY(hipMalloc(&d_aux_b_, sizeof(uint32_t) * max_pairs_));
     }
-    ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta)));
-    ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta)));
+    ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta) * 2));
+    ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta) * 2));
+    balanced_steps_ = 0;
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
     ND_HIP_TRY(hipMalloc(&d_skip_flag_, (size_t)invalid_ + 1));
     ND_HIP_TRY(hipMemset(d_skip_flag_, 0, (size_t)invalid_ + 1));
@@ -943,15 +949,17 @@ class Engine : public EngineBase {
         } else {
           tick();
           const unsigned pair_blocks = (n_pairs + 255) / 256;
-          mark_run_heads<<<dim3(pair_blocks), dim3(256), 0, stream_>>>(sorted_keys, live_now, d_run_start_of_, d_meta_);
+          RunsMeta* meta = d_meta_ + (balanced_steps_ & 1);
+          RunsMeta* meta_next = d_meta_ + ((balanced_steps_ + 1) & 1);
+          balanced_steps_++;
           if (n_pairs >= kClassifyLargeFrom) {
             const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
             classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                sorted_keys, live_now, meta, meta_next, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
                 d_skip_flag_);
           } else {
             classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, d_run_start_of_, d_meta_, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                sorted_keys, live_now, meta, meta_next, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
                 d_skip_flag_);
           }
           tock(&times.load_balancing);
@@ -962,7 +970,7 @@ class Engine : public EngineBase {
           tick();
           unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
           step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
-              P, d_chunks_, d_meta_, chunk_capacity_, d_skip_flag_);
+              P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
           tock(&times.workgroup_kernel);
           times.workgroup_launches++;
         }
@@ -1101,7 +1109,6 @@ class Engine : public EngineBase {
     release(d_vals_b_);
     release(d_hist_);
     release(d_scratch_);
-    release(d_run_start_of_);
     release(d_live_);
     release(d_emit_keys_);
     release(d_emit_slots_);
@@ -1149,12 +1156,12 @@ class Engine : public EngineBase {
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
-  uint32_t* d_run_start_of_ = nullptr;  // per transit vertex: first position of its run in the sorted map
   uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
   bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false;
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
-  RunsMeta* d_meta_ = nullptr;
+  RunsMeta* d_meta_ = nullptr;          // two work-item counters, alternating between load-balanced steps
+  uint64_t balanced_steps_ = 0;        // ... counted over the life of the buffers, so the parity never repeats
   uint32_t* d_chunks_ = nullptr;
   uint8_t* d_skip_flag_ = nullptr;
   int32_t* d_distinct_counts_ = nullptr;
