@@ -560,6 +560,10 @@ __global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
 // ---------------------------------------------------------------------------------------
 
 constexpr int kMaxSteps = 128;
+#ifndef ND_ASSEMBLE_ROWS
+#define ND_ASSEMBLE_ROWS 64
+#endif
+constexpr uint32_t kAssembleRows = ND_ASSEMBLE_ROWS;  // rows a workgroup of the final assembly stages at most
 
 struct StepLayout {
   int n_steps;
@@ -605,6 +609,38 @@ __global__ __launch_bounds__(256) void assemble_final_rows(const int32_t* __rest
   for (uint32_t e = threadIdx.x; e < nb * final_size; e += 256) {
     const uint32_t s = e / final_size;
     dst[e] = s_rows[s * row_pitch + (e - s * final_size)];
+  }
+}
+
+// The same for walks (every step contributes one id per sample: step_out[k * n_samples + s]),
+// without the index arithmetic of the general case: a wavefront reads 64 consecutive samples
+// of one step, and the rows are written out with running (row, column) counters.
+__global__ __launch_bounds__(256) void assemble_walk_rows(const int32_t* __restrict__ step_out,
+                                                          int32_t* __restrict__ final_samples, uint32_t n_samples,
+                                                          uint32_t n_steps, uint32_t row_pitch,
+                                                          uint32_t samples_per_block) {
+  extern __shared__ int32_t s_rows[];
+  const uint32_t s0 = blockIdx.x * samples_per_block;
+  const uint32_t nb = n_samples - s0 < samples_per_block ? n_samples - s0 : samples_per_block;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  for (uint32_t first = 0; first < nb; first += 64u) {
+    const uint32_t s = first + lane;
+    if (s < nb)
+      for (uint32_t k = wave; k < n_steps; k += 4u) s_rows[s * row_pitch + k] = step_out[(size_t)k * n_samples + s0 + s];
+  }
+  __syncthreads();
+  int32_t* dst = final_samples + (size_t)s0 * n_steps;
+  const uint32_t total = nb * n_steps;
+  uint32_t row = threadIdx.x / n_steps, col = threadIdx.x - row * n_steps;
+  const uint32_t row_step = 256u / n_steps, col_step = 256u - row_step * n_steps;
+  for (uint32_t e = threadIdx.x; e < total; e += 256u) {
+    dst[e] = s_rows[row * row_pitch + col];
+    row += row_step;
+    col += col_step;
+    if (col >= n_steps) {
+      col -= n_steps;
+      row++;
+    }
   }
 }
 
@@ -798,9 +834,11 @@ class Engine : public EngineBase {
     // rows staged per workgroup by the final assembly: as many as fit 64 KiB of LDS
     row_pitch_ = (uint32_t)(F | 1);
     rows_per_block_ = (uint32_t)(65536 / (row_pitch_ * sizeof(int32_t)));
-    if (rows_per_block_ > 64) rows_per_block_ = 64;
+    if (rows_per_block_ > kAssembleRows) rows_per_block_ = kAssembleRows;
     if (rows_per_block_ > 0) {
       ND_HIP_TRY(hipFuncSetAttribute((const void*)assemble_final_rows, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     65536));
+      ND_HIP_TRY(hipFuncSetAttribute((const void*)assemble_walk_rows, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      65536));
     }
     allocated_ = true;
@@ -988,6 +1026,11 @@ class Engine : public EngineBase {
     tick();
     if (rows_direct_) {
       // the step kernels wrote the rows themselves
+    } else if (walk_mode_ && rows_per_block_ > 0) {
+      const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
+      const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
+      assemble_walk_rows<<<dim3(blocks), dim3(256), lds, stream_>>>(d_step_out_, d_final_, (uint32_t)n_samples_,
+                                                                    (uint32_t)n_steps, row_pitch_, rows_per_block_);
     } else if (rows_per_block_ > 0) {
       const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
