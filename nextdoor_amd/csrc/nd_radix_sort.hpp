@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   for (int w = 0; w < kSortWaves; ++w) s_wave_count[w][tid] = 0;
   __syncthreads();
 
-  uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
+  uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], aux[kAux ? kSortItems : 1];
   bool live[kSortItems];
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
@@ -156,6 +156,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
     live[it] = inside && key[it] != drop_key;
     if (kIotaValues) val[it] = (uint32_t)(tile_start + off);
     else val[it] = inside ? vals_in[tile_start + off] : 0u;
+    if (kAux) aux[it] = inside ? aux_in[tile_start + off] : 0u;  // fetched with the pair: no second round trip
   }
 
   const uint64_t lanes_below = (1ull << lane) - 1ull;
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
     __syncthreads();
 #pragma unroll
     for (int it = 0; it < kSortItems; ++it) {
-      if (live[it]) s_vals[rank[it]] = aux_in[tile_start + (uint32_t)tile_offset<kSortItems>(wave, it, lane)];
+      if (live[it]) s_vals[rank[it]] = aux[it];
     }
     __syncthreads();
     for (uint32_t p = tid; p < live_in_tile; p += kSortThreads) {
