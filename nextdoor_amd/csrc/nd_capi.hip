@@ -12,6 +12,7 @@
 #include "nd_apps_layer.hpp"
 #include "nd_apps_walks.hpp"
 #include "nd_engine.hpp"
+#include "nd_sharded_engine.hpp"
 #include "nd_layer_engine.hpp"
 #include "nd_graph.hpp"
 
@@ -40,7 +41,7 @@ struct AppEntry {
 
 template <class SampleType, class App>
 nd::EngineBase* make_engine(const char* name) {
-  return new nd::Engine<SampleType, App>(name);
+  return new nd::ShardedEngine<SampleType, App>(name);
 }
 
 template <class SampleType, class App>

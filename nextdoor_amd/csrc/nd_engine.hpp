@@ -28,7 +28,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <chrono>
+#include <memory>
 #include <string>
+#include <thread>
 #include <type_traits>
 #include <vector>
 
@@ -707,15 +710,29 @@ class Engine : public EngineBase {
   // structures the app asks for (interleaved edges, edge index).
   int set_graph(const CSR* graph) override {
     graph_ = nullptr;
-    if (!dgraph_.upload(graph, app_uses_weights<App>::value, app_uses_edge_lookup<App>::value, &last_error)) return -1;
+    dgraph_ = std::make_shared<DeviceGraph>();
+    if (!dgraph_->upload(graph, app_uses_weights<App>::value, app_uses_edge_lookup<App>::value, &last_error)) return -1;
     graph_ = graph;
-    view_ = dgraph_.view;
+    view_ = dgraph_->view;
     return 0;
   }
 
+  // The device graph another engine of the same app has uploaded (engines that each sample
+  // a range of the samples share one copy).
+  void share_graph(const Engine& other) {
+    dgraph_ = other.dgraph_;
+    graph_ = other.graph_;
+    view_ = other.view_;
+  }
+
+  int alloc(uint64_t seed) override { return alloc_range(seed, 0, -1); }
+
   // allocNextDoorDataOnGPU: run the host half of the App (numSamples, initializeSample,
   // initialSample) and allocate every per-run buffer once.
-  int alloc(uint64_t seed) override {
+  // Allocates for samples [first, first + count) of the app's samples (count < 0: all).
+  // Sample indices, roots and random streams are those of the whole run, so the ranges of
+  // several engines put together are the bytes one engine produces for everything.
+  int alloc_range(uint64_t seed, int64_t first, int64_t count) {
     if (!graph_) { last_error = "alloc before set_graph"; return -1; }
     free_run_buffers();
     seed_ = seed;
@@ -726,7 +743,13 @@ class Engine : public EngineBase {
     if (n_steps < 1 || n_steps > kMaxSteps) { last_error = "steps() must be in [1, 128]"; return -2; }
     for (int k = 0; k < n_steps; ++k)
       if (app.stepSize(k) <= 0) { last_error = "stepSize must be positive (ALL_NEIGHBORS is not supported)"; return -2; }
-    n_samples_ = app.numSamples(csr);
+    const int64_t all_samples = app.numSamples(csr);
+    if (first < 0 || first > all_samples || (count >= 0 && first + count > all_samples)) {
+      last_error = "sample range outside the app's samples";
+      return -2;
+    }
+    first_sample_ = first;
+    n_samples_ = count < 0 ? all_samples - first : count;
     init_size_ = app.initialSampleSize(csr);
     if (n_samples_ <= 0 || init_size_ <= 0) { last_error = "app yields no samples"; return -2; }
     invalid_ = graph_->get_n_vertices();  // nextdoor.cu:1993
@@ -738,8 +761,8 @@ class Engine : public EngineBase {
     samples_.reserve((size_t)n_samples_);
     initialContents.reserve((size_t)n_samples_ * init_size_);
     for (int64_t s = 0; s < n_samples_; ++s) {
-      samples_.push_back(app.template initializeSample<SampleType>(csr, (VertexID_t)s));
-      std::vector<VertexID_t> roots = app.initialSample((int)s, csr, samples_.back());
+      samples_.push_back(app.template initializeSample<SampleType>(csr, (VertexID_t)(first_sample_ + s)));
+      std::vector<VertexID_t> roots = app.initialSample((int)(first_sample_ + s), csr, samples_.back());
       if ((EdgePos_t)roots.size() != init_size_) {
         last_error = "initialSample size differs from initialSampleSize";  // nextdoor.cu:1964-1969
         return -2;
@@ -892,8 +915,8 @@ class Engine : public EngineBase {
       P.invalid = invalid_;
       P.is_last = step == n_steps - 1;
       P.seed = seed_;
-      P.first_slot = 0;
-      P.first_sample = 0;
+      P.first_slot = (uint64_t)first_sample_ * transits_per_sample * m;  // outputs of the samples before ours
+      P.first_sample = (uint32_t)first_sample_;
       P.n_pairs = n_pairs;
       P.live_pairs = nullptr;
       if (rows_direct_) {
@@ -904,7 +927,7 @@ class Engine : public EngineBase {
         P.out_pitch = layout_.seg_len[step];
       }
       P.samples = d_samples_;
-      P.paired_edges = dgraph_.paired;
+      P.paired_edges = dgraph_->paired;
       const bool emits = walk_mode_ && step + 1 < n_steps;
       P.state_travels = state_travels_;
       P.pair_state = nullptr;
@@ -993,11 +1016,11 @@ class Engine : public EngineBase {
           if (n_pairs >= kClassifyLargeFrom) {
             const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
             classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, meta, meta_next, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
                 d_skip_flag_);
           } else {
             classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, meta, meta_next, dgraph_.row_ptr(), m, d_chunks_, chunk_capacity_,
+                sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
                 d_skip_flag_);
           }
           tock(&times.load_balancing);
@@ -1053,12 +1076,16 @@ class Engine : public EngineBase {
   }
 
   // getFinalSamples: device -> hFinalSamples
-  int fetch_final_samples() override {
+  int fetch_final_samples() override { return fetch_final_samples_into(hFinalSamples.data()); }
+
+  int fetch_final_samples_into(VertexID_t* dst) {
     if (!allocated_) { last_error = "no device data"; return -1; }
-    ND_HIP_TRY(hipMemcpy(hFinalSamples.data(), d_final_, sizeof(VertexID_t) * hFinalSamples.size(),
+    ND_HIP_TRY(hipMemcpy(dst, d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * (size_t)final_sample_size(),
                          hipMemcpyDeviceToHost));
     return 0;
   }
+
+  bool is_walk() const { return walk_mode_; }
 
   int fetch_sample_states(void* dst, size_t bytes) override {
     if (!allocated_ || std::is_empty<SampleType>::value) { last_error = "no sample state"; return -1; }
@@ -1136,7 +1163,7 @@ class Engine : public EngineBase {
   }
 
   void free_graph() {
-    dgraph_.release();
+    dgraph_.reset();
     graph_ = nullptr;
   }
 
@@ -1175,7 +1202,8 @@ class Engine : public EngineBase {
   const char* name_;
   const CSR* graph_ = nullptr;
   CSRPartition view_{};
-  DeviceGraph dgraph_;
+  std::shared_ptr<DeviceGraph> dgraph_;
+  int64_t first_sample_ = 0;  // index of our first sample among the app's samples
 
   std::vector<SampleType> samples_;
   int64_t n_samples_ = 0;

@@ -187,3 +187,17 @@ def test_layer_sampling_app_is_khop_10_25(oracle):
     g = graphs.random_graph(n=400, mean_degree=5, seed=21)
     got = run_and_compare(oracle, "Layer", oracle.KHOP, g)
     assert got.shape == (400, 10 + 250)
+
+
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("PPRPerVertex", "PPR", False),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+])
+def test_two_sample_ranges_give_the_bytes_of_one(oracle, app, kind_name, state, monkeypatch):
+    # large walks are sampled as two ranges of samples on two streams; forced here on a small
+    # graph (odd sample count: ranges of different length)
+    monkeypatch.setenv("ND_SAMPLE_RANGES", "2")
+    g = graphs.random_graph(n=1501, mean_degree=6, seed=17, hub=4, isolated_every=11)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, inversion_period=0)
