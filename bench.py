@@ -28,16 +28,16 @@ HBM_PEAK_GBS = 8000.0
 # this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
 # known size).  None where no such run has been recorded.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 1.245e9,     # step_flat_kernel
-    "uniform_walk_chunglu57k": 4.27e6,       # step_flat_kernel
-    "khop_rmat21": 1.94e9,                   # step kernels of one hop (2 x flat 0.688e9 + workgroup 2.495e9, over 2 hops)
-    "fastgcn_importance_rmat22": 8.101e10,   # collective_mark, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 5.242e10,  # collective_mark, average over its 12 launches per pass
+    "weighted_node2vec_rmat22": 1.246e9,     # step_flat_kernel
+    "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
+    "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
+    "fastgcn_importance_rmat22": 8.104e10,   # collective_mark, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 5.241e10,  # collective_mark, average over its 12 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
-    "weighted_node2vec_rmat22": 165.4e9, "uniform_walk_chunglu57k": 0.98e9, "khop_rmat21": 14.8e9,
-    "fastgcn_importance_rmat22": 270.2e9, "ladies_importance_chunglu3m": 2128.9e9,
+    "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
+    "fastgcn_importance_rmat22": 270.6e9, "ladies_importance_chunglu3m": 2128.7e9,
 }
 
 WORKLOADS = {
@@ -162,6 +162,8 @@ def main():
     ap.add_argument("--inversion-period", type=int, default=1,
                     help="walks: invert the sample->transit map before every p-th step (1: every step, as the "
                          "reference; 0: the engine decides); the samples do not depend on it")
+    ap.add_argument("--skip-engine-choice", action="store_true",
+                    help="walks: do not also measure the pass with the engine-chosen inversion period")
     ap.add_argument("--seed", type=int, default=42)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -199,7 +201,7 @@ def main():
     # walks, for information only (not the headline): the same pass when the engine chooses how
     # often to invert; the samples must come out the same
     adaptive = None
-    if sampler.step_size(0) == 1 and sampler.steps > 1 and args.inversion_period == 1:
+    if sampler.step_size(0) == 1 and sampler.steps > 1 and args.inversion_period == 1 and not args.skip_engine_choice:
         sampler.set_inversion_period(0)
         sampler.do_transit_parallel(lb)
         t0 = time.perf_counter()
