@@ -350,6 +350,127 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
   if (i < n) dst[i] = value;
 }
 
+// ---- the best m keys of every sample, without sorting everything ----
+//
+// Only the first stepSize ranked vertices of a sample are ever read, out of up to millions of
+// distinct ones.  A two-level radix select on the upper 16 bits of the sort key finds, per
+// sample, the smallest 16-bit prefix T such that at least m keys have a prefix <= T; the
+// entries with a prefix <= T (m and a few more) are copied out in order and only those are
+// sorted.  Entries are grouped by sample, so a workgroup counts into an LDS histogram for the
+// sample its tile begins with and falls back to global atomics for the few entries beyond.
+constexpr uint32_t kSelectTile = 2048;  // entries per workgroup (256 lanes x 8)
+
+// level 0: hist[s][key >> 24]; level 1: hist[s][(key >> 16) & 255] over entries whose upper 8
+// bits equal prefix8[s]
+__global__ __launch_bounds__(256) void select_histogram(const uint32_t* __restrict__ key_bits,
+                                                        const uint32_t* __restrict__ distinct_sample, uint32_t n,
+                                                        int level, const uint32_t* __restrict__ prefix8,
+                                                        uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_hist[256];
+  s_hist[threadIdx.x] = 0;
+  const uint32_t tile_begin = blockIdx.x * kSelectTile;
+  const uint32_t first_sample = distinct_sample[tile_begin];
+  __syncthreads();
+  for (uint32_t k = 0; k < kSelectTile / 256; ++k) {
+    const uint32_t i = tile_begin + k * 256 + threadIdx.x;
+    if (i >= n) break;
+    const uint32_t key = key_bits[i];
+    const uint32_t s = distinct_sample[i];
+    uint32_t bin = key >> 24;
+    if (level == 1) {
+      if (bin != prefix8[s]) continue;
+      bin = (key >> 16) & 255u;
+    }
+    if (s == first_sample) atomicAdd(&s_hist[bin], 1u);
+    else atomicAdd(&hist[(size_t)s * 256 + bin], 1u);
+  }
+  __syncthreads();
+  const uint32_t c = s_hist[threadIdx.x];
+  if (c) atomicAdd(&hist[(size_t)first_sample * 256 + threadIdx.x], c);
+}
+
+// One lane per sample walks its 256 bins.  level 0: prefix8[s] = bin holding the need-th
+// smallest key, need[s] = what is still needed inside that bin, kept[s] = keys in the bins
+// before it.  level 1: threshold16[s] = (prefix8 << 8) | bin, kept[s] += keys up to and
+// including that bin.  A sample with fewer keys than needed keeps everything.
+__global__ void select_pick(const uint32_t* __restrict__ hist, uint32_t n_samples, int level, uint32_t wanted,
+                            uint32_t* __restrict__ prefix8, uint32_t* __restrict__ need,
+                            uint32_t* __restrict__ kept, uint32_t* __restrict__ threshold16) {
+  const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= n_samples) return;
+  const uint32_t* h = hist + (size_t)s * 256;
+  const uint32_t target = level == 0 ? wanted : need[s];
+  uint32_t before = 0, bin = 0;
+  for (; bin < 256; ++bin) {
+    const uint32_t c = h[bin];
+    if (before + c >= target) break;
+    before += c;
+  }
+  if (level == 0) {
+    if (bin == 256) {  // fewer keys than wanted: everything stays
+      prefix8[s] = 255;
+      need[s] = 0xFFFFFFFFu;
+      kept[s] = before - h[255];
+    } else {
+      prefix8[s] = bin;
+      need[s] = target - before;
+      kept[s] = before;
+    }
+  } else {
+    if (bin == 256) bin = 255;
+    threshold16[s] = (prefix8[s] << 8) | bin;
+    uint32_t through = 0;
+    for (uint32_t b = 0; b <= bin; ++b) through += h[b];
+    kept[s] += through;
+  }
+}
+
+__device__ __forceinline__ bool select_keeps(const uint32_t* key_bits, const uint32_t* distinct_sample,
+                                             const uint32_t* threshold16, uint32_t i) {
+  return (key_bits[i] >> 16) <= threshold16[distinct_sample[i]];
+}
+
+__global__ __launch_bounds__(256) void select_count(const uint32_t* __restrict__ key_bits,
+                                                    const uint32_t* __restrict__ distinct_sample,
+                                                    const uint32_t* __restrict__ threshold16, uint32_t n,
+                                                    uint32_t* __restrict__ tile_counts) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const uint32_t base = blockIdx.x * kSelectTile + threadIdx.x * 8u;
+  uint32_t mine = 0;
+  for (uint32_t k = 0; k < 8; ++k)
+    if (base + k < n && select_keeps(key_bits, distinct_sample, threshold16, base + k)) mine++;
+  uint32_t total;
+  block_exclusive_scan_256(mine, s_wave, &total);
+  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+}
+
+// Copies the kept entries out, in order: key, sample and vertex id.
+__global__ __launch_bounds__(256) void select_compact(const uint32_t* __restrict__ key_bits,
+                                                      const uint32_t* __restrict__ distinct_sample,
+                                                      const int32_t* __restrict__ distinct_ids,
+                                                      const uint32_t* __restrict__ threshold16, uint32_t n,
+                                                      const uint32_t* __restrict__ tile_offsets,
+                                                      uint32_t* __restrict__ kept_key, uint32_t* __restrict__ kept_sample,
+                                                      int32_t* __restrict__ kept_id) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const uint32_t base = blockIdx.x * kSelectTile + threadIdx.x * 8u;
+  bool keep[8];
+  uint32_t mine = 0;
+  for (uint32_t k = 0; k < 8; ++k) {
+    keep[k] = base + k < n && select_keeps(key_bits, distinct_sample, threshold16, base + k);
+    mine += keep[k] ? 1u : 0u;
+  }
+  uint32_t total;
+  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
+  for (uint32_t k = 0; k < 8; ++k) {
+    if (!keep[k]) continue;
+    kept_key[r] = key_bits[base + k];
+    kept_sample[r] = distinct_sample[base + k];
+    kept_id[r] = distinct_ids[base + k];
+    ++r;
+  }
+}
+
 // log2 of a positive normal float from exponent extraction and an atanh series; every step
 // is a single IEEE operation so that host and device agree bit for bit.
 __host__ __device__ __forceinline__ float det_log2(float x) {
@@ -608,6 +729,15 @@ class LayerEngine : public EngineBase {
     if (App::kNeighborhoodForm != apps::kConcatenated) {
       ND_HIP_TRY(hipMalloc(&d_distinct_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     }
+    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+      const size_t per_sample = sizeof(uint32_t) * ((size_t)n_samples_ + 1);
+      ND_HIP_TRY(hipMalloc(&d_ranked_start_, per_sample));
+      ND_HIP_TRY(hipMalloc(&d_select_prefix_, per_sample));
+      ND_HIP_TRY(hipMalloc(&d_select_need_, per_sample));
+      ND_HIP_TRY(hipMalloc(&d_select_kept_, per_sample));
+      ND_HIP_TRY(hipMalloc(&d_select_threshold_, per_sample));
+      ND_HIP_TRY(hipMalloc(&d_select_hist_, sizeof(uint32_t) * 256 * (size_t)n_samples_));
+    }
     return 0;
   }
 
@@ -774,7 +904,7 @@ class LayerEngine : public EngineBase {
     P.nbr_cols = d_nbr_cols_;
     P.nbr_weights = d_nbr_weights_;
     if (form != apps::kConcatenated) {
-      P.distinct_start = d_distinct_start_;
+      P.distinct_start = form == apps::kRankedByLadiesImportance ? d_ranked_start_ : d_distinct_start_;
       P.distinct_ids = form == apps::kRankedByLadiesImportance ? d_ranked_ids_ : d_distinct_ids_;
       P.running_sums = d_running_sums_;
     }
@@ -830,21 +960,47 @@ class LayerEngine : public EngineBase {
       ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
           d_importance_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_, (uint64_t)s0, (uint32_t)invalid_,
           (uint32_t)step, d_key_bits_);
-      // order the distinct vertices of every sample by descending key: the list is in
+      // per sample, the entries that can be among its first `wanted` in key order (radix select
+      // on the upper 16 bits of the key), copied out in (sample, vertex) order
+      const uint32_t wanted = (uint32_t)App().stepSize(step);
+      const unsigned tiles = (n_distinct + kSelectTile - 1) / kSelectTile;
+      const unsigned sample_blocks = (n + 255) / 256;
+      for (int level = 0; level < 2; ++level) {
+        ND_HIP_TRY(hipMemsetAsync(d_select_hist_, 0, sizeof(uint32_t) * 256 * (size_t)n, stream_));
+        select_histogram<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, n_distinct, level,
+                                                                 d_select_prefix_, d_select_hist_);
+        select_pick<<<dim3(sample_blocks), dim3(256), 0, stream_>>>(d_select_hist_, n, level, wanted, d_select_prefix_,
+                                                                    d_select_need_, d_select_kept_, d_select_threshold_);
+      }
+      // where every sample's ranked list starts: exclusive scan of the kept counts
+      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
+      ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
+      select_count<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, d_select_threshold_,
+                                                           n_distinct, d_scratch_);
+      scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
+      select_compact<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, d_distinct_ids_,
+                                                             d_select_threshold_, n_distinct, d_scratch_, d_kept_key_,
+                                                             d_kept_sample_, d_kept_id_);
+      uint32_t n_kept = 0;
+      ND_HIP_TRY(hipMemcpyAsync(&n_kept, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
+      ND_HIP_TRY(hipStreamSynchronize(stream_));
+      // order the kept vertices of every sample by descending key: the list is in
       // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
       // ascending vertex id among equal keys
-      const SortPlan by_key = make_sort_plan(n_distinct, 32);
-      uint32_t *k3 = nullptr, *j3 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_key, d_key_bits_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
-                                  d_scratch_, stream_, &k3, &j3));
-      const unsigned blocks = (n_distinct + 255) / 256;
-      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_distinct_sample_, j3, n_distinct, d_key2_, d_index2_);
-      const SortPlan by_sample = make_sort_plan(n_distinct, chunk_bits);
-      uint32_t *k4 = nullptr, *j4 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
-                                  d_scratch_, stream_, &k4, &j4));
-      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_distinct_ids_, j4, n_distinct,
-                                                          (uint32_t*)d_ranked_ids_, nullptr);
+      if (n_kept > 0) {
+        const SortPlan by_key = make_sort_plan(n_kept, 32);
+        uint32_t *k3 = nullptr, *j3 = nullptr;
+        ND_HIP_TRY(radix_sort_pairs(by_key, d_kept_key_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                    d_scratch_, stream_, &k3, &j3));
+        const unsigned blocks = (n_kept + 255) / 256;
+        gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_kept_sample_, j3, n_kept, d_key2_, d_index2_);
+        const SortPlan by_sample = make_sort_plan(n_kept, chunk_bits);
+        uint32_t *k4 = nullptr, *j4 = nullptr;
+        ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                    d_scratch_, stream_, &k4, &j4));
+        gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_kept_id_, j4, n_kept,
+                                                            (uint32_t*)d_ranked_ids_, nullptr);
+      }
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
   }
@@ -866,6 +1022,9 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_kept_key_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_kept_sample_, sizeof(uint32_t) * cap));
+      ND_HIP_TRY(hipMalloc(&d_kept_id_, sizeof(int32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * cap));
@@ -873,7 +1032,9 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_key2_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_index2_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(cap)));
-      ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * make_sort_plan(cap, 32).scratch_elems));
+      size_t scratch = make_sort_plan(cap, 32).scratch_elems;
+      if (cap / kSelectTile + 2 > scratch) scratch = cap / kSelectTile + 2;  // tile counts of the selection
+      ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
     }
     distinct_capacity_ = cap;
     return 0;
@@ -895,6 +1056,7 @@ class LayerEngine : public EngineBase {
     release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
+    release(d_kept_key_); release(d_kept_sample_); release(d_kept_id_);
     distinct_capacity_ = 0;
   }
 
@@ -911,6 +1073,8 @@ class LayerEngine : public EngineBase {
     release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
     release(d_item_count_); release(d_item_start_);
     release(d_distinct_start_);
+    release(d_ranked_start_); release(d_select_prefix_); release(d_select_need_); release(d_select_kept_);
+    release(d_select_threshold_); release(d_select_hist_);
     release_neighborhood_buffers();
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
@@ -956,6 +1120,11 @@ class LayerEngine : public EngineBase {
   uint32_t *d_sizes_ = nullptr, *d_offsets_ = nullptr, *d_row_offsets_ = nullptr, *d_small_scratch_ = nullptr;
   uint32_t *d_item_count_ = nullptr, *d_item_start_ = nullptr;
   uint32_t* d_distinct_start_ = nullptr;
+  // LADIES form: the selection of the best keys per sample
+  uint32_t *d_ranked_start_ = nullptr, *d_select_prefix_ = nullptr, *d_select_need_ = nullptr;
+  uint32_t *d_select_kept_ = nullptr, *d_select_threshold_ = nullptr, *d_select_hist_ = nullptr;
+  uint32_t *d_kept_key_ = nullptr, *d_kept_sample_ = nullptr;
+  int32_t* d_kept_id_ = nullptr;
   int32_t* d_nbr_cols_ = nullptr;
   float* d_nbr_weights_ = nullptr;
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
