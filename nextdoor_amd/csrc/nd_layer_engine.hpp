@@ -291,37 +291,49 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
                                                       unsigned long long* __restrict__ importance,
                                                       uint32_t* __restrict__ distinct_sample) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
+  __shared__ uint32_t s_before[kScanThreads];  // set bits of the tile before word 8 * t
   const uint32_t sample = blockIdx.x / tiles_per_sample;
   const uint32_t tile = blockIdx.x - sample * tiles_per_sample;
   const uint32_t* words = bitmap + (size_t)blockIdx.x * kBitmapTileWords;
-  uint32_t running = tile_offsets[blockIdx.x];
-  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = running;
-  // 256 consecutive words per round, one per lane: the ids a wavefront writes in a round
-  // are one contiguous stretch of the output
-  for (uint32_t round = 0; round < kBitmapTileWords / 256; ++round) {
-    const uint32_t w = round * 256 + threadIdx.x;
-    uint32_t bits = words[w];
+  {
+    const uint4* mine = (const uint4*)words + threadIdx.x * 2;
+    const uint4 a = mine[0], b = mine[1];
+    const uint32_t count = __popc(a.x) + __popc(a.y) + __popc(a.z) + __popc(a.w) + __popc(b.x) + __popc(b.y) +
+                           __popc(b.z) + __popc(b.w);
     uint32_t total;
-    uint32_t r = running + block_exclusive_scan_256((uint32_t)__popc(bits), s_wave, &total);
-    running += total;
-    const uint32_t first_vertex = (tile * kBitmapTileWords + w) * 32u;
-    while (bits) {
-      const uint32_t v = first_vertex + (uint32_t)__ffs((int)bits) - 1u;
-      bits &= bits - 1u;
-      distinct_ids[r] = (int32_t)v;
+    s_before[threadIdx.x] = block_exclusive_scan_256(count, s_wave, &total);
+  }
+  __syncthreads();
+  const uint32_t first = tile_offsets[blockIdx.x];
+  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = first;
+  // A wavefront walks its quarter of the tile 64 vertices at a time, one vertex per lane, so
+  // that the reads (row extents, accumulators) and the writes of a round are contiguous.
+  constexpr uint32_t kWordsPerWave = kBitmapTileWords / (kScanThreads / kWave);
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t first_word = wave * kWordsPerWave;
+  uint32_t r = first + s_before[first_word / 8];
+  for (uint32_t w = first_word; w < first_word + kWordsPerWave; w += 2) {
+    const uint32_t word = words[w + (lane >> 5)];
+    const bool set = (word >> (lane & 31u)) & 1u;
+    const uint64_t mask = __ballot(set);
+    if (mask == 0) continue;  // the same for every lane
+    if (set) {
+      const uint32_t v = (tile * kBitmapTileWords + w) * 32u + lane;
+      const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+      distinct_ids[at] = (int32_t)v;
       if (degree_sq) {
         const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-        degree_sq[r] = d * d;
+        degree_sq[at] = d * d;
       }
       if (sums) {
         // collect the vertex's importance and leave the accumulator clear for the next chunk
         unsigned long long* acc = sums + (size_t)sample * sums_per_sample + v;
-        importance[r] = *acc;
+        importance[at] = *acc;
         *acc = 0;
-        distinct_sample[r] = sample;
+        distinct_sample[at] = sample;
       }
-      ++r;
     }
+    r += (uint32_t)__popcll(mask);
   }
 }
 
