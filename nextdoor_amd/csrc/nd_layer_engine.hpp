@@ -204,23 +204,29 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   uint32_t* sample_bits = bitmap + (size_t)s * words_per_sample;
   const uint32_t first = item * kBuildItemEntries;
   const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
-  uint32_t cur = 0;
+  // the transit whose adjacency holds the lane's entry changes rarely: its range inside the
+  // concatenation, its first edge and its row sum stay in registers
+  uint32_t cur_begin = 0, cur_end = 0;
+  EdgePos_t cur_edges = 0;
+  int32_t t = 0;
   const uint32_t lane = threadIdx.x & 63u;
   for (uint32_t e0 = first; e0 < last; e0 += 256) {  // the same trip count for every lane
     const uint32_t e = e0 + threadIdx.x;
     uint32_t word_index = 0xFFFFFFFFu, bits = 0, vertex = 0xFFFFFFFFu;
     unsigned long long term = 0;
     if (e < last) {
-      if (!(s_start[cur] <= e && e < s_start[cur + 1])) {
+      if (!(cur_begin <= e && e < cur_end)) {
         uint32_t lo = 0, hi = tv.count;
         while (hi - lo > 1) {
           const uint32_t mid = lo + (hi - lo) / 2;
           if (s_start[mid] <= e) lo = mid; else hi = mid;
         }
-        cur = lo;
+        cur_begin = s_start[lo];
+        cur_end = s_start[lo + 1];
+        t = transits[lo];
+        cur_edges = csr.row_ptr[t];
       }
-      const int32_t t = transits[cur];
-      const EdgePos_t src = csr.row_ptr[t] + (EdgePos_t)(e - s_start[cur]);
+      const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
       vertex = (uint32_t)csr.edges[src];
       word_index = vertex >> 5;
       bits = 1u << (vertex & 31u);
