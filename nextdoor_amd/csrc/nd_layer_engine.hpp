@@ -17,9 +17,9 @@
 //    nullptr, nextdoor.cu:1441-1446).  Here offsets are an exclusive scan over samples
 //    (deterministic), the buffers are grown once and reused, and next() receives the
 //    neighbourhood in the form the app declares (nd::apps::NeighborhoodForm).
-//  * For kDistinctByDegreeSquared the concatenation is never stored: every entry sets a bit
-//    in a per-sample bitmap over the vertices, the set bits in ascending order are the
-//    distinct vertices, and a 64-bit inclusive scan of degree^2 gives the running sums the
+//  * For kDistinctByDegreeSquared the concatenation is never stored: every entry marks its
+//    vertex in a per-sample presence map (one byte per vertex), the marked vertices in
+//    ascending order are the distinct vertices, and a 64-bit inclusive scan of degree^2 gives the running sums the
 //    app inverts.
 //  * For kRankedByLadiesImportance each entry of the concatenation carries
 //    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed as 2^53
@@ -152,16 +152,24 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
   return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
 }
 
-// ---- distinct vertices of a collective neighbourhood through a bitmap ----
+// ---- distinct vertices of a collective neighbourhood through a presence map ----
 //
-// One bitmap of |V| bits per sample of the chunk (words_per_sample words, a multiple of the
-// tile below).  collective_mark walks the neighbourhood exactly as collective_build does,
-// but instead of copying an entry it sets the entry's bit; nothing of the concatenation is
-// stored.  A neighbourhood that sits on hubs repeats its vertices many times over (3.8e10
-// entries hold 2.0e9 distinct pairs at FastGCN's full size), so the bit is tested with a
-// plain load first and the atomic is issued only when the bit reads clear.  A stale read
-// costs one redundant atomic, never a wrong bit.
-constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words
+// Per sample of the chunk a map over the vertices (words_per_sample 32-bit words, a multiple
+// of the tile below).  collective_mark walks the neighbourhood exactly as collective_build
+// does, but instead of copying an entry it marks the entry's vertex; nothing of the
+// concatenation is stored.  A neighbourhood that sits on hubs repeats its vertices many
+// times over (3.8e10 entries hold 2.0e9 distinct pairs at FastGCN's full size), so the map
+// is read first and only written where the vertex is not marked yet; a stale read costs one
+// redundant write, never a wrong mark.
+//
+// Two layouts.  One BIT per vertex (FastGCN form): 8 times smaller to clear, count and
+// compact, and the lanes of a dense row share a few words; the price is one atomic OR per new
+// word-stretch.  One BYTE per vertex (LADIES form, kWithImportance): every writer stores the
+// same value 1, so plain stores do.  Atomics of any width top out at ~24 G/s on this part,
+// and the LADIES form already spends that on its importance sums: with bits, marking 3.8e10
+// entries took 477 ms there, with bytes 403 ms; for FastGCN the bit map wins (143 vs 152 ms
+// per pass) because the byte maps of 4096 batches are 17 GB to clear, count and compact.
+constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words: 65536 vertices as bits, 8192 as bytes
 
 // kWithImportance (LADIES form): every entry also adds (weight / row_sums[transit])^2, as a
 // fixed-point integer, to sums[sample * sums_per_sample + vertex].  Parallel edges make a
@@ -201,7 +209,7 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   if (threadIdx.x == 0) s_start[tv.count] = carry;
   __syncthreads();
   const uint32_t size = s_start[tv.count];
-  uint32_t* sample_bits = bitmap + (size_t)s * words_per_sample;
+  uint32_t* present_of_sample = bitmap + (size_t)s * words_per_sample;
   const uint32_t first = item * kBuildItemEntries;
   const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
   // the transit whose adjacency holds the lane's entry changes rarely: its range inside the
@@ -212,7 +220,7 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   const uint32_t lane = threadIdx.x & 63u;
   for (uint32_t e0 = first; e0 < last; e0 += 256) {  // the same trip count for every lane
     const uint32_t e = e0 + threadIdx.x;
-    uint32_t word_index = 0xFFFFFFFFu, bits = 0, vertex = 0xFFFFFFFFu;
+    uint32_t vertex = 0xFFFFFFFFu;
     unsigned long long term = 0;
     if (e < last) {
       if (!(cur_begin <= e && e < cur_end)) {
@@ -228,8 +236,6 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
       }
       const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
       vertex = (uint32_t)csr.edges[src];
-      word_index = vertex >> 5;
-      bits = 1u << (vertex & 31u);
       if (kWithImportance) {
         const float p = csr.weights[src] / row_sums[t];
         term = importance_term_fixed(p * p);
@@ -252,25 +258,37 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
       if (vertex != 0xFFFFFFFFu && term != 0 && (lane == 63u || right != vertex))
         atomicAdd(sums + (size_t)s * sums_per_sample + vertex, term);
     }
-    // Adjacencies are sorted, so neighbouring lanes mostly hit the same word: OR the bits
-    // of equal words along the wave and let the last lane of each stretch do the memory
-    // work (a dense hub row then costs 8 words per wavefront instead of 64).
+    if (kWithImportance) {
+      if (vertex != 0xFFFFFFFFu) {
+        uint8_t* mark = (uint8_t*)present_of_sample + vertex;
+        if (*mark == 0) *mark = 1;
+      }
+    } else {
+      // Adjacencies are sorted, so neighbouring lanes mostly hit the same word: OR the bits
+      // of equal words along the wave and let the last lane of each stretch do the memory
+      // work (a dense hub row then costs 8 words per wavefront instead of 64).
+      uint32_t word_index = 0xFFFFFFFFu, bits = 0;
+      if (vertex != 0xFFFFFFFFu) {
+        word_index = vertex >> 5;
+        bits = 1u << (vertex & 31u);
+      }
 #pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const uint32_t up_index = __shfl_up(word_index, d, kWave);
-      const uint32_t up_bits = __shfl_up(bits, d, kWave);
-      if (lane >= (uint32_t)d && up_index == word_index) bits |= up_bits;
-    }
-    const uint32_t next_index = __shfl_down(word_index, 1, kWave);
-    const bool last_of_stretch = lane == 63u || next_index != word_index;
-    if (bits != 0 && last_of_stretch) {
-      uint32_t* word = sample_bits + word_index;
-      if ((*word & bits) != bits) atomicOr(word, bits);
+      for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t up_index = __shfl_up(word_index, d, kWave);
+        const uint32_t up_bits = __shfl_up(bits, d, kWave);
+        if (lane >= (uint32_t)d && up_index == word_index) bits |= up_bits;
+      }
+      const uint32_t next_index = __shfl_down(word_index, 1, kWave);
+      if (bits != 0 && (lane == 63u || next_index != word_index)) {
+        uint32_t* word = present_of_sample + word_index;
+        if ((*word & bits) != bits) atomicOr(word, bits);
+      }
     }
   }
 }
 
-// tile_counts[s * tiles_per_sample + t] = bits set in tile t of sample s's bitmap
+// tile_counts[s * tiles_per_sample + t] = vertices marked in tile t of sample s's presence map
+// (a marked byte is 1, so the population count of a word counts marks in either layout)
 __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __restrict__ bitmap,
                                                           uint32_t* __restrict__ tile_counts) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
@@ -283,10 +301,11 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
   if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
-// The set bits of every sample's bitmap, in ascending order, become the sample's distinct
+// The marked vertices of every sample, in ascending order, become the sample's distinct
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
 // tile of a sample is where the sample's list starts).  Per distinct vertex either
 // degree^2 (degree_sq given) or the importance accumulated in sums (sums given).
+template <bool kBytes>
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t tiles_per_sample, const EdgePos_t* __restrict__ row_ptr,
@@ -318,13 +337,15 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t first_word = wave * kWordsPerWave;
   uint32_t r = first + s_before[first_word / 8];
-  for (uint32_t w = first_word; w < first_word + kWordsPerWave; w += 2) {
-    const uint32_t word = words[w + (lane >> 5)];
-    const bool set = (word >> (lane & 31u)) & 1u;
+  const uint8_t* bytes = (const uint8_t*)words;
+  constexpr uint32_t kWordsPerRound = kBytes ? 16u : 2u;     // 64 vertices
+  constexpr uint32_t kVerticesPerWord = kBytes ? 4u : 32u;
+  for (uint32_t w = first_word; w < first_word + kWordsPerWave; w += kWordsPerRound) {
+    const bool set = kBytes ? bytes[w * 4u + lane] != 0 : ((words[w + (lane >> 5)] >> (lane & 31u)) & 1u) != 0;
     const uint64_t mask = __ballot(set);
     if (mask == 0) continue;  // the same for every lane
     if (set) {
-      const uint32_t v = (tile * kBitmapTileWords + w) * 32u + lane;
+      const uint32_t v = (tile * kBitmapTileWords + w) * kVerticesPerWord + lane;
       const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       distinct_ids[at] = (int32_t)v;
       if (degree_sq) {
@@ -623,9 +644,9 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
 // Entries of concatenated neighbourhood one chunk of samples may hold (about 70 bytes of
 // device memory per entry across all work arrays).
 constexpr uint64_t kLayerChunkEntries = 96ull << 20;
-// Bitmap form: nothing is stored per entry, so a chunk is bounded by the memory of its
-// bitmaps and by the number of marking work items (entries / kBuildItemEntries) of one launch.
-constexpr uint64_t kBitmapBudgetBytes = 4ull << 30;
+// Importance forms: nothing is stored per entry, so a chunk is bounded by the memory of its
+// presence maps (and accumulators) and by the number of marking work items (entries / kBuildItemEntries) of one launch.
+constexpr uint64_t kBitmapBudgetBytes = 24ull << 30;
 constexpr uint64_t kBitmapChunkEntries = 1ull << 40;
 
 template <class SampleType, class App>
@@ -713,7 +734,10 @@ class LayerEngine : public EngineBase {
       const long long v = atoll(env);
       if (v > 0) chunk_entries_ = bitmap_chunk_entries_ = (uint64_t)v;
     }
-    bitmap_words_ = (((uint32_t)invalid_ + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
+    // one byte per vertex for the LADIES form, one bit for the FastGCN form
+    const uint32_t per_word = App::kNeighborhoodForm == apps::kRankedByLadiesImportance ? 4u : 32u;
+    bitmap_words_ = (((uint32_t)invalid_ + per_word - 1u) / per_word + kBitmapTileWords - 1) / kBitmapTileWords *
+                    kBitmapTileWords;
     // LADIES form: one 64-bit importance accumulator per vertex next to the bitmap
     sums_per_sample_ = App::kNeighborhoodForm == apps::kRankedByLadiesImportance ? (uint32_t)invalid_ : 0u;
     const uint64_t fit = kBitmapBudgetBytes / ((uint64_t)bitmap_words_ * sizeof(uint32_t) +
@@ -966,7 +990,7 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
-    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
+    bitmap_compact<ladies><<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
         d_bitmap_, d_tile_offsets_, tiles_per_sample, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
         d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
@@ -1117,7 +1141,7 @@ class LayerEngine : public EngineBase {
   uint64_t seed_ = 0;
   bool allocated_ = false;
   size_t capacity_ = 0;
-  uint32_t bitmap_words_ = 0;          // words of one sample's bitmap (a multiple of kBitmapTileWords)
+  uint32_t bitmap_words_ = 0;          // 32-bit words of one sample's presence map (a multiple of kBitmapTileWords)
   uint32_t bitmap_chunk_samples_ = 0;  // samples whose bitmaps fit the budget
   uint64_t bitmap_chunk_entries_ = 0;
   uint32_t bitmap_samples_ = 0;        // samples the allocated bitmaps hold
