@@ -82,12 +82,11 @@ inline bool doTransitParallelSampling(CSR*, NextDoorData& data, bool enableLoadB
 }
 
 // doSampleParallelSampling(csr, data), src/nextdoor.cu:3009-3209: the reference's baseline
-// mode, every sample on its own lane.  For walks the engine then never brings the samples
-// into transit order (it only drops ended walks now and then); other apps have no such mode
-// here and run as above without load balancing.  The samples are the same bytes either way.
+// mode, every sample's work in sample order: the engine never brings the pairs into transit
+// order (it only drops the dead ones) and does no load balancing.  The samples are the same
+// bytes either way.
 inline bool doSampleParallelSampling(CSR*, NextDoorData& data) {
-  return data.sampler && nd_sampler_set_inversion_period(data.sampler, 32) == 0 &&
-         nd_sampler_do_transit_parallel(data.sampler, 0) == 0;
+  return data.sampler && nd_sampler_do_sample_parallel(data.sampler) == 0;
 }
 
 // getFinalSamples(data), src/nextdoor.cu:3211-3237.

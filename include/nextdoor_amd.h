@@ -65,6 +65,13 @@ int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g);
 int nd_sampler_alloc(nd_sampler* s, uint64_t seed);
 /* doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006. */
 int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing);
+/* doSampleParallelSampling(csr, data), src/nextdoor.cu:3009-3209: the reference's baseline
+ * mode.  The (sample -> transit) map is never sorted by transit: before a step the pairs whose
+ * transit is INVALID are dropped (one stable compaction, sample order kept) and every remaining
+ * pair gets its lanes; no load balancing.  Walks advance several steps per launch between
+ * compactions.  Layer-wise apps have one schedule only and run it.  Same samples, byte for
+ * byte, as the transit-parallel modes. */
+int nd_sampler_do_sample_parallel(nd_sampler* s);
 /* How often walks re-invert the (sample -> transit) map.  The reference inverts before every
  * step (src/nextdoor.cu:2924-2939), which is period 1 and the default.  period p > 1: the walks
  * are not brought into transit order (no load balancing); before step 1 and then every p-th
@@ -113,6 +120,19 @@ int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, in
  * of all collective neighbourhoods built, 1 = distinct (sample, vertex) pairs found,
  * 2 = chunks of samples processed; other apps return 0. */
 int64_t nd_sampler_counter(const nd_sampler* s, int which);
+/* The validators the reference's apps pass to nextdoor() as checkResultsFunc
+ * (src/check_results.cu): checkSampledVerticesResult (162-299) for the per-transit apps and
+ * importance samplers, checkAdjacencyMatrixResult (46-160) for the layer-wise apps that record
+ * an adjacency matrix.  Runs on the host over the fetched final samples (and sample states).
+ * *ok = 1 when the samples pass; 0 with the first violation in nd_last_error(). */
+int nd_sampler_check_results(nd_sampler* s, int* ok);
+/* The same rule over caller-supplied arrays (no device needed): final_samples is
+ * [n_samples][F], initial [n_samples][initial_size]; collective != 0: step k holds
+ * step_sizes[k] vertices (CollectiveNeighborhood layout), else T_k * step_sizes[k].
+ * Returns 1 (pass), 0 (violation, text in nd_last_error()) or a negative error. */
+int nd_check_sampled_vertices(const nd_graph* g, int n_steps, const int32_t* step_sizes, int initial_size,
+                              int collective, int64_t n_samples, const int32_t* initial,
+                              const int32_t* final_samples, int32_t invalid);
 /* freeDeviceData(data), src/nextdoor.cu:2088-2115. */
 void nd_sampler_free_device(nd_sampler* s);
 void nd_sampler_destroy(nd_sampler* s);

@@ -22,12 +22,30 @@ from . import _capi
 from ._capi import NextDoorError, check, lib
 
 __all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
-           "sort_pairs", "unique_transits", "collective_neighborhood"]
+           "sort_pairs", "unique_transits", "collective_neighborhood", "check_sampled_vertices"]
 
 
 def app_names():
     L = lib()
     return [L.nd_app_name(i).decode() for i in range(L.nd_num_apps())]
+
+
+def check_sampled_vertices(graph, step_sizes, initial, final_samples, invalid=None, collective=False):
+    """The reference's checkSampledVerticesResult rule (src/check_results.cu:162-299) on host
+    arrays: ``initial`` is (num_samples, initial_size), ``final_samples`` (num_samples, F).
+    Returns (True, "") or (False, first violation)."""
+    initial = _as(initial, np.int32)
+    final_samples = _as(final_samples, np.int32)
+    n_samples = final_samples.shape[0]
+    initial = initial.reshape(n_samples, -1) if n_samples else initial.reshape(0, 1)
+    sizes = _as(step_sizes, np.int32)
+    rc = lib().nd_check_sampled_vertices(graph._h, len(sizes), _ptr(sizes, C.c_int32), max(initial.shape[1], 1),
+                                         int(collective), n_samples, _ptr(initial, C.c_int32),
+                                         _ptr(final_samples, C.c_int32),
+                                         graph.n_vertices if invalid is None else invalid)
+    if rc < 0:
+        raise NextDoorError(lib().nd_last_error().decode())
+    return (True, "") if rc == 1 else (False, lib().nd_last_error().decode())
 
 
 def _as(arr, dtype):
@@ -172,6 +190,17 @@ class Sampler:
 
     def do_transit_parallel(self, load_balancing=True):
         check(lib().nd_sampler_do_transit_parallel(self._h, int(load_balancing)))
+
+    def do_sample_parallel(self):
+        """The reference's baseline mode: no transit order, no load balancing; same samples."""
+        check(lib().nd_sampler_do_sample_parallel(self._h))
+
+    def check_results(self):
+        """The reference's result validators (src/check_results.cu) on the host.  Returns
+        (True, "") or (False, first violation)."""
+        ok = C.c_int()
+        check(lib().nd_sampler_check_results(self._h, C.byref(ok)))
+        return (True, "") if ok.value else (False, lib().nd_last_error().decode())
 
     def final_samples(self):
         """(num_samples, final_sample_size) int32 array; INVALID entries equal n_vertices."""

@@ -32,6 +32,10 @@ SIGNATURES = {
     "nd_sampler_set_graph": (C.c_int, [C.c_void_p, C.c_void_p]),
     "nd_sampler_alloc": (C.c_int, [C.c_void_p, C.c_uint64]),
     "nd_sampler_do_transit_parallel": (C.c_int, [C.c_void_p, C.c_int]),
+    "nd_sampler_do_sample_parallel": (C.c_int, [C.c_void_p]),
+    "nd_sampler_check_results": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
+    "nd_check_sampled_vertices": (C.c_int, [C.c_void_p, C.c_int, c_i32p, C.c_int, C.c_int, C.c_int64, c_i32p, c_i32p,
+                                            C.c_int32]),
     "nd_sampler_get_final_samples": (C.c_int, [C.c_void_p, C.POINTER(c_i32p), c_i64p]),
     "nd_sampler_final_sample_size": (C.c_int, [C.c_void_p]),
     "nd_sampler_num_samples": (C.c_int64, [C.c_void_p]),

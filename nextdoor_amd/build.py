@@ -7,7 +7,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libnextdoor_amd.so")
 
-SOURCES = ["nd_capi.hip", "nd_graph.cpp"]
+SOURCES = ["nd_capi.hip", "nd_graph.cpp", "nd_check.cpp"]
 
 # -ffp-contract=off: the samplers compare single IEEE float operations bit for bit with
 # the CPU checker.  The target-feature pair switches packed-fp32 code generation off.

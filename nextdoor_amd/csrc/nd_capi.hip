@@ -15,6 +15,7 @@
 #include "nd_sharded_engine.hpp"
 #include "nd_layer_engine.hpp"
 #include "nd_graph.hpp"
+#include "nd_check.hpp"
 
 struct nd_graph {
   CSR csr;
@@ -224,6 +225,12 @@ int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing) {
   return rc == 0 ? 0 : fail(s->engine->last_error, rc);
 }
 
+int nd_sampler_do_sample_parallel(nd_sampler* s) {
+  if (!s) return fail("null sampler");
+  const int rc = s->engine->sample(nd::kSampleParallel);
+  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+}
+
 int nd_sampler_get_final_samples(nd_sampler* s, const int32_t** data, int64_t* length) {
   if (!s || !data || !length) return fail("null argument");
   const int rc = s->engine->fetch_final_samples();
@@ -300,6 +307,55 @@ int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, in
 }
 
 int64_t nd_sampler_counter(const nd_sampler* s, int which) { return s ? s->engine->counter(which) : 0; }
+
+int nd_check_sampled_vertices(const nd_graph* g, int n_steps, const int32_t* step_sizes, int initial_size,
+                              int collective, int64_t n_samples, const int32_t* initial,
+                              const int32_t* final_samples, int32_t invalid) {
+  if (!g || !step_sizes || n_steps < 1 || initial_size < 1 || n_samples < 0 ||
+      (n_samples > 0 && (!initial || !final_samples)))
+    return fail("bad argument");
+  nd::SampleShape shape;
+  shape.step_size.assign(step_sizes, step_sizes + n_steps);
+  shape.initial_size = initial_size;
+  shape.collective = collective != 0;
+  std::string report;
+  if (nd::check_sampled_vertices(g->csr, shape, n_samples, initial, final_samples, invalid, &report)) return 1;
+  g_error = report;
+  return 0;
+}
+
+int nd_sampler_check_results(nd_sampler* s, int* ok) {
+  if (!s || !ok) return fail("null argument");
+  if (!s->graph) return fail("no graph set");
+  nd::EngineBase& e = *s->engine;
+  const int rc = e.fetch_final_samples();
+  if (rc != 0) return fail(e.last_error, rc);
+  nd::SampleShape shape;
+  for (int k = 0; k < e.steps(); ++k) shape.step_size.push_back(e.step_size(k));
+  shape.initial_size = e.initial_sample_size();
+  shape.collective = e.sampling_type() == SamplingType::CollectiveNeighborhood;
+  std::string report;
+  bool pass;
+  // a layer-wise app whose sample state is the per-layer adjacency matrix
+  // {len[L], row[L][B*B], col[L][B*B], val[L][B*B]} records edges instead of sampling along them
+  const size_t layers = shape.step_size.size(), cells = (size_t)shape.step_size[0] * shape.step_size[0];
+  const size_t matrix_ints = layers + 3 * layers * cells;
+  if (shape.collective && e.sample_state_bytes() == sizeof(int32_t) * matrix_ints * (size_t)e.num_samples()) {
+    std::vector<int32_t> states((size_t)e.num_samples() * matrix_ints);
+    const int rc2 = e.fetch_sample_states(states.data(), states.size() * sizeof(int32_t));
+    if (rc2 != 0) return fail(e.last_error, rc2);
+    pass = nd::check_layer_adjacency_matrix(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+                                            e.hFinalSamples.data(), states.data() + layers,
+                                            states.data() + layers + layers * cells, matrix_ints, e.invalid_vertex(),
+                                            &report);
+  } else {
+    pass = nd::check_sampled_vertices(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+                                      e.hFinalSamples.data(), e.invalid_vertex(), &report);
+  }
+  *ok = pass ? 1 : 0;
+  if (!pass) g_error = report;
+  return 0;
+}
 
 void nd_sampler_free_device(nd_sampler* s) {
   if (s) s->engine->free_device();

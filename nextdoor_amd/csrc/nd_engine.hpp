@@ -47,7 +47,10 @@ namespace nd {
 // Host-visible, app-independent interface (what the C ABI talks to)
 // ---------------------------------------------------------------------------------------
 
-enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1 };
+// kSampleParallel: the reference's baseline (src/nextdoor.cu:3009-3209), every sample's work in
+// sample order: the (sample -> transit) map is never sorted by transit, the pairs whose transit
+// is INVALID are only dropped (one stable compaction), and there is no load balancing.
+enum KernelMode { kTransitParallel = 0, kTransitParallelLoadBalanced = 1, kSampleParallel = 2 };
 
 struct PhaseTimes {  // milliseconds, accumulated over one sample() call when profiling is on
   float end_to_end = 0, inversion = 0, load_balancing = 0, flat_kernel = 0, workgroup_kernel = 0, assemble = 0, distinct = 0;
@@ -900,6 +903,8 @@ class Engine : public EngineBase {
     int sort_period = inversion_period;
     if (sort_period <= 0)
       sort_period = (double)n_samples_ < kWalksPerVertexForInversion * (double)invalid_ ? kSparseInversionPeriod : 1;
+    const bool sample_parallel = mode == kSampleParallel;
+    if (sample_parallel && sort_period <= 1) sort_period = kSparseInversionPeriod;
     const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
     KeyLayout transits_layout;             // and how it is laid out
     for (int step = 0; step < n_steps; ++step) {
@@ -957,7 +962,7 @@ class Engine : public EngineBase {
         // Walks that invert only now and then gain nothing from the transit order (few of them
         // share a transit, and the order is stale one step later): they only drop the walks
         // that have ended, keeping slot order, in which the writes of a step's results coalesce.
-        const bool compact_only = walk_mode_ && sort_period > 1;
+        const bool compact_only = sample_parallel || (walk_mode_ && sort_period > 1);
         const SortPlan plan = make_sort_plan(n_pairs, compact_only ? 0 : max_bits_);
         SortJob job;
         if (walk_mode_) {
@@ -990,7 +995,7 @@ class Engine : public EngineBase {
         P.live_pairs = live_now;
         live_last = live_now;
         sorts_done++;
-        if (compact_only) {
+        if (compact_only && walk_mode_) {
           // the walks keep their lanes until the next compaction
           const int stretch = n_steps - step < sort_period ? n_steps - step : sort_period;
           P.emit_keys = d_emit_keys_;
@@ -1002,7 +1007,7 @@ class Engine : public EngineBase {
           tock(&times.flat_kernel);
           times.flat_launches++;
           step += stretch - 1;
-        } else if (!balance) {
+        } else if (!balance || compact_only) {
           tick();
           launch_flat(P, flat_grid, nullptr);
           tock(&times.flat_kernel);

@@ -59,6 +59,10 @@ def test_layer_literal_matches_oracle(oracle, app, layers, batch):
         assert np.all(st[:, :layers] == 0)
     # the reference's own validator on the GPU result
     assert oracle.check_adjacency_matrix(og, d, roots, got, got_rows, got_cols, s.invalid_vertex)
+    assert s.check_results() == (True, "")  # and the library's
+    print("app", app, "sample parallel", flush=True)
+    s.do_sample_parallel()
+    assert np.array_equal(s.final_samples(), want)
     s.close()
 
 
@@ -88,6 +92,7 @@ def test_fastgcn_importance_matches_oracle(oracle, app, gname):
             prev = cur
     s.do_transit_parallel(True)
     assert np.array_equal(s.final_samples(), want)
+    assert s.check_results() == (True, "")
     s.close()
 
 
@@ -121,6 +126,7 @@ def test_ladies_importance_matches_oracle(oracle, app, gname):
             seg = row[k * B:(k + 1) * B]
             seg = seg[seg != s.invalid_vertex]
             assert len(set(seg.tolist())) == len(seg)
+    assert s.check_results() == (True, "")
     s.close()
 
 

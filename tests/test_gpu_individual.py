@@ -30,7 +30,10 @@ def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)
         assert want.shape == (s.num_samples, s.final_sample_size)
         for lb in modes:
             print("app", app, "V", g.n_vertices, "E", g.n_edges, "lb", lb, flush=True)
-            s.do_transit_parallel(load_balancing=lb)
+            if lb == "sample_parallel":
+                s.do_sample_parallel()
+            else:
+                s.do_transit_parallel(load_balancing=lb)
             got = s.final_samples()
             if not np.array_equal(got, want):
                 bad = np.argwhere(got != want)
@@ -45,6 +48,7 @@ def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)
         # PPR unchecked: src/tests/singleGPU/ppr.cu:12-30)
         if kind != oracle.PPR:
             assert oracle.check_sampled_vertices(og, d, roots, got, s.invalid_vertex)
+            assert s.check_results() == (True, "")  # the library's own validator
         assert oracle.check_exact_transits(og, d, roots, got, s.invalid_vertex)
         return got
     finally:
@@ -64,6 +68,46 @@ def test_samples_do_not_depend_on_the_inversion_period(oracle, app, kind_name, s
     # sees fit) give the bytes of the oracle too; for other apps the setting changes nothing
     g = graphs.random_graph(n=1500, mean_degree=6, seed=9, hub=4, isolated_every=11)
     run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, inversion_period=period)
+
+
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("DeepWalkPerVertex", "DEEPWALK", False),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+    ("KHop", "KHOP", False),
+    ("KHop4x3x2", "KHOP", False),
+])
+def test_sample_parallel_mode_gives_the_same_samples(oracle, app, kind_name, state):
+    # the reference's baseline schedule (no transit order, no load balancing), then the
+    # transit-parallel one on the same sampler
+    g = graphs.random_graph(n=1500, mean_degree=6, seed=9, hub=4, isolated_every=11)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state,
+                    modes=("sample_parallel", True, "sample_parallel"))
+
+
+def test_command_line_runs_checks_and_prints(oracle, tmp_path):
+    import io
+    from nextdoor_amd import __main__ as cli
+    g = graphs.random_graph(n=120, mean_degree=4, seed=12)
+    rec = np.zeros(g.n_edges, dtype=[("s", "<i4"), ("d", "<i4"), ("w", "<f4")])
+    rec["s"] = np.repeat(np.arange(g.n_vertices), np.diff(g.row_ptr))
+    rec["d"], rec["w"] = g.col, g.weight
+    path = tmp_path / "g.data"
+    rec.tofile(path)
+    for kernel, extra in (("TransitParallel", ["-l"]), ("SampleParallel", [])):
+        out = io.StringIO()
+        print("cli KHop3x2", kernel, flush=True)
+        rc = cli.run(["KHop3x2", "-g", str(path), "-t", "edge-list", "-f", "binary", "-n", "2", "-c", "-p",
+                      "-k", kernel] + extra, out=out)
+        text = out.getvalue()
+        assert rc == 0, text
+        assert "Graph has %d edges and %d vertices" % (g.n_edges, g.n_vertices) in text
+        assert text.count("Contents of sample") == g.n_vertices and "Results Checked" in text
+        d = oracle.app_desc(oracle.KHOP, 2, [3, 2])
+        want, _ = oracle.sample_individual(graphs.oracle_view(g), d, 42, np.arange(g.n_vertices, dtype=np.int32))
+        assert "totalSampledVertices %d" % np.count_nonzero(want != g.n_vertices) in text
+        first = [l for l in text.splitlines() if l.startswith("Contents of sample 0 ")][0]
+        assert first == "Contents of sample 0 [%s]" % "".join("%d, " % v for v in want[0])
 
 
 GRAPHS = {
@@ -171,9 +215,12 @@ def test_multirw_matches_oracle(oracle, app, n_roots, steps, period):
         roots = oracle.multirw_roots(s.num_samples, n_roots, g.n_vertices)
         assert np.array_equal(s.initial_contents, roots[:, 0])
         want, want_walkers, want_last, _ = oracle.sample_multirw(og, SEED, roots, steps)
-        for lb in (False, True):
+        for lb in (False, True, "sample_parallel"):
             print("app", app, "period", period, "lb", lb, flush=True)
-            s.do_transit_parallel(load_balancing=lb)
+            if lb == "sample_parallel":
+                s.do_sample_parallel()
+            else:
+                s.do_transit_parallel(load_balancing=lb)
             assert np.array_equal(s.final_samples(), want)
             state = s.sample_states().view(np.int32).reshape(s.num_samples, n_roots + 1)
             assert np.array_equal(state[:, :n_roots], want_walkers)
