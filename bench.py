@@ -61,6 +61,10 @@ WORKLOADS = {
     "ladies_importance_chunglu3m_b8": dict(app="LADIESImportanceB8", kind="LADIES_IMPORTANCE",
                                            graph=("chung_lu", dict(n_vertices=3072441, n_edges=117000000,
                                                                    exponent=2.0))),
+    # edge-list apps of the reference (src/apps/mvs, src/apps/clustergcn) on the headline graph
+    "mvs_rmat22": dict(app="MVS", kind="SUBGRAPH", graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
+    "clustergcn_rmat22": dict(app="ClusterGCN", kind="SUBGRAPH",
+                              graph=("rmat", dict(scale=22, edge_factor=16, symmetrise=True))),
 }
 
 
@@ -251,6 +255,19 @@ def main():
         if not args.skip_cpu_baseline:
             result["cpu_baseline"] = cpu_baseline_layers(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
         args.skip_cpu_baseline = True  # the walk/k-hop accounting below does not apply to layer-wise apps
+    if w["kind"] == "SUBGRAPH":
+        listed = sampler.counter(0)
+        result["config"]["edges_listed"] = listed
+        result["config"]["edges_listed_per_s"] = listed / (ms_per_step / 1000.0)
+        # minimal traffic of a pass: the result rows and the lists written once; MVS also reads
+        # every listed edge once, ClusterGCN the 32 row extents and vertices of every sample
+        rows_bytes = 4.0 * edges_per_pass
+        reads = 4.0 * listed if w["app"] == "MVS" else sampler.num_samples * 32 * 12.0
+        achieved = (rows_bytes + 8.0 * listed + reads) / (np.mean(gpu_ms) / 1000.0) / 1e9
+        result["roofline"] = {"bound": "hbm", "kernel": "subgraph_step_kernel (count + write passes)",
+                              "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+        args.skip_cpu_baseline = True
     if w["kind"] == "KHOP":
         counts = sampler.distinct()
         result["config"]["distinct_ms"] = sampler.phase_times()["distinct_ms"]

@@ -108,6 +108,16 @@ int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
  * [10] milliseconds in the kernel that walks the collective neighbourhoods, [11] its launches. */
 int nd_sampler_set_profiling(nd_sampler* s, int on);
 int nd_sampler_phase_times(const nd_sampler* s, float out[12]);
+/* Apps whose outputFormat() is AdjacencyMatrix on per-transit sampling (MVS, ClusterGCN:
+ * src/apps/mvs/mvsSampling.cu, src/apps/clustergcn/clusterGCNSampling.cu) leave one edge list
+ * per sample.  The reference keeps them in dRowStorage / dColStorage at
+ * sample.posInStorage / adjMatrixPos with sample.length / adjacencyMatrixLen entries, in the
+ * order its atomics happened to run.  Here the lists are packed back to back in sample order:
+ * sample i owns entries [list_start[i], list_start[i + 1]) of rows / cols (list_start has
+ * n_samples + 1 entries), ordered by step, transit index, neighbour slot and emit order.
+ * Borrowed host pointers, valid until the next call.  Other apps: error. */
+int nd_sampler_get_adjacency(nd_sampler* s, const int32_t** rows, const int32_t** cols, int64_t* n_edges,
+                             const uint32_t** list_start, int64_t* n_samples);
 /* Distinct post-pass for SampledVertices results (GraphSAGE: draw with replacement, then
  * distinct): every hop segment of every sample is replaced, on the device, by its ascending
  * unique valid ids packed left and INVALID-padded; counts[sample * steps + hop] = ids kept.

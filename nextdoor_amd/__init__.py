@@ -209,6 +209,18 @@ class Sampler:
         flat = np.ctypeslib.as_array(p, shape=(n.value,)).copy()
         return flat.reshape(self.num_samples, self.final_sample_size)
 
+    def adjacency(self):
+        """Edge lists of the apps with AdjacencyMatrix output on per-transit sampling (MVS,
+        ClusterGCN): (rows, cols, list_start); sample i owns rows/cols[list_start[i]:list_start[i+1]]."""
+        rows, cols = C.POINTER(C.c_int32)(), C.POINTER(C.c_int32)()
+        start = C.POINTER(C.c_uint32)()
+        n_edges, n_samples = C.c_int64(), C.c_int64()
+        check(lib().nd_sampler_get_adjacency(self._h, C.byref(rows), C.byref(cols), C.byref(n_edges), C.byref(start),
+                                             C.byref(n_samples)))
+        take = lambda p, n, dt: (np.ctypeslib.as_array(p, shape=(n,)).copy() if n else np.zeros(0, dtype=dt))
+        return (take(rows, n_edges.value, np.int32), take(cols, n_edges.value, np.int32),
+                take(start, n_samples.value + 1, np.uint32))
+
     def distinct(self):
         """Distinct post-pass on the device rows; returns counts[num_samples, steps]."""
         check(lib().nd_sampler_distinct(self._h))

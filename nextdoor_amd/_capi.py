@@ -51,6 +51,8 @@ SIGNATURES = {
     "nd_sampler_set_inversion_period": (C.c_int, [C.c_void_p, C.c_int]),
     "nd_sampler_set_profiling": (C.c_int, [C.c_void_p, C.c_int]),
     "nd_sampler_phase_times": (C.c_int, [C.c_void_p, c_f32p]),
+    "nd_sampler_get_adjacency": (C.c_int, [C.c_void_p, C.POINTER(c_i32p), C.POINTER(c_i32p), c_i64p,
+                                           C.POINTER(C.POINTER(C.c_uint32)), c_i64p]),
     "nd_sampler_distinct": (C.c_int, [C.c_void_p]),
     "nd_sampler_get_distinct_counts": (C.c_int, [C.c_void_p, C.POINTER(c_i32p), c_i64p]),
     "nd_sampler_counter": (C.c_int64, [C.c_void_p, C.c_int]),

@@ -9,11 +9,13 @@
 
 #include "nd_apps_khop.hpp"
 #include "nd_apps_multirw.hpp"
+#include "nd_apps_subgraph.hpp"
 #include "nd_apps_layer.hpp"
 #include "nd_apps_walks.hpp"
 #include "nd_engine.hpp"
 #include "nd_sharded_engine.hpp"
 #include "nd_layer_engine.hpp"
+#include "nd_subgraph_engine.hpp"
 #include "nd_graph.hpp"
 #include "nd_check.hpp"
 
@@ -46,6 +48,11 @@ nd::EngineBase* make_engine(const char* name) {
 }
 
 template <class SampleType, class App>
+nd::EngineBase* make_subgraph_engine(const char* name) {
+  return new nd::SubgraphEngine<SampleType, App>(name);
+}
+
+template <class SampleType, class App>
 nd::EngineBase* make_layer_engine(const char* name) {
   return new nd::LayerEngine<SampleType, App>(name);
 }
@@ -74,6 +81,12 @@ const AppEntry kApps[] = {
     {"Layer", make_engine<LayerSample, LayerSamplingApp>},
     {"MultiRW", make_engine<MultiRWSample, MultiRWApp>},
     {"MultiRW4x6", make_engine<MultiRWSampleT<4>, MultiRWAppT<4, 6>>},
+    // edge-list results: the reference's MVS (batches of 32 vertices) and ClusterGCN (two clusters
+    // of 16), and small variants
+    {"MVS", make_subgraph_engine<MVSSample, MVSSamplingApp>},
+    {"ClusterGCN", make_subgraph_engine<SubGraphSample, SubGraphSamplingAppI>},
+    {"MVS5", make_subgraph_engine<SubgraphSampleT<5>, MVSSamplingAppT<5>>},
+    {"ClusterGCN3x2", make_subgraph_engine<SubgraphSampleT<6>, SubGraphSamplingAppT<3, 2>>},
     // layer-wise apps: the reference's FastGCN / LADIES (5 layers of 64, 10000 samples) ...
     {"FastGCN", make_layer_engine<FastGCNSample, FastGCNSamplingApp>},
     {"LADIES", make_layer_engine<ImportanceSample, ImportanceSampleApp>},
@@ -293,6 +306,19 @@ int nd_sampler_phase_times(const nd_sampler* s, float out[12]) {
   return 0;
 }
 
+int nd_sampler_get_adjacency(nd_sampler* s, const int32_t** rows, const int32_t** cols, int64_t* n_edges,
+                             const uint32_t** list_start, int64_t* n_samples) {
+  if (!s || !rows || !cols || !n_edges || !list_start || !n_samples) return fail("null argument");
+  const int rc = s->engine->fetch_adjacency();
+  if (rc != 0) return fail(s->engine->last_error, rc);
+  *rows = s->engine->hListRows.data();
+  *cols = s->engine->hListCols.data();
+  *n_edges = (int64_t)s->engine->hListRows.size();
+  *list_start = s->engine->hListStart.data();
+  *n_samples = s->engine->num_samples();
+  return 0;
+}
+
 int nd_sampler_distinct(nd_sampler* s) {
   if (!s) return fail("null sampler");
   const int rc = s->engine->distinct();
@@ -338,6 +364,15 @@ int nd_sampler_check_results(nd_sampler* s, int* ok) {
   bool pass;
   // a layer-wise app whose sample state is the per-layer adjacency matrix
   // {len[L], row[L][B*B], col[L][B*B], val[L][B*B]} records edges instead of sampling along them
+  if (e.lists_edges()) {
+    const int rc2 = e.fetch_adjacency();
+    if (rc2 != 0) return fail(e.last_error, rc2);
+    pass = nd::check_subgraph_edge_lists(s->graph->csr, e.num_samples(), shape.initial_size, e.initialContents.data(),
+                                         e.hListStart.data(), e.hListRows.data(), e.hListCols.data(), &report);
+    *ok = pass ? 1 : 0;
+    if (!pass) g_error = report;
+    return 0;
+  }
   const size_t layers = shape.step_size.size(), cells = (size_t)shape.step_size[0] * shape.step_size[0];
   const size_t matrix_ints = layers + 3 * layers * cells;
   if (shape.collective && e.sample_state_bytes() == sizeof(int32_t) * matrix_ints * (size_t)e.num_samples()) {

@@ -177,4 +177,39 @@ bool check_layer_adjacency_matrix(const CSR& graph, const SampleShape& shape, in
   return !verdict.failed();
 }
 
+bool check_subgraph_edge_lists(const CSR& graph, int64_t n_samples, int vertices_per_sample, const int32_t* vertices,
+                               const uint32_t* list_start, const int32_t* rows, const int32_t* cols,
+                               std::string* report) {
+  Verdict verdict;
+  for_each_sample(n_samples, verdict, [&](int64_t s) {
+    const uint32_t begin = list_start[s], end = list_start[s + 1];
+    for (uint32_t e = begin; e < end; ++e) {
+      if (!adjacent(graph, rows[e], cols[e])) {
+        std::ostringstream msg;
+        msg << "Sample '" << s << "': no edge '" << rows[e] << "' -> '" << cols[e] << "' in graph";
+        verdict.fail(msg.str());
+        return;
+      }
+    }
+    const int32_t* mine = vertices + s * vertices_per_sample;
+    for (int a = 0; a < vertices_per_sample; ++a) {
+      for (int b = 0; b < vertices_per_sample; ++b) {
+        const int32_t v1 = mine[a], v2 = mine[b];
+        if (v1 == v2 || !adjacent(graph, v1, v2)) continue;
+        bool listed = false;
+        for (uint32_t e = begin; e < end && !listed; ++e) listed = rows[e] == v1 && cols[e] == v2;
+        if (!listed) {
+          std::ostringstream msg;
+          msg << "Sample '" << s << "': Edge '" << v1 << "'->'" << v2 << "' exists in graph but not in sample of length '"
+              << (end - begin) << "'";
+          verdict.fail(msg.str());
+          return;
+        }
+      }
+    }
+  });
+  if (verdict.failed() && report) *report = verdict.report();
+  return !verdict.failed();
+}
+
 }  // namespace nd

@@ -39,4 +39,13 @@ bool check_layer_adjacency_matrix(const CSR& graph, const SampleShape& shape, in
                                   const int32_t* initial, const int32_t* final_samples, const int32_t* rows,
                                   const int32_t* cols, size_t state_stride, int32_t invalid, std::string* report);
 
+// checkMVSResult / checkSubGraphResult (src/tests/multiGPU/mvs.cu:12-101,
+// src/tests/multiGPU/clustergcn.cu:10-93): sample s owns entries [list_start[s], list_start[s+1])
+// of rows / cols and the vertices[s * vertices_per_sample ...] it was built from.  Every listed
+// (row, col) must be an edge of the graph, and every edge of the graph between two different
+// vertices of the sample must be listed.
+bool check_subgraph_edge_lists(const CSR& graph, int64_t n_samples, int vertices_per_sample, const int32_t* vertices,
+                               const uint32_t* list_start, const int32_t* rows, const int32_t* cols,
+                               std::string* report);
+
 }  // namespace nd

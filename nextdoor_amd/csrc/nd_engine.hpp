@@ -89,10 +89,21 @@ class EngineBase {
   // engine-specific sizes of the last run (layer engine: 0 = entries of all collective
   // neighbourhoods, 1 = distinct (sample, vertex) pairs, 2 = chunks); 0 where not applicable
   virtual int64_t counter(int) const { return 0; }
+  // Apps with AdjacencyMatrix output on the per-transit engine (MVS, ClusterGCN): device ->
+  // hListStart / hListRows / hListCols
+  virtual bool lists_edges() const { return false; }
+  virtual int fetch_adjacency() {
+    last_error = "this app does not produce edge lists";
+    return -2;
+  }
 
   std::vector<VertexID_t> hFinalSamples;       // as NextDoorData::hFinalSamples (libNextDoor.hpp:17)
   std::vector<VertexID_t> initialContents;     // as NextDoorData::initialContents (libNextDoor.hpp:18)
   std::vector<int32_t> hDistinctCounts;        // [num_samples * steps] ids kept by distinct()
+  // edge lists of all samples, packed in sample order: sample s owns entries
+  // [hListStart[s], hListStart[s + 1]) of hListRows / hListCols
+  std::vector<uint32_t> hListStart;
+  std::vector<VertexID_t> hListRows, hListCols;
   std::string last_error;
   bool profiling = false;
   PhaseTimes times;

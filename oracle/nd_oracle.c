@@ -863,3 +863,88 @@ int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, ui
   }
   return 0;
 }
+
+/* ------------------------------------------------------------------------- */
+/* Edge-list apps: MVS and ClusterGCN                                         */
+/* ------------------------------------------------------------------------- */
+
+int64_t ndo_subgraph_num_samples(const ndo_graph* g, int vertices_per_sample, int64_t cap) {
+  if (g->n_edges > 100000000) return 800000;
+  const int64_t wanted = ((int64_t)g->n_vertices * 8 + vertices_per_sample - 1) / vertices_per_sample;
+  return wanted < cap ? wanted : cap;
+}
+
+void ndo_mvs_vertices(const ndo_graph* g, int64_t n_samples, int batch, int32_t* vertices) {
+  for (int64_t s = 0; s < n_samples; ++s)
+    for (int i = 0; i < batch; ++i) vertices[s * batch + i] = (int32_t)((s * batch + i) % g->n_vertices);
+}
+
+void ndo_clustergcn_vertices(const ndo_graph* g, int64_t n_samples, int cluster_size, int clusters_per_sample,
+                             int32_t* vertices) {
+  const int64_t n_clusters = g->n_vertices / cluster_size;
+  for (int64_t s = 0; s < n_samples; ++s) {
+    int32_t* mine = vertices + s * cluster_size * clusters_per_sample;
+    for (int i = 0; i < clusters_per_sample; ++i) {
+      const int64_t c = (s * clusters_per_sample + i) % n_clusters;
+      for (int v = 0; v < cluster_size; ++v) *mine++ = (int32_t)(c * cluster_size + v);
+    }
+  }
+}
+
+int64_t ndo_sample_mvs(const ndo_graph* g, int64_t n_samples, int batch, const int32_t* vertices,
+                       uint32_t* list_start, int32_t* rows, int32_t* cols) {
+  const int64_t lanes = (int64_t)batch * batch;  /* lane l = j * batch + nbr */
+  int64_t at = 0;
+  for (int64_t s = 0; s < n_samples; ++s) {
+    list_start[s] = (uint32_t)at;
+    for (int64_t first = 0; first < lanes; first += 64) {
+      const int64_t last = first + 64 < lanes ? first + 64 : lanes;
+      /* the i-th append of every lane of the group, lane after lane, for i = 0, 1, ... */
+      for (int32_t i = 0;; ++i) {
+        int any = 0;
+        for (int64_t l = first; l < last; ++l) {
+          const int32_t v = vertices[s * batch + l / batch];
+          const int32_t e = (int32_t)(l % batch) + i * batch;   /* mvsSampling.cu:36 */
+          if (e >= degree_of(g, v)) continue;
+          any = 1;
+          if (rows) { rows[at] = v; cols[at] = g->col[g->row_ptr[v] + e]; }
+          at++;
+        }
+        if (!any) break;
+      }
+    }
+  }
+  list_start[n_samples] = (uint32_t)at;
+  return at;
+}
+
+int64_t ndo_sample_clustergcn(const ndo_graph* g, int64_t n_samples, int n, const int32_t* vertices,
+                              int32_t* final_samples, uint32_t* list_start, int32_t* rows, int32_t* cols) {
+  const int32_t invalid = g->n_vertices;
+  const int64_t F = (int64_t)n + (int64_t)n * n;
+  int64_t at = 0;
+  for (int64_t s = 0; s < n_samples; ++s) {
+    const int32_t* mine = vertices + s * n;
+    list_start[s] = (uint32_t)at;
+    if (final_samples) {
+      for (int64_t i = 0; i < F; ++i) final_samples[s * F + i] = invalid;
+      /* step 0: next() returns the transit; it only runs for a transit with edges */
+      for (int j = 0; j < n; ++j)
+        if (degree_of(g, mine[j]) > 0) final_samples[s * F + j] = mine[j];
+    }
+    /* step 1: transits are the step-0 outputs */
+    for (int j = 0; j < n; ++j) {
+      const int32_t v1 = mine[j];
+      if (degree_of(g, v1) == 0) continue;
+      for (int nbr = 0; nbr < n; ++nbr) {
+        const int32_t v2 = mine[nbr];
+        if (ndo_has_edge(g, v1, v2)) {               /* clusterGCNSampling.cu:49-57 */
+          if (rows) { rows[at] = v1; cols[at] = v2; }
+          at++;
+        }
+      }
+    }
+  }
+  list_start[n_samples] = (uint32_t)at;
+  return at;
+}

@@ -232,6 +232,47 @@ int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, ui
                                  int64_t n_samples, int64_t first_sample, const int32_t* initial,
                                  int32_t* final_samples, ndo_stats* stats, int n_threads);
 
+/* ---- edge-list apps: MVS and ClusterGCN ----
+ * Both leave, per sample, a list of edges (row, col).  The reference appends to the list with
+ * atomicAdd(&sample->length, 1) (mvsSampling.cu:36-39, clusterGCNSampling.cu:52-57), so only
+ * the CONTENT of a list is fixed by it; the order used here is this repo's definition: the
+ * slots l = j * stepSize + nbr (transit index j, neighbour slot nbr) are taken in groups of 64
+ * consecutive l, and inside a group the appends are interleaved: the first append of every
+ * slot in slot order, then the second append of every slot, ...  (With at most one append per
+ * slot, as in ClusterGCN, that is plain slot order.)  Lists are packed in sample order: list_start[s] = edges of the samples before s,
+ * list_start[n_samples] = total.  rows / cols may be NULL (sizes only).  Return the total. */
+
+/* numSamples of both apps (mvsSampling.cu:57-60 cap 1500000, clusterGCNSampling.cu:84-87 cap
+ * 2000000): 800000 for graphs of more than 1e8 edges, else min(cap, ceil(8 V / vertices)). */
+int64_t ndo_subgraph_num_samples(const ndo_graph* g, int vertices_per_sample, int64_t cap);
+
+/* initialSample of MVS (mvsSampling.cu:74-94): vertex i of sample s = (s * batch + i) mod V. */
+void ndo_mvs_vertices(const ndo_graph* g, int64_t n_samples, int batch, int32_t* vertices);
+
+/* initialSample of ClusterGCN (clusterGCNSampling.cu:107-122, clusters built at 166-172):
+ * cluster c = vertices c*cluster_size .. +cluster_size-1, V / cluster_size clusters; sample s
+ * = clusters (s * n_clusters_per_sample + i) mod #clusters. */
+void ndo_clustergcn_vertices(const ndo_graph* g, int64_t n_samples, int cluster_size, int clusters_per_sample,
+                             int32_t* vertices);
+
+/* MVSSamplingApp::next (mvsSampling.cu:27-46): one step of `batch` slots per transit; slot nbr
+ * of transit v appends (v, adj(v)[e]) for e = nbr, nbr + batch, ...
+ * pinned by: the multiset of a sample's list equals the concatenated adjacencies of its
+ * vertices (numpy), and the reference's checkMVSResult rules (src/tests/multiGPU/mvs.cu:12-101). */
+int64_t ndo_sample_mvs(const ndo_graph* g, int64_t n_samples, int batch, const int32_t* vertices,
+                       uint32_t* list_start, int32_t* rows, int32_t* cols);
+
+/* SubGraphSamplingAppI::next (clusterGCNSampling.cu:32-73): step 0 returns the transit
+ * (an isolated vertex never reaches next(): INVALID, nextdoor.cu:250-262); step 1, slot nbr of
+ * transit v1 appends (v1, vertices[nbr]) when v1's adjacency holds vertices[nbr].
+ * final_samples: [n_samples][n + n*n], n = vertices per sample: the step-0 outputs, then
+ * INVALID (next returns -1 at step 1).
+ * pinned by: a dense adjacency-matrix brute force on small graphs (numpy) and the reference's
+ * checkSubGraphResult rules (src/tests/multiGPU/clustergcn.cu:10-93). */
+int64_t ndo_sample_clustergcn(const ndo_graph* g, int64_t n_samples, int vertices_per_sample,
+                              const int32_t* vertices, int32_t* final_samples, uint32_t* list_start,
+                              int32_t* rows, int32_t* cols);
+
 /* log2 of a positive normal float from exponent extraction and an atanh series; every step
  * is one IEEE single-precision operation.  pinned against libm (absolute error < 2e-6). */
 float ndo_det_log2(float x);

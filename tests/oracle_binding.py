@@ -77,6 +77,15 @@ def lib():
                                                C.c_int64, i32p, i32p, i32p, i32p, C.c_int]
         L.ndo_check_adjacency_matrix.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_int64, i32p, i32p,
                                                  i32p, i32p, C.c_int32]
+        u32p = C.POINTER(C.c_uint32)
+        L.ndo_subgraph_num_samples.restype = C.c_int64
+        L.ndo_subgraph_num_samples.argtypes = [C.POINTER(GraphStruct), C.c_int, C.c_int64]
+        L.ndo_mvs_vertices.argtypes = [C.POINTER(GraphStruct), C.c_int64, C.c_int, i32p]
+        L.ndo_clustergcn_vertices.argtypes = [C.POINTER(GraphStruct), C.c_int64, C.c_int, C.c_int, i32p]
+        L.ndo_sample_mvs.restype = C.c_int64
+        L.ndo_sample_mvs.argtypes = [C.POINTER(GraphStruct), C.c_int64, C.c_int, i32p, u32p, i32p, i32p]
+        L.ndo_sample_clustergcn.restype = C.c_int64
+        L.ndo_sample_clustergcn.argtypes = [C.POINTER(GraphStruct), C.c_int64, C.c_int, i32p, i32p, u32p, i32p, i32p]
         L.ndo_det_log2.restype = C.c_float
         L.ndo_det_log2.argtypes = [C.c_float]
         L.ndo_sample_ladies_importance.argtypes = [C.POINTER(GraphStruct), C.POINTER(AppDesc), C.c_uint64,
@@ -296,3 +305,47 @@ def sample_multirw(graph, seed, roots, steps, first_sample=0):
                               _p(last, C.c_int32), _p(final, C.c_int32), _p(transits, C.c_int32))
     assert rc == 0
     return final, walkers, last, transits
+
+
+def subgraph_num_samples(graph, vertices_per_sample, cap):
+    return lib().ndo_subgraph_num_samples(C.byref(graph.struct), vertices_per_sample, cap)
+
+
+def mvs_vertices(graph, n_samples, batch):
+    out = np.empty((n_samples, batch), dtype=np.int32)
+    lib().ndo_mvs_vertices(C.byref(graph.struct), n_samples, batch, _p(out, C.c_int32))
+    return out
+
+
+def clustergcn_vertices(graph, n_samples, cluster_size, clusters_per_sample):
+    out = np.empty((n_samples, cluster_size * clusters_per_sample), dtype=np.int32)
+    lib().ndo_clustergcn_vertices(C.byref(graph.struct), n_samples, cluster_size, clusters_per_sample,
+                                  _p(out, C.c_int32))
+    return out
+
+
+def sample_mvs(graph, vertices):
+    """(rows, cols, list_start) of MVS over vertices[n_samples][batch]."""
+    vertices = np.ascontiguousarray(vertices, dtype=np.int32)
+    n, batch = vertices.shape
+    start = np.zeros(n + 1, dtype=np.uint32)
+    total = lib().ndo_sample_mvs(C.byref(graph.struct), n, batch, _p(vertices, C.c_int32), _p(start, C.c_uint32),
+                                 None, None)
+    rows, cols = np.empty(total, dtype=np.int32), np.empty(total, dtype=np.int32)
+    lib().ndo_sample_mvs(C.byref(graph.struct), n, batch, _p(vertices, C.c_int32), _p(start, C.c_uint32),
+                         _p(rows, C.c_int32), _p(cols, C.c_int32))
+    return rows, cols, start
+
+
+def sample_clustergcn(graph, vertices):
+    """(final, rows, cols, list_start) of ClusterGCN over vertices[n_samples][n]."""
+    vertices = np.ascontiguousarray(vertices, dtype=np.int32)
+    n, per = vertices.shape
+    start = np.zeros(n + 1, dtype=np.uint32)
+    final = np.empty((n, per + per * per), dtype=np.int32)
+    total = lib().ndo_sample_clustergcn(C.byref(graph.struct), n, per, _p(vertices, C.c_int32), _p(final, C.c_int32),
+                                        _p(start, C.c_uint32), None, None)
+    rows, cols = np.empty(total, dtype=np.int32), np.empty(total, dtype=np.int32)
+    lib().ndo_sample_clustergcn(C.byref(graph.struct), n, per, _p(vertices, C.c_int32), _p(final, C.c_int32),
+                                _p(start, C.c_uint32), _p(rows, C.c_int32), _p(cols, C.c_int32))
+    return final, rows, cols, start
