@@ -287,6 +287,152 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   }
 }
 
+// The same marking with the presence map (and the importance sums) of one stretch of the vertex
+// range held in LDS: one workgroup per (sample, stretch).  Adjacencies are sorted by
+// destination, so the part of a transit's adjacency that falls into the stretch is one
+// sub-range, found by two binary searches; the workgroup streams the sub-ranges of all the
+// sample's transits, marks and adds in LDS, and writes the stretch out once - plain stores
+// that cover the whole map, so nothing is cleared beforehand and no atomic reaches memory
+// (global atomics stop at ~24 G/s on this part; the LADIES form needs 4.2e9 of them).
+constexpr uint32_t kBinThreads = 1024;
+constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
+constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
+
+template <bool kWithImportance>
+__global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
+    CSRPartition csr, TransitView tv, int32_t invalid, uint32_t bins_per_sample, uint32_t* __restrict__ bitmap,
+    uint32_t words_per_sample, const float* __restrict__ row_sums, unsigned long long* __restrict__ sums,
+    uint32_t sums_per_sample) {
+  constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
+  constexpr uint32_t kBinVertices = kBinWords * 32u;
+  // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
+  // packed into bits on the way out; LADIES form: bits and 64-bit sums, LDS atomics
+  __shared__ uint32_t s_bits[kWithImportance ? kBinWords : kBinVertices / 4u];
+  __shared__ unsigned long long s_acc[kWithImportance ? kBinVerticesSums : 1];
+  uint8_t* s_bytes = (uint8_t*)s_bits;
+  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i's sub-range in the stretch's entries
+  __shared__ EdgePos_t s_edge[kMaxLayerTransits];      // its first edge
+  const uint32_t s = blockIdx.x / bins_per_sample;
+  const uint32_t bin = blockIdx.x - s * bins_per_sample;
+  const uint32_t v_lo = bin * kBinVertices;
+  const int32_t* transits = tv.base + (size_t)s * tv.stride;
+  const uint32_t lane = threadIdx.x & 63u;
+  for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
+  if (kWithImportance)
+    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
+  for (uint32_t i = threadIdx.x; i < tv.count; i += kBinThreads) {
+    const int32_t t = transits[i];
+    EdgePos_t from = 0, to = 0;
+    if (t != invalid && t != -1) {
+      const EdgePos_t end = csr.row_ptr[t + 1];
+      // first edge whose destination is >= v_lo, then the first that is >= v_lo + kBinVertices
+      EdgePos_t lo = csr.row_ptr[t], hi = end;
+      while (lo < hi) {
+        const EdgePos_t mid = lo + (hi - lo) / 2;
+        if ((uint32_t)csr.edges[mid] < v_lo) lo = mid + 1; else hi = mid;
+      }
+      from = lo;
+      hi = end;
+      while (lo < hi) {
+        const EdgePos_t mid = lo + (hi - lo) / 2;
+        if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
+      }
+      to = lo;
+    }
+    s_start[i] = (uint32_t)(to - from);
+    s_edge[i] = from;
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {  // lengths -> starts
+    uint32_t carry = 0;
+    for (uint32_t c = 0; c < tv.count; c += 64) {
+      const uint32_t i = c + lane;
+      const uint32_t len = i < tv.count ? s_start[i] : 0u;
+      const uint32_t through = wave_inclusive_scan(len);
+      if (i < tv.count) s_start[i] = carry + through - len;
+      carry += __shfl(through, 63, kWave);
+    }
+    if (lane == 0) s_start[tv.count] = carry;
+  }
+  __syncthreads();
+  const uint32_t size = s_start[tv.count];
+  uint32_t cur_begin = 0, cur_end = 0;
+  EdgePos_t cur_edges = 0;
+  int32_t t = 0;
+  for (uint32_t e0 = 0; e0 < size; e0 += kBinThreads) {  // the same trip count for every lane
+    const uint32_t e = e0 + threadIdx.x;
+    uint32_t local = 0xFFFFFFFFu;  // vertex - v_lo
+    unsigned long long term = 0;
+    if (e < size) {
+      if (!(cur_begin <= e && e < cur_end)) {
+        uint32_t lo = 0, hi = tv.count;
+        while (hi - lo > 1) {
+          const uint32_t mid = lo + (hi - lo) / 2;
+          if (s_start[mid] <= e) lo = mid; else hi = mid;
+        }
+        cur_begin = s_start[lo];
+        cur_end = s_start[lo + 1];
+        cur_edges = s_edge[lo];
+        if (kWithImportance) t = transits[lo];
+      }
+      const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
+      local = (uint32_t)csr.edges[src] - v_lo;
+      if (kWithImportance) {
+        const float p = csr.weights[src] / row_sums[t];
+        term = importance_term_fixed(p * p);
+      }
+    }
+    if (kWithImportance) {
+      // parallel edges sit in neighbouring lanes: add their terms along the wave, when the
+      // wave holds any
+      const uint32_t left = __shfl_up(local, 1, kWave);
+      bool closed = lane == 0 || left != local;  // this lane starts a segment
+      bool last_of_segment = true;
+      if (__ballot(!closed && local != 0xFFFFFFFFu) != 0) {
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+          const uint32_t lo = __shfl_up((uint32_t)term, d, kWave);
+          const uint32_t hi = __shfl_up((uint32_t)(term >> 32), d, kWave);
+          const int up_closed = __shfl_up((int)closed, d, kWave);
+          if (lane >= (uint32_t)d) {
+            if (!closed) term += ((unsigned long long)hi << 32) | lo;
+            closed = closed || up_closed;
+          }
+        }
+        const uint32_t right = __shfl_down(local, 1, kWave);
+        last_of_segment = lane == 63u || right != local;
+      }
+      if (local != 0xFFFFFFFFu && last_of_segment) {
+        if (term != 0) atomicAdd(&s_acc[local], term);
+        atomicOr(&s_bits[local >> 5], 1u << (local & 31u));
+      }
+    } else if (local != 0xFFFFFFFFu) {
+      s_bytes[local] = 1;
+    }
+  }
+  __syncthreads();
+  const uint32_t first_word = bin * kBinWords;
+  uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
+  for (uint32_t i = threadIdx.x; i < kBinWords && first_word + i < words_per_sample; i += kBinThreads) {
+    uint32_t word = 0;
+    if (kWithImportance) {
+      word = s_bits[i];
+    } else {
+#pragma unroll
+      for (uint32_t q = 0; q < 8; ++q) {  // 32 bytes, each 0 or 1 -> 32 bits
+        const uint32_t four = s_bits[i * 8u + q];
+        word |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
+      }
+    }
+    out[i] = word;
+  }
+  if (kWithImportance) {
+    // only the sums of marked vertices are ever read
+    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads)
+      if ((s_bits[i >> 5] >> (i & 31u)) & 1u) sums[(size_t)s * sums_per_sample + v_lo + i] = s_acc[i];
+  }
+}
+
 // tile_counts[s * tiles_per_sample + t] = vertices marked in tile t of sample s's presence map
 // (a marked byte is 1, so the population count of a word counts marks in either layout)
 __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __restrict__ bitmap,
@@ -353,10 +499,8 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
         degree_sq[at] = d * d;
       }
       if (sums) {
-        // collect the vertex's importance and leave the accumulator clear for the next chunk
         unsigned long long* acc = sums + (size_t)sample * sums_per_sample + v;
         importance[at] = *acc;
-        *acc = 0;
         distinct_sample[at] = sample;
       }
     }
@@ -735,7 +879,7 @@ class LayerEngine : public EngineBase {
       if (v > 0) chunk_entries_ = bitmap_chunk_entries_ = (uint64_t)v;
     }
     // one byte per vertex for the LADIES form, one bit for the FastGCN form
-    const uint32_t per_word = App::kNeighborhoodForm == apps::kRankedByLadiesImportance ? 4u : 32u;
+    const uint32_t per_word = 32u;
     bitmap_words_ = (((uint32_t)invalid_ + per_word - 1u) / per_word + kBitmapTileWords - 1) / kBitmapTileWords *
                     kBitmapTileWords;
     // LADIES form: one 64-bit importance accumulator per vertex next to the bitmap
@@ -969,18 +1113,19 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
       ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
       if (ladies) {
-        // cleared once: the compaction leaves every accumulator it reads at zero again
+        // never cleared: the sum of a vertex is written whenever the vertex is marked, and read only then
         const size_t bytes = sizeof(unsigned long long) * (size_t)n * sums_per_sample_;
         ND_HIP_TRY(hipMalloc(&d_sums_, bytes));
-        ND_HIP_TRY(hipMemsetAsync(d_sums_, 0, bytes, stream_));
       }
       bitmap_samples_ = n;
     }
-    ND_HIP_TRY(hipMemsetAsync(d_bitmap_, 0, sizeof(uint32_t) * (size_t)n * bitmap_words_, stream_));
+    (void)n_items;
+    constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
+    const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
+    if ((uint64_t)n * bins >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
     tick();
-    collective_mark<ladies><<<dim3(n_items), dim3(256), 0, stream_>>>(dgraph_.view, tv, invalid_, d_item_start_, n,
-                                                                      d_bitmap_, bitmap_words_, d_row_sums_, d_sums_,
-                                                                      sums_per_sample_);
+    collective_mark_binned<ladies><<<dim3(n * bins), dim3(kBinThreads), 0, stream_>>>(
+        dgraph_.view, tv, invalid_, bins, d_bitmap_, bitmap_words_, d_row_sums_, d_sums_, sums_per_sample_);
     tock();
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
     ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
@@ -990,7 +1135,7 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
-    bitmap_compact<ladies><<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
+    bitmap_compact<false><<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
         d_bitmap_, d_tile_offsets_, tiles_per_sample, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
         d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
