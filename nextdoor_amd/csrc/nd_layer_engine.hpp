@@ -287,6 +287,51 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
   }
 }
 
+// ---- wave-wide data movement on the VALU (DPP), no LDS traffic ----
+// The value of the lane `shift` below inside the lane's row of 16; lanes without one get `fill`.
+template <int kShift>
+__device__ __forceinline__ uint32_t row_shift_up(uint32_t fill, uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, 0x110 | kShift, 0xF, 0xF, false);
+}
+// Lane 15 of the row below, for the rows chosen by kRowMask (row_bcast:15 / row_bcast:31).
+template <int kControl, int kRowMask>
+__device__ __forceinline__ uint32_t row_broadcast(uint32_t fill, uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, kControl, kRowMask, 0xF, false);
+}
+// The value of lane - 1 / lane + 1 across the whole wavefront; the end lanes get `fill`.
+__device__ __forceinline__ uint32_t wave_from_below(uint32_t fill, uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, 0x138, 0xF, 0xF, false);  // wave_shr:1
+}
+__device__ __forceinline__ uint32_t wave_from_above(uint32_t fill, uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, 0x130, 0xF, 0xF, false);  // wave_shl:1
+}
+
+// One step of a segmented inclusive sum along the wavefront: (closed, term) of this lane
+// takes in (up_closed, up_term) of a lane further down.  A lane is closed once its sum has
+// reached the start of its segment.
+__device__ __forceinline__ void take_in(uint32_t up_closed, uint32_t up_lo, uint32_t up_hi, uint32_t& closed,
+                                        unsigned long long& term) {
+  if (!closed) term += ((unsigned long long)up_hi << 32) | up_lo;
+  closed |= up_closed;
+}
+
+template <int kShift>
+__device__ __forceinline__ void segmented_row_step(uint32_t& closed, unsigned long long& term) {
+  // lanes without a source take in the neutral element (open, 0)
+  const uint32_t c = row_shift_up<kShift>(0u, closed);
+  const uint32_t lo = row_shift_up<kShift>(0u, (uint32_t)term);
+  const uint32_t hi = row_shift_up<kShift>(0u, (uint32_t)(term >> 32));
+  take_in(c, lo, hi, closed, term);
+}
+
+template <int kControl, int kRowMask>
+__device__ __forceinline__ void segmented_broadcast_step(uint32_t& closed, unsigned long long& term) {
+  const uint32_t c = row_broadcast<kControl, kRowMask>(0u, closed);
+  const uint32_t lo = row_broadcast<kControl, kRowMask>(0u, (uint32_t)term);
+  const uint32_t hi = row_broadcast<kControl, kRowMask>(0u, (uint32_t)(term >> 32));
+  take_in(c, lo, hi, closed, term);
+}
+
 // The same marking with the presence map (and the importance sums) of one stretch of the vertex
 // range held in LDS: one workgroup per (sample, stretch).  Adjacencies are sorted by
 // destination, so the part of a transit's adjacency that falls into the stretch is one
@@ -294,7 +339,13 @@ __global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, Transit
 // sample's transits, marks and adds in LDS, and writes the stretch out once - plain stores
 // that cover the whole map, so nothing is cleared beforehand and no atomic reaches memory
 // (global atomics stop at ~24 G/s on this part; the LADIES form needs 4.2e9 of them).
+// The LDS pipeline is what this kernel runs out of (counters: a wavefront waits for LDS a
+// third of its time), so it is kept for the map itself: every wavefront walks a contiguous
+// part of the stretch's entries, which lets a lane step from one sub-range to the next instead
+// of searching the table for every entry, and the sums along the wavefront move through DPP.
 constexpr uint32_t kBinThreads = 1024;
+constexpr uint32_t kBinWaves = kBinThreads / 64;
+constexpr uint32_t kBinAhead = 4;             // entries a lane fetches before it works on the first
 constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
@@ -310,19 +361,26 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __shared__ uint32_t s_bits[kWithImportance ? kBinWords : kBinVertices / 4u];
   __shared__ unsigned long long s_acc[kWithImportance ? kBinVerticesSums : 1];
   uint8_t* s_bytes = (uint8_t*)s_bits;
-  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i's sub-range in the stretch's entries
+  // the sub-ranges that hold entries, in transit order
+  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // first entry of sub-range k among the stretch's entries
   __shared__ EdgePos_t s_edge[kMaxLayerTransits];      // its first edge
+  __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // the weights of its transit added up
+  __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
+  __shared__ uint32_t s_ranges;                        // sub-ranges kept
   const uint32_t s = blockIdx.x / bins_per_sample;
   const uint32_t bin = blockIdx.x - s * bins_per_sample;
   const uint32_t v_lo = bin * kBinVertices;
   const int32_t* transits = tv.base + (size_t)s * tv.stride;
   const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = threadIdx.x >> 6;
   for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
   if (kWithImportance)
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
-  for (uint32_t i = threadIdx.x; i < tv.count; i += kBinThreads) {
-    const int32_t t = transits[i];
-    EdgePos_t from = 0, to = 0;
+  EdgePos_t my_from = 0;  // tv.count <= kBinThreads: a lane keeps its transit's sub-range
+  float my_row_sum = 1.0f;
+  if (threadIdx.x < tv.count) {
+    const int32_t t = transits[threadIdx.x];
+    EdgePos_t to = 0;
     if (t != invalid && t != -1) {
       const EdgePos_t end = csr.row_ptr[t + 1];
       // first edge whose destination is >= v_lo, then the first that is >= v_lo + kBinVertices
@@ -331,83 +389,127 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
         const EdgePos_t mid = lo + (hi - lo) / 2;
         if ((uint32_t)csr.edges[mid] < v_lo) lo = mid + 1; else hi = mid;
       }
-      from = lo;
+      my_from = lo;
       hi = end;
       while (lo < hi) {
         const EdgePos_t mid = lo + (hi - lo) / 2;
         if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
       }
       to = lo;
+      if (kWithImportance) my_row_sum = row_sums[t];
     }
-    s_start[i] = (uint32_t)(to - from);
-    s_edge[i] = from;
+    s_length[threadIdx.x] = (uint32_t)(to - my_from);
+    s_edge[threadIdx.x] = my_from;  // by transit for now
+    if (kWithImportance) s_row_sum[threadIdx.x] = my_row_sum;
   }
   __syncthreads();
-  if (threadIdx.x < 64) {  // lengths -> starts
-    uint32_t carry = 0;
+  // wave 0: drop the empty sub-ranges, turn lengths into starts (the tables are rewritten in
+  // place: an entry moves down or stays, and a round only writes below what it has read)
+  if (wave == 0) {
+    uint32_t kept = 0, entries = 0;
     for (uint32_t c = 0; c < tv.count; c += 64) {
       const uint32_t i = c + lane;
-      const uint32_t len = i < tv.count ? s_start[i] : 0u;
+      const uint32_t len = i < tv.count ? s_length[i] : 0u;
+      const EdgePos_t edge = i < tv.count ? s_edge[i] : 0;
+      const float row_sum = kWithImportance && i < tv.count ? s_row_sum[i] : 1.0f;
+      const uint64_t holds = __ballot(len != 0);
       const uint32_t through = wave_inclusive_scan(len);
-      if (i < tv.count) s_start[i] = carry + through - len;
-      carry += __shfl(through, 63, kWave);
+      if (len != 0) {
+        const uint32_t k = kept + (uint32_t)__popcll(holds & ((1ull << lane) - 1ull));
+        s_start[k] = entries + through - len;
+        s_edge[k] = edge;
+        if (kWithImportance) s_row_sum[k] = row_sum;
+      }
+      kept += (uint32_t)__popcll(holds);
+      entries += __shfl(through, 63, kWave);
     }
-    if (lane == 0) s_start[tv.count] = carry;
+    if (lane == 0) {
+      s_start[kept] = entries;
+      s_ranges = kept;
+    }
   }
   __syncthreads();
-  const uint32_t size = s_start[tv.count];
-  uint32_t cur_begin = 0, cur_end = 0;
+  const uint32_t ranges = s_ranges;
+  const uint32_t size = s_start[ranges];
+  // every wavefront walks a contiguous part of the entries, 64 * kBinAhead per round
+  constexpr uint32_t kRound = 64u * kBinAhead;
+  const uint32_t part = (size + kBinWaves * kRound - 1) / (kBinWaves * kRound) * kRound;
+  const uint32_t part_begin = wave * part;
+  const uint32_t part_end = part_begin + part < size ? part_begin + part : size;
+  uint32_t cur = 0, cur_begin = 0, cur_end = 0;
   EdgePos_t cur_edges = 0;
-  int32_t t = 0;
-  for (uint32_t e0 = 0; e0 < size; e0 += kBinThreads) {  // the same trip count for every lane
-    const uint32_t e = e0 + threadIdx.x;
-    uint32_t local = 0xFFFFFFFFu;  // vertex - v_lo
-    unsigned long long term = 0;
-    if (e < size) {
-      if (!(cur_begin <= e && e < cur_end)) {
-        uint32_t lo = 0, hi = tv.count;
-        while (hi - lo > 1) {
-          const uint32_t mid = lo + (hi - lo) / 2;
-          if (s_start[mid] <= e) lo = mid; else hi = mid;
+  float cur_row_sum = 1.0f;
+  if (part_begin + lane < part_end) {  // the sub-range of the lane's first entry
+    const uint32_t e = part_begin + lane;
+    uint32_t lo = 0, hi = ranges;
+    while (hi - lo > 1) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (s_start[mid] <= e) lo = mid; else hi = mid;
+    }
+    cur = lo;
+    cur_begin = s_start[lo];
+    cur_end = s_start[lo + 1];
+    cur_edges = s_edge[lo];
+    if (kWithImportance) cur_row_sum = s_row_sum[lo];
+  }
+  for (uint32_t e0 = part_begin; e0 < part_end; e0 += kRound) {  // the same trip count for every lane of a wave
+    uint32_t locals[kBinAhead];  // vertex - v_lo
+    float weights[kBinAhead], sums_of_row[kBinAhead];
+#pragma unroll
+    for (uint32_t a = 0; a < kBinAhead; ++a) {
+      const uint32_t e = e0 + a * 64u + lane;
+      locals[a] = 0xFFFFFFFFu;
+      weights[a] = 0.0f;
+      sums_of_row[a] = 1.0f;
+      if (e < part_end) {
+        if (e >= cur_end) {
+          do {  // no sub-range is empty: at most a few steps
+            ++cur;
+            cur_begin = cur_end;
+            cur_end = s_start[cur + 1];
+          } while (e >= cur_end);
+          cur_edges = s_edge[cur];
+          if (kWithImportance) cur_row_sum = s_row_sum[cur];
         }
-        cur_begin = s_start[lo];
-        cur_end = s_start[lo + 1];
-        cur_edges = s_edge[lo];
-        if (kWithImportance) t = transits[lo];
-      }
-      const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
-      local = (uint32_t)csr.edges[src] - v_lo;
-      if (kWithImportance) {
-        const float p = csr.weights[src] / row_sums[t];
-        term = importance_term_fixed(p * p);
+        const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
+        locals[a] = (uint32_t)csr.edges[src] - v_lo;
+        if (kWithImportance) {
+          weights[a] = csr.weights[src];
+          sums_of_row[a] = cur_row_sum;
+        }
       }
     }
-    if (kWithImportance) {
-      // parallel edges sit in neighbouring lanes: add their terms along the wave, when the
-      // wave holds any
-      const uint32_t left = __shfl_up(local, 1, kWave);
-      bool closed = lane == 0 || left != local;  // this lane starts a segment
-      bool last_of_segment = true;
-      if (__ballot(!closed && local != 0xFFFFFFFFu) != 0) {
 #pragma unroll
-        for (int d = 1; d < kWave; d <<= 1) {
-          const uint32_t lo = __shfl_up((uint32_t)term, d, kWave);
-          const uint32_t hi = __shfl_up((uint32_t)(term >> 32), d, kWave);
-          const int up_closed = __shfl_up((int)closed, d, kWave);
-          if (lane >= (uint32_t)d) {
-            if (!closed) term += ((unsigned long long)hi << 32) | lo;
-            closed = closed || up_closed;
-          }
+    for (uint32_t a = 0; a < kBinAhead; ++a) {
+      const uint32_t local = locals[a];
+      if (kWithImportance) {
+        unsigned long long term = 0;
+        if (local != 0xFFFFFFFFu) {
+          const float p = weights[a] / sums_of_row[a];
+          term = importance_term_fixed(p * p);
         }
-        const uint32_t right = __shfl_down(local, 1, kWave);
-        last_of_segment = lane == 63u || right != local;
+        // parallel edges sit in neighbouring lanes: add their terms along the wave, when the
+        // wave holds any.  0xFFFFFFFE: no lane holds it, so lane 0 always starts a segment.
+        const uint32_t left = wave_from_below(0xFFFFFFFEu, local);
+        uint32_t closed = left != local ? 1u : 0u;
+        bool last_of_segment = true;
+        if (__ballot(closed == 0 && local != 0xFFFFFFFFu) != 0) {
+          segmented_row_step<1>(closed, term);
+          segmented_row_step<2>(closed, term);
+          segmented_row_step<4>(closed, term);
+          segmented_row_step<8>(closed, term);
+          segmented_broadcast_step<0x142, 0xA>(closed, term);  // rows 1 and 3 take in the row below
+          segmented_broadcast_step<0x143, 0xC>(closed, term);  // rows 2 and 3 take in lane 31
+          const uint32_t right = wave_from_above(0xFFFFFFFEu, local);
+          last_of_segment = right != local;
+        }
+        if (local != 0xFFFFFFFFu && last_of_segment) {
+          if (term != 0) atomicAdd(&s_acc[local], term);
+          atomicOr(&s_bits[local >> 5], 1u << (local & 31u));
+        }
+      } else if (local != 0xFFFFFFFFu) {
+        s_bytes[local] = 1;
       }
-      if (local != 0xFFFFFFFFu && last_of_segment) {
-        if (term != 0) atomicAdd(&s_acc[local], term);
-        atomicOr(&s_bits[local >> 5], 1u << (local & 31u));
-      }
-    } else if (local != 0xFFFFFFFFu) {
-      s_bytes[local] = 1;
     }
   }
   __syncthreads();
