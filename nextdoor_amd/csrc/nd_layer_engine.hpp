@@ -144,159 +144,39 @@ __global__ __launch_bounds__(256) void collective_build(CSRPartition csr, Transi
   }
 }
 
-// (weight / rowsum)^2 as a 2^53 fixed-point integer: sums of up to 1024 of them fit 64 bits
-// and, unlike float sums, do not depend on the order of the additions.
+// (weight * (1 / rowsum))^2 as a 2^53 fixed-point integer, truncated: sums of up to 1024 of
+// them fit 64 bits and, unlike float sums, do not depend on the order of the additions.
+// A float in (0, 1) is (2^23 + m) * 2^(e - 150) with exponent field e and mantissa m, so the
+// product with 2^53 is the 24-bit mantissa shifted by e - 97; the same integer as
+// (unsigned long long)(term * 2^53f), without a float -> 64-bit conversion.
 __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(float term) {
-  if (!(term > 0.0f)) return 0ull;
-  if (term >= 1.0f) return 1ull << 53;
-  return (unsigned long long)(term * 9007199254740992.0f);  // * 2^53: exact, then truncated
+  uint32_t bits;
+  __builtin_memcpy(&bits, &term, sizeof(bits));
+  if ((int32_t)bits <= 0) return 0ull;  // zero or negative
+  if (bits >= 0x3F800000u) return bits > 0x7F800000u ? 0ull : 1ull << 53;  // >= 1 (NaN: 0)
+  const uint32_t e = bits >> 23;
+  const uint32_t mantissa = (bits & 0x7FFFFFu) | (e ? 0x800000u : 0u);
+  const int shift = (int)e - 97;
+  if (shift >= 0) return (unsigned long long)mantissa << shift;
+  return shift > -24 ? (unsigned long long)(mantissa >> -shift) : 0ull;
 }
 
 // ---- distinct vertices of a collective neighbourhood through a presence map ----
 //
-// Per sample of the chunk a map over the vertices (words_per_sample 32-bit words, a multiple
-// of the tile below).  collective_mark walks the neighbourhood exactly as collective_build
-// does, but instead of copying an entry it marks the entry's vertex; nothing of the
-// concatenation is stored.  A neighbourhood that sits on hubs repeats its vertices many
-// times over (3.8e10 entries hold 2.0e9 distinct pairs at FastGCN's full size), so the map
-// is read first and only written where the vertex is not marked yet; a stale read costs one
-// redundant write, never a wrong mark.
-//
-// Two layouts.  One BIT per vertex (FastGCN form): 8 times smaller to clear, count and
-// compact, and the lanes of a dense row share a few words; the price is one atomic OR per new
-// word-stretch.  One BYTE per vertex (LADIES form, kWithImportance): every writer stores the
-// same value 1, so plain stores do.  Atomics of any width top out at ~24 G/s on this part,
-// and the LADIES form already spends that on its importance sums: with bits, marking 3.8e10
-// entries took 477 ms there, with bytes 403 ms; for FastGCN the bit map wins (143 vs 152 ms
-// per pass) because the byte maps of 4096 batches are 17 GB to clear, count and compact.
-constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words: 65536 vertices as bits, 8192 as bytes
-
-// kWithImportance (LADIES form): every entry also adds (weight / row_sums[transit])^2, as a
-// fixed-point integer, to sums[sample * sums_per_sample + vertex].  Parallel edges make a
-// vertex repeat in neighbouring lanes; their terms are added up along the wavefront first
-// (a segmented scan in which a lane whose vertex differs from its left neighbour's starts a
-// new segment) and the last lane of each segment issues the one atomic.
-template <bool kWithImportance>
-__global__ __launch_bounds__(256) void collective_mark(CSRPartition csr, TransitView tv, int32_t invalid,
-                                                       const uint32_t* __restrict__ item_start, uint32_t n_samples,
-                                                       uint32_t* __restrict__ bitmap, uint32_t words_per_sample,
-                                                       const float* __restrict__ row_sums,
-                                                       unsigned long long* __restrict__ sums,
-                                                       uint32_t sums_per_sample) {
-  __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // start of transit i inside the sample's concatenation
-  __shared__ uint32_t s_scan_tmp[4];
-  uint32_t lo_s = 0, hi_s = n_samples;
-  while (hi_s - lo_s > 1) {
-    const uint32_t mid = lo_s + (hi_s - lo_s) / 2;
-    if (item_start[mid] <= blockIdx.x) lo_s = mid; else hi_s = mid;
-  }
-  const uint32_t s = lo_s;
-  const uint32_t item = blockIdx.x - item_start[s];
-  const int32_t* transits = tv.base + (size_t)s * tv.stride;
-  uint32_t carry = 0;
-  for (uint32_t chunk = 0; chunk < tv.count; chunk += 256) {
-    const uint32_t i = chunk + threadIdx.x;
-    uint32_t deg = 0;
-    if (i < tv.count) {
-      const int32_t t = transits[i];
-      if (t != invalid && t != -1) deg = (uint32_t)(csr.row_ptr[t + 1] - csr.row_ptr[t]);
-    }
-    uint32_t total;
-    const uint32_t excl = block_exclusive_scan_256(deg, s_scan_tmp, &total);
-    if (i < tv.count) s_start[i] = carry + excl;
-    carry += total;
-  }
-  if (threadIdx.x == 0) s_start[tv.count] = carry;
-  __syncthreads();
-  const uint32_t size = s_start[tv.count];
-  uint32_t* present_of_sample = bitmap + (size_t)s * words_per_sample;
-  const uint32_t first = item * kBuildItemEntries;
-  const uint32_t last = first + kBuildItemEntries < size ? first + kBuildItemEntries : size;
-  // the transit whose adjacency holds the lane's entry changes rarely: its range inside the
-  // concatenation, its first edge and its row sum stay in registers
-  uint32_t cur_begin = 0, cur_end = 0;
-  EdgePos_t cur_edges = 0;
-  int32_t t = 0;
-  const uint32_t lane = threadIdx.x & 63u;
-  for (uint32_t e0 = first; e0 < last; e0 += 256) {  // the same trip count for every lane
-    const uint32_t e = e0 + threadIdx.x;
-    uint32_t vertex = 0xFFFFFFFFu;
-    unsigned long long term = 0;
-    if (e < last) {
-      if (!(cur_begin <= e && e < cur_end)) {
-        uint32_t lo = 0, hi = tv.count;
-        while (hi - lo > 1) {
-          const uint32_t mid = lo + (hi - lo) / 2;
-          if (s_start[mid] <= e) lo = mid; else hi = mid;
-        }
-        cur_begin = s_start[lo];
-        cur_end = s_start[lo + 1];
-        t = transits[lo];
-        cur_edges = csr.row_ptr[t];
-      }
-      const EdgePos_t src = cur_edges + (EdgePos_t)(e - cur_begin);
-      vertex = (uint32_t)csr.edges[src];
-      if (kWithImportance) {
-        const float p = csr.weights[src] / row_sums[t];
-        term = importance_term_fixed(p * p);
-      }
-    }
-    if (kWithImportance) {
-      const uint32_t left = __shfl_up(vertex, 1, kWave);
-      bool closed = lane == 0 || left != vertex;  // this lane starts a segment
-#pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t lo = __shfl_up((uint32_t)term, d, kWave);
-        const uint32_t hi = __shfl_up((uint32_t)(term >> 32), d, kWave);
-        const int up_closed = __shfl_up((int)closed, d, kWave);
-        if (lane >= (uint32_t)d) {
-          if (!closed) term += ((unsigned long long)hi << 32) | lo;
-          closed = closed || up_closed;
-        }
-      }
-      const uint32_t right = __shfl_down(vertex, 1, kWave);
-      if (vertex != 0xFFFFFFFFu && term != 0 && (lane == 63u || right != vertex))
-        atomicAdd(sums + (size_t)s * sums_per_sample + vertex, term);
-    }
-    if (kWithImportance) {
-      if (vertex != 0xFFFFFFFFu) {
-        uint8_t* mark = (uint8_t*)present_of_sample + vertex;
-        if (*mark == 0) *mark = 1;
-      }
-    } else {
-      // Adjacencies are sorted, so neighbouring lanes mostly hit the same word: OR the bits
-      // of equal words along the wave and let the last lane of each stretch do the memory
-      // work (a dense hub row then costs 8 words per wavefront instead of 64).
-      uint32_t word_index = 0xFFFFFFFFu, bits = 0;
-      if (vertex != 0xFFFFFFFFu) {
-        word_index = vertex >> 5;
-        bits = 1u << (vertex & 31u);
-      }
-#pragma unroll
-      for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t up_index = __shfl_up(word_index, d, kWave);
-        const uint32_t up_bits = __shfl_up(bits, d, kWave);
-        if (lane >= (uint32_t)d && up_index == word_index) bits |= up_bits;
-      }
-      const uint32_t next_index = __shfl_down(word_index, 1, kWave);
-      if (bits != 0 && (lane == 63u || next_index != word_index)) {
-        uint32_t* word = present_of_sample + word_index;
-        if ((*word & bits) != bits) atomicOr(word, bits);
-      }
-    }
-  }
-}
+// Per sample of the chunk a bitmap over the vertices (words_per_sample 32-bit words, a multiple
+// of the tile below).  collective_mark_binned walks the neighbourhood as collective_build does,
+// but instead of copying an entry it marks the entry's vertex; nothing of the concatenation is
+// stored.  A neighbourhood that sits on hubs repeats its vertices many times over (3.8e10
+// entries hold 2.0e9 distinct pairs at FastGCN's full size).
+// LADIES form (kWithImportance): every entry also adds (weight * inverse_row_sum[transit])^2, as
+// a 2^53 fixed-point integer, to the 64-bit sum of (sample, vertex).
+constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words: 65536 vertices
 
 // ---- wave-wide data movement on the VALU (DPP), no LDS traffic ----
 // The value of the lane `shift` below inside the lane's row of 16; lanes without one get `fill`.
 template <int kShift>
 __device__ __forceinline__ uint32_t row_shift_up(uint32_t fill, uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, 0x110 | kShift, 0xF, 0xF, false);
-}
-// Lane 15 of the row below, for the rows chosen by kRowMask (row_bcast:15 / row_bcast:31).
-template <int kControl, int kRowMask>
-__device__ __forceinline__ uint32_t row_broadcast(uint32_t fill, uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, kControl, kRowMask, 0xF, false);
 }
 // The value of lane - 1 / lane + 1 across the whole wavefront; the end lanes get `fill`.
 __device__ __forceinline__ uint32_t wave_from_below(uint32_t fill, uint32_t x) {
@@ -306,7 +186,7 @@ __device__ __forceinline__ uint32_t wave_from_above(uint32_t fill, uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)x, 0x130, 0xF, 0xF, false);  // wave_shl:1
 }
 
-// One step of a segmented inclusive sum along the wavefront: (closed, term) of this lane
+// One step of a segmented inclusive sum along a row of 16 lanes: (closed, term) of this lane
 // takes in (up_closed, up_term) of a lane further down.  A lane is closed once its sum has
 // reached the start of its segment.
 __device__ __forceinline__ void take_in(uint32_t up_closed, uint32_t up_lo, uint32_t up_hi, uint32_t& closed,
@@ -321,14 +201,6 @@ __device__ __forceinline__ void segmented_row_step(uint32_t& closed, unsigned lo
   const uint32_t c = row_shift_up<kShift>(0u, closed);
   const uint32_t lo = row_shift_up<kShift>(0u, (uint32_t)term);
   const uint32_t hi = row_shift_up<kShift>(0u, (uint32_t)(term >> 32));
-  take_in(c, lo, hi, closed, term);
-}
-
-template <int kControl, int kRowMask>
-__device__ __forceinline__ void segmented_broadcast_step(uint32_t& closed, unsigned long long& term) {
-  const uint32_t c = row_broadcast<kControl, kRowMask>(0u, closed);
-  const uint32_t lo = row_broadcast<kControl, kRowMask>(0u, (uint32_t)term);
-  const uint32_t hi = row_broadcast<kControl, kRowMask>(0u, (uint32_t)(term >> 32));
   take_in(c, lo, hi, closed, term);
 }
 
@@ -352,7 +224,8 @@ constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit su
 template <bool kWithImportance>
 __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t bins_per_sample, uint32_t* __restrict__ bitmap,
-    uint32_t words_per_sample, const float* __restrict__ row_sums, unsigned long long* __restrict__ sums,
+    uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
+    unsigned long long* __restrict__ sums,
     uint32_t sums_per_sample) {
   constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
   constexpr uint32_t kBinVertices = kBinWords * 32u;
@@ -364,7 +237,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   // the sub-ranges that hold entries, in transit order
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // first entry of sub-range k among the stretch's entries
   __shared__ EdgePos_t s_edge[kMaxLayerTransits];      // its first edge
-  __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // the weights of its transit added up
+  __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // 1 / (the weights of its transit added up)
   __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
   __shared__ uint32_t s_ranges;                        // sub-ranges kept
   const uint32_t s = blockIdx.x / bins_per_sample;
@@ -396,7 +269,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
         if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
       }
       to = lo;
-      if (kWithImportance) my_row_sum = row_sums[t];
+      if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
     s_length[threadIdx.x] = (uint32_t)(to - my_from);
     s_edge[threadIdx.x] = my_from;  // by transit for now
@@ -485,25 +358,26 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
       if (kWithImportance) {
         unsigned long long term = 0;
         if (local != 0xFFFFFFFFu) {
-          const float p = weights[a] / sums_of_row[a];
+          const float p = weights[a] * sums_of_row[a];
           term = importance_term_fixed(p * p);
         }
-        // parallel edges sit in neighbouring lanes: add their terms along the wave, when the
-        // wave holds any.  0xFFFFFFFE: no lane holds it, so lane 0 always starts a segment.
+        // Parallel edges sit in neighbouring lanes.  A few of them may as well hit the same
+        // LDS word one after the other; a run of four or more somewhere in the wave (hub pairs
+        // are joined by thousands of edges) is added up first, inside the rows of 16 lanes.
+        // 0xFFFFFFFE: no lane holds it, so lane 0 always starts a segment.
         const uint32_t left = wave_from_below(0xFFFFFFFEu, local);
-        uint32_t closed = left != local ? 1u : 0u;
-        bool last_of_segment = true;
-        if (__ballot(closed == 0 && local != 0xFFFFFFFFu) != 0) {
+        uint32_t closed = (left != local || (lane & 15u) == 0) ? 1u : 0u;
+        const uint64_t repeats = __ballot(left == local && local != 0xFFFFFFFFu);
+        bool adds = true;  // this lane adds its term to the vertex's sum
+        if ((repeats & (repeats >> 1) & (repeats >> 2)) != 0) {
           segmented_row_step<1>(closed, term);
           segmented_row_step<2>(closed, term);
           segmented_row_step<4>(closed, term);
           segmented_row_step<8>(closed, term);
-          segmented_broadcast_step<0x142, 0xA>(closed, term);  // rows 1 and 3 take in the row below
-          segmented_broadcast_step<0x143, 0xC>(closed, term);  // rows 2 and 3 take in lane 31
           const uint32_t right = wave_from_above(0xFFFFFFFEu, local);
-          last_of_segment = right != local;
+          adds = right != local || (lane & 15u) == 15u;
         }
-        if (local != 0xFFFFFFFFu && last_of_segment) {
+        if (local != 0xFFFFFFFFu && adds) {
           if (term != 0) atomicAdd(&s_acc[local], term);
           atomicOr(&s_bits[local >> 5], 1u << (local & 31u));
         }
@@ -536,7 +410,6 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
 }
 
 // tile_counts[s * tiles_per_sample + t] = vertices marked in tile t of sample s's presence map
-// (a marked byte is 1, so the population count of a word counts marks in either layout)
 __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __restrict__ bitmap,
                                                           uint32_t* __restrict__ tile_counts) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
@@ -553,7 +426,6 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
 // tile of a sample is where the sample's list starts).  Per distinct vertex either
 // degree^2 (degree_sq given) or the importance accumulated in sums (sums given).
-template <bool kBytes>
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t tiles_per_sample, const EdgePos_t* __restrict__ row_ptr,
@@ -585,11 +457,10 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t first_word = wave * kWordsPerWave;
   uint32_t r = first + s_before[first_word / 8];
-  const uint8_t* bytes = (const uint8_t*)words;
-  constexpr uint32_t kWordsPerRound = kBytes ? 16u : 2u;     // 64 vertices
-  constexpr uint32_t kVerticesPerWord = kBytes ? 4u : 32u;
+  constexpr uint32_t kWordsPerRound = 2u;  // 64 vertices
+  constexpr uint32_t kVerticesPerWord = 32u;
   for (uint32_t w = first_word; w < first_word + kWordsPerWave; w += kWordsPerRound) {
-    const bool set = kBytes ? bytes[w * 4u + lane] != 0 : ((words[w + (lane >> 5)] >> (lane & 31u)) & 1u) != 0;
+    const bool set = ((words[w + (lane >> 5)] >> (lane & 31u)) & 1u) != 0;
     const uint64_t mask = __ballot(set);
     if (mask == 0) continue;  // the same for every lane
     if (set) {
@@ -919,13 +790,13 @@ class LayerEngine : public EngineBase {
     release(d_row_sums_);
     if (!dgraph_.upload(graph, false, app_uses_edge_lookup<App>::value, &last_error)) return -1;
     if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
-      // weights of every vertex summed in edge order (sequential float adds)
+      // 1 / (weights of every vertex summed in edge order, sequential float adds)
       const size_t V = (size_t)graph->get_n_vertices();
       std::vector<float> sums(V);
       for (size_t v = 0; v < V; ++v) {
         float acc = 0.0f;
         for (EdgePos_t x = graph->row_ptr[v]; x < graph->row_ptr[v + 1]; ++x) acc = acc + graph->weight[x];
-        sums[v] = acc;
+        sums[v] = 1.0f / acc;  // the kernels multiply by the inverse
       }
       ND_HIP_TRY(hipMalloc(&d_row_sums_, sizeof(float) * V));
       ND_HIP_TRY(hipMemcpy(d_row_sums_, sums.data(), sizeof(float) * V, hipMemcpyHostToDevice));
@@ -1237,7 +1108,7 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
-    bitmap_compact<false><<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
+    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
         d_bitmap_, d_tile_offsets_, tiles_per_sample, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
         d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);

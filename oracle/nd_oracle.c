@@ -762,7 +762,7 @@ static uint32_t descending_key_bits(float key) {
   return ~b;
 }
 
-/* (weight / rowsum)^2 as a 2^53 fixed-point integer (exact scaling, truncation) */
+/* (weight * (1 / rowsum))^2 as a 2^53 fixed-point integer (exact scaling, truncation) */
 static uint64_t term_fixed(float term) {
   if (!(term > 0.0f)) return 0;
   if (term >= 1.0f) return (uint64_t)1 << 53;
@@ -816,7 +816,7 @@ int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, ui
         const int32_t u = transits[i];
         if (u == invalid || u == -1) continue;
         for (int32_t x = g->row_ptr[u]; x < g->row_ptr[u + 1]; ++x) {
-          const float p = g->weight[x] / rowsum[u];
+          const float p = g->weight[x] * (1.0f / rowsum[u]);
           term[at] = p * p;
           occ[at].vertex = g->col[x];
           occ[at].pos = at;

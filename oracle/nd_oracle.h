@@ -217,8 +217,8 @@ int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, u
 /* LADIES-style layer-dependent importance sampling (own definition; parity unpinned by
  * the reference, whose LADIES app is the literal one above).  For a layer with frontier
  * (transits) U: every occurrence (u, x) of an edge u -> v = col[x], u a valid transit, in
- * contributes term = (w_x / rowsum_u)^2 (float), rowsum_u = the weights of u summed in edge
- * order (float, sequential).  importance(v) = the terms of v's occurrences, each truncated
+ * contributes term = (w_x * (1 / rowsum_u))^2 (float; the inverse rounded once per row),
+ * rowsum_u = the weights of u summed in edge order (float, sequential).  importance(v) = the terms of v's occurrences, each truncated
  * to a 2^53 fixed-point integer and summed exactly (so the sum does not depend on the order
  * of the additions), converted to float: the squared column norm of the row-normalised
  * adjacency restricted to the frontier, times 2^53.  m_k vertices are drawn WITHOUT replacement with probability
