@@ -218,6 +218,7 @@ __device__ __forceinline__ void segmented_row_step(uint32_t& closed, unsigned lo
 constexpr uint32_t kBinThreads = 1024;
 constexpr uint32_t kBinWaves = kBinThreads / 64;
 constexpr uint32_t kBinAhead = 4;             // entries a lane fetches before it works on the first
+constexpr uint32_t kBinsPerGroup = 8;         // consecutive stretches of a sample one workgroup takes
 constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
@@ -240,38 +241,55 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // 1 / (the weights of its transit added up)
   __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
   __shared__ uint32_t s_ranges;                        // sub-ranges kept
-  const uint32_t s = blockIdx.x / bins_per_sample;
-  const uint32_t bin = blockIdx.x - s * bins_per_sample;
-  const uint32_t v_lo = bin * kBinVertices;
+  // A workgroup takes kBinsPerGroup consecutive stretches of one sample, one after the other:
+  // where a transit's sub-range ends in one stretch it begins in the next, and the end is
+  // then only a short gallop away instead of a search of the whole adjacency.
+  const uint32_t groups_per_sample = (bins_per_sample + kBinsPerGroup - 1) / kBinsPerGroup;
+  const uint32_t s = blockIdx.x / groups_per_sample;
+  const uint32_t first_bin = (blockIdx.x - s * groups_per_sample) * kBinsPerGroup;
   const int32_t* transits = tv.base + (size_t)s * tv.stride;
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = threadIdx.x >> 6;
-  for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
-  if (kWithImportance)
-    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
-  EdgePos_t my_from = 0;  // tv.count <= kBinThreads: a lane keeps its transit's sub-range
+  // tv.count <= kBinThreads: lane i keeps transit i's adjacency and how far the stretches
+  // before this one reach into it
+  EdgePos_t my_end = 0, my_reach = 0;
   float my_row_sum = 1.0f;
   if (threadIdx.x < tv.count) {
     const int32_t t = transits[threadIdx.x];
-    EdgePos_t to = 0;
     if (t != invalid && t != -1) {
-      const EdgePos_t end = csr.row_ptr[t + 1];
-      // first edge whose destination is >= v_lo, then the first that is >= v_lo + kBinVertices
-      EdgePos_t lo = csr.row_ptr[t], hi = end;
+      my_end = csr.row_ptr[t + 1];
+      EdgePos_t lo = csr.row_ptr[t], hi = my_end;  // first edge whose destination is in the first stretch or above
+      const uint32_t v_first = first_bin * kBinVertices;
       while (lo < hi) {
         const EdgePos_t mid = lo + (hi - lo) / 2;
-        if ((uint32_t)csr.edges[mid] < v_lo) lo = mid + 1; else hi = mid;
+        if ((uint32_t)csr.edges[mid] < v_first) lo = mid + 1; else hi = mid;
       }
-      my_from = lo;
-      hi = end;
-      while (lo < hi) {
-        const EdgePos_t mid = lo + (hi - lo) / 2;
-        if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
-      }
-      to = lo;
+      my_reach = lo;
       if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
-    s_length[threadIdx.x] = (uint32_t)(to - my_from);
+  }
+  for (uint32_t bin = first_bin; bin < first_bin + kBinsPerGroup && bin < bins_per_sample; ++bin) {
+  const uint32_t v_lo = bin * kBinVertices;
+  for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
+  if (kWithImportance)
+    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
+  if (threadIdx.x < tv.count) {
+    const EdgePos_t my_from = my_reach;
+    // first edge at or after my_from whose destination is >= v_lo + kBinVertices: gallop, then bisect
+    EdgePos_t lo = my_from, width = 64;
+    while (lo < my_end) {
+      const EdgePos_t probe = lo + width < my_end ? lo + width : my_end;
+      if ((uint32_t)csr.edges[probe - 1] >= v_lo + kBinVertices) break;
+      lo = probe;
+      width <<= 1;
+    }
+    EdgePos_t hi = lo + width < my_end ? lo + width : my_end;
+    while (lo < hi) {
+      const EdgePos_t mid = lo + (hi - lo) / 2;
+      if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
+    }
+    my_reach = lo;
+    s_length[threadIdx.x] = (uint32_t)(my_reach - my_from);
     s_edge[threadIdx.x] = my_from;  // by transit for now
     if (kWithImportance) s_row_sum[threadIdx.x] = my_row_sum;
   }
@@ -406,6 +424,8 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     // only the sums of marked vertices are ever read
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads)
       if ((s_bits[i >> 5] >> (i & 31u)) & 1u) sums[(size_t)s * sums_per_sample + v_lo + i] = s_acc[i];
+  }
+  __syncthreads();  // the next stretch clears what this one has just read
   }
 }
 
@@ -1095,9 +1115,10 @@ class LayerEngine : public EngineBase {
     (void)n_items;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
-    if ((uint64_t)n * bins >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
+    const uint32_t groups = (bins + kBinsPerGroup - 1) / kBinsPerGroup;
+    if ((uint64_t)n * groups >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
     tick();
-    collective_mark_binned<ladies><<<dim3(n * bins), dim3(kBinThreads), 0, stream_>>>(
+    collective_mark_binned<ladies><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
         dgraph_.view, tv, invalid_, bins, d_bitmap_, bitmap_words_, d_row_sums_, d_sums_, sums_per_sample_);
     tock();
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
