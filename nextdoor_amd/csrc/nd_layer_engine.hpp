@@ -218,13 +218,17 @@ __device__ __forceinline__ void segmented_row_step(uint32_t& closed, unsigned lo
 constexpr uint32_t kBinThreads = 1024;
 constexpr uint32_t kBinWaves = kBinThreads / 64;
 constexpr uint32_t kBinAhead = 4;             // entries a lane fetches before it works on the first
-constexpr uint32_t kBinsPerGroup = 8;         // consecutive stretches of a sample one workgroup takes
+// consecutive stretches of a sample one workgroup takes (FastGCN form: few, large stretches per
+// sample, and the low ones hold most entries; LADIES form: hundreds of small ones)
+constexpr uint32_t kBinsPerGroupBits = 8;
+constexpr uint32_t kBinsPerGroupSums = 16;
 constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
 template <bool kWithImportance>
 __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
-    CSRPartition csr, TransitView tv, int32_t invalid, uint32_t bins_per_sample, uint32_t* __restrict__ bitmap,
+    CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
+    uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
     unsigned long long* __restrict__ sums,
     uint32_t sums_per_sample) {
@@ -244,9 +248,11 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   // A workgroup takes kBinsPerGroup consecutive stretches of one sample, one after the other:
   // where a transit's sub-range ends in one stretch it begins in the next, and the end is
   // then only a short gallop away instead of a search of the whole adjacency.
-  const uint32_t groups_per_sample = (bins_per_sample + kBinsPerGroup - 1) / kBinsPerGroup;
-  const uint32_t s = blockIdx.x / groups_per_sample;
-  const uint32_t first_bin = (blockIdx.x - s * groups_per_sample) * kBinsPerGroup;
+  constexpr uint32_t kBinsPerGroup = kWithImportance ? kBinsPerGroupSums : kBinsPerGroupBits;
+  // the low stretches hold the hubs and take longest: all samples' first groups start first
+  const uint32_t group = blockIdx.x / n_samples;
+  const uint32_t s = blockIdx.x - group * n_samples;
+  const uint32_t first_bin = group * kBinsPerGroup;
   const int32_t* transits = tv.base + (size_t)s * tv.stride;
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t wave = threadIdx.x >> 6;
@@ -1115,11 +1121,12 @@ class LayerEngine : public EngineBase {
     (void)n_items;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
-    const uint32_t groups = (bins + kBinsPerGroup - 1) / kBinsPerGroup;
+    constexpr uint32_t per_group = ladies ? kBinsPerGroupSums : kBinsPerGroupBits;
+    const uint32_t groups = (bins + per_group - 1) / per_group;
     if ((uint64_t)n * groups >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
     tick();
     collective_mark_binned<ladies><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, bins, d_bitmap_, bitmap_words_, d_row_sums_, d_sums_, sums_per_sample_);
+        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, d_row_sums_, d_sums_, sums_per_sample_);
     tock();
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
     ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
