@@ -133,7 +133,15 @@ __device__ __forceinline__ uint64_t block_exclusive_scan_256_u64(uint64_t v, uin
   return before + incl - v;
 }
 
-__global__ __launch_bounds__(kScanThreads) void scan64_tile_totals(const uint64_t* __restrict__ in, size_t n,
+// The input of the 64-bit scan is a functor, so that values can be computed on the way in
+// (e.g. degree^2 of a listed vertex) instead of being stored first.
+struct LoadU64 {
+  const uint64_t* p;
+  __device__ __forceinline__ uint64_t operator()(size_t i) const { return p[i]; }
+};
+
+template <class Load>
+__global__ __launch_bounds__(kScanThreads) void scan64_tile_totals(Load in, size_t n,
                                                                    uint64_t* __restrict__ tile_totals) {
   __shared__ uint64_t s_wave[kScanThreads / kWave];
   const size_t base = (size_t)blockIdx.x * kScanTile;
@@ -141,29 +149,41 @@ __global__ __launch_bounds__(kScanThreads) void scan64_tile_totals(const uint64_
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
     const size_t idx = base + (size_t)i * kScanThreads + threadIdx.x;
-    if (idx < n) sum += in[idx];
+    if (idx < n) sum += in(idx);
   }
   uint64_t total;
   block_exclusive_scan_256_u64(sum, s_wave, &total);
   if (threadIdx.x == 0) tile_totals[blockIdx.x] = total;
 }
 
+// One workgroup; a thread takes kTotalsPerThread consecutive totals per round.
+constexpr int kTotalsPerThread = 16;
 __global__ __launch_bounds__(kScanThreads) void scan64_of_totals(uint64_t* __restrict__ tile_totals, size_t num_tiles) {
   __shared__ uint64_t s_wave[kScanThreads / kWave];
   uint64_t carry = 0;
-  for (size_t start = 0; start < num_tiles; start += kScanThreads) {
-    const size_t idx = start + threadIdx.x;
-    const uint64_t v = idx < num_tiles ? tile_totals[idx] : 0ull;
+  for (size_t start = 0; start < num_tiles; start += (size_t)kScanThreads * kTotalsPerThread) {
+    const size_t first = start + (size_t)threadIdx.x * kTotalsPerThread;
+    uint64_t v[kTotalsPerThread];
+    uint64_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kTotalsPerThread; ++i) {
+      v[i] = first + i < num_tiles ? tile_totals[first + i] : 0ull;
+      sum += v[i];
+    }
     uint64_t total;
-    const uint64_t excl = block_exclusive_scan_256_u64(v, s_wave, &total);
-    if (idx < num_tiles) tile_totals[idx] = carry + excl;
+    uint64_t running = carry + block_exclusive_scan_256_u64(sum, s_wave, &total);
+#pragma unroll
+    for (int i = 0; i < kTotalsPerThread; ++i) {
+      if (first + i < num_tiles) tile_totals[first + i] = running;
+      running += v[i];
+    }
     carry += total;
   }
   if (threadIdx.x == 0) tile_totals[num_tiles] = carry;
 }
 
-__global__ __launch_bounds__(kScanThreads) void scan64_apply_inclusive(const uint64_t* __restrict__ in,
-                                                                       uint64_t* __restrict__ out, size_t n,
+template <class Load>
+__global__ __launch_bounds__(kScanThreads) void scan64_apply_inclusive(Load in, uint64_t* __restrict__ out, size_t n,
                                                                        const uint64_t* __restrict__ tile_offsets) {
   __shared__ uint64_t s_wave[kScanThreads / kWave];
   const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
@@ -171,7 +191,7 @@ __global__ __launch_bounds__(kScanThreads) void scan64_apply_inclusive(const uin
   uint64_t sum = 0;
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
-    v[i] = base + i < n ? in[base + i] : 0ull;
+    v[i] = base + i < n ? in(base + i) : 0ull;
     sum += v[i];
   }
   uint64_t total;
@@ -185,15 +205,21 @@ __global__ __launch_bounds__(kScanThreads) void scan64_apply_inclusive(const uin
 
 inline size_t scan_num_tiles(size_t n) { return (n + kScanTile - 1) / kScanTile; }
 
-// out[i] = sum of in[0..i]; in and out may alias.  scratch needs scan_num_tiles(n) + 1 uint64.
-inline hipError_t inclusive_scan_u64(const uint64_t* in, uint64_t* out, size_t n, uint64_t* scratch,
-                                     hipStream_t stream) {
+// out[i] = in(0) + ... + in(i).  scratch needs scan_num_tiles(n) + 1 uint64.
+template <class Load>
+inline hipError_t inclusive_scan_u64_of(Load in, uint64_t* out, size_t n, uint64_t* scratch, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   const size_t tiles = (n + kScanTile - 1) / kScanTile;
-  scan64_tile_totals<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, n, scratch);
+  scan64_tile_totals<Load><<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, n, scratch);
   scan64_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream>>>(scratch, tiles);
-  scan64_apply_inclusive<<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, out, n, scratch);
+  scan64_apply_inclusive<Load><<<dim3((unsigned)tiles), dim3(kScanThreads), 0, stream>>>(in, out, n, scratch);
   return hipGetLastError();
+}
+
+// out[i] = sum of in[0..i]; in and out may alias.
+inline hipError_t inclusive_scan_u64(const uint64_t* in, uint64_t* out, size_t n, uint64_t* scratch,
+                                     hipStream_t stream) {
+  return inclusive_scan_u64_of(LoadU64{in}, out, n, scratch, stream);
 }
 
 // Scratch needed by exclusive_scan_u32 for n elements, in uint32 units.

@@ -448,15 +448,24 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
   if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
+// degree(ids[i])^2, computed where the running sums are formed instead of being stored
+struct DegreeSquaredOf {
+  const int32_t* ids;
+  const EdgePos_t* row_ptr;
+  __device__ __forceinline__ uint64_t operator()(size_t i) const {
+    const int32_t v = ids[i];
+    const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+    return d * d;
+  }
+};
+
 // The marked vertices of every sample, in ascending order, become the sample's distinct
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
-// tile of a sample is where the sample's list starts).  Per distinct vertex either
-// degree^2 (degree_sq given) or the importance accumulated in sums (sums given).
+// tile of a sample is where the sample's list starts).  With sums given, the importance
+// accumulated for the vertex is copied next to it.
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
-                                                      uint32_t tiles_per_sample, const EdgePos_t* __restrict__ row_ptr,
-                                                      int32_t* __restrict__ distinct_ids,
-                                                      uint64_t* __restrict__ degree_sq,
+                                                      uint32_t tiles_per_sample, int32_t* __restrict__ distinct_ids,
                                                       uint32_t* __restrict__ distinct_start,
                                                       unsigned long long* __restrict__ sums, uint32_t sums_per_sample,
                                                       unsigned long long* __restrict__ importance,
@@ -493,10 +502,6 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
       const uint32_t v = (tile * kBitmapTileWords + w) * kVerticesPerWord + lane;
       const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       distinct_ids[at] = (int32_t)v;
-      if (degree_sq) {
-        const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-        degree_sq[at] = d * d;
-      }
       if (sums) {
         unsigned long long* acc = sums + (size_t)sample * sums_per_sample + v;
         importance[at] = *acc;
@@ -1137,11 +1142,11 @@ class LayerEngine : public EngineBase {
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
     bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
-        d_bitmap_, d_tile_offsets_, tiles_per_sample, dgraph_.row_ptr(), d_distinct_ids_, d_degree_sq_,
-        d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
+        d_bitmap_, d_tile_offsets_, tiles_per_sample, d_distinct_ids_, d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
     if (!ladies) {
-      ND_HIP_TRY(inclusive_scan_u64(d_degree_sq_, d_running_sums_, n_distinct, d_scratch64_, stream_));
+      ND_HIP_TRY(inclusive_scan_u64_of(DegreeSquaredOf{d_distinct_ids_, dgraph_.row_ptr()}, d_running_sums_, n_distinct,
+                                       d_scratch64_, stream_));
     } else if (n_distinct > 0) {
       int chunk_bits = 1;
       while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
@@ -1201,7 +1206,6 @@ class LayerEngine : public EngineBase {
     release_distinct_buffers();
     ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
     if (form == apps::kDistinctByDegreeSquared) {
-      ND_HIP_TRY(hipMalloc(&d_degree_sq_, sizeof(uint64_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
     }
@@ -1240,7 +1244,7 @@ class LayerEngine : public EngineBase {
   }
 
   void release_distinct_buffers() {
-    release(d_distinct_ids_); release(d_degree_sq_); release(d_running_sums_); release(d_scratch64_);
+    release(d_distinct_ids_); release(d_running_sums_); release(d_scratch64_);
     release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
@@ -1318,7 +1322,7 @@ class LayerEngine : public EngineBase {
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t *d_key2_ = nullptr, *d_index2_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
-  uint64_t *d_degree_sq_ = nullptr, *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
+  uint64_t *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
   unsigned long long* d_importance_ = nullptr;
   uint32_t *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
   int32_t* d_ranked_ids_ = nullptr;
