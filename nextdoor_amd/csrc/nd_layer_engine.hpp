@@ -448,6 +448,54 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
   if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
+// log2 of a positive normal float from exponent extraction and an atanh series; every step
+// is a single IEEE operation so that host and device agree bit for bit.
+__host__ __device__ __forceinline__ float det_log2(float x) {
+  uint32_t bits;
+#if defined(__HIP_DEVICE_COMPILE__)
+  bits = __float_as_uint(x);
+#else
+  memcpy(&bits, &x, sizeof(bits));
+#endif
+  int e = (int)(bits >> 23) - 127;
+  const uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
+  float m;
+#if defined(__HIP_DEVICE_COMPILE__)
+  m = __uint_as_float(mbits);
+#else
+  memcpy(&m, &mbits, sizeof(m));
+#endif
+  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
+  const float z = (m - 1.0f) / (m + 1.0f);
+  const float z2 = z * z;
+  float poly = z2 * 0.142857149f;
+  poly = poly + 0.2f;
+  poly = poly * z2;
+  poly = poly + 0.333333343f;
+  poly = poly * z2;
+  poly = poly + 1.0f;
+  float ln_m = z * poly;
+  ln_m = ln_m * 2.0f;
+  return (float)e + ln_m * 1.44269502f;
+}
+
+// Efraimidis-Spirakis key of (sample, vertex): log2(u) / importance with u from Philox at slot
+// sample * |V| + vertex and importance the fixed-point sum of the vertex's terms (the common
+// 2^53 scale does not change the order of the keys); as sortable bits, inverted so that an
+// ascending sort yields descending keys.
+__device__ __forceinline__ uint32_t ladies_key_bits(unsigned long long importance_fixed, uint64_t slot, uint32_t step,
+                                                    uint64_t seed) {
+  const float importance = (float)importance_fixed;
+  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
+                                        (uint32_t)(seed >> 32));
+  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+  float key = -__builtin_inff();
+  if (importance > 0.0f) key = det_log2(u) / importance;
+  uint32_t b = __float_as_uint(key);
+  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  return ~b;
+}
+
 // degree(ids[i])^2, computed where the running sums are formed instead of being stored
 struct DegreeSquaredOf {
   const int32_t* ids;
@@ -461,14 +509,15 @@ struct DegreeSquaredOf {
 
 // The marked vertices of every sample, in ascending order, become the sample's distinct
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
-// tile of a sample is where the sample's list starts).  With sums given, the importance
-// accumulated for the vertex is copied next to it.
+// tile of a sample is where the sample's list starts).  With sums given (LADIES form), the
+// vertex's sampling key is formed from the importance accumulated for it.
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t tiles_per_sample, int32_t* __restrict__ distinct_ids,
                                                       uint32_t* __restrict__ distinct_start,
-                                                      unsigned long long* __restrict__ sums, uint32_t sums_per_sample,
-                                                      unsigned long long* __restrict__ importance,
+                                                      const unsigned long long* __restrict__ sums,
+                                                      uint32_t sums_per_sample, uint64_t seed, uint64_t first_sample,
+                                                      uint32_t step, uint32_t* __restrict__ key_bits,
                                                       uint32_t* __restrict__ distinct_sample) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t s_before[kScanThreads];  // set bits of the tile before word 8 * t
@@ -503,8 +552,8 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
       const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       distinct_ids[at] = (int32_t)v;
       if (sums) {
-        unsigned long long* acc = sums + (size_t)sample * sums_per_sample + v;
-        importance[at] = *acc;
+        const uint64_t slot = (first_sample + sample) * (uint64_t)sums_per_sample + v;  // sums_per_sample = |V|
+        key_bits[at] = ladies_key_bits(sums[(size_t)sample * sums_per_sample + v], slot, step, seed);
         distinct_sample[at] = sample;
       }
     }
@@ -656,60 +705,6 @@ __global__ __launch_bounds__(256) void select_compact(const uint32_t* __restrict
     kept_id[r] = distinct_ids[base + k];
     ++r;
   }
-}
-
-// log2 of a positive normal float from exponent extraction and an atanh series; every step
-// is a single IEEE operation so that host and device agree bit for bit.
-__host__ __device__ __forceinline__ float det_log2(float x) {
-  uint32_t bits;
-#if defined(__HIP_DEVICE_COMPILE__)
-  bits = __float_as_uint(x);
-#else
-  memcpy(&bits, &x, sizeof(bits));
-#endif
-  int e = (int)(bits >> 23) - 127;
-  const uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
-  float m;
-#if defined(__HIP_DEVICE_COMPILE__)
-  m = __uint_as_float(mbits);
-#else
-  memcpy(&m, &mbits, sizeof(m));
-#endif
-  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
-  const float z = (m - 1.0f) / (m + 1.0f);
-  const float z2 = z * z;
-  float poly = z2 * 0.142857149f;
-  poly = poly + 0.2f;
-  poly = poly * z2;
-  poly = poly + 0.333333343f;
-  poly = poly * z2;
-  poly = poly + 1.0f;
-  float ln_m = z * poly;
-  ln_m = ln_m * 2.0f;
-  return (float)e + ln_m * 1.44269502f;
-}
-
-// One lane per distinct (sample, vertex): Efraimidis-Spirakis key log2(u) / importance with u
-// from Philox at slot sample * |V| + vertex and importance the fixed-point sum of the
-// vertex's terms (the common 2^53 scale does not change the order of the keys); stored as
-// sortable bits, inverted so that an ascending sort yields descending keys.
-__global__ __launch_bounds__(256) void ladies_keys(const unsigned long long* __restrict__ importance_fixed,
-                                                   const int32_t* __restrict__ distinct_ids,
-                                                   const uint32_t* __restrict__ distinct_sample, uint32_t n_distinct,
-                                                   uint64_t seed, uint64_t first_sample, uint32_t n_vertices,
-                                                   uint32_t step, uint32_t* __restrict__ key_bits) {
-  const uint32_t j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= n_distinct) return;
-  const float importance = (float)importance_fixed[j];
-  const uint64_t slot = (first_sample + distinct_sample[j]) * (uint64_t)n_vertices + (uint32_t)distinct_ids[j];
-  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
-                                        (uint32_t)(seed >> 32));
-  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
-  float key = -__builtin_inff();
-  if (importance > 0.0f) key = det_log2(u) / importance;
-  uint32_t b = __float_as_uint(key);
-  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-  key_bits[j] = ~b;
 }
 
 // running sums of one sample's distinct ids, as the WeightArray handed to next()
@@ -1142,7 +1137,8 @@ class LayerEngine : public EngineBase {
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
     bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
-        d_bitmap_, d_tile_offsets_, tiles_per_sample, d_distinct_ids_, d_distinct_start_, d_sums_, sums_per_sample_, d_importance_, d_distinct_sample_);
+        d_bitmap_, d_tile_offsets_, tiles_per_sample, d_distinct_ids_, d_distinct_start_, d_sums_, sums_per_sample_, seed_,
+        (uint64_t)s0, (uint32_t)step, d_key_bits_, d_distinct_sample_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
     if (!ladies) {
       ND_HIP_TRY(inclusive_scan_u64_of(DegreeSquaredOf{d_distinct_ids_, dgraph_.row_ptr()}, d_running_sums_, n_distinct,
@@ -1150,9 +1146,6 @@ class LayerEngine : public EngineBase {
     } else if (n_distinct > 0) {
       int chunk_bits = 1;
       while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
-      ladies_keys<<<dim3((n_distinct + 255) / 256), dim3(256), 0, stream_>>>(
-          d_importance_, d_distinct_ids_, d_distinct_sample_, n_distinct, seed_, (uint64_t)s0, (uint32_t)invalid_,
-          (uint32_t)step, d_key_bits_);
       // per sample, the entries that can be among its first `wanted` in key order (radix select
       // on the upper 16 bits of the key), copied out in (sample, vertex) order
       const uint32_t wanted = (uint32_t)App().stepSize(step);
@@ -1210,7 +1203,6 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
     }
     if (form == apps::kRankedByLadiesImportance) {
-      ND_HIP_TRY(hipMalloc(&d_importance_, sizeof(unsigned long long) * cap));
       ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
@@ -1245,7 +1237,7 @@ class LayerEngine : public EngineBase {
 
   void release_distinct_buffers() {
     release(d_distinct_ids_); release(d_running_sums_); release(d_scratch64_);
-    release(d_importance_); release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
+    release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
     release(d_kept_key_); release(d_kept_sample_); release(d_kept_id_);
@@ -1323,7 +1315,6 @@ class LayerEngine : public EngineBase {
   uint32_t *d_key2_ = nullptr, *d_index2_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
   uint64_t *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
-  unsigned long long* d_importance_ = nullptr;
   uint32_t *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
   int32_t* d_ranked_ids_ = nullptr;
 };
