@@ -31,13 +31,13 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "weighted_node2vec_rmat22": 1.246e9,     # step_flat_kernel
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
-    "fastgcn_importance_rmat22": 8.103e10,   # collective_mark, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 5.241e10,  # collective_mark, average over its 12 launches per pass
+    "fastgcn_importance_rmat22": 6.953e9,    # collective_mark_binned, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 1.787e11,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
     "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 253.7e9, "ladies_importance_chunglu3m": 859.8e9,
+    "fastgcn_importance_rmat22": 165.7e9, "ladies_importance_chunglu3m": 500.7e9,
 }
 
 WORKLOADS = {
@@ -238,15 +238,15 @@ def main():
         result["config"]["distinct_pairs"] = distinct
         result["config"]["chunks"] = sampler.counter(2)
         result["config"]["neighbourhood_entries_per_s"] = entries / (ms_per_step / 1000.0)
-        # dominant kernel: collective_mark walks every entry of every collective neighbourhood
-        # once.  Minimal traffic: the entry's vertex id (4 B; + 4 B weight for LADIES) and one
-        # bit (FastGCN) or one bit + a 64-bit accumulator (LADIES) per distinct pair.
+        # dominant kernel: collective_mark_binned walks every entry of every collective
+        # neighbourhood once.  Minimal traffic: the entry's vertex id (4 B; + 4 B weight for
+        # LADIES) and one bit (FastGCN) or one bit + a 64-bit sum (LADIES) per distinct pair.
         ladies = w["kind"] == "LADIES_IMPORTANCE"
         mark_bytes = entries * (8 if ladies else 4) + distinct * (8.125 if ladies else 0.125)
         launches = max(prof["neighbourhood_launches"], 1)
         achieved = mark_bytes / (prof["neighbourhood_ms"] / 1000.0) / 1e9
         result["roofline"] = {
-            "bound": "hbm", "kernel": "collective_mark", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "bound": "hbm", "kernel": "collective_mark_binned", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "algorithmic_bytes_per_launch": mark_bytes / launches,
             "avg_launch_ms": prof["neighbourhood_ms"] / launches,

@@ -140,7 +140,7 @@ struct FastGCNImportanceAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSample
 };
 
 // LADIES-style layer-dependent importance sampling WITHOUT replacement.  With U the
-// previous layer, importance(v) = sum over edges u -> v, u in U, of (w_uv / rowsum(u))^2.
+// previous layer, importance(v) = sum over edges u -> v, u in U, of (w_uv * (1 / rowsum(u)))^2 (the inverse rounded to float once per row).
 // The engine computes it over the collective neighbourhood, draws one Efraimidis-Spirakis
 // key log2(uniform) / importance per distinct vertex (uniform from Philox at slot
 // sample * |V| + v) and hands next() the vertices in descending key order: the first

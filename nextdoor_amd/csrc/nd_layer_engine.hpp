@@ -18,15 +18,14 @@
 //    (deterministic), the buffers are grown once and reused, and next() receives the
 //    neighbourhood in the form the app declares (nd::apps::NeighborhoodForm).
 //  * For kDistinctByDegreeSquared the concatenation is never stored: every entry marks its
-//    vertex in a per-sample presence map (one byte per vertex), the marked vertices in
-//    ascending order are the distinct vertices, and a 64-bit inclusive scan of degree^2 gives the running sums the
-//    app inverts.
-//  * For kRankedByLadiesImportance each entry of the concatenation carries
-//    (weight / rowsum(transit))^2; the terms of a distinct vertex are summed as 2^53
-//    fixed-point integers, Efraimidis-Spirakis keys are computed per distinct vertex
-//    and two more stable sorts order the distinct vertices of every sample by descending key.
-//    (The concatenation is sorted by (sample, vertex) with two stable radix sorts; run heads
-//    give the distinct vertices.)
+//    vertex in a per-sample bitmap, built stretch by stretch in LDS; the marked vertices in
+//    ascending order are the distinct vertices, and a 64-bit inclusive scan of degree^2 over
+//    them gives the running sums the app inverts.
+//  * For kRankedByLadiesImportance each entry also carries (weight * (1 / rowsum(transit)))^2;
+//    the terms of a vertex are summed as 2^53 fixed-point integers next to the bitmap (in LDS),
+//    the Efraimidis-Spirakis key of every distinct vertex is formed from its sum, a radix
+//    select keeps the entries that can be among a sample's first picks, and two stable sorts
+//    order those by descending key.
 //  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
 //    of entries, so a layer whose frontier sits on hubs cannot outgrow memory.
 //  * Random numbers: Philox keyed by the output slot s * stepSize(k) + nbr and the layer.
