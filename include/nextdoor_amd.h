@@ -100,6 +100,12 @@ int nd_sampler_sampling_type(const nd_sampler* s);
  * SampleType structs.  nd_sampler_sample_state_bytes is 0 for an empty SampleType. */
 int64_t nd_sampler_sample_state_bytes(const nd_sampler* s);
 int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes);
+/* No counterpart in the reference (whose step loop waits for the host several times per step,
+ * src/nextdoor.cu:2498-2636).  A pass here is a fixed sequence of launches with all varying
+ * sizes in device memory, so it can be recorded once as a HIP graph and replayed: mode 1 on,
+ * 0 off (default: measured, the replay gains nothing here).  Samples are the same bytes either
+ * way; per-phase profiling runs eagerly. */
+int nd_sampler_set_launch_graph(nd_sampler* s, int mode);
 /* The per-phase wall-clock breakdown the reference prints (src/nextdoor.cu:2963-2966),
  * measured with events on the sampler's stream when profiling is on.
  * out[0] end to end, [1] inversion, [2] load balancing, [3] flat (identity / sub-wavefront)

@@ -242,6 +242,11 @@ class Sampler:
         engine decide.  The samples do not depend on it."""
         check(lib().nd_sampler_set_inversion_period(self._h, int(period)))
 
+    def set_launch_graph(self, mode):
+        """1: replay every pass as a recorded HIP graph; 0 (default): enqueue the launches one
+        by one.  The samples are the same."""
+        check(lib().nd_sampler_set_launch_graph(self._h, int(mode)))
+
     def set_profiling(self, on):
         check(lib().nd_sampler_set_profiling(self._h, int(on)))
 

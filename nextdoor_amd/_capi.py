@@ -49,6 +49,7 @@ SIGNATURES = {
     "nd_sampler_sample_state_bytes": (C.c_int64, [C.c_void_p]),
     "nd_sampler_get_sample_states": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64]),
     "nd_sampler_set_inversion_period": (C.c_int, [C.c_void_p, C.c_int]),
+    "nd_sampler_set_launch_graph": (C.c_int, [C.c_void_p, C.c_int]),
     "nd_sampler_set_profiling": (C.c_int, [C.c_void_p, C.c_int]),
     "nd_sampler_phase_times": (C.c_int, [C.c_void_p, c_f32p]),
     "nd_sampler_get_adjacency": (C.c_int, [C.c_void_p, C.POINTER(c_i32p), C.POINTER(c_i32p), c_i64p,

@@ -287,6 +287,13 @@ int nd_sampler_set_inversion_period(nd_sampler* s, int period) {
   return 0;
 }
 
+int nd_sampler_set_launch_graph(nd_sampler* s, int mode) {
+  if (!s) return fail("null sampler");
+  if (mode != 0 && mode != 1) return fail("launch graph mode is 0 (off) or 1 (on)");
+  s->engine->launch_graph = mode;
+  return 0;
+}
+
 int nd_sampler_set_profiling(nd_sampler* s, int on) {
   if (!s) return fail("null sampler");
   s->engine->profiling = on != 0;

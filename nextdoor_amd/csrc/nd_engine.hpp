@@ -73,6 +73,9 @@ class EngineBase {
   // compaction in slot order), and there is no load balancing.  0: the engine decides from
   // the walks-per-vertex ratio.  Results do not depend on it.  Other apps always invert.
   int inversion_period = 1;
+  // 1: replay a pass as a recorded HIP graph instead of enqueueing its launches one by one;
+  // 0 (default): enqueue.  Layer-wise and edge-list apps have few, long launches and ignore it.
+  int launch_graph = 0;
   virtual int fetch_final_samples() = 0;
   virtual void free_device() = 0;
   virtual int64_t num_samples() const = 0;
@@ -886,10 +889,6 @@ class Engine : public EngineBase {
   // the only host wait is at the end.
   int sample(int mode) override {
     if (!allocated_) { last_error = "sample before alloc"; return -1; }
-    const bool balance = mode == kTransitParallelLoadBalanced;
-    App app;
-    const int n_steps = app.steps();
-    const size_t F = (size_t)final_sample_size();
     times = PhaseTimes();
     if (!std::is_empty<SampleType>::value) {
       ND_HIP_TRY(hipMemcpyAsync(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
@@ -897,7 +896,20 @@ class Engine : public EngineBase {
     }
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
+    const int rc = wants_launch_graph() ? replay_pass(mode) : enqueue_pass(mode);
+    if (rc != 0) return rc;
+    ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
+    return 0;
+  }
 
+  // Every launch of one pass, in order, on stream_; no host wait in between.
+  int enqueue_pass(int mode) {
+    const bool balance = mode == kTransitParallelLoadBalanced;
+    App app;
+    const int n_steps = app.steps();
+    const size_t F = (size_t)final_sample_size();
     // pairs whose transit is INVALID are dropped by the inversion and never reach a step
     // kernel: their outputs keep this fill
     {
@@ -1085,10 +1097,59 @@ class Engine : public EngineBase {
     }
     tock(&times.assemble);
     ND_HIP_TRY(hipGetLastError());
-    ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
-    ND_HIP_TRY(hipStreamSynchronize(stream_));
-    ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
     return 0;
+  }
+
+  // A pass can be recorded once as a HIP graph and replayed: nothing in it depends on the host
+  // (sizes that change from step to step live in device memory), so the graph of one pass is
+  // the graph of every pass with the same mode, inversion period and load-balancing parity.
+  // No memset nodes: buffers are cleared by fill kernels.  Off by default: on the pass it was
+  // meant for (56,944 walks, ~1300 launches of 3-9 us each) the replay takes 4.72 ms against
+  // 4.8 ms enqueued one by one - the kernels' own durations add up to the pass, not the gaps.
+  bool wants_launch_graph() const { return launch_graph == 1 && !profiling; }
+
+  int replay_pass(int mode) {
+    const int parity = balanced_steps_ & 1;
+    RecordedPass* pass = nullptr;
+    for (RecordedPass& r : recorded_)
+      if (r.mode == mode && r.inversion_period == inversion_period && r.parity == parity) pass = &r;
+    if (!pass) {
+      RecordedPass r;
+      r.mode = mode;
+      r.inversion_period = inversion_period;
+      r.parity = parity;
+      const uint64_t before = balanced_steps_;
+      ND_HIP_TRY(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
+      const int rc = enqueue_pass(mode);
+      hipGraph_t graph = nullptr;
+      const hipError_t ended = hipStreamEndCapture(stream_, &graph);
+      r.balanced_steps = balanced_steps_ - before;
+      balanced_steps_ = before;  // advanced below, as for every replay
+      if (rc != 0 || ended != hipSuccess) {
+        if (graph) (void)hipGraphDestroy(graph);
+        if (rc == 0) last_error = std::string("hipStreamEndCapture: ") + hipGetErrorString(ended);
+        return rc != 0 ? rc : -1;
+      }
+      const hipError_t made = hipGraphInstantiate(&r.exec, graph, nullptr, nullptr, 0);
+      (void)hipGraphDestroy(graph);
+      if (made != hipSuccess) {
+        last_error = std::string("hipGraphInstantiate: ") + hipGetErrorString(made);
+        return -1;
+      }
+      r.counts = times;
+      recorded_.push_back(r);
+      pass = &recorded_.back();
+    }
+    times = pass->counts;  // launch counts of the recorded pass; durations stay zero
+    balanced_steps_ += pass->balanced_steps;
+    ND_HIP_TRY(hipGraphLaunch(pass->exec, stream_));
+    return 0;
+  }
+
+  void drop_recorded_passes() {
+    for (RecordedPass& r : recorded_)
+      if (r.exec) (void)hipGraphExecDestroy(r.exec);
+    recorded_.clear();
   }
 
   // getFinalSamples: device -> hFinalSamples
@@ -1184,6 +1245,7 @@ class Engine : public EngineBase {
   }
 
   void free_run_buffers() {
+    drop_recorded_passes();
     release(d_initial_);
     release(d_samples_);
     release(d_samples_init_);
@@ -1248,6 +1310,13 @@ class Engine : public EngineBase {
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;          // two work-item counters, alternating between load-balanced steps
+  struct RecordedPass {
+    int mode = 0, inversion_period = 0, parity = 0;
+    uint64_t balanced_steps = 0;  // load-balanced steps of the pass
+    PhaseTimes counts;            // its launch counts
+    hipGraphExec_t exec = nullptr;
+  };
+  std::vector<RecordedPass> recorded_;
   uint64_t balanced_steps_ = 0;        // ... counted over the life of the buffers, so the parity never repeats
   uint32_t* d_chunks_ = nullptr;
   uint8_t* d_skip_flag_ = nullptr;

@@ -88,6 +88,7 @@ class ShardedEngine : public EngineBase {
   int sample(int mode) override {
     for (auto& p : parts_) {
       p->inversion_period = inversion_period;
+      p->launch_graph = launch_graph;
       p->profiling = profiling;
     }
     times = PhaseTimes();

@@ -85,6 +85,40 @@ def test_sample_parallel_mode_gives_the_same_samples(oracle, app, kind_name, sta
                     modes=("sample_parallel", True, "sample_parallel"))
 
 
+@pytest.mark.parametrize("app,kind_name,period", [
+    ("UniformRandomWalk", "UNIFORM_WALK", 1),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", 1),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", 0),
+    ("KHop", "KHOP", 1),
+])
+def test_recorded_passes_replay_to_the_same_samples(oracle, app, kind_name, period):
+    # a pass recorded as a HIP graph, replayed several times with eager passes, fetches and
+    # other modes in between: every replay must give the oracle's bytes
+    g = graphs.random_graph(n=1500, mean_degree=6, seed=9, hub=4, isolated_every=11)
+    og = graphs.oracle_view(g)
+    s = nd.Sampler(app, g, seed=SEED)
+    try:
+        d = desc_for(oracle, s, getattr(oracle, kind_name))
+        want, _ = oracle.sample_individual(og, d, SEED, s.initial_contents)
+        s.set_inversion_period(period)
+        s.set_launch_graph(1)
+        for turn in range(7):
+            lb = turn % 3 != 2
+            eager = turn == 3
+            print("app", app, "period", period, "turn", turn, "lb", lb, "eager", eager, flush=True)
+            if eager:
+                s.set_profiling(True)  # per-phase events: launches go out one by one
+            s.do_transit_parallel(load_balancing=lb)
+            if eager:
+                s.set_profiling(False)
+            assert np.array_equal(s.final_samples(), want), f"turn {turn}"
+        s.set_launch_graph(0)
+        s.do_transit_parallel(load_balancing=True)
+        assert np.array_equal(s.final_samples(), want)
+    finally:
+        s.close()
+
+
 def test_command_line_runs_checks_and_prints(oracle, tmp_path):
     import io
     from nextdoor_amd import __main__ as cli
