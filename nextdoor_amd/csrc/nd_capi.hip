@@ -361,6 +361,10 @@ int nd_sampler_check_results(nd_sampler* s, int* ok) {
   if (!s || !ok) return fail("null argument");
   if (!s->graph) return fail("no graph set");
   nd::EngineBase& e = *s->engine;
+  // the rule "adjacent to a vertex of the previous step" presumes that the previous step's
+  // samples are the transits (the reference checks its MultiRW app with a rule of its own,
+  // src/tests/multiGPU/multirw.cu:12-137, against the walkers left in the sample state)
+  if (e.has_explicit_transits()) return fail("no validator for apps that choose their own transits");
   const int rc = e.fetch_final_samples();
   if (rc != 0) return fail(e.last_error, rc);
   nd::SampleShape shape;

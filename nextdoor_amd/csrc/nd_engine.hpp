@@ -95,6 +95,8 @@ class EngineBase {
   // Apps with AdjacencyMatrix output on the per-transit engine (MVS, ClusterGCN): device ->
   // hListStart / hListRows / hListCols
   virtual bool lists_edges() const { return false; }
+  // App::hasExplicitTransits(): the transits of a step are not the previous step's samples
+  virtual bool has_explicit_transits() const { return false; }
   virtual int fetch_adjacency() {
     last_error = "this app does not produce edge lists";
     return -2;
@@ -713,6 +715,7 @@ class Engine : public EngineBase {
   const char* app_name() const override { return name_; }
   int64_t num_samples() const override { return n_samples_; }
   int final_sample_size() const override { return nd::final_sample_size<App>(); }
+  bool has_explicit_transits() const override { return App().hasExplicitTransits(); }
   int steps() const override { return App().steps(); }
   int step_size(int k) const override { return App().stepSize(k); }
   int initial_sample_size() const override { return App().initialSampleSize(nullptr); }

@@ -38,6 +38,7 @@ class ShardedEngine : public EngineBase {
   int step_size(int k) const override { return parts_[0]->step_size(k); }
   int initial_sample_size() const override { return parts_[0]->initial_sample_size(); }
   int sampling_type() const override { return parts_[0]->sampling_type(); }
+  bool has_explicit_transits() const override { return parts_[0]->has_explicit_transits(); }
   int32_t invalid_vertex() const override { return parts_[0]->invalid_vertex(); }
   int max_bits() const override { return parts_[0]->max_bits(); }
   size_t sample_state_bytes() const override {
