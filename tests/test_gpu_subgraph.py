@@ -72,6 +72,31 @@ def test_clustergcn_matches_oracle(oracle, app, cluster, per_sample, gname):
         s.close()
 
 
+def test_power_law_graph_with_long_hub_lists(oracle):
+    # R-MAT scale 14: the low vertex ids are hubs with thousands of edges, so single lanes of
+    # MVS copy hundreds of edges and whole units interleave many rounds
+    g = nd.Graph.rmat(14, 16, seed=7, symmetrise=True)
+    og = graphs.oracle_view(g)
+    assert np.diff(g.row_ptr).max() > 2000
+    for app in ("MVS", "ClusterGCN"):
+        s = nd.Sampler(app, g, seed=3)
+        try:
+            print("app", app, "rmat14", flush=True)
+            s.do_transit_parallel()
+            rows, cols, start = s.adjacency()
+            if app == "MVS":
+                want_rows, want_cols, want_start = oracle.sample_mvs(og, oracle.mvs_vertices(og, s.num_samples, 32))
+            else:
+                verts = oracle.clustergcn_vertices(og, s.num_samples, 16, 2)
+                want_final, want_rows, want_cols, want_start = oracle.sample_clustergcn(og, verts)
+                assert np.array_equal(s.final_samples(), want_final)
+            assert np.array_equal(start, want_start)
+            assert np.array_equal(rows, want_rows) and np.array_equal(cols, want_cols)
+            assert s.check_results() == (True, "")
+        finally:
+            s.close()
+
+
 def test_graph_without_edges_gives_empty_lists():
     g = nd.Graph.from_edges([], [], [], n_vertices=64)
     for app in ("MVS", "ClusterGCN"):
