@@ -171,6 +171,58 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
 // a 2^53 fixed-point integer, to the 64-bit sum of (sample, vertex).
 constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words: 65536 vertices
 
+// log2 of a positive normal float from exponent extraction and an atanh series; every step
+// is a single IEEE operation so that host and device agree bit for bit.
+__host__ __device__ __forceinline__ float det_log2(float x) {
+  uint32_t bits;
+#if defined(__HIP_DEVICE_COMPILE__)
+  bits = __float_as_uint(x);
+#else
+  memcpy(&bits, &x, sizeof(bits));
+#endif
+  int e = (int)(bits >> 23) - 127;
+  const uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
+  float m;
+#if defined(__HIP_DEVICE_COMPILE__)
+  m = __uint_as_float(mbits);
+#else
+  memcpy(&m, &mbits, sizeof(m));
+#endif
+  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
+  const float z = (m - 1.0f) / (m + 1.0f);
+  const float z2 = z * z;
+  float poly = z2 * 0.142857149f;
+  poly = poly + 0.2f;
+  poly = poly * z2;
+  poly = poly + 0.333333343f;
+  poly = poly * z2;
+  poly = poly + 1.0f;
+  float ln_m = z * poly;
+  ln_m = ln_m * 2.0f;
+  return (float)e + ln_m * 1.44269502f;
+}
+
+// Efraimidis-Spirakis key of (sample, vertex): log2(u) / importance with u from Philox at slot
+// sample * |V| + vertex and importance the fixed-point sum of the vertex's terms (the common
+// 2^53 scale does not change the order of the keys); as sortable bits, inverted so that an
+// ascending sort yields descending keys.  No key is 0xFFFFFFFF (it would be a negative NaN):
+// kAbsentKey marks the vertices a sample's neighbourhood does not hold.
+constexpr uint32_t kAbsentKey = 0xFFFFFFFFu;
+// importance sums stay below 2^63 (at most 1024 transits, each adding at most 2^53)
+constexpr unsigned long long kAbsentSum = ~0ull;
+__device__ __forceinline__ uint32_t ladies_key_bits(unsigned long long importance_fixed, uint64_t slot, uint32_t step,
+                                                    uint64_t seed) {
+  const float importance = (float)importance_fixed;
+  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
+                                        (uint32_t)(seed >> 32));
+  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+  float key = -__builtin_inff();
+  if (importance > 0.0f) key = det_log2(u) / importance;
+  uint32_t b = __float_as_uint(key);
+  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  return ~b;
+}
+
 // ---- wave-wide data movement on the VALU (DPP), no LDS traffic ----
 // The value of the lane `shift` below inside the lane's row of 16; lanes without one get `fill`.
 template <int kShift>
@@ -229,8 +281,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
-    unsigned long long* __restrict__ sums,
-    uint32_t sums_per_sample) {
+    unsigned long long* __restrict__ sums, uint32_t keys_per_sample) {
   constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
   constexpr uint32_t kBinVertices = kBinWords * 32u;
   // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
@@ -410,25 +461,27 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     }
   }
   __syncthreads();
-  const uint32_t first_word = bin * kBinWords;
-  uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
-  for (uint32_t i = threadIdx.x; i < kBinWords && first_word + i < words_per_sample; i += kBinThreads) {
-    uint32_t word = 0;
-    if (kWithImportance) {
-      word = s_bits[i];
-    } else {
+  if (kWithImportance) {
+    // LADIES form: what leaves the workgroup is the importance sum of every vertex of the
+    // stretch (kAbsentSum where the neighbourhood does not hold the vertex); no bitmap.  (The
+    // sampling keys are formed by the first pass of the selection: done here, next to the
+    // streaming of the other workgroup of the compute unit, the same arithmetic took 100 ms
+    // instead of 13.)
+    unsigned long long* out = sums + (size_t)s * keys_per_sample + v_lo;
+    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads)
+      __builtin_nontemporal_store(((s_bits[i >> 5] >> (i & 31u)) & 1u) ? s_acc[i] : kAbsentSum, &out[i]);
+  } else {
+    const uint32_t first_word = bin * kBinWords;
+    uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
+    for (uint32_t i = threadIdx.x; i < kBinWords && first_word + i < words_per_sample; i += kBinThreads) {
+      uint32_t word = 0;
 #pragma unroll
       for (uint32_t q = 0; q < 8; ++q) {  // 32 bytes, each 0 or 1 -> 32 bits
         const uint32_t four = s_bits[i * 8u + q];
         word |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
       }
+      out[i] = word;
     }
-    out[i] = word;
-  }
-  if (kWithImportance) {
-    // only the sums of marked vertices are ever read
-    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads)
-      if ((s_bits[i >> 5] >> (i & 31u)) & 1u) sums[(size_t)s * sums_per_sample + v_lo + i] = s_acc[i];
   }
   __syncthreads();  // the next stretch clears what this one has just read
   }
@@ -447,54 +500,6 @@ __global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __rest
   if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
 }
 
-// log2 of a positive normal float from exponent extraction and an atanh series; every step
-// is a single IEEE operation so that host and device agree bit for bit.
-__host__ __device__ __forceinline__ float det_log2(float x) {
-  uint32_t bits;
-#if defined(__HIP_DEVICE_COMPILE__)
-  bits = __float_as_uint(x);
-#else
-  memcpy(&bits, &x, sizeof(bits));
-#endif
-  int e = (int)(bits >> 23) - 127;
-  const uint32_t mbits = (bits & 0x7FFFFFu) | 0x3F800000u;
-  float m;
-#if defined(__HIP_DEVICE_COMPILE__)
-  m = __uint_as_float(mbits);
-#else
-  memcpy(&m, &mbits, sizeof(m));
-#endif
-  if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
-  const float z = (m - 1.0f) / (m + 1.0f);
-  const float z2 = z * z;
-  float poly = z2 * 0.142857149f;
-  poly = poly + 0.2f;
-  poly = poly * z2;
-  poly = poly + 0.333333343f;
-  poly = poly * z2;
-  poly = poly + 1.0f;
-  float ln_m = z * poly;
-  ln_m = ln_m * 2.0f;
-  return (float)e + ln_m * 1.44269502f;
-}
-
-// Efraimidis-Spirakis key of (sample, vertex): log2(u) / importance with u from Philox at slot
-// sample * |V| + vertex and importance the fixed-point sum of the vertex's terms (the common
-// 2^53 scale does not change the order of the keys); as sortable bits, inverted so that an
-// ascending sort yields descending keys.
-__device__ __forceinline__ uint32_t ladies_key_bits(unsigned long long importance_fixed, uint64_t slot, uint32_t step,
-                                                    uint64_t seed) {
-  const float importance = (float)importance_fixed;
-  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
-                                        (uint32_t)(seed >> 32));
-  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
-  float key = -__builtin_inff();
-  if (importance > 0.0f) key = det_log2(u) / importance;
-  uint32_t b = __float_as_uint(key);
-  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-  return ~b;
-}
-
 // degree(ids[i])^2, computed where the running sums are formed instead of being stored
 struct DegreeSquaredOf {
   const int32_t* ids;
@@ -508,16 +513,11 @@ struct DegreeSquaredOf {
 
 // The marked vertices of every sample, in ascending order, become the sample's distinct
 // vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
-// tile of a sample is where the sample's list starts).  With sums given (LADIES form), the
-// vertex's sampling key is formed from the importance accumulated for it.
+// tile of a sample is where the sample's list starts).
 __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t tiles_per_sample, int32_t* __restrict__ distinct_ids,
-                                                      uint32_t* __restrict__ distinct_start,
-                                                      const unsigned long long* __restrict__ sums,
-                                                      uint32_t sums_per_sample, uint64_t seed, uint64_t first_sample,
-                                                      uint32_t step, uint32_t* __restrict__ key_bits,
-                                                      uint32_t* __restrict__ distinct_sample) {
+                                                      uint32_t* __restrict__ distinct_start) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t s_before[kScanThreads];  // set bits of the tile before word 8 * t
   const uint32_t sample = blockIdx.x / tiles_per_sample;
@@ -550,11 +550,6 @@ __global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict
       const uint32_t v = (tile * kBitmapTileWords + w) * kVerticesPerWord + lane;
       const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       distinct_ids[at] = (int32_t)v;
-      if (sums) {
-        const uint64_t slot = (first_sample + sample) * (uint64_t)sums_per_sample + v;  // sums_per_sample = |V|
-        key_bits[at] = ladies_key_bits(sums[(size_t)sample * sums_per_sample + v], slot, step, seed);
-        distinct_sample[at] = sample;
-      }
     }
     r += (uint32_t)__popcll(mask);
   }
@@ -593,35 +588,59 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
 // entries with a prefix <= T (m and a few more) are copied out in order and only those are
 // sorted.  Entries are grouped by sample, so a workgroup counts into an LDS histogram for the
 // sample its tile begins with and falls back to global atomics for the few entries beyond.
-constexpr uint32_t kSelectTile = 2048;  // entries per workgroup (256 lanes x 8)
+// The keys of a chunk are dense: keys[s * keys_per_sample + v] for every vertex v (kAbsentKey
+// where sample s does not hold v), so position tells sample and vertex and no list of the
+// distinct pairs is ever written.  A workgroup takes kSelectTile consecutive vertices of one
+// sample: blockIdx.x = tile of the sample, blockIdx.y = sample.
+constexpr uint32_t kSelectPerLane = 32;
+constexpr uint32_t kSelectTile = 256 * kSelectPerLane;
 
-// level 0: hist[s][key >> 24]; level 1: hist[s][(key >> 16) & 255] over entries whose upper 8
-// bits equal prefix8[s]
-__global__ __launch_bounds__(256) void select_histogram(const uint32_t* __restrict__ key_bits,
-                                                        const uint32_t* __restrict__ distinct_sample, uint32_t n,
-                                                        int level, const uint32_t* __restrict__ prefix8,
-                                                        uint32_t* __restrict__ hist) {
+// level 0: forms the keys - keys[s][v] from sums[s][v], Philox slot (first_sample + s) * |V| + v -
+// and counts hist[s][key >> 24] over the sample's present keys, present[s] = how many there
+// are; level 1: hist[s][(key >> 16) & 255] over the keys whose upper 8 bits equal prefix8[s]
+__global__ __launch_bounds__(256) void select_histogram(const unsigned long long* __restrict__ sums,
+                                                        uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+                                                        int level, uint32_t n_vertices, uint64_t seed,
+                                                        uint64_t first_sample, uint32_t step,
+                                                        const uint32_t* __restrict__ prefix8,
+                                                        uint32_t* __restrict__ hist, uint32_t* __restrict__ present) {
   __shared__ uint32_t s_hist[256];
+  __shared__ uint32_t s_present;
   s_hist[threadIdx.x] = 0;
+  if (threadIdx.x == 0) s_present = 0;
+  const uint32_t s = blockIdx.y;
+  uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  const unsigned long long* my_sums = sums + (size_t)s * keys_per_sample;
   const uint32_t tile_begin = blockIdx.x * kSelectTile;
-  const uint32_t first_sample = distinct_sample[tile_begin];
+  const uint32_t want8 = level == 1 ? prefix8[s] : 0u;
   __syncthreads();
-  for (uint32_t k = 0; k < kSelectTile / 256; ++k) {
-    const uint32_t i = tile_begin + k * 256 + threadIdx.x;
-    if (i >= n) break;
-    const uint32_t key = key_bits[i];
-    const uint32_t s = distinct_sample[i];
+  uint32_t seen = 0;
+  for (uint32_t k = 0; k < kSelectPerLane; ++k) {
+    const uint32_t v = tile_begin + k * 256 + threadIdx.x;
+    if (v >= keys_per_sample) break;
+    uint32_t key;
+    if (level == 0) {
+      const unsigned long long sum = my_sums[v];
+      key = sum == kAbsentSum ? kAbsentKey
+                              : ladies_key_bits(sum, (first_sample + s) * (uint64_t)n_vertices + v, step, seed);
+      mine[v] = key;
+    } else {
+      key = mine[v];
+    }
+    if (key == kAbsentKey) continue;
+    ++seen;
     uint32_t bin = key >> 24;
     if (level == 1) {
-      if (bin != prefix8[s]) continue;
+      if (bin != want8) continue;
       bin = (key >> 16) & 255u;
     }
-    if (s == first_sample) atomicAdd(&s_hist[bin], 1u);
-    else atomicAdd(&hist[(size_t)s * 256 + bin], 1u);
+    atomicAdd(&s_hist[bin], 1u);
   }
+  if (level == 0 && seen) atomicAdd(&s_present, seen);
   __syncthreads();
   const uint32_t c = s_hist[threadIdx.x];
-  if (c) atomicAdd(&hist[(size_t)first_sample * 256 + threadIdx.x], c);
+  if (c) atomicAdd(&hist[(size_t)s * 256 + threadIdx.x], c);
+  if (level == 0 && threadIdx.x == 0 && s_present) atomicAdd(&present[s], s_present);
 }
 
 // One lane per sample walks its 256 bins.  level 0: prefix8[s] = bin holding the need-th
@@ -660,49 +679,66 @@ __global__ void select_pick(const uint32_t* __restrict__ hist, uint32_t n_sample
   }
 }
 
-__device__ __forceinline__ bool select_keeps(const uint32_t* key_bits, const uint32_t* distinct_sample,
-                                             const uint32_t* threshold16, uint32_t i) {
-  return (key_bits[i] >> 16) <= threshold16[distinct_sample[i]];
+__device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold16) {
+  return key != kAbsentKey && (key >> 16) <= threshold16;
 }
 
-__global__ __launch_bounds__(256) void select_count(const uint32_t* __restrict__ key_bits,
-                                                    const uint32_t* __restrict__ distinct_sample,
-                                                    const uint32_t* __restrict__ threshold16, uint32_t n,
+// tile_counts[s * gridDim.x + tile] = keys of the tile that stay
+__global__ __launch_bounds__(256) void select_count(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+                                                    const uint32_t* __restrict__ threshold16,
                                                     uint32_t* __restrict__ tile_counts) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
-  const uint32_t base = blockIdx.x * kSelectTile + threadIdx.x * 8u;
-  uint32_t mine = 0;
-  for (uint32_t k = 0; k < 8; ++k)
-    if (base + k < n && select_keeps(key_bits, distinct_sample, threshold16, base + k)) mine++;
+  const uint32_t s = blockIdx.y;
+  const uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  const uint32_t threshold = threshold16[s];
+  const uint32_t tile_begin = blockIdx.x * kSelectTile;
+  uint32_t stay = 0;
+  for (uint32_t k = 0; k < kSelectPerLane; ++k) {
+    const uint32_t v = tile_begin + k * 256 + threadIdx.x;
+    if (v < keys_per_sample && select_keeps(mine[v], threshold)) stay++;
+  }
   uint32_t total;
-  block_exclusive_scan_256(mine, s_wave, &total);
-  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+  block_exclusive_scan_256(stay, s_wave, &total);
+  if (threadIdx.x == 0) tile_counts[(size_t)s * gridDim.x + blockIdx.x] = total;
 }
 
-// Copies the kept entries out, in order: key, sample and vertex id.
-__global__ __launch_bounds__(256) void select_compact(const uint32_t* __restrict__ key_bits,
-                                                      const uint32_t* __restrict__ distinct_sample,
-                                                      const int32_t* __restrict__ distinct_ids,
-                                                      const uint32_t* __restrict__ threshold16, uint32_t n,
+// Copies the kept entries out, in (sample, vertex) order: key, sample and vertex id.  A
+// wavefront takes a quarter of the tile, 64 consecutive vertices per round: once to count what
+// it keeps, once more to write.
+__global__ __launch_bounds__(256) void select_compact(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+                                                      const uint32_t* __restrict__ threshold16,
                                                       const uint32_t* __restrict__ tile_offsets,
                                                       uint32_t* __restrict__ kept_key, uint32_t* __restrict__ kept_sample,
                                                       int32_t* __restrict__ kept_id) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
-  const uint32_t base = blockIdx.x * kSelectTile + threadIdx.x * 8u;
-  bool keep[8];
-  uint32_t mine = 0;
-  for (uint32_t k = 0; k < 8; ++k) {
-    keep[k] = base + k < n && select_keeps(key_bits, distinct_sample, threshold16, base + k);
-    mine += keep[k] ? 1u : 0u;
+  __shared__ uint32_t s_kept_by_wave[kScanThreads / kWave];
+  constexpr uint32_t kPerWave = kSelectTile / (kScanThreads / kWave);
+  const uint32_t s = blockIdx.y;
+  const uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  const uint32_t threshold = threshold16[s];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t begin = blockIdx.x * kSelectTile + wave * kPerWave;
+  uint32_t kept = 0;
+  for (uint32_t v0 = begin; v0 < begin + kPerWave; v0 += 64) {
+    const uint32_t v = v0 + lane;
+    kept += (uint32_t)__popcll(__ballot(v < keys_per_sample && select_keeps(mine[v], threshold)));
   }
-  uint32_t total;
-  uint32_t r = block_exclusive_scan_256(mine, s_wave, &total) + tile_offsets[blockIdx.x];
-  for (uint32_t k = 0; k < 8; ++k) {
-    if (!keep[k]) continue;
-    kept_key[r] = key_bits[base + k];
-    kept_sample[r] = distinct_sample[base + k];
-    kept_id[r] = distinct_ids[base + k];
-    ++r;
+  if (lane == 0) s_kept_by_wave[wave] = kept;
+  __syncthreads();
+  uint32_t r = tile_offsets[(size_t)s * gridDim.x + blockIdx.x];
+  for (uint32_t w = 0; w < wave; ++w) r += s_kept_by_wave[w];
+  if (kept == 0) return;
+  for (uint32_t v0 = begin; v0 < begin + kPerWave; v0 += 64) {
+    const uint32_t v = v0 + lane;
+    const uint32_t key = v < keys_per_sample ? mine[v] : kAbsentKey;
+    const bool stays = select_keeps(key, threshold);
+    const uint64_t mask = __ballot(stays);
+    if (stays) {
+      const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+      kept_key[at] = key;
+      kept_sample[at] = s;
+      kept_id[at] = (int32_t)v;
+    }
+    r += (uint32_t)__popcll(mask);
   }
 }
 
@@ -788,7 +824,7 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
 constexpr uint64_t kLayerChunkEntries = 96ull << 20;
 // Importance forms: nothing is stored per entry, so a chunk is bounded by the memory of its
 // presence maps (and accumulators) and by the number of marking work items (entries / kBuildItemEntries) of one launch.
-constexpr uint64_t kBitmapBudgetBytes = 24ull << 30;
+constexpr uint64_t kBitmapBudgetBytes = 48ull << 30;
 constexpr uint64_t kBitmapChunkEntries = 1ull << 40;
 
 template <class SampleType, class App>
@@ -880,10 +916,15 @@ class LayerEngine : public EngineBase {
     const uint32_t per_word = 32u;
     bitmap_words_ = (((uint32_t)invalid_ + per_word - 1u) / per_word + kBitmapTileWords - 1) / kBitmapTileWords *
                     kBitmapTileWords;
-    // LADIES form: one 64-bit importance accumulator per vertex next to the bitmap
-    sums_per_sample_ = App::kNeighborhoodForm == apps::kRankedByLadiesImportance ? (uint32_t)invalid_ : 0u;
-    const uint64_t fit = kBitmapBudgetBytes / ((uint64_t)bitmap_words_ * sizeof(uint32_t) +
-                                               (uint64_t)sums_per_sample_ * sizeof(unsigned long long));
+    // bytes a sample of a chunk holds: its bitmap (FastGCN form) or one key per vertex, padded
+    // to whole stretches (LADIES form)
+    uint64_t bytes_per_sample = (uint64_t)bitmap_words_ * sizeof(uint32_t);
+    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+      const uint32_t bin_words = kBinVerticesSums / 32u;
+      bytes_per_sample = (uint64_t)((bitmap_words_ + bin_words - 1) / bin_words) * kBinVerticesSums *
+                         (sizeof(uint32_t) + sizeof(unsigned long long));
+    }
+    const uint64_t fit = kBitmapBudgetBytes / bytes_per_sample;
     bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
@@ -921,6 +962,7 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_select_kept_, per_sample));
       ND_HIP_TRY(hipMalloc(&d_select_threshold_, per_sample));
       ND_HIP_TRY(hipMalloc(&d_select_hist_, sizeof(uint32_t) * 256 * (size_t)n_samples_));
+      ND_HIP_TRY(hipMalloc(&d_select_present_, per_sample));
     }
     return 0;
   }
@@ -1098,34 +1140,37 @@ class LayerEngine : public EngineBase {
     return 0;
   }
 
-  // Distinct vertices of every sample of the chunk, ascending: mark bits (and add up
-  // importance), count the bits per tile, scan, write the ids out.  Then running sums of
-  // degree^2, or the ranking by Efraimidis-Spirakis key.
+  // What next() of the importance forms is handed, for every sample of the chunk.
   int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n, unsigned n_items) {
-    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
-    const uint32_t tiles_per_sample = bitmap_words_ / kBitmapTileWords;
-    const size_t n_tiles = (size_t)n * tiles_per_sample;
-    if (n > bitmap_samples_) {
-      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_sums_);
-      ND_HIP_TRY(hipMalloc(&d_bitmap_, sizeof(uint32_t) * (size_t)n * bitmap_words_));
-      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
-      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
-      if (ladies) {
-        // never cleared: the sum of a vertex is written whenever the vertex is marked, and read only then
-        const size_t bytes = sizeof(unsigned long long) * (size_t)n * sums_per_sample_;
-        ND_HIP_TRY(hipMalloc(&d_sums_, bytes));
-      }
-      bitmap_samples_ = n;
-    }
     (void)n_items;
+    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
     constexpr uint32_t per_group = ladies ? kBinsPerGroupSums : kBinsPerGroupBits;
     const uint32_t groups = (bins + per_group - 1) / per_group;
     if ((uint64_t)n * groups >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
+    if constexpr (ladies) {
+      return rank_by_keys(step, s0, tv, n, bins, groups);
+    } else {
+      return list_distinct(tv, n, bins, groups);
+    }
+  }
+
+  // FastGCN form: the distinct vertices of every sample, ascending (mark bits, count them per
+  // tile, scan, write the ids out), and the running sums of degree^2 over them.
+  int list_distinct(const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
+    const uint32_t tiles_per_sample = bitmap_words_ / kBitmapTileWords;
+    const size_t n_tiles = (size_t)n * tiles_per_sample;
+    if (n > bitmap_samples_) {
+      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
+      ND_HIP_TRY(hipMalloc(&d_bitmap_, sizeof(uint32_t) * (size_t)n * bitmap_words_));
+      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
+      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
+      bitmap_samples_ = n;
+    }
     tick();
-    collective_mark_binned<ladies><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, d_row_sums_, d_sums_, sums_per_sample_);
+    collective_mark_binned<false><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
+        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u);
     tock();
     bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
     ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
@@ -1135,62 +1180,85 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     distinct_total_ += n_distinct;
     if (ensure_distinct_capacity(n_distinct) != 0) return -1;
-    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(
-        d_bitmap_, d_tile_offsets_, tiles_per_sample, d_distinct_ids_, d_distinct_start_, d_sums_, sums_per_sample_, seed_,
-        (uint64_t)s0, (uint32_t)step, d_key_bits_, d_distinct_sample_);
+    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_, tiles_per_sample,
+                                                                       d_distinct_ids_, d_distinct_start_);
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
-    if (!ladies) {
-      ND_HIP_TRY(inclusive_scan_u64_of(DegreeSquaredOf{d_distinct_ids_, dgraph_.row_ptr()}, d_running_sums_, n_distinct,
-                                       d_scratch64_, stream_));
-    } else if (n_distinct > 0) {
+    ND_HIP_TRY(inclusive_scan_u64_of(DegreeSquaredOf{d_distinct_ids_, dgraph_.row_ptr()}, d_running_sums_, n_distinct,
+                                     d_scratch64_, stream_));
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
+
+  // LADIES form: the marking leaves one sampling key per (sample, vertex); per sample, the
+  // vertices that can be among its first `wanted` in key order are picked by a radix select on
+  // the upper 16 bits of the key and ordered by descending key.  The distinct pairs of a
+  // sample (2.4 M per batch at full size) are never listed.
+  int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
+    const uint32_t keys_per_sample = bins * kBinVerticesSums;
+    const uint32_t tiles_per_sample = (keys_per_sample + kSelectTile - 1) / kSelectTile;
+    const size_t n_tiles = (size_t)n * tiles_per_sample;
+    if (n > bitmap_samples_) {
+      release(d_keys_dense_); release(d_sums_dense_); release(d_tile_offsets_); release(d_tile_scratch_);
+      ND_HIP_TRY(hipMalloc(&d_keys_dense_, sizeof(uint32_t) * (size_t)n * keys_per_sample));
+      ND_HIP_TRY(hipMalloc(&d_sums_dense_, sizeof(unsigned long long) * (size_t)n * keys_per_sample));
+      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
+      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
+      bitmap_samples_ = n;
+    }
+    tick();
+    collective_mark_binned<true><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
+        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample);
+    tock();
+    const uint32_t wanted = (uint32_t)App().stepSize(step);
+    const dim3 tiles(tiles_per_sample, n);
+    const unsigned sample_blocks = (n + 255) / 256;
+    ND_HIP_TRY(hipMemsetAsync(d_select_present_, 0, sizeof(uint32_t) * (size_t)n, stream_));
+    for (int level = 0; level < 2; ++level) {
+      ND_HIP_TRY(hipMemsetAsync(d_select_hist_, 0, sizeof(uint32_t) * 256 * (size_t)n, stream_));
+      select_histogram<<<tiles, dim3(256), 0, stream_>>>(d_sums_dense_, d_keys_dense_, keys_per_sample, level,
+                                                         (uint32_t)invalid_, seed_, (uint64_t)s0, (uint32_t)step,
+                                                         d_select_prefix_, d_select_hist_, d_select_present_);
+      select_pick<<<dim3(sample_blocks), dim3(256), 0, stream_>>>(d_select_hist_, n, level, wanted, d_select_prefix_,
+                                                                  d_select_need_, d_select_kept_, d_select_threshold_);
+    }
+    // where every sample's ranked list starts: exclusive scan of the kept counts
+    fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
+    ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
+    select_count<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_, d_tile_offsets_);
+    ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
+    uint32_t n_kept = 0;
+    ND_HIP_TRY(hipMemcpyAsync(&n_kept, d_tile_scratch_ + scan_num_tiles(n_tiles), sizeof(uint32_t),
+                              hipMemcpyDeviceToHost, stream_));
+    std::vector<uint32_t> present(n);
+    ND_HIP_TRY(hipMemcpyAsync(present.data(), d_select_present_, sizeof(uint32_t) * n, hipMemcpyDeviceToHost, stream_));
+    ND_HIP_TRY(hipStreamSynchronize(stream_));
+    for (uint32_t c : present) distinct_total_ += c;
+    if (ensure_distinct_capacity(n_kept) != 0) return -1;
+    select_compact<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_,
+                                                     d_tile_offsets_, d_kept_key_, d_kept_sample_, d_kept_id_);
+    // order the kept vertices of every sample by descending key: the list is in
+    // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
+    // ascending vertex id among equal keys
+    if (n_kept > 0) {
       int chunk_bits = 1;
       while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
-      // per sample, the entries that can be among its first `wanted` in key order (radix select
-      // on the upper 16 bits of the key), copied out in (sample, vertex) order
-      const uint32_t wanted = (uint32_t)App().stepSize(step);
-      const unsigned tiles = (n_distinct + kSelectTile - 1) / kSelectTile;
-      const unsigned sample_blocks = (n + 255) / 256;
-      for (int level = 0; level < 2; ++level) {
-        ND_HIP_TRY(hipMemsetAsync(d_select_hist_, 0, sizeof(uint32_t) * 256 * (size_t)n, stream_));
-        select_histogram<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, n_distinct, level,
-                                                                 d_select_prefix_, d_select_hist_);
-        select_pick<<<dim3(sample_blocks), dim3(256), 0, stream_>>>(d_select_hist_, n, level, wanted, d_select_prefix_,
-                                                                    d_select_need_, d_select_kept_, d_select_threshold_);
-      }
-      // where every sample's ranked list starts: exclusive scan of the kept counts
-      fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
-      ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
-      select_count<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, d_select_threshold_,
-                                                           n_distinct, d_scratch_);
-      scan_of_totals<<<dim3(1), dim3(kScanThreads), 0, stream_>>>(d_scratch_, tiles);
-      select_compact<<<dim3(tiles), dim3(256), 0, stream_>>>(d_key_bits_, d_distinct_sample_, d_distinct_ids_,
-                                                             d_select_threshold_, n_distinct, d_scratch_, d_kept_key_,
-                                                             d_kept_sample_, d_kept_id_);
-      uint32_t n_kept = 0;
-      ND_HIP_TRY(hipMemcpyAsync(&n_kept, d_scratch_ + tiles, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_));
-      ND_HIP_TRY(hipStreamSynchronize(stream_));
-      // order the kept vertices of every sample by descending key: the list is in
-      // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
-      // ascending vertex id among equal keys
-      if (n_kept > 0) {
-        const SortPlan by_key = make_sort_plan(n_kept, 32);
-        uint32_t *k3 = nullptr, *j3 = nullptr;
-        ND_HIP_TRY(radix_sort_pairs(by_key, d_kept_key_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
-                                    d_scratch_, stream_, &k3, &j3));
-        const unsigned blocks = (n_kept + 255) / 256;
-        gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_kept_sample_, j3, n_kept, d_key2_, d_index2_);
-        const SortPlan by_sample = make_sort_plan(n_kept, chunk_bits);
-        uint32_t *k4 = nullptr, *j4 = nullptr;
-        ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
-                                    d_scratch_, stream_, &k4, &j4));
-        gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_kept_id_, j4, n_kept,
-                                                            (uint32_t*)d_ranked_ids_, nullptr);
-      }
+      const SortPlan by_key = make_sort_plan(n_kept, 32);
+      uint32_t *k3 = nullptr, *j3 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_key, d_kept_key_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                  d_scratch_, stream_, &k3, &j3));
+      const unsigned blocks = (n_kept + 255) / 256;
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_kept_sample_, j3, n_kept, d_key2_, d_index2_);
+      const SortPlan by_sample = make_sort_plan(n_kept, chunk_bits);
+      uint32_t *k4 = nullptr, *j4 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_sample, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+                                  d_scratch_, stream_, &k4, &j4));
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>((const uint32_t*)d_kept_id_, j4, n_kept,
+                                                          (uint32_t*)d_ranked_ids_, nullptr);
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
   }
 
-  // Arrays with one entry per distinct (sample, vertex) pair of a chunk.
+  // Arrays with one entry per listed (sample, vertex) pair of a chunk: the distinct pairs
+  // (FastGCN form) or the pairs the selection keeps (LADIES form).
   int ensure_distinct_capacity(uint32_t n_distinct) {
     if (n_distinct <= distinct_capacity_ && distinct_capacity_ > 0) return 0;
     constexpr int form = App::kNeighborhoodForm;
@@ -1202,8 +1270,6 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
     }
     if (form == apps::kRankedByLadiesImportance) {
-      ND_HIP_TRY(hipMalloc(&d_distinct_sample_, sizeof(uint32_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_key_bits_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_kept_key_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_kept_sample_, sizeof(uint32_t) * cap));
@@ -1216,7 +1282,6 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_index2_, sizeof(uint32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_hist_, sizeof(uint32_t) * sort_hist_capacity(cap)));
       size_t scratch = make_sort_plan(cap, 32).scratch_elems;
-      if (cap / kSelectTile + 2 > scratch) scratch = cap / kSelectTile + 2;  // tile counts of the selection
       ND_HIP_TRY(hipMalloc(&d_scratch_, sizeof(uint32_t) * scratch));
     }
     distinct_capacity_ = cap;
@@ -1236,7 +1301,7 @@ class LayerEngine : public EngineBase {
 
   void release_distinct_buffers() {
     release(d_distinct_ids_); release(d_running_sums_); release(d_scratch64_);
-    release(d_distinct_sample_); release(d_key_bits_); release(d_ranked_ids_);
+    release(d_ranked_ids_);
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
     release(d_kept_key_); release(d_kept_sample_); release(d_kept_id_);
@@ -1245,7 +1310,7 @@ class LayerEngine : public EngineBase {
 
   void release_neighborhood_buffers() {
     release(d_nbr_cols_); release(d_nbr_weights_);
-    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_sums_);
+    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_keys_dense_); release(d_sums_dense_);
     release_distinct_buffers();
     capacity_ = 0;
     bitmap_samples_ = 0;
@@ -1257,7 +1322,7 @@ class LayerEngine : public EngineBase {
     release(d_item_count_); release(d_item_start_);
     release(d_distinct_start_);
     release(d_ranked_start_); release(d_select_prefix_); release(d_select_need_); release(d_select_kept_);
-    release(d_select_threshold_); release(d_select_hist_);
+    release(d_select_threshold_); release(d_select_hist_); release(d_select_present_);
     release_neighborhood_buffers();
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
@@ -1288,8 +1353,9 @@ class LayerEngine : public EngineBase {
   uint32_t bitmap_samples_ = 0;        // samples the allocated bitmaps hold
   size_t distinct_capacity_ = 0;
   uint32_t *d_bitmap_ = nullptr, *d_tile_offsets_ = nullptr, *d_tile_scratch_ = nullptr;
-  unsigned long long* d_sums_ = nullptr;  // LADIES form: importance accumulators, [sample][vertex]
-  uint32_t sums_per_sample_ = 0;
+  // LADIES form: importance sums and sampling keys, [sample][vertex, padded to whole stretches]
+  unsigned long long* d_sums_dense_ = nullptr;
+  uint32_t* d_keys_dense_ = nullptr;
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
   uint64_t chunk_entries_ = kLayerChunkEntries;
   bool progress_ = false;
@@ -1306,6 +1372,7 @@ class LayerEngine : public EngineBase {
   // LADIES form: the selection of the best keys per sample
   uint32_t *d_ranked_start_ = nullptr, *d_select_prefix_ = nullptr, *d_select_need_ = nullptr;
   uint32_t *d_select_kept_ = nullptr, *d_select_threshold_ = nullptr, *d_select_hist_ = nullptr;
+  uint32_t* d_select_present_ = nullptr;  // present[s]: distinct vertices of sample s's neighbourhood
   uint32_t *d_kept_key_ = nullptr, *d_kept_sample_ = nullptr;
   int32_t* d_kept_id_ = nullptr;
   int32_t* d_nbr_cols_ = nullptr;
@@ -1314,7 +1381,6 @@ class LayerEngine : public EngineBase {
   uint32_t *d_key2_ = nullptr, *d_index2_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
   int32_t* d_distinct_ids_ = nullptr;
   uint64_t *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
-  uint32_t *d_distinct_sample_ = nullptr, *d_key_bits_ = nullptr;
   int32_t* d_ranked_ids_ = nullptr;
 };
 
