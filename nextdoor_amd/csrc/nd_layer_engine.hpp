@@ -683,62 +683,36 @@ __device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold16)
   return key != kAbsentKey && (key >> 16) <= threshold16;
 }
 
-// tile_counts[s * gridDim.x + tile] = keys of the tile that stay
-__global__ __launch_bounds__(256) void select_count(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
-                                                    const uint32_t* __restrict__ threshold16,
-                                                    uint32_t* __restrict__ tile_counts) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
+// Copies the kept entries of sample s into its stretch [ranked_start[s], ranked_start[s + 1]) of
+// kept_key / kept_id, in whatever order the wavefronts get there (a wavefront claims room for
+// the entries of a round with one atomic; a few hundred of a sample's millions of keys stay,
+// so most rounds claim nothing).  The sorts that follow fix the order.
+__global__ __launch_bounds__(256) void select_collect(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+                                                      const uint32_t* __restrict__ threshold16,
+                                                      const uint32_t* __restrict__ ranked_start,
+                                                      uint32_t* __restrict__ claimed, uint32_t* __restrict__ kept_key,
+                                                      uint32_t* __restrict__ kept_sample, int32_t* __restrict__ kept_id) {
   const uint32_t s = blockIdx.y;
   const uint32_t* mine = keys + (size_t)s * keys_per_sample;
   const uint32_t threshold = threshold16[s];
+  const uint32_t first = ranked_start[s];
+  const uint32_t lane = threadIdx.x & 63u;
   const uint32_t tile_begin = blockIdx.x * kSelectTile;
-  uint32_t stay = 0;
   for (uint32_t k = 0; k < kSelectPerLane; ++k) {
     const uint32_t v = tile_begin + k * 256 + threadIdx.x;
-    if (v < keys_per_sample && select_keeps(mine[v], threshold)) stay++;
-  }
-  uint32_t total;
-  block_exclusive_scan_256(stay, s_wave, &total);
-  if (threadIdx.x == 0) tile_counts[(size_t)s * gridDim.x + blockIdx.x] = total;
-}
-
-// Copies the kept entries out, in (sample, vertex) order: key, sample and vertex id.  A
-// wavefront takes a quarter of the tile, 64 consecutive vertices per round: once to count what
-// it keeps, once more to write.
-__global__ __launch_bounds__(256) void select_compact(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
-                                                      const uint32_t* __restrict__ threshold16,
-                                                      const uint32_t* __restrict__ tile_offsets,
-                                                      uint32_t* __restrict__ kept_key, uint32_t* __restrict__ kept_sample,
-                                                      int32_t* __restrict__ kept_id) {
-  __shared__ uint32_t s_kept_by_wave[kScanThreads / kWave];
-  constexpr uint32_t kPerWave = kSelectTile / (kScanThreads / kWave);
-  const uint32_t s = blockIdx.y;
-  const uint32_t* mine = keys + (size_t)s * keys_per_sample;
-  const uint32_t threshold = threshold16[s];
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t begin = blockIdx.x * kSelectTile + wave * kPerWave;
-  uint32_t kept = 0;
-  for (uint32_t v0 = begin; v0 < begin + kPerWave; v0 += 64) {
-    const uint32_t v = v0 + lane;
-    kept += (uint32_t)__popcll(__ballot(v < keys_per_sample && select_keeps(mine[v], threshold)));
-  }
-  if (lane == 0) s_kept_by_wave[wave] = kept;
-  __syncthreads();
-  uint32_t r = tile_offsets[(size_t)s * gridDim.x + blockIdx.x];
-  for (uint32_t w = 0; w < wave; ++w) r += s_kept_by_wave[w];
-  if (kept == 0) return;
-  for (uint32_t v0 = begin; v0 < begin + kPerWave; v0 += 64) {
-    const uint32_t v = v0 + lane;
     const uint32_t key = v < keys_per_sample ? mine[v] : kAbsentKey;
     const bool stays = select_keeps(key, threshold);
     const uint64_t mask = __ballot(stays);
+    if (mask == 0) continue;  // the same for every lane of the wavefront
+    uint32_t base = 0;
+    if (lane == (uint32_t)__ffsll((long long)mask) - 1u) base = atomicAdd(&claimed[s], (uint32_t)__popcll(mask));
+    base = __shfl(base, __ffsll((long long)mask) - 1, kWave);
     if (stays) {
-      const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+      const uint32_t at = first + base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       kept_key[at] = key;
       kept_sample[at] = s;
       kept_id[at] = (int32_t)v;
     }
-    r += (uint32_t)__popcll(mask);
   }
 }
 
@@ -1195,13 +1169,10 @@ class LayerEngine : public EngineBase {
   int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
     const uint32_t keys_per_sample = bins * kBinVerticesSums;
     const uint32_t tiles_per_sample = (keys_per_sample + kSelectTile - 1) / kSelectTile;
-    const size_t n_tiles = (size_t)n * tiles_per_sample;
     if (n > bitmap_samples_) {
-      release(d_keys_dense_); release(d_sums_dense_); release(d_tile_offsets_); release(d_tile_scratch_);
+      release(d_keys_dense_); release(d_sums_dense_);
       ND_HIP_TRY(hipMalloc(&d_keys_dense_, sizeof(uint32_t) * (size_t)n * keys_per_sample));
       ND_HIP_TRY(hipMalloc(&d_sums_dense_, sizeof(unsigned long long) * (size_t)n * keys_per_sample));
-      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
-      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
       bitmap_samples_ = n;
     }
     tick();
@@ -1223,29 +1194,33 @@ class LayerEngine : public EngineBase {
     // where every sample's ranked list starts: exclusive scan of the kept counts
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
     ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
-    select_count<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_, d_tile_offsets_);
-    ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
     uint32_t n_kept = 0;
-    ND_HIP_TRY(hipMemcpyAsync(&n_kept, d_tile_scratch_ + scan_num_tiles(n_tiles), sizeof(uint32_t),
+    ND_HIP_TRY(hipMemcpyAsync(&n_kept, d_small_scratch_ + scan_num_tiles((size_t)n + 1), sizeof(uint32_t),
                               hipMemcpyDeviceToHost, stream_));
     std::vector<uint32_t> present(n);
     ND_HIP_TRY(hipMemcpyAsync(present.data(), d_select_present_, sizeof(uint32_t) * n, hipMemcpyDeviceToHost, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     for (uint32_t c : present) distinct_total_ += c;
     if (ensure_distinct_capacity(n_kept) != 0) return -1;
-    select_compact<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_,
-                                                     d_tile_offsets_, d_kept_key_, d_kept_sample_, d_kept_id_);
-    // order the kept vertices of every sample by descending key: the list is in
-    // (sample, vertex) order; a stable sort by key and a stable sort by sample keep
-    // ascending vertex id among equal keys
+    ND_HIP_TRY(hipMemsetAsync(d_select_present_, 0, sizeof(uint32_t) * (size_t)n, stream_));  // now: room claimed
+    select_collect<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_,
+                                                     d_ranked_start_, d_select_present_, d_kept_key_, d_kept_sample_,
+                                                     d_kept_id_);
+    // order the kept vertices of every sample by descending key, equal keys by ascending
+    // vertex id: stable sorts by vertex, then by key, then by sample
     if (n_kept > 0) {
       int chunk_bits = 1;
       while (((uint64_t)n >> chunk_bits) != 0) chunk_bits++;
+      const unsigned blocks = (n_kept + 255) / 256;
+      const SortPlan by_vertex = make_sort_plan(n_kept, max_bits_);
+      uint32_t *k2 = nullptr, *j2 = nullptr;
+      ND_HIP_TRY(radix_sort_pairs(by_vertex, (const uint32_t*)d_kept_id_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_,
+                                  d_vals_b_, d_hist_, d_scratch_, stream_, &k2, &j2));
+      gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_kept_key_, j2, n_kept, d_key2_, d_index2_);
       const SortPlan by_key = make_sort_plan(n_kept, 32);
       uint32_t *k3 = nullptr, *j3 = nullptr;
-      ND_HIP_TRY(radix_sort_pairs(by_key, d_kept_key_, nullptr, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
+      ND_HIP_TRY(radix_sort_pairs(by_key, d_key2_, d_index2_, d_keys_a_, d_vals_a_, d_keys_b_, d_vals_b_, d_hist_,
                                   d_scratch_, stream_, &k3, &j3));
-      const unsigned blocks = (n_kept + 255) / 256;
       gather_u32<<<dim3(blocks), dim3(256), 0, stream_>>>(d_kept_sample_, j3, n_kept, d_key2_, d_index2_);
       const SortPlan by_sample = make_sort_plan(n_kept, chunk_bits);
       uint32_t *k4 = nullptr, *j4 = nullptr;
