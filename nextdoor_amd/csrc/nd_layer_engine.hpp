@@ -615,26 +615,39 @@ __global__ __launch_bounds__(256) void select_histogram(const unsigned long long
   const uint32_t want8 = level == 1 ? prefix8[s] : 0u;
   __syncthreads();
   uint32_t seen = 0;
-  for (uint32_t k = 0; k < kSelectPerLane; ++k) {
-    const uint32_t v = tile_begin + k * 256 + threadIdx.x;
-    if (v >= keys_per_sample) break;
-    uint32_t key;
-    if (level == 0) {
-      const unsigned long long sum = my_sums[v];
-      key = sum == kAbsentSum ? kAbsentKey
-                              : ladies_key_bits(sum, (first_sample + s) * (uint64_t)n_vertices + v, step, seed);
-      mine[v] = key;
-    } else {
-      key = mine[v];
+  if (level == 0) {
+    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 4) {
+      unsigned long long batch[4];  // four loads under way before the arithmetic starts
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        batch[k] = v < keys_per_sample ? my_sums[v] : kAbsentSum;
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        if (v >= keys_per_sample) continue;
+        uint32_t key = kAbsentKey;
+        if (batch[k] != kAbsentSum) {
+          key = ladies_key_bits(batch[k], (first_sample + s) * (uint64_t)n_vertices + v, step, seed);
+          ++seen;
+          atomicAdd(&s_hist[key >> 24], 1u);
+        }
+        mine[v] = key;
+      }
     }
-    if (key == kAbsentKey) continue;
-    ++seen;
-    uint32_t bin = key >> 24;
-    if (level == 1) {
-      if (bin != want8) continue;
-      bin = (key >> 16) & 255u;
+  } else {
+    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
+      uint32_t batch[8];
+#pragma unroll
+      for (uint32_t k = 0; k < 8; ++k) {
+        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < 8; ++k)
+        if (batch[k] != kAbsentKey && (batch[k] >> 24) == want8) atomicAdd(&s_hist[(batch[k] >> 16) & 255u], 1u);
     }
-    atomicAdd(&s_hist[bin], 1u);
   }
   if (level == 0 && seen) atomicAdd(&s_present, seen);
   __syncthreads();
@@ -698,20 +711,29 @@ __global__ __launch_bounds__(256) void select_collect(const uint32_t* __restrict
   const uint32_t first = ranked_start[s];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t tile_begin = blockIdx.x * kSelectTile;
-  for (uint32_t k = 0; k < kSelectPerLane; ++k) {
-    const uint32_t v = tile_begin + k * 256 + threadIdx.x;
-    const uint32_t key = v < keys_per_sample ? mine[v] : kAbsentKey;
-    const bool stays = select_keeps(key, threshold);
-    const uint64_t mask = __ballot(stays);
-    if (mask == 0) continue;  // the same for every lane of the wavefront
-    uint32_t base = 0;
-    if (lane == (uint32_t)__ffsll((long long)mask) - 1u) base = atomicAdd(&claimed[s], (uint32_t)__popcll(mask));
-    base = __shfl(base, __ffsll((long long)mask) - 1, kWave);
-    if (stays) {
-      const uint32_t at = first + base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-      kept_key[at] = key;
-      kept_sample[at] = s;
-      kept_id[at] = (int32_t)v;
+  for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
+    uint32_t batch[8];  // eight loads under way before the first is looked at
+#pragma unroll
+    for (uint32_t k = 0; k < 8; ++k) {
+      const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+      batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 8; ++k) {
+      const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+      const uint32_t key = batch[k];
+      const bool stays = select_keeps(key, threshold);
+      const uint64_t mask = __ballot(stays);
+      if (mask == 0) continue;  // the same for every lane of the wavefront
+      uint32_t base = 0;
+      if (lane == (uint32_t)__ffsll((long long)mask) - 1u) base = atomicAdd(&claimed[s], (uint32_t)__popcll(mask));
+      base = __shfl(base, __ffsll((long long)mask) - 1, kWave);
+      if (stays) {
+        const uint32_t at = first + base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+        kept_key[at] = key;
+        kept_sample[at] = s;
+        kept_id[at] = (int32_t)v;
+      }
     }
   }
 }
