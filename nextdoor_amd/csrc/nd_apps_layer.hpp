@@ -30,8 +30,10 @@ namespace apps {
 // What the engine hands a CollectiveNeighborhood app's next() as transitEdges /
 // transitEdgeWeights / numEdges:
 //   kConcatenated  the adjacencies of the sample's transits, concatenated (ids, float weights)
-//   kDistinctByDegreeSquared  the ascending distinct ids of that neighbourhood and the
-//                  running sums (uint64) of degree(id)^2 over them
+//   kDistinctByDegreeSquared  transitEdges is a view of the distinct ids of that neighbourhood
+//                  weighted by degree(id)^2: total() is the sum of the weights and
+//                  first_exceeding(t) the smallest id whose running sum (ids ascending) exceeds t;
+//                  numEdges = how many distinct ids there are; no weight array
 //   kRankedByLadiesImportance  the distinct ids ordered by descending Efraimidis-Spirakis key
 //                  for the LADIES importance (squared column norm of the row-normalised
 //                  adjacency restricted to the transits); no weights
@@ -93,7 +95,8 @@ struct LayerSamplingAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSamples> {
 // with replacement, from the distinct vertices D of the union neighbourhood of the previous
 // layer, vertex v with probability degree(v)^2 / sum_{D} degree^2 (the squared degree
 // normalised over D).  Exact integer inverse CDF: r = top 24 bits of the slot's first
-// Philox word, target = (r * total) >> 24, pick the first id whose running sum exceeds it.
+// Philox word, target = (r * total) >> 24, pick the first id (ascending) whose running sum
+// exceeds it.
 // Roots of a batch are drawn uniformly from all vertices from a fixed Philox stream.
 template <int kLayers, int kBatch, int kNumSamples>
 struct FastGCNImportanceAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSamples> {
@@ -105,22 +108,17 @@ struct FastGCNImportanceAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSample
 
   template <typename SampleType, typename EdgeArray, typename WeightArray>
   __device__ inline VertexID next(int, CSRPartition*, const VertexID*, const VertexID, SampleType*, const float,
-                                  EdgeArray& distinctIds, WeightArray& runningSums, const EdgePos_t numDistinct,
+                                  EdgeArray& distinctByDegreeSquared, WeightArray&, const EdgePos_t numDistinct,
                                   const VertexID_t, curandState* state) {
     if (numDistinct == 0) return -1;
-    const uint64_t total = runningSums[numDistinct - 1];
+    const uint64_t total = distinctByDegreeSquared.total();
     if (total == 0) return -1;
     const uint64_t r = state->next_word() >> 8;
     // (r * total) >> 24 with the 88-bit product held as (hi, lo)
     const uint64_t lo = r * total;
     const uint64_t hi = __umul64hi(r, total);
     const uint64_t target = (hi << 40) | (lo >> 24);
-    EdgePos_t first = 0, last = numDistinct;  // first index whose running sum exceeds target
-    while (first < last) {
-      const EdgePos_t mid = first + (last - first) / 2;
-      if (runningSums[mid] > target) last = mid; else first = mid + 1;
-    }
-    return distinctIds[first];
+    return distinctByDegreeSquared.first_exceeding(target);
   }
 
   template <class SampleType>

@@ -487,73 +487,114 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   }
 }
 
-// tile_counts[s * tiles_per_sample + t] = vertices marked in tile t of sample s's presence map
-__global__ __launch_bounds__(256) void bitmap_tile_counts(const uint32_t* __restrict__ bitmap,
-                                                          uint32_t* __restrict__ tile_counts) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
-  const uint4* words = (const uint4*)(bitmap + (size_t)blockIdx.x * kBitmapTileWords) + threadIdx.x * 2;
+// ---- FastGCN form: the marked vertices of a sample weighted by degree^2, without a list ----
+//
+// The app draws "the first marked vertex, ascending, whose running sum of degree^2 exceeds a
+// target".  Listing the marked vertices with their running sums costs 20 bytes for each of
+// the 2.0e9 distinct pairs of a full-size pass; instead the bitmap is kept and summed at two
+// levels - groups of 256 vertices (8 words) and parts of 64 groups - so that a draw searches
+// the parts of its sample, then the groups of one part, then walks one group's set bits.
+constexpr uint32_t kGroupWords = 8;
+constexpr uint32_t kGroupsPerPart = 64;
+constexpr uint32_t kPartWords = kGroupWords * kGroupsPerPart;  // 16384 vertices
+
+// One wavefront per part, one lane per group: group_through[part * 64 + g] = degree^2 of the
+// marked vertices of groups 0..g of the part; part_total[part]; marked[s] += marked vertices.
+__global__ __launch_bounds__(256) void bitmap_group_sums(const uint32_t* __restrict__ bitmap, uint32_t words_per_sample,
+                                                         uint32_t n_parts, const EdgePos_t* __restrict__ row_ptr,
+                                                         uint64_t* __restrict__ group_through,
+                                                         uint64_t* __restrict__ part_total,
+                                                         uint32_t* __restrict__ marked) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t part = blockIdx.x * (256 / kWave) + (threadIdx.x >> 6);  // over all samples
+  if (part >= n_parts) return;  // a whole wavefront
+  const uint32_t parts_per_sample = words_per_sample / kPartWords;
+  const uint32_t s = part / parts_per_sample;
+  const uint32_t first_word = (part - s * parts_per_sample) * kPartWords + lane * kGroupWords;
+  const uint4* words = (const uint4*)(bitmap + (size_t)s * words_per_sample + first_word);
   const uint4 a = words[0], b = words[1];
-  const uint32_t mine = __popc(a.x) + __popc(a.y) + __popc(a.z) + __popc(a.w) + __popc(b.x) + __popc(b.y) +
-                        __popc(b.z) + __popc(b.w);
-  uint32_t total;
-  block_exclusive_scan_256(mine, s_wave, &total);
-  if (threadIdx.x == 0) tile_counts[blockIdx.x] = total;
+  const uint32_t w[kGroupWords] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  uint64_t sum = 0;
+  uint32_t count = 0;
+#pragma unroll
+  for (uint32_t k = 0; k < kGroupWords; ++k) {
+    uint32_t bits = w[k];
+    count += __popc(bits);
+    while (bits) {
+      const uint32_t v = (first_word + k) * 32u + (uint32_t)__ffs((int)bits) - 1u;
+      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+      sum += d * d;
+      bits &= bits - 1u;
+    }
+  }
+  const uint64_t through = wave_inclusive_scan_u64(sum);
+  group_through[(size_t)part * kGroupsPerPart + lane] = through;
+  if (lane == 63) part_total[part] = through;
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) count += __shfl_xor(count, d, kWave);
+  if (lane == 0 && count) atomicAdd(&marked[s], count);
 }
 
-// degree(ids[i])^2, computed where the running sums are formed instead of being stored
-struct DegreeSquaredOf {
-  const int32_t* ids;
+// One wavefront per sample: part_before[s * (parts + 1) + p] = degree^2 of the marked vertices
+// of the sample's parts before p; entry `parts` is the sample's total.
+__global__ __launch_bounds__(64) void sample_part_sums(const uint64_t* __restrict__ part_total, uint32_t parts,
+                                                       uint64_t* __restrict__ part_before) {
+  const uint32_t s = blockIdx.x, lane = threadIdx.x;
+  uint64_t carry = 0;
+  for (uint32_t p0 = 0; p0 < parts; p0 += 64) {
+    const uint32_t p = p0 + lane;
+    const uint64_t mine = p < parts ? part_total[(size_t)s * parts + p] : 0ull;
+    const uint64_t through = wave_inclusive_scan_u64(mine);
+    if (p < parts) part_before[(size_t)s * (parts + 1) + p] = carry + through - mine;
+    const uint32_t lo = __shfl((uint32_t)through, 63, kWave), hi = __shfl((uint32_t)(through >> 32), 63, kWave);
+    carry += ((uint64_t)hi << 32) | lo;
+  }
+  if (lane == 0) part_before[(size_t)s * (parts + 1) + parts] = carry;
+}
+
+// What next() of a kDistinctByDegreeSquared app receives as transitEdges.
+struct DistinctByDegreeSquared {
+  const uint32_t* bits;           // the sample's bitmap
+  const uint64_t* part_before;    // the sample's parts + 1 entries
+  const uint64_t* group_through;  // the sample's parts * 64 entries
   const EdgePos_t* row_ptr;
-  __device__ __forceinline__ uint64_t operator()(size_t i) const {
-    const int32_t v = ids[i];
-    const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-    return d * d;
+  uint32_t parts;
+
+  __device__ __forceinline__ uint64_t total() const { return part_before[parts]; }
+
+  // the smallest marked vertex whose running sum of degree^2 (marked vertices ascending)
+  // exceeds target; target < total()
+  __device__ inline VertexID first_exceeding(uint64_t target) const {
+    uint32_t lo = 0, hi = parts;  // last part whose sum-before is <= target
+    while (hi - lo > 1) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (part_before[mid] <= target) lo = mid; else hi = mid;
+    }
+    const uint32_t part = lo;
+    target -= part_before[part];
+    const uint64_t* through = group_through + (size_t)part * kGroupsPerPart;
+    uint32_t first = 0, last = kGroupsPerPart - 1;  // first group whose sum-through exceeds target
+    while (first < last) {
+      const uint32_t mid = first + (last - first) / 2;
+      if (through[mid] > target) last = mid; else first = mid + 1;
+    }
+    if (first) target -= through[first - 1];
+    const uint32_t first_word = part * kPartWords + first * kGroupWords;
+    uint64_t running = 0;
+    VertexID found = -1;
+    for (uint32_t k = 0; k < kGroupWords && found < 0; ++k) {
+      uint32_t word = bits[first_word + k];
+      while (word) {
+        const uint32_t v = (first_word + k) * 32u + (uint32_t)__ffs((int)word) - 1u;
+        const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
+        running += d * d;
+        if (running > target) { found = (VertexID)v; break; }
+        word &= word - 1u;
+      }
+    }
+    return found;
   }
 };
-
-// The marked vertices of every sample, in ascending order, become the sample's distinct
-// vertices; tile_offsets is the exclusive scan of the tile counts (its entry at the first
-// tile of a sample is where the sample's list starts).
-__global__ __launch_bounds__(256) void bitmap_compact(const uint32_t* __restrict__ bitmap,
-                                                      const uint32_t* __restrict__ tile_offsets,
-                                                      uint32_t tiles_per_sample, int32_t* __restrict__ distinct_ids,
-                                                      uint32_t* __restrict__ distinct_start) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
-  __shared__ uint32_t s_before[kScanThreads];  // set bits of the tile before word 8 * t
-  const uint32_t sample = blockIdx.x / tiles_per_sample;
-  const uint32_t tile = blockIdx.x - sample * tiles_per_sample;
-  const uint32_t* words = bitmap + (size_t)blockIdx.x * kBitmapTileWords;
-  {
-    const uint4* mine = (const uint4*)words + threadIdx.x * 2;
-    const uint4 a = mine[0], b = mine[1];
-    const uint32_t count = __popc(a.x) + __popc(a.y) + __popc(a.z) + __popc(a.w) + __popc(b.x) + __popc(b.y) +
-                           __popc(b.z) + __popc(b.w);
-    uint32_t total;
-    s_before[threadIdx.x] = block_exclusive_scan_256(count, s_wave, &total);
-  }
-  __syncthreads();
-  const uint32_t first = tile_offsets[blockIdx.x];
-  if (tile == 0 && threadIdx.x == 0) distinct_start[sample] = first;
-  // A wavefront walks its quarter of the tile 64 vertices at a time, one vertex per lane, so
-  // that the reads (row extents, accumulators) and the writes of a round are contiguous.
-  constexpr uint32_t kWordsPerWave = kBitmapTileWords / (kScanThreads / kWave);
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t first_word = wave * kWordsPerWave;
-  uint32_t r = first + s_before[first_word / 8];
-  constexpr uint32_t kWordsPerRound = 2u;  // 64 vertices
-  constexpr uint32_t kVerticesPerWord = 32u;
-  for (uint32_t w = first_word; w < first_word + kWordsPerWave; w += kWordsPerRound) {
-    const bool set = ((words[w + (lane >> 5)] >> (lane & 31u)) & 1u) != 0;
-    const uint64_t mask = __ballot(set);
-    if (mask == 0) continue;  // the same for every lane
-    if (set) {
-      const uint32_t v = (tile * kBitmapTileWords + w) * kVerticesPerWord + lane;
-      const uint32_t at = r + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-      distinct_ids[at] = (int32_t)v;
-    }
-    r += (uint32_t)__popcll(mask);
-  }
-}
 
 // item_count[s] = work items of sample s (at least one, so that row offsets get written)
 __global__ void build_item_counts(const uint32_t* __restrict__ sizes, uint32_t n, uint32_t* __restrict__ item_count) {
@@ -738,13 +779,6 @@ __global__ __launch_bounds__(256) void select_collect(const uint32_t* __restrict
   }
 }
 
-// running sums of one sample's distinct ids, as the WeightArray handed to next()
-struct SegmentRunningSums {
-  const uint64_t* sums;  // global inclusive sums, already offset to the sample's first distinct id
-  uint64_t before;       // inclusive sum just before the sample's first distinct id
-  __device__ __forceinline__ uint64_t operator[](EdgePos_t i) const { return sums[i] - before; }
-};
-
 struct LayerParams {
   CSRPartition csr;
   TransitView transits;   // base already points at the first sample of the chunk
@@ -763,10 +797,16 @@ struct LayerParams {
   const uint32_t* offsets;
   const int32_t* nbr_cols;
   const float* nbr_weights;
-  // kDistinctByDegreeSquared / kRankedByLadiesImportance
-  const uint32_t* distinct_start;
-  const int32_t* distinct_ids;   // ascending ids, or ids in descending key order
-  const uint64_t* running_sums;
+  // kRankedByLadiesImportance: the kept ids of sample ls in descending key order are
+  // ranked_ids[ranked_start[ls] .. ranked_start[ls + 1])
+  const uint32_t* ranked_start;
+  const int32_t* ranked_ids;
+  // kDistinctByDegreeSquared: bitmaps and their two levels of degree^2 sums
+  const uint32_t* bitmap;
+  uint32_t words_per_sample;
+  const uint64_t* part_before;
+  const uint64_t* group_through;
+  const uint32_t* marked;        // marked vertices per sample
 };
 
 template <class SampleType, class App>
@@ -796,20 +836,22 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
       neighbor = r == -1 ? P.invalid : r;
     }
   } else if constexpr (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
-    const uint32_t begin = P.distinct_start[ls];
-    const CSR::Edge* ids = P.distinct_ids + begin;
-    SegmentRunningSums sums{P.running_sums + begin, begin ? P.running_sums[begin - 1] : 0ull};
-    const VertexID r = App().template next<SampleType, const CSR::Edge*, SegmentRunningSums>(
-        P.step, &csr, transits, sample_id, state, 0.0f, ids, sums, (EdgePos_t)(P.distinct_start[ls + 1] - begin),
+    const uint32_t parts = P.words_per_sample / kPartWords;
+    DistinctByDegreeSquared distinct{P.bitmap + (size_t)ls * P.words_per_sample,
+                                     P.part_before + (size_t)ls * (parts + 1),
+                                     P.group_through + (size_t)ls * parts * kGroupsPerPart, csr.row_ptr, parts};
+    const float* no_weights = nullptr;
+    const VertexID r = App().template next<SampleType, DistinctByDegreeSquared, const float*>(
+        P.step, &csr, transits, sample_id, state, 0.0f, distinct, no_weights, (EdgePos_t)P.marked[ls],
         (VertexID_t)nbr, &rng);
     neighbor = r == -1 ? P.invalid : r;
   } else {
-    const uint32_t begin = P.distinct_start[ls];
-    const CSR::Edge* ranked = P.distinct_ids + begin;
+    const uint32_t begin = P.ranked_start[ls];
+    const CSR::Edge* ranked = P.ranked_ids + begin;
     const float* no_weights = nullptr;
     const VertexID r = App().template next<SampleType, const CSR::Edge*, const float*>(
         P.step, &csr, transits, sample_id, state, 0.0f, ranked, no_weights,
-        (EdgePos_t)(P.distinct_start[ls + 1] - begin), (VertexID_t)nbr, &rng);
+        (EdgePos_t)(P.ranked_start[ls + 1] - begin), (VertexID_t)nbr, &rng);
     neighbor = r == -1 ? P.invalid : r;
   }
   P.final_samples[(size_t)s * P.final_size + P.out_base + nbr] = neighbor;
@@ -947,9 +989,6 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_item_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_row_offsets_, sizeof(uint32_t) * (size_t)n_samples_ * widest));
     ND_HIP_TRY(hipMalloc(&d_small_scratch_, sizeof(uint32_t) * scan_scratch_elems((size_t)n_samples_ + 1)));
-    if (App::kNeighborhoodForm != apps::kConcatenated) {
-      ND_HIP_TRY(hipMalloc(&d_distinct_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
-    }
     if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
       const size_t per_sample = sizeof(uint32_t) * ((size_t)n_samples_ + 1);
       ND_HIP_TRY(hipMalloc(&d_ranked_start_, per_sample));
@@ -1126,9 +1165,13 @@ class LayerEngine : public EngineBase {
     P.nbr_cols = d_nbr_cols_;
     P.nbr_weights = d_nbr_weights_;
     if (form != apps::kConcatenated) {
-      P.distinct_start = form == apps::kRankedByLadiesImportance ? d_ranked_start_ : d_distinct_start_;
-      P.distinct_ids = form == apps::kRankedByLadiesImportance ? d_ranked_ids_ : d_distinct_ids_;
-      P.running_sums = d_running_sums_;
+      P.ranked_start = d_ranked_start_;
+      P.ranked_ids = d_ranked_ids_;
+      P.bitmap = d_bitmap_;
+      P.words_per_sample = bitmap_words_;
+      P.part_before = d_part_before_;
+      P.group_through = d_group_through_;
+      P.marked = d_marked_;
     }
     const uint64_t outputs = (uint64_t)n * P.step_size;
     layer_execute_kernel<SampleType, App><<<dim3((unsigned)((outputs + 255) / 256)), dim3(256), 0, stream_>>>(P);
@@ -1152,35 +1195,33 @@ class LayerEngine : public EngineBase {
     }
   }
 
-  // FastGCN form: the distinct vertices of every sample, ascending (mark bits, count them per
-  // tile, scan, write the ids out), and the running sums of degree^2 over them.
+  // FastGCN form: mark the vertices of every sample's neighbourhood in its bitmap and add up
+  // degree^2 over the marked vertices at two levels (groups of 256 vertices, parts of 64 groups).
   int list_distinct(const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
-    const uint32_t tiles_per_sample = bitmap_words_ / kBitmapTileWords;
-    const size_t n_tiles = (size_t)n * tiles_per_sample;
+    const uint32_t parts_per_sample = bitmap_words_ / kPartWords;
+    const size_t n_parts = (size_t)n * parts_per_sample;
+    if (n_parts >= (1ull << 32)) { last_error = "a chunk needs 2^32 or more bitmap parts"; return -1; }
     if (n > bitmap_samples_) {
-      release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_);
+      release(d_bitmap_); release(d_group_through_); release(d_part_total_); release(d_part_before_); release(d_marked_);
       ND_HIP_TRY(hipMalloc(&d_bitmap_, sizeof(uint32_t) * (size_t)n * bitmap_words_));
-      ND_HIP_TRY(hipMalloc(&d_tile_offsets_, sizeof(uint32_t) * (n_tiles + 1)));
-      ND_HIP_TRY(hipMalloc(&d_tile_scratch_, sizeof(uint32_t) * scan_scratch_elems(n_tiles)));
+      ND_HIP_TRY(hipMalloc(&d_group_through_, sizeof(uint64_t) * n_parts * kGroupsPerPart));
+      ND_HIP_TRY(hipMalloc(&d_part_total_, sizeof(uint64_t) * n_parts));
+      ND_HIP_TRY(hipMalloc(&d_part_before_, sizeof(uint64_t) * (size_t)n * (parts_per_sample + 1)));
+      ND_HIP_TRY(hipMalloc(&d_marked_, sizeof(uint32_t) * (size_t)n));
       bitmap_samples_ = n;
     }
     tick();
     collective_mark_binned<false><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
         dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u);
     tock();
-    bitmap_tile_counts<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_);
-    ND_HIP_TRY(exclusive_scan_u32(d_tile_offsets_, d_tile_offsets_, n_tiles, d_tile_scratch_, stream_));
-    uint32_t n_distinct = 0;
-    ND_HIP_TRY(hipMemcpyAsync(&n_distinct, d_tile_scratch_ + scan_num_tiles(n_tiles), sizeof(uint32_t),
-                              hipMemcpyDeviceToHost, stream_));
+    ND_HIP_TRY(hipMemsetAsync(d_marked_, 0, sizeof(uint32_t) * (size_t)n, stream_));
+    bitmap_group_sums<<<dim3((unsigned)((n_parts + 3) / 4)), dim3(256), 0, stream_>>>(
+        d_bitmap_, bitmap_words_, (uint32_t)n_parts, dgraph_.row_ptr(), d_group_through_, d_part_total_, d_marked_);
+    sample_part_sums<<<dim3(n), dim3(64), 0, stream_>>>(d_part_total_, parts_per_sample, d_part_before_);
+    std::vector<uint32_t> marked(n);
+    ND_HIP_TRY(hipMemcpyAsync(marked.data(), d_marked_, sizeof(uint32_t) * n, hipMemcpyDeviceToHost, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
-    distinct_total_ += n_distinct;
-    if (ensure_distinct_capacity(n_distinct) != 0) return -1;
-    bitmap_compact<<<dim3((unsigned)n_tiles), dim3(256), 0, stream_>>>(d_bitmap_, d_tile_offsets_, tiles_per_sample,
-                                                                       d_distinct_ids_, d_distinct_start_);
-    fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_distinct_start_ + n, 1, n_distinct);
-    ND_HIP_TRY(inclusive_scan_u64_of(DegreeSquaredOf{d_distinct_ids_, dgraph_.row_ptr()}, d_running_sums_, n_distinct,
-                                     d_scratch64_, stream_));
+    for (uint32_t c : marked) distinct_total_ += c;
     return hipGetLastError() == hipSuccess ? 0 : -1;
   }
 
@@ -1261,11 +1302,6 @@ class LayerEngine : public EngineBase {
     constexpr int form = App::kNeighborhoodForm;
     const size_t cap = (size_t)n_distinct + n_distinct / 8 + 1024;
     release_distinct_buffers();
-    ND_HIP_TRY(hipMalloc(&d_distinct_ids_, sizeof(int32_t) * cap));
-    if (form == apps::kDistinctByDegreeSquared) {
-      ND_HIP_TRY(hipMalloc(&d_running_sums_, sizeof(uint64_t) * cap));
-      ND_HIP_TRY(hipMalloc(&d_scratch64_, sizeof(uint64_t) * (scan_num_tiles(cap) + 1)));
-    }
     if (form == apps::kRankedByLadiesImportance) {
       ND_HIP_TRY(hipMalloc(&d_ranked_ids_, sizeof(int32_t) * cap));
       ND_HIP_TRY(hipMalloc(&d_kept_key_, sizeof(uint32_t) * cap));
@@ -1297,7 +1333,6 @@ class LayerEngine : public EngineBase {
   }
 
   void release_distinct_buffers() {
-    release(d_distinct_ids_); release(d_running_sums_); release(d_scratch64_);
     release(d_ranked_ids_);
     release(d_keys_a_); release(d_vals_a_); release(d_keys_b_); release(d_vals_b_);
     release(d_key2_); release(d_index2_); release(d_hist_); release(d_scratch_);
@@ -1307,7 +1342,8 @@ class LayerEngine : public EngineBase {
 
   void release_neighborhood_buffers() {
     release(d_nbr_cols_); release(d_nbr_weights_);
-    release(d_bitmap_); release(d_tile_offsets_); release(d_tile_scratch_); release(d_keys_dense_); release(d_sums_dense_);
+    release(d_bitmap_); release(d_keys_dense_); release(d_sums_dense_);
+    release(d_group_through_); release(d_part_total_); release(d_part_before_); release(d_marked_);
     release_distinct_buffers();
     capacity_ = 0;
     bitmap_samples_ = 0;
@@ -1317,7 +1353,6 @@ class LayerEngine : public EngineBase {
     release(d_initial_); release(d_samples_); release(d_samples_init_); release(d_final_);
     release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
     release(d_item_count_); release(d_item_start_);
-    release(d_distinct_start_);
     release(d_ranked_start_); release(d_select_prefix_); release(d_select_need_); release(d_select_kept_);
     release(d_select_threshold_); release(d_select_hist_); release(d_select_present_);
     release_neighborhood_buffers();
@@ -1349,7 +1384,7 @@ class LayerEngine : public EngineBase {
   uint64_t bitmap_chunk_entries_ = 0;
   uint32_t bitmap_samples_ = 0;        // samples the allocated bitmaps hold
   size_t distinct_capacity_ = 0;
-  uint32_t *d_bitmap_ = nullptr, *d_tile_offsets_ = nullptr, *d_tile_scratch_ = nullptr;
+  uint32_t* d_bitmap_ = nullptr;
   // LADIES form: importance sums and sampling keys, [sample][vertex, padded to whole stretches]
   unsigned long long* d_sums_dense_ = nullptr;
   uint32_t* d_keys_dense_ = nullptr;
@@ -1365,7 +1400,6 @@ class LayerEngine : public EngineBase {
   VertexID_t* d_final_ = nullptr;
   uint32_t *d_sizes_ = nullptr, *d_offsets_ = nullptr, *d_row_offsets_ = nullptr, *d_small_scratch_ = nullptr;
   uint32_t *d_item_count_ = nullptr, *d_item_start_ = nullptr;
-  uint32_t* d_distinct_start_ = nullptr;
   // LADIES form: the selection of the best keys per sample
   uint32_t *d_ranked_start_ = nullptr, *d_select_prefix_ = nullptr, *d_select_need_ = nullptr;
   uint32_t *d_select_kept_ = nullptr, *d_select_threshold_ = nullptr, *d_select_hist_ = nullptr;
@@ -1376,8 +1410,9 @@ class LayerEngine : public EngineBase {
   float* d_nbr_weights_ = nullptr;
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t *d_key2_ = nullptr, *d_index2_ = nullptr, *d_hist_ = nullptr, *d_scratch_ = nullptr;
-  int32_t* d_distinct_ids_ = nullptr;
-  uint64_t *d_running_sums_ = nullptr, *d_scratch64_ = nullptr;
+  // FastGCN form: degree^2 of the marked vertices, by group inside a part, by part, by sample
+  uint64_t *d_group_through_ = nullptr, *d_part_total_ = nullptr, *d_part_before_ = nullptr;
+  uint32_t* d_marked_ = nullptr;
   int32_t* d_ranked_ids_ = nullptr;
 };
 
