@@ -399,7 +399,42 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     cur_edges = s_edge[lo];
     if (kWithImportance) cur_row_sum = s_row_sum[lo];
   }
-  for (uint32_t e0 = part_begin; e0 < part_end; e0 += kRound) {  // the same trip count for every lane of a wave
+  if (!kWithImportance) {
+    // FastGCN form: nothing is shared between neighbouring entries, so a lane takes four
+    // consecutive entries per round - one 16-byte load and one round of index arithmetic for
+    // four marks (the kernel is bound by instruction issue: its edge stream comes from the
+    // caches) - unless its four entries straddle the end of a sub-range or of the part.
+    struct __attribute__((packed, aligned(4))) FourIds { uint32_t id[4]; };
+    for (uint32_t e0 = part_begin; e0 < part_end; e0 += kRound) {
+      const uint32_t e = e0 + lane * kBinAhead;
+      if (e >= part_end) continue;
+      if (e >= cur_end) {
+        do {
+          ++cur;
+          cur_begin = cur_end;
+          cur_end = s_start[cur + 1];
+        } while (e >= cur_end);
+        cur_edges = s_edge[cur];
+      }
+      if (e + kBinAhead <= cur_end && e + kBinAhead <= part_end) {
+        FourIds four;
+        __builtin_memcpy(&four, csr.edges + cur_edges + (EdgePos_t)(e - cur_begin), sizeof(four));
+#pragma unroll
+        for (uint32_t a = 0; a < kBinAhead; ++a) s_bytes[four.id[a] - v_lo] = 1;
+      } else {
+        for (uint32_t a = 0; a < kBinAhead && e + a < part_end; ++a) {
+          while (e + a >= cur_end) {
+            ++cur;
+            cur_begin = cur_end;
+            cur_end = s_start[cur + 1];
+            cur_edges = s_edge[cur];
+          }
+          s_bytes[(uint32_t)csr.edges[cur_edges + (EdgePos_t)(e + a - cur_begin)] - v_lo] = 1;
+        }
+      }
+    }
+  }
+  for (uint32_t e0 = part_begin; kWithImportance && e0 < part_end; e0 += kRound) {  // the same trip count for every lane of a wave
     uint32_t locals[kBinAhead];  // vertex - v_lo
     float weights[kBinAhead], sums_of_row[kBinAhead];
 #pragma unroll
