@@ -31,13 +31,13 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "weighted_node2vec_rmat22": 1.246e9,     # step_flat_kernel
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
-    "fastgcn_importance_rmat22": 6.953e9,    # collective_mark_binned, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 1.787e11,  # collective_mark_binned, average over its 2 launches per pass
+    "fastgcn_importance_rmat22": 6.872e9,    # collective_mark_binned, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 1.864e11,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
     "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 165.7e9, "ladies_importance_chunglu3m": 500.7e9,
+    "fastgcn_importance_rmat22": 19.6e9, "ladies_importance_chunglu3m": 499.8e9,
 }
 
 WORKLOADS = {
@@ -251,6 +251,10 @@ def main():
             "algorithmic_bytes_per_launch": mark_bytes / launches,
             "avg_launch_ms": prof["neighbourhood_ms"] / launches,
             "whole_pass": {"measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
+            # `achieved` prices every entry as if it came from HBM; `traffic` is what the counters
+            # saw: where it is far lower (FastGCN: the hubs' adjacencies sit in the caches), HBM
+            # is not what bounds the kernel
+            "note": "achieved = algorithmic bytes / time; compare traffic for what HBM really served",
         }
         if not args.skip_cpu_baseline:
             result["cpu_baseline"] = cpu_baseline_layers(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
