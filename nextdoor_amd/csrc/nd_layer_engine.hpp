@@ -17,15 +17,15 @@
 //    nullptr, nextdoor.cu:1441-1446).  Here offsets are an exclusive scan over samples
 //    (deterministic), the buffers are grown once and reused, and next() receives the
 //    neighbourhood in the form the app declares (nd::apps::NeighborhoodForm).
-//  * For kDistinctByDegreeSquared the concatenation is never stored: every entry marks its
-//    vertex in a per-sample bitmap, built stretch by stretch in LDS; the marked vertices in
-//    ascending order are the distinct vertices, and a 64-bit inclusive scan of degree^2 over
-//    them gives the running sums the app inverts.
+//  * For kDistinctByDegreeSquared the concatenation is never stored, nor a list of its distinct
+//    vertices: every entry marks its vertex in a per-sample bitmap, built stretch by stretch
+//    in LDS; degree^2 of the marked vertices is summed over groups and parts of the bitmap,
+//    and a draw searches those sums.
 //  * For kRankedByLadiesImportance each entry also carries (weight * (1 / rowsum(transit)))^2;
-//    the terms of a vertex are summed as 2^53 fixed-point integers next to the bitmap (in LDS),
-//    the Efraimidis-Spirakis key of every distinct vertex is formed from its sum, a radix
-//    select keeps the entries that can be among a sample's first picks, and two stable sorts
-//    order those by descending key.
+//    the terms of a vertex are summed as 2^53 fixed-point integers (in LDS) into one sum per
+//    (sample, vertex), its Efraimidis-Spirakis key is formed from the sum, a radix select keeps
+//    the few entries that can be among a sample's first picks, and stable sorts order those by
+//    descending key.
 //  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
 //    of entries, so a layer whose frontier sits on hubs cannot outgrow memory.
 //  * Random numbers: Philox keyed by the output slot s * stepSize(k) + nbr and the layer.
@@ -160,16 +160,17 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
   return shift > -24 ? (unsigned long long)(mantissa >> -shift) : 0ull;
 }
 
-// ---- distinct vertices of a collective neighbourhood through a presence map ----
+// ---- the distinct vertices of a collective neighbourhood, marked stretch by stretch ----
 //
-// Per sample of the chunk a bitmap over the vertices (words_per_sample 32-bit words, a multiple
-// of the tile below).  collective_mark_binned walks the neighbourhood as collective_build does,
-// but instead of copying an entry it marks the entry's vertex; nothing of the concatenation is
-// stored.  A neighbourhood that sits on hubs repeats its vertices many times over (3.8e10
-// entries hold 2.0e9 distinct pairs at FastGCN's full size).
-// LADIES form (kWithImportance): every entry also adds (weight * inverse_row_sum[transit])^2, as
-// a 2^53 fixed-point integer, to the 64-bit sum of (sample, vertex).
-constexpr uint32_t kBitmapTileWords = 2048;  // 256 lanes x 8 words: 65536 vertices
+// collective_mark_binned walks the neighbourhood as collective_build does, but instead of
+// copying an entry it marks the entry's vertex; nothing of the concatenation is stored.  A
+// neighbourhood that sits on hubs repeats its vertices many times over (3.8e10 entries hold
+// 2.0e9 distinct pairs at FastGCN's full size).  FastGCN form: the result is a bitmap per
+// sample (words_per_sample 32-bit words, a multiple of the tile below).  LADIES form
+// (kWithImportance): every entry also adds (weight * inverse_row_sum[transit])^2, as a 2^53
+// fixed-point integer, to the 64-bit sum of (sample, vertex); the result is that sum for every
+// vertex of every sample, kAbsentSum where the sample's neighbourhood does not hold the vertex.
+constexpr uint32_t kBitmapTileWords = 2048;  // bitmaps are padded to whole tiles of 65536 vertices (4 parts)
 
 // log2 of a positive normal float from exponent extraction and an atanh series; every step
 // is a single IEEE operation so that host and device agree bit for bit.
