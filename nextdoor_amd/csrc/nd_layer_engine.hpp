@@ -556,11 +556,29 @@ __global__ __launch_bounds__(256) void bitmap_group_sums(const uint32_t* __restr
   for (uint32_t k = 0; k < kGroupWords; ++k) {
     uint32_t bits = w[k];
     count += __popc(bits);
+    const uint32_t base = (first_word + k) * 32u;
     while (bits) {
-      const uint32_t v = (first_word + k) * 32u + (uint32_t)__ffs((int)bits) - 1u;
-      const uint64_t d = (uint64_t)(row_ptr[v + 1] - row_ptr[v]);
-      sum += d * d;
-      bits &= bits - 1u;
+      // four row extents are fetched before the first is used: one at a time, a lane spent
+      // its time waiting for each in turn
+      uint32_t v[4];
+      bool has[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        has[q] = bits != 0;
+        v[q] = base + (has[q] ? (uint32_t)__ffs((int)bits) - 1u : 0u);
+        bits &= bits - 1u;  // 0 stays 0
+      }
+      EdgePos_t from[4], to[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        from[q] = has[q] ? row_ptr[v[q]] : 0;
+        to[q] = has[q] ? row_ptr[v[q] + 1] : 0;
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint64_t d = (uint64_t)(to[q] - from[q]);
+        sum += d * d;
+      }
     }
   }
   const uint64_t through = wave_inclusive_scan_u64(sum);
