@@ -1178,18 +1178,18 @@ class LayerEngine : public EngineBase {
     constexpr int form = App::kNeighborhoodForm;
     TransitView tv = all;
     tv.base = all.base + (size_t)s0 * all.stride;
-    // work items of the build: long neighbourhoods are spread over several workgroups
-    uint64_t n_items = 0;
-    for (uint32_t s = s0; s < s1; ++s) {
-      const uint64_t items = ((uint64_t)h_sizes_[s] + kBuildItemEntries - 1) / kBuildItemEntries;
-      n_items += items ? items : 1;
-    }
-    if (n_items >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more work items"; return -2; }
-    build_item_counts<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_sizes_ + s0, n, d_item_count_);
-    ND_HIP_TRY(exclusive_scan_u32(d_item_count_, d_item_start_, (size_t)n + 1, d_small_scratch_, stream_));
     if (form != apps::kConcatenated) {
-      if (build_distinct_by_bitmap(step, s0, tv, n, (unsigned)n_items) != 0) return -1;
+      if (build_distinct_by_bitmap(step, s0, tv, n) != 0) return -1;
     } else {
+      // work items of the build: long neighbourhoods are spread over several workgroups
+      uint64_t n_items = 0;
+      for (uint32_t s = s0; s < s1; ++s) {
+        const uint64_t items = ((uint64_t)h_sizes_[s] + kBuildItemEntries - 1) / kBuildItemEntries;
+        n_items += items ? items : 1;
+      }
+      if (n_items >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more work items"; return -2; }
+      build_item_counts<<<dim3((n + 1 + 255) / 256), dim3(256), 0, stream_>>>(d_sizes_ + s0, n, d_item_count_);
+      ND_HIP_TRY(exclusive_scan_u32(d_item_count_, d_item_start_, (size_t)n + 1, d_small_scratch_, stream_));
       if (ensure_neighborhood_capacity((uint32_t)total) != 0) return -1;
       // offsets of the chunk's samples, relative to the chunk (element n = total)
       ND_HIP_TRY(exclusive_scan_u32(d_sizes_ + s0, d_offsets_, (size_t)n + 1, d_small_scratch_, stream_));
@@ -1234,8 +1234,7 @@ class LayerEngine : public EngineBase {
   }
 
   // What next() of the importance forms is handed, for every sample of the chunk.
-  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n, unsigned n_items) {
-    (void)n_items;
+  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n) {
     constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
