@@ -1018,6 +1018,9 @@ class LayerEngine : public EngineBase {
     }
     const uint64_t fit = kBitmapBudgetBytes / bytes_per_sample;
     bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
+    // the selection kernels of the LADIES form index the samples of a chunk by blockIdx.y
+    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance && bitmap_chunk_samples_ > 65535u)
+      bitmap_chunk_samples_ = 65535u;
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
