@@ -35,7 +35,8 @@ struct NextDoorData {
   const char* appName;
   uint64_t seed;
   nd_sampler* sampler = nullptr;
-  CSR* csr = nullptr;
+  CSR* csr = nullptr;                       // the caller's graph; stays set after freeDeviceData
+  bool graphOnDevice = false;
   std::vector<VertexID_t> hFinalSamples;    // libNextDoor.hpp:17
   std::vector<VertexID_t> initialContents;  // libNextDoor.hpp:18
   VertexID_t INVALID_VERTEX = 0;            // libNextDoor.hpp:35
@@ -57,13 +58,14 @@ inline bool transferCSRToGPUs(NextDoorData& data, CSR* csr) {
   if (!data.sampler && nd_sampler_create(data.appName, &data.sampler) != 0) return false;
   if (nd_sampler_set_graph(data.sampler, csr) != 0) return false;
   data.csr = csr;
+  data.graphOnDevice = true;
   return true;
 }
 
 // allocNextDoorDataOnGPU(csr, data), src/nextdoor.cu:1931-2086.  Transfers the graph first
 // when the caller has not done so.
 inline bool allocNextDoorDataOnGPU(CSR* csr, NextDoorData& data) {
-  if (data.csr != csr && !transferCSRToGPUs(data, csr)) return false;
+  if ((data.csr != csr || !data.graphOnDevice) && !transferCSRToGPUs(data, csr)) return false;
   if (nd_sampler_alloc(data.sampler, data.seed) != 0) return false;
   const VertexID_t* roots = nullptr;
   int64_t n = 0;
@@ -105,7 +107,40 @@ inline int getFinalSampleSize(const NextDoorData& data) {
 // freeDeviceData(data), src/nextdoor.cu:2088-2115.
 inline void freeDeviceData(NextDoorData& data) {
   if (data.sampler) nd_sampler_free_device(data.sampler);
-  data.csr = nullptr;
+  data.graphOnDevice = false;
+}
+
+// checkSampledVerticesResult<SampleType, App>(data), src/check_results.cu:162-299: the checker
+// the reference's per-transit apps hand to nextdoor().  Works on the host copies
+// (data.hFinalSamples, data.initialContents, data.csr), so also after freeDeviceData.
+inline bool checkSampledVerticesResult(NextDoorData& data) {
+  if (!data.sampler || !data.csr) return false;
+  const int steps = nd_sampler_steps(data.sampler);
+  std::vector<int32_t> sizes((size_t)(steps > 0 ? steps : 0));
+  for (int k = 0; k < steps; ++k) sizes[(size_t)k] = nd_sampler_step_size(data.sampler, k);
+  const int initial = nd_sampler_initial_sample_size(data.sampler);
+  const int64_t n_samples = initial > 0 ? (int64_t)data.initialContents.size() / initial : 0;
+  const int verdict = nd_check_sampled_vertices(data.csr, steps, sizes.data(), initial,
+                                                nd_sampler_sampling_type(data.sampler) == 1, n_samples,
+                                                data.initialContents.data(), data.hFinalSamples.data(),
+                                                data.INVALID_VERTEX);
+  if (verdict != 1) fprintf(stderr, "%s\n", nd_last_error());
+  return verdict == 1;
+}
+
+// The edge lists of the apps whose outputFormat() is AdjacencyMatrix on per-transit sampling
+// (MVS, ClusterGCN; the reference reads dRowStorage / dColStorage at sample.posInStorage):
+// sample i owns rows/cols[list_start[i] .. list_start[i + 1]).
+inline bool getAdjacency(NextDoorData& data, std::vector<VertexID_t>& rows, std::vector<VertexID_t>& cols,
+                         std::vector<uint32_t>& list_start) {
+  const int32_t *r = nullptr, *c = nullptr;
+  const uint32_t* start = nullptr;
+  int64_t n_edges = 0, n_samples = 0;
+  if (!data.sampler || nd_sampler_get_adjacency(data.sampler, &r, &c, &n_edges, &start, &n_samples) != 0) return false;
+  rows.assign(r, r + n_edges);
+  cols.assign(c, c + n_edges);
+  list_start.assign(start, start + n_samples + 1);
+  return true;
 }
 
 // nextdoor<SampleType, App>(file, type, format, nruns, chk, print, kernelType, lb, checker),

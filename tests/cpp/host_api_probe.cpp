@@ -28,7 +28,9 @@ int main(int argc, char** argv) {
                            [&](NextDoorData& data) {
                              final_size = getFinalSampleSize(data);
                              n_values = data.hFinalSamples.size();
-                             return final_size == 8 && n_values == data.initialContents.size() * 8;
+                             // the library's validator, on the host copies after freeDeviceData
+                             return final_size == 8 && n_values == data.initialContents.size() * 8 &&
+                                    checkSampledVerticesResult(data);
                            });
   printf("final_size %d values %zu\n", final_size, n_values);
   if (!ok) return 7;
@@ -45,5 +47,24 @@ int main(int argc, char** argv) {
   }
   if (transit_parallel.empty() || transit_parallel != sample_parallel) return 10;
   printf("kernel types agree\n");
+  {  // an edge-list app: every listed edge leaves a vertex of its sample
+    CSR* g = loadGraph(graph_file, "edge-list", "text");
+    NextDoorData data("MVS5");
+    std::vector<VertexID_t> rows, cols;
+    std::vector<uint32_t> start;
+    if (!g || !allocNextDoorDataOnGPU(g, data) || !doTransitParallelSampling(g, data, true)) return 11;
+    if (!getAdjacency(data, rows, cols, start) || rows.size() != cols.size() || start.empty() ||
+        start.back() != rows.size())
+      return 12;
+    for (size_t s = 0; s + 1 < start.size(); ++s)
+      for (uint32_t e = start[s]; e < start[s + 1]; ++e) {
+        bool mine = false;
+        for (int i = 0; i < 5; ++i) mine = mine || data.initialContents[s * 5 + (size_t)i] == rows[e];
+        if (!mine) return 13;
+      }
+    printf("edge lists %zu\n", rows.size());
+    freeDeviceData(data);
+    nd_graph_free(g);
+  }
   return 0;
 }

@@ -46,3 +46,4 @@ def test_nextdoor_entry_runs_on_the_gpu(tmp_path):
     assert "totalSampledVertices 96" in out.stdout  # 12 walks x 8 steps, no dead ends
     assert "final_size 8 values 96" in out.stdout
     assert "kernel types agree" in out.stdout
+    assert "edge lists 300" in out.stdout  # MVS5: 20 batches of 5 vertices with 3 out-edges each
