@@ -81,7 +81,7 @@ class ShardedEngine : public EngineBase {
       first += count;
     }
     if (n_parts > 1)
-      for (auto& p : parts_) std::vector<VertexID_t>().swap(p->hFinalSamples);  // the rows come home through ours
+      for (auto& p : parts_) p->hFinalSamples.clear();  // the rows come home through ours
     hFinalSamples.assign((size_t)n * (size_t)final_sample_size(), invalid_vertex());
     return 0;
   }
