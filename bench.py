@@ -279,6 +279,14 @@ def main():
     if not args.skip_cpu_baseline:
         base, run = cpu_baseline(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
         result["cpu_baseline"] = base
+        # the reference's only CPU path over the samples is its validator (src/check_results.cu:162-299):
+        # ours, over every output of the pass just sampled, on the same host cores
+        t0 = time.perf_counter()
+        ok, why = sampler.check_results()
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"]["validator"] = {"passed": bool(ok), "seconds": round(dt, 2),
+                                               "outputs_checked_per_s": edges_per_pass / dt,
+                                               "report": None if ok else why}
         weighted = w["kind"] in ("WEIGHTED_NODE2VEC", "DEEPWALK", "PPR")
         second = w["kind"] in ("WEIGHTED_NODE2VEC", "NODE2VEC")
         step_bytes, sort_bytes = algorithmic_bytes_per_pass(sampler, run, weighted, second)
