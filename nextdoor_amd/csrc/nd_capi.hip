@@ -3,7 +3,9 @@
 
 #include <string.h>
 
+#include <exception>
 #include <memory>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -35,6 +37,21 @@ thread_local std::string g_error;
 int fail(const std::string& msg, int code = -1) {
   g_error = msg;
   return code;
+}
+
+// No exception leaves the library: a body that throws (host memory, a container's range
+// check) reports through the error text like any other failure.
+template <class Body>
+int guarded(Body body) {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return fail("out of host memory");
+  } catch (const std::exception& e) {
+    return fail(std::string("internal error: ") + e.what());
+  } catch (...) {
+    return fail("internal error");
+  }
 }
 
 struct AppEntry {
@@ -147,51 +164,61 @@ const char* nd_app_name(int index) { return index >= 0 && index < kNumApps ? kAp
 // ---- graphs ---------------------------------------------------------------------------
 
 int nd_graph_load(const char* path, const char* graph_type, const char* graph_format, nd_graph** out) {
-  if (!out) return fail("null out");
-  std::unique_ptr<nd_graph> g(new nd_graph);
-  std::string err;
-  if (nd::load_graph_file(g->csr, path, graph_type, graph_format, &err) != 0) return fail(err);
-  *out = g.release();
-  return 0;
+  return guarded([&]() -> int {
+    if (!out) return fail("null out");
+    std::unique_ptr<nd_graph> g(new nd_graph);
+    std::string err;
+    if (nd::load_graph_file(g->csr, path, graph_type, graph_format, &err) != 0) return fail(err);
+    *out = g.release();
+    return 0;
+  });
 }
 
 int nd_graph_from_edges(int32_t n_vertices, int64_t n_edges, const int32_t* src, const int32_t* dst,
                         const float* weight, nd_graph** out) {
-  if (!out || n_edges < 0 || (n_edges > 0 && (!src || !dst))) return fail("bad argument");
-  std::unique_ptr<nd_graph> g(new nd_graph);
-  std::string err;
-  if (nd::csr_from_edges(g->csr, n_vertices, (size_t)n_edges, src, dst, weight, &err) != 0) return fail(err);
-  *out = g.release();
-  return 0;
+  return guarded([&]() -> int {
+    if (!out || n_edges < 0 || (n_edges > 0 && (!src || !dst))) return fail("bad argument");
+    std::unique_ptr<nd_graph> g(new nd_graph);
+    std::string err;
+    if (nd::csr_from_edges(g->csr, n_vertices, (size_t)n_edges, src, dst, weight, &err) != 0) return fail(err);
+    *out = g.release();
+    return 0;
+  });
 }
 
 int nd_graph_from_csr(int32_t n_vertices, int64_t n_edges, const int32_t* row_ptr, const int32_t* col,
                       const float* weight, nd_graph** out) {
-  if (!out || !row_ptr || (n_edges > 0 && !col)) return fail("bad argument");
-  std::unique_ptr<nd_graph> g(new nd_graph);
-  std::string err;
-  if (nd::csr_from_arrays(g->csr, n_vertices, n_edges, row_ptr, col, weight, &err) != 0) return fail(err);
-  *out = g.release();
-  return 0;
+  return guarded([&]() -> int {
+    if (!out || !row_ptr || (n_edges > 0 && !col)) return fail("bad argument");
+    std::unique_ptr<nd_graph> g(new nd_graph);
+    std::string err;
+    if (nd::csr_from_arrays(g->csr, n_vertices, n_edges, row_ptr, col, weight, &err) != 0) return fail(err);
+    *out = g.release();
+    return 0;
+  });
 }
 
 int nd_graph_rmat(int scale, int edge_factor, double a, double b, double c, uint64_t seed, int symmetrise,
                   nd_graph** out) {
-  if (!out) return fail("null out");
-  std::unique_ptr<nd_graph> g(new nd_graph);
-  std::string err;
-  if (nd::generate_rmat(g->csr, scale, edge_factor, a, b, c, seed, symmetrise != 0, &err) != 0) return fail(err);
-  *out = g.release();
-  return 0;
+  return guarded([&]() -> int {
+    if (!out) return fail("null out");
+    std::unique_ptr<nd_graph> g(new nd_graph);
+    std::string err;
+    if (nd::generate_rmat(g->csr, scale, edge_factor, a, b, c, seed, symmetrise != 0, &err) != 0) return fail(err);
+    *out = g.release();
+    return 0;
+  });
 }
 
 int nd_graph_chung_lu(int32_t n_vertices, int64_t n_edges, double exponent, uint64_t seed, nd_graph** out) {
-  if (!out) return fail("null out");
-  std::unique_ptr<nd_graph> g(new nd_graph);
-  std::string err;
-  if (nd::generate_chung_lu(g->csr, n_vertices, n_edges, exponent, seed, &err) != 0) return fail(err);
-  *out = g.release();
-  return 0;
+  return guarded([&]() -> int {
+    if (!out) return fail("null out");
+    std::unique_ptr<nd_graph> g(new nd_graph);
+    std::string err;
+    if (nd::generate_chung_lu(g->csr, n_vertices, n_edges, exponent, seed, &err) != 0) return fail(err);
+    *out = g.release();
+    return 0;
+  });
 }
 
 int32_t nd_graph_num_vertices(const nd_graph* g) { return g ? g->csr.get_n_vertices() : 0; }
@@ -205,52 +232,64 @@ void nd_graph_free(nd_graph* g) { delete g; }
 // ---- sampler --------------------------------------------------------------------------
 
 int nd_sampler_create(const char* app_name, nd_sampler** out) {
-  if (!app_name || !out) return fail("null argument");
-  for (int i = 0; i < kNumApps; ++i) {
-    if (strcmp(kApps[i].name, app_name) == 0) {
-      nd_sampler* s = new nd_sampler;
-      s->engine.reset(kApps[i].make(kApps[i].name));
-      *out = s;
-      return 0;
+  return guarded([&]() -> int {
+    if (!app_name || !out) return fail("null argument");
+    for (int i = 0; i < kNumApps; ++i) {
+      if (strcmp(kApps[i].name, app_name) == 0) {
+        nd_sampler* s = new nd_sampler;
+        s->engine.reset(kApps[i].make(kApps[i].name));
+        *out = s;
+        return 0;
+      }
     }
-  }
-  return fail(std::string("unknown app '") + app_name + "'");
+    return fail(std::string("unknown app '") + app_name + "'");
+  });
 }
 
 int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g) {
-  if (!s || !g) return fail("null argument");
-  int n_devices = 0;
-  if (hipGetDeviceCount(&n_devices) != hipSuccess || n_devices < 1) return fail("no HIP device available");
-  s->graph = g;
-  const int rc = s->engine->set_graph(&g->csr);
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s || !g) return fail("null argument");
+    int n_devices = 0;
+    if (hipGetDeviceCount(&n_devices) != hipSuccess || n_devices < 1) return fail("no HIP device available");
+    s->graph = g;
+    const int rc = s->engine->set_graph(&g->csr);
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_alloc(nd_sampler* s, uint64_t seed) {
-  if (!s) return fail("null sampler");
-  const int rc = s->engine->alloc(seed);
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s) return fail("null sampler");
+    const int rc = s->engine->alloc(seed);
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_do_transit_parallel(nd_sampler* s, int enable_load_balancing) {
-  if (!s) return fail("null sampler");
-  const int rc = s->engine->sample(enable_load_balancing ? nd::kTransitParallelLoadBalanced : nd::kTransitParallel);
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s) return fail("null sampler");
+    const int rc = s->engine->sample(enable_load_balancing ? nd::kTransitParallelLoadBalanced : nd::kTransitParallel);
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_do_sample_parallel(nd_sampler* s) {
-  if (!s) return fail("null sampler");
-  const int rc = s->engine->sample(nd::kSampleParallel);
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s) return fail("null sampler");
+    const int rc = s->engine->sample(nd::kSampleParallel);
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_get_final_samples(nd_sampler* s, const int32_t** data, int64_t* length) {
-  if (!s || !data || !length) return fail("null argument");
-  const int rc = s->engine->fetch_final_samples();
-  if (rc != 0) return fail(s->engine->last_error, rc);
-  *data = s->engine->hFinalSamples.data();
-  *length = (int64_t)s->engine->hFinalSamples.size();
-  return 0;
+  return guarded([&]() -> int {
+    if (!s || !data || !length) return fail("null argument");
+    const int rc = s->engine->fetch_final_samples();
+    if (rc != 0) return fail(s->engine->last_error, rc);
+    *data = s->engine->hFinalSamples.data();
+    *length = (int64_t)s->engine->hFinalSamples.size();
+    return 0;
+  });
 }
 
 int nd_sampler_final_sample_size(const nd_sampler* s) { return s ? s->engine->final_sample_size() : -1; }
@@ -275,9 +314,11 @@ int nd_sampler_sampling_type(const nd_sampler* s) { return s ? s->engine->sampli
 int64_t nd_sampler_sample_state_bytes(const nd_sampler* s) { return s ? (int64_t)s->engine->sample_state_bytes() : -1; }
 
 int nd_sampler_get_sample_states(nd_sampler* s, void* dst, int64_t bytes) {
-  if (!s || !dst) return fail("null argument");
-  const int rc = s->engine->fetch_sample_states(dst, (size_t)bytes);
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s || !dst) return fail("null argument");
+    const int rc = s->engine->fetch_sample_states(dst, (size_t)bytes);
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_set_inversion_period(nd_sampler* s, int period) {
@@ -315,21 +356,25 @@ int nd_sampler_phase_times(const nd_sampler* s, float out[12]) {
 
 int nd_sampler_get_adjacency(nd_sampler* s, const int32_t** rows, const int32_t** cols, int64_t* n_edges,
                              const uint32_t** list_start, int64_t* n_samples) {
-  if (!s || !rows || !cols || !n_edges || !list_start || !n_samples) return fail("null argument");
-  const int rc = s->engine->fetch_adjacency();
-  if (rc != 0) return fail(s->engine->last_error, rc);
-  *rows = s->engine->hListRows.data();
-  *cols = s->engine->hListCols.data();
-  *n_edges = (int64_t)s->engine->hListRows.size();
-  *list_start = s->engine->hListStart.data();
-  *n_samples = s->engine->num_samples();
-  return 0;
+  return guarded([&]() -> int {
+    if (!s || !rows || !cols || !n_edges || !list_start || !n_samples) return fail("null argument");
+    const int rc = s->engine->fetch_adjacency();
+    if (rc != 0) return fail(s->engine->last_error, rc);
+    *rows = s->engine->hListRows.data();
+    *cols = s->engine->hListCols.data();
+    *n_edges = (int64_t)s->engine->hListRows.size();
+    *list_start = s->engine->hListStart.data();
+    *n_samples = s->engine->num_samples();
+    return 0;
+  });
 }
 
 int nd_sampler_distinct(nd_sampler* s) {
-  if (!s) return fail("null sampler");
-  const int rc = s->engine->distinct();
-  return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  return guarded([&]() -> int {
+    if (!s) return fail("null sampler");
+    const int rc = s->engine->distinct();
+    return rc == 0 ? 0 : fail(s->engine->last_error, rc);
+  });
 }
 
 int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length) {
@@ -344,63 +389,67 @@ int64_t nd_sampler_counter(const nd_sampler* s, int which) { return s ? s->engin
 int nd_check_sampled_vertices(const nd_graph* g, int n_steps, const int32_t* step_sizes, int initial_size,
                               int collective, int64_t n_samples, const int32_t* initial,
                               const int32_t* final_samples, int32_t invalid) {
-  if (!g || !step_sizes || n_steps < 1 || initial_size < 1 || n_samples < 0 ||
-      (n_samples > 0 && (!initial || !final_samples)))
-    return fail("bad argument");
-  nd::SampleShape shape;
-  shape.step_size.assign(step_sizes, step_sizes + n_steps);
-  shape.initial_size = initial_size;
-  shape.collective = collective != 0;
-  std::string report;
-  if (nd::check_sampled_vertices(g->csr, shape, n_samples, initial, final_samples, invalid, &report)) return 1;
-  g_error = report;
-  return 0;
+  return guarded([&]() -> int {
+    if (!g || !step_sizes || n_steps < 1 || initial_size < 1 || n_samples < 0 ||
+        (n_samples > 0 && (!initial || !final_samples)))
+      return fail("bad argument");
+    nd::SampleShape shape;
+    shape.step_size.assign(step_sizes, step_sizes + n_steps);
+    shape.initial_size = initial_size;
+    shape.collective = collective != 0;
+    std::string report;
+    if (nd::check_sampled_vertices(g->csr, shape, n_samples, initial, final_samples, invalid, &report)) return 1;
+    g_error = report;
+    return 0;
+  });
 }
 
 int nd_sampler_check_results(nd_sampler* s, int* ok) {
-  if (!s || !ok) return fail("null argument");
-  if (!s->graph) return fail("no graph set");
-  nd::EngineBase& e = *s->engine;
-  // the rule "adjacent to a vertex of the previous step" presumes that the previous step's
-  // samples are the transits (the reference checks its MultiRW app with a rule of its own,
-  // src/tests/multiGPU/multirw.cu:12-137, against the walkers left in the sample state)
-  if (e.has_explicit_transits()) return fail("no validator for apps that choose their own transits");
-  const int rc = e.fetch_final_samples();
-  if (rc != 0) return fail(e.last_error, rc);
-  nd::SampleShape shape;
-  for (int k = 0; k < e.steps(); ++k) shape.step_size.push_back(e.step_size(k));
-  shape.initial_size = e.initial_sample_size();
-  shape.collective = e.sampling_type() == SamplingType::CollectiveNeighborhood;
-  std::string report;
-  bool pass;
-  // a layer-wise app whose sample state is the per-layer adjacency matrix
-  // {len[L], row[L][B*B], col[L][B*B], val[L][B*B]} records edges instead of sampling along them
-  if (e.lists_edges()) {
-    const int rc2 = e.fetch_adjacency();
-    if (rc2 != 0) return fail(e.last_error, rc2);
-    pass = nd::check_subgraph_edge_lists(s->graph->csr, e.num_samples(), shape.initial_size, e.initialContents.data(),
-                                         e.hListStart.data(), e.hListRows.data(), e.hListCols.data(), &report);
+  return guarded([&]() -> int {
+    if (!s || !ok) return fail("null argument");
+    if (!s->graph) return fail("no graph set");
+    nd::EngineBase& e = *s->engine;
+    // the rule "adjacent to a vertex of the previous step" presumes that the previous step's
+    // samples are the transits (the reference checks its MultiRW app with a rule of its own,
+    // src/tests/multiGPU/multirw.cu:12-137, against the walkers left in the sample state)
+    if (e.has_explicit_transits()) return fail("no validator for apps that choose their own transits");
+    const int rc = e.fetch_final_samples();
+    if (rc != 0) return fail(e.last_error, rc);
+    nd::SampleShape shape;
+    for (int k = 0; k < e.steps(); ++k) shape.step_size.push_back(e.step_size(k));
+    shape.initial_size = e.initial_sample_size();
+    shape.collective = e.sampling_type() == SamplingType::CollectiveNeighborhood;
+    std::string report;
+    bool pass;
+    // a layer-wise app whose sample state is the per-layer adjacency matrix
+    // {len[L], row[L][B*B], col[L][B*B], val[L][B*B]} records edges instead of sampling along them
+    if (e.lists_edges()) {
+      const int rc2 = e.fetch_adjacency();
+      if (rc2 != 0) return fail(e.last_error, rc2);
+      pass = nd::check_subgraph_edge_lists(s->graph->csr, e.num_samples(), shape.initial_size, e.initialContents.data(),
+                                           e.hListStart.data(), e.hListRows.data(), e.hListCols.data(), &report);
+      *ok = pass ? 1 : 0;
+      if (!pass) g_error = report;
+      return 0;
+    }
+    const size_t layers = shape.step_size.size(), cells = (size_t)shape.step_size[0] * shape.step_size[0];
+    const size_t matrix_ints = layers + 3 * layers * cells;
+    if (shape.collective && e.sample_state_bytes() == sizeof(int32_t) * matrix_ints * (size_t)e.num_samples()) {
+      std::vector<int32_t> states((size_t)e.num_samples() * matrix_ints);
+      const int rc2 = e.fetch_sample_states(states.data(), states.size() * sizeof(int32_t));
+      if (rc2 != 0) return fail(e.last_error, rc2);
+      pass = nd::check_layer_adjacency_matrix(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+                                              e.hFinalSamples.data(), states.data() + layers,
+                                              states.data() + layers + layers * cells, matrix_ints, e.invalid_vertex(),
+                                              &report);
+    } else {
+      pass = nd::check_sampled_vertices(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+                                        e.hFinalSamples.data(), e.invalid_vertex(), &report);
+    }
     *ok = pass ? 1 : 0;
     if (!pass) g_error = report;
     return 0;
-  }
-  const size_t layers = shape.step_size.size(), cells = (size_t)shape.step_size[0] * shape.step_size[0];
-  const size_t matrix_ints = layers + 3 * layers * cells;
-  if (shape.collective && e.sample_state_bytes() == sizeof(int32_t) * matrix_ints * (size_t)e.num_samples()) {
-    std::vector<int32_t> states((size_t)e.num_samples() * matrix_ints);
-    const int rc2 = e.fetch_sample_states(states.data(), states.size() * sizeof(int32_t));
-    if (rc2 != 0) return fail(e.last_error, rc2);
-    pass = nd::check_layer_adjacency_matrix(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
-                                            e.hFinalSamples.data(), states.data() + layers,
-                                            states.data() + layers + layers * cells, matrix_ints, e.invalid_vertex(),
-                                            &report);
-  } else {
-    pass = nd::check_sampled_vertices(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
-                                      e.hFinalSamples.data(), e.invalid_vertex(), &report);
-  }
-  *ok = pass ? 1 : 0;
-  if (!pass) g_error = report;
-  return 0;
+  });
 }
 
 void nd_sampler_free_device(nd_sampler* s) {
@@ -419,18 +468,20 @@ void nd_free_device_memory(void) {
 }
 
 int nd_init_sampling(const char* app_name, const char* graph_path, uint64_t seed) {
-  nd_free_device_memory();
-  int rc = nd_graph_load(graph_path, "edge-list", "binary", &g_module_graph);
-  if (rc != 0) return rc;
-  rc = nd_sampler_create(app_name, &g_module_sampler);
-  if (rc == 0) rc = nd_sampler_set_graph(g_module_sampler, g_module_graph);
-  if (rc == 0) rc = nd_sampler_alloc(g_module_sampler, seed);
-  if (rc != 0) {
-    const std::string keep = g_error;
+  return guarded([&]() -> int {
     nd_free_device_memory();
-    g_error = keep;
-  }
-  return rc;
+    int rc = nd_graph_load(graph_path, "edge-list", "binary", &g_module_graph);
+    if (rc != 0) return rc;
+    rc = nd_sampler_create(app_name, &g_module_sampler);
+    if (rc == 0) rc = nd_sampler_set_graph(g_module_sampler, g_module_graph);
+    if (rc == 0) rc = nd_sampler_alloc(g_module_sampler, seed);
+    if (rc != 0) {
+      const std::string keep = g_error;
+      nd_free_device_memory();
+      g_error = keep;
+    }
+    return rc;
+  });
 }
 
 int nd_sample(void) {
@@ -454,133 +505,151 @@ const int32_t* nd_final_samples_array(void) {
 
 int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, int64_t n_slots, int draws_per_slot,
                            float* out) {
-  if (n_slots < 0 || draws_per_slot < 1 || (n_slots > 0 && !out)) return fail("bad argument");
-  if (n_slots == 0) return 0;
-  DeviceBuffer d;
-  const size_t bytes = sizeof(float) * (size_t)n_slots * draws_per_slot;
-  CAPI_HIP(d.alloc(bytes));
-  philox_fill_kernel<<<dim3((unsigned)((n_slots + 255) / 256)), dim3(256), 0, 0>>>(seed, step, first_slot,
-                                                                                  (size_t)n_slots, draws_per_slot,
-                                                                                  d.as<float>());
-  CAPI_HIP(hipGetLastError());
-  CAPI_HIP(hipMemcpy(out, d.p, bytes, hipMemcpyDeviceToHost));
-  return 0;
+  return guarded([&]() -> int {
+    if (n_slots < 0 || draws_per_slot < 1 || (n_slots > 0 && !out)) return fail("bad argument");
+    if (n_slots == 0) return 0;
+    DeviceBuffer d;
+    const size_t bytes = sizeof(float) * (size_t)n_slots * draws_per_slot;
+    CAPI_HIP(d.alloc(bytes));
+    philox_fill_kernel<<<dim3((unsigned)((n_slots + 255) / 256)), dim3(256), 0, 0>>>(seed, step, first_slot,
+                                                                                    (size_t)n_slots, draws_per_slot,
+                                                                                    d.as<float>());
+    CAPI_HIP(hipGetLastError());
+    CAPI_HIP(hipMemcpy(out, d.p, bytes, hipMemcpyDeviceToHost));
+    return 0;
+  });
 }
 
 int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_bits, int32_t* keys_out,
                   int32_t* vals_out) {
-  if (n < 0 || key_bits < 1 || key_bits > 32 || (n > 0 && (!keys || !keys_out || !vals_out)))
-    return fail("bad argument");
-  if (n == 0) return 0;
-  if (n >= (int64_t)1 << 31) return fail("too many pairs");
-  const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);
-  DeviceBuffer k_in, v_in, k_a, v_a, k_b, v_b, hist, scratch;
-  const size_t bytes = sizeof(uint32_t) * (size_t)n;
-  CAPI_HIP(k_in.alloc(bytes));
-  CAPI_HIP(k_a.alloc(bytes));
-  CAPI_HIP(v_a.alloc(bytes));
-  CAPI_HIP(k_b.alloc(bytes));
-  CAPI_HIP(v_b.alloc(bytes));
-  CAPI_HIP(hist.alloc(sizeof(uint32_t) * plan.hist_elems));
-  CAPI_HIP(scratch.alloc(sizeof(uint32_t) * plan.scratch_elems));
-  CAPI_HIP(hipMemcpy(k_in.p, keys, bytes, hipMemcpyHostToDevice));
-  if (vals) {
-    CAPI_HIP(v_in.alloc(bytes));
-    CAPI_HIP(hipMemcpy(v_in.p, vals, bytes, hipMemcpyHostToDevice));
-  }
-  uint32_t *k_sorted = nullptr, *v_sorted = nullptr;
-  CAPI_HIP(nd::radix_sort_pairs(plan, k_in.as<uint32_t>(), vals ? v_in.as<uint32_t>() : nullptr, k_a.as<uint32_t>(),
-                                v_a.as<uint32_t>(), k_b.as<uint32_t>(), v_b.as<uint32_t>(), hist.as<uint32_t>(),
-                                scratch.as<uint32_t>(), 0, &k_sorted, &v_sorted));
-  CAPI_HIP(hipDeviceSynchronize());
-  CAPI_HIP(hipMemcpy(keys_out, k_sorted, bytes, hipMemcpyDeviceToHost));
-  CAPI_HIP(hipMemcpy(vals_out, v_sorted, bytes, hipMemcpyDeviceToHost));
-  return 0;
+  return guarded([&]() -> int {
+    if (n < 0 || key_bits < 1 || key_bits > 32 || (n > 0 && (!keys || !keys_out || !vals_out)))
+      return fail("bad argument");
+    if (n == 0) return 0;
+    if (n >= (int64_t)1 << 31) return fail("too many pairs");
+    const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);
+    DeviceBuffer k_in, v_in, k_a, v_a, k_b, v_b, hist, scratch;
+    const size_t bytes = sizeof(uint32_t) * (size_t)n;
+    CAPI_HIP(k_in.alloc(bytes));
+    CAPI_HIP(k_a.alloc(bytes));
+    CAPI_HIP(v_a.alloc(bytes));
+    CAPI_HIP(k_b.alloc(bytes));
+    CAPI_HIP(v_b.alloc(bytes));
+    CAPI_HIP(hist.alloc(sizeof(uint32_t) * plan.hist_elems));
+    CAPI_HIP(scratch.alloc(sizeof(uint32_t) * plan.scratch_elems));
+    CAPI_HIP(hipMemcpy(k_in.p, keys, bytes, hipMemcpyHostToDevice));
+    if (vals) {
+      CAPI_HIP(v_in.alloc(bytes));
+      CAPI_HIP(hipMemcpy(v_in.p, vals, bytes, hipMemcpyHostToDevice));
+    }
+    uint32_t *k_sorted = nullptr, *v_sorted = nullptr;
+    CAPI_HIP(nd::radix_sort_pairs(plan, k_in.as<uint32_t>(), vals ? v_in.as<uint32_t>() : nullptr, k_a.as<uint32_t>(),
+                                  v_a.as<uint32_t>(), k_b.as<uint32_t>(), v_b.as<uint32_t>(), hist.as<uint32_t>(),
+                                  scratch.as<uint32_t>(), 0, &k_sorted, &v_sorted));
+    CAPI_HIP(hipDeviceSynchronize());
+    CAPI_HIP(hipMemcpy(keys_out, k_sorted, bytes, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(vals_out, v_sorted, bytes, hipMemcpyDeviceToHost));
+    return 0;
+  });
 }
 
 int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
                        int32_t* offsets, int64_t* n_runs, int64_t* n_valid) {
-  if (n < 0 || !n_runs || !n_valid || (n > 0 && (!sorted_keys || !uniq || !counts || !offsets)))
-    return fail("bad argument");
-  *n_runs = 0;
-  *n_valid = 0;
-  if (n == 0) return 0;
-  const size_t bytes = sizeof(uint32_t) * (size_t)n;
-  DeviceBuffer keys, run_key, run_start, run_count, meta, scratch;
-  CAPI_HIP(keys.alloc(bytes));
-  CAPI_HIP(run_key.alloc(bytes));
-  CAPI_HIP(run_start.alloc(bytes + sizeof(uint32_t)));
-  CAPI_HIP(run_count.alloc(bytes));
-  CAPI_HIP(meta.alloc(sizeof(nd::RunsMeta)));
-  CAPI_HIP(scratch.alloc(sizeof(uint32_t) * nd::runs_scratch_elems((size_t)n)));
-  CAPI_HIP(hipMemcpy(keys.p, sorted_keys, bytes, hipMemcpyHostToDevice));
-  CAPI_HIP(nd::find_transit_runs(keys.as<uint32_t>(), (size_t)n, (uint32_t)invalid, run_key.as<uint32_t>(),
-                                 run_start.as<uint32_t>(), meta.as<nd::RunsMeta>(), scratch.as<uint32_t>(), 0));
-  run_counts_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(run_start.as<uint32_t>(),
-                                                                           meta.as<nd::RunsMeta>(),
-                                                                           run_count.as<uint32_t>());
-  CAPI_HIP(hipGetLastError());
-  nd::RunsMeta h;
-  CAPI_HIP(hipMemcpy(&h, meta.p, sizeof(h), hipMemcpyDeviceToHost));
-  *n_runs = h.n_runs;
-  *n_valid = h.n_valid;
-  if (h.n_runs) {
-    CAPI_HIP(hipMemcpy(uniq, run_key.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
-    CAPI_HIP(hipMemcpy(counts, run_count.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
-    CAPI_HIP(hipMemcpy(offsets, run_start.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
-  }
-  return 0;
+  return guarded([&]() -> int {
+    if (n < 0 || !n_runs || !n_valid || (n > 0 && (!sorted_keys || !uniq || !counts || !offsets)))
+      return fail("bad argument");
+    *n_runs = 0;
+    *n_valid = 0;
+    if (n == 0) return 0;
+    const size_t bytes = sizeof(uint32_t) * (size_t)n;
+    DeviceBuffer keys, run_key, run_start, run_count, meta, scratch;
+    CAPI_HIP(keys.alloc(bytes));
+    CAPI_HIP(run_key.alloc(bytes));
+    CAPI_HIP(run_start.alloc(bytes + sizeof(uint32_t)));
+    CAPI_HIP(run_count.alloc(bytes));
+    CAPI_HIP(meta.alloc(sizeof(nd::RunsMeta)));
+    CAPI_HIP(scratch.alloc(sizeof(uint32_t) * nd::runs_scratch_elems((size_t)n)));
+    CAPI_HIP(hipMemcpy(keys.p, sorted_keys, bytes, hipMemcpyHostToDevice));
+    CAPI_HIP(nd::find_transit_runs(keys.as<uint32_t>(), (size_t)n, (uint32_t)invalid, run_key.as<uint32_t>(),
+                                   run_start.as<uint32_t>(), meta.as<nd::RunsMeta>(), scratch.as<uint32_t>(), 0));
+    run_counts_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(run_start.as<uint32_t>(),
+                                                                             meta.as<nd::RunsMeta>(),
+                                                                             run_count.as<uint32_t>());
+    CAPI_HIP(hipGetLastError());
+    nd::RunsMeta h;
+    CAPI_HIP(hipMemcpy(&h, meta.p, sizeof(h), hipMemcpyDeviceToHost));
+    *n_runs = h.n_runs;
+    *n_valid = h.n_valid;
+    if (h.n_runs) {
+      CAPI_HIP(hipMemcpy(uniq, run_key.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+      CAPI_HIP(hipMemcpy(counts, run_count.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+      CAPI_HIP(hipMemcpy(offsets, run_start.p, sizeof(uint32_t) * h.n_runs, hipMemcpyDeviceToHost));
+    }
+    return 0;
+  });
 }
 
 int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64_t n_samples,
                                int32_t transits_per_sample, int32_t invalid, int32_t* sizes, int32_t* offsets,
                                int32_t* cols, float* weights, int64_t capacity, int32_t* row_offsets) {
-  if (!g || !transits || n_samples < 1 || transits_per_sample < 1 || !sizes || !offsets || !cols || !weights ||
-      !row_offsets || (uint32_t)transits_per_sample > nd::kMaxLayerTransits || n_samples >= (1ll << 31))
-    return fail("bad argument");
-  nd::DeviceGraph dg;
-  std::string err;
-  if (!dg.upload(&g->csr, false, false, &err)) return fail(err);
-  const uint32_t S = (uint32_t)n_samples;
-  const size_t n_tr = (size_t)S * transits_per_sample;
-  DeviceBuffer d_tr, d_sizes, d_offsets, d_scratch, d_cols, d_weights, d_rows;
-  CAPI_HIP(d_tr.alloc(sizeof(int32_t) * n_tr));
-  CAPI_HIP(d_sizes.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
-  CAPI_HIP(d_offsets.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
-  CAPI_HIP(d_scratch.alloc(sizeof(uint32_t) * nd::scan_scratch_elems((size_t)S + 1)));
-  CAPI_HIP(d_rows.alloc(sizeof(uint32_t) * n_tr));
-  CAPI_HIP(hipMemcpy(d_tr.p, transits, sizeof(int32_t) * n_tr, hipMemcpyHostToDevice));
-  CAPI_HIP(hipMemset(d_sizes.p, 0, sizeof(uint32_t) * ((size_t)S + 1)));
-  nd::TransitView tv{d_tr.as<int32_t>(), (uint32_t)transits_per_sample, (uint32_t)transits_per_sample};
-  nd::collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, 0>>>(dg.view, tv, S, invalid, d_sizes.as<uint32_t>());
-  CAPI_HIP(nd::exclusive_scan_u32(d_sizes.as<uint32_t>(), d_offsets.as<uint32_t>(), (size_t)S + 1,
-                                  d_scratch.as<uint32_t>(), 0));
-  CAPI_HIP(hipMemcpy(sizes, d_sizes.p, sizeof(uint32_t) * S, hipMemcpyDeviceToHost));
-  CAPI_HIP(hipMemcpy(offsets, d_offsets.p, sizeof(uint32_t) * ((size_t)S + 1), hipMemcpyDeviceToHost));
-  const int64_t total = offsets[S];
-  if (total > capacity) return fail("collective neighbourhood larger than the capacity given");
-  CAPI_HIP(d_cols.alloc(sizeof(int32_t) * (size_t)total));
-  CAPI_HIP(d_weights.alloc(sizeof(float) * (size_t)total));
-  DeviceBuffer d_item_count, d_item_start;
-  CAPI_HIP(d_item_count.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
-  CAPI_HIP(d_item_start.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
-  uint64_t n_items = 0;
-  for (uint32_t i = 0; i < S; ++i) {
-    const uint64_t items = ((uint64_t)(uint32_t)sizes[i] + nd::kBuildItemEntries - 1) / nd::kBuildItemEntries;
-    n_items += items ? items : 1;
-  }
-  nd::build_item_counts<<<dim3((S + 1 + 255) / 256), dim3(256), 0, 0>>>(d_sizes.as<uint32_t>(), S,
-                                                                       d_item_count.as<uint32_t>());
-  CAPI_HIP(nd::exclusive_scan_u32(d_item_count.as<uint32_t>(), d_item_start.as<uint32_t>(), (size_t)S + 1,
-                                  d_scratch.as<uint32_t>(), 0));
-  nd::collective_build<<<dim3((unsigned)n_items), dim3(256), 0, 0>>>(
-      dg.view, tv, invalid, d_offsets.as<uint32_t>(), d_item_start.as<uint32_t>(), S, d_cols.as<int32_t>(),
-      d_weights.as<float>(), d_rows.as<uint32_t>());
-  CAPI_HIP(hipGetLastError());
-  CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
-  CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));
-  CAPI_HIP(hipMemcpy(row_offsets, d_rows.p, sizeof(uint32_t) * n_tr, hipMemcpyDeviceToHost));
-  return 0;
+  return guarded([&]() -> int {
+    if (!g || !transits || n_samples < 1 || transits_per_sample < 1 || !sizes || !offsets || !cols || !weights ||
+        !row_offsets || (uint32_t)transits_per_sample > nd::kMaxLayerTransits || n_samples >= (1ll << 31))
+      return fail("bad argument");
+    const uint32_t S = (uint32_t)n_samples;
+    const size_t n_tr = (size_t)S * transits_per_sample;
+    // the kernels index the row extents with every transit that is not a "no vertex" value
+    uint64_t entries = 0;
+    for (size_t i = 0; i < n_tr; ++i) {
+      const int32_t t = transits[i];
+      if (t == invalid || t == -1) continue;
+      if (!g->csr.has_vertex(t)) return fail("transit " + std::to_string(t) + " is not a vertex of the graph");
+      entries += (uint64_t)g->csr.n_edges_for_vertex(t);
+    }
+    if (entries >= (1ull << 31)) return fail("collective neighbourhoods of more than 2^31 entries");
+    if ((int64_t)entries > capacity) return fail("collective neighbourhood larger than the capacity given");
+    nd::DeviceGraph dg;
+    std::string err;
+    if (!dg.upload(&g->csr, false, false, &err)) return fail(err);
+    DeviceBuffer d_tr, d_sizes, d_offsets, d_scratch, d_cols, d_weights, d_rows;
+    CAPI_HIP(d_tr.alloc(sizeof(int32_t) * n_tr));
+    CAPI_HIP(d_sizes.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+    CAPI_HIP(d_offsets.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+    CAPI_HIP(d_scratch.alloc(sizeof(uint32_t) * nd::scan_scratch_elems((size_t)S + 1)));
+    CAPI_HIP(d_rows.alloc(sizeof(uint32_t) * n_tr));
+    CAPI_HIP(hipMemcpy(d_tr.p, transits, sizeof(int32_t) * n_tr, hipMemcpyHostToDevice));
+    CAPI_HIP(hipMemset(d_sizes.p, 0, sizeof(uint32_t) * ((size_t)S + 1)));
+    nd::TransitView tv{d_tr.as<int32_t>(), (uint32_t)transits_per_sample, (uint32_t)transits_per_sample};
+    nd::collective_sizes<<<dim3((S + 3) / 4), dim3(256), 0, 0>>>(dg.view, tv, S, invalid, d_sizes.as<uint32_t>());
+    CAPI_HIP(nd::exclusive_scan_u32(d_sizes.as<uint32_t>(), d_offsets.as<uint32_t>(), (size_t)S + 1,
+                                    d_scratch.as<uint32_t>(), 0));
+    CAPI_HIP(hipMemcpy(sizes, d_sizes.p, sizeof(uint32_t) * S, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(offsets, d_offsets.p, sizeof(uint32_t) * ((size_t)S + 1), hipMemcpyDeviceToHost));
+    const int64_t total = offsets[S];
+    if (total > capacity) return fail("collective neighbourhood larger than the capacity given");
+    CAPI_HIP(d_cols.alloc(sizeof(int32_t) * (size_t)total));
+    CAPI_HIP(d_weights.alloc(sizeof(float) * (size_t)total));
+    DeviceBuffer d_item_count, d_item_start;
+    CAPI_HIP(d_item_count.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+    CAPI_HIP(d_item_start.alloc(sizeof(uint32_t) * ((size_t)S + 1)));
+    uint64_t n_items = 0;
+    for (uint32_t i = 0; i < S; ++i) {
+      const uint64_t items = ((uint64_t)(uint32_t)sizes[i] + nd::kBuildItemEntries - 1) / nd::kBuildItemEntries;
+      n_items += items ? items : 1;
+    }
+    nd::build_item_counts<<<dim3((S + 1 + 255) / 256), dim3(256), 0, 0>>>(d_sizes.as<uint32_t>(), S,
+                                                                         d_item_count.as<uint32_t>());
+    CAPI_HIP(nd::exclusive_scan_u32(d_item_count.as<uint32_t>(), d_item_start.as<uint32_t>(), (size_t)S + 1,
+                                    d_scratch.as<uint32_t>(), 0));
+    nd::collective_build<<<dim3((unsigned)n_items), dim3(256), 0, 0>>>(
+        dg.view, tv, invalid, d_offsets.as<uint32_t>(), d_item_start.as<uint32_t>(), S, d_cols.as<int32_t>(),
+        d_weights.as<float>(), d_rows.as<uint32_t>());
+    CAPI_HIP(hipGetLastError());
+    CAPI_HIP(hipMemcpy(cols, d_cols.p, sizeof(int32_t) * (size_t)total, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(weights, d_weights.p, sizeof(float) * (size_t)total, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(row_offsets, d_rows.p, sizeof(uint32_t) * n_tr, hipMemcpyDeviceToHost));
+    return 0;
+  });
 }
 
 }  // extern "C"

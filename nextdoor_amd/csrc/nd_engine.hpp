@@ -108,6 +108,15 @@ class HostArray {
   bool pinned_ = false;
 };
 
+// Roots index the row extents in the kernels: each must be a vertex, or the "no vertex" value
+// (the number of vertices).  The reference does not check (a root outside the graph reads past
+// its arrays there).
+inline bool roots_are_vertices(const std::vector<VertexID_t>& roots, int32_t n_vertices) {
+  for (VertexID_t r : roots)
+    if (r < 0 || r > n_vertices) return false;
+  return true;
+}
+
 class EngineBase {
  public:
   virtual ~EngineBase() {}
@@ -833,6 +842,10 @@ class Engine : public EngineBase {
       std::vector<VertexID_t> roots = app.initialSample((int)(first_sample_ + s), csr, samples_.back());
       if ((EdgePos_t)roots.size() != init_size_) {
         last_error = "initialSample size differs from initialSampleSize";  // nextdoor.cu:1964-1969
+        return -2;
+      }
+      if (!roots_are_vertices(roots, graph_->get_n_vertices())) {
+        last_error = "initialSample returned a root that is not a vertex of the graph";
         return -2;
       }
       initialContents.insert(initialContents.end(), roots.begin(), roots.end());

@@ -992,6 +992,10 @@ class LayerEngine : public EngineBase {
         last_error = "initialSample size differs from initialSampleSize";
         return -2;
       }
+      if (!roots_are_vertices(roots, graph_->get_n_vertices())) {
+        last_error = "initialSample returned a root that is not a vertex of the graph";
+        return -2;
+      }
       initialContents.insert(initialContents.end(), roots.begin(), roots.end());
     }
     const size_t F = (size_t)final_sample_size();

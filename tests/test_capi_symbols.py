@@ -45,3 +45,21 @@ def test_unknown_app_is_an_error_not_an_abort():
     g = nextdoor_amd.Graph.from_edges([0, 1], [1, 0])
     with pytest.raises(nextdoor_amd.NextDoorError):
         nextdoor_amd.Sampler("NoSuchApp", g)
+
+
+def test_bad_arguments_are_refused_before_anything_reaches_a_device():
+    import numpy as np
+    import nextdoor_amd
+    import pytest
+    g = nextdoor_amd.Graph.from_edges([0, 1, 2], [1, 2, 0])
+    # a transit that is neither a vertex nor a "no vertex" value
+    with pytest.raises(nextdoor_amd.NextDoorError, match="not a vertex"):
+        nextdoor_amd.collective_neighborhood(g, np.array([[0, 7]], np.int32), 2, invalid=3, capacity=16)
+    # room for fewer entries than the neighbourhoods hold
+    with pytest.raises(nextdoor_amd.NextDoorError, match="capacity"):
+        nextdoor_amd.collective_neighborhood(g, np.array([[0, 1]], np.int32), 2, invalid=3, capacity=1)
+    # row offsets that run backwards, a column outside the graph
+    with pytest.raises(nextdoor_amd.NextDoorError, match="monotone"):
+        nextdoor_amd.Graph.from_csr([0, 2, 1, 3], [1, 2, 0])
+    with pytest.raises(nextdoor_amd.NextDoorError, match="out of range"):
+        nextdoor_amd.Graph.from_csr([0, 1, 2, 3], [1, 2, 9])
