@@ -534,59 +534,73 @@ constexpr uint32_t kGroupWords = 8;
 constexpr uint32_t kGroupsPerPart = 64;
 constexpr uint32_t kPartWords = kGroupWords * kGroupsPerPart;  // 16384 vertices
 
-// One wavefront per part, one lane per group: group_through[part * 64 + g] = degree^2 of the
-// marked vertices of groups 0..g of the part; part_total[part]; marked[s] += marked vertices.
-__global__ __launch_bounds__(256) void bitmap_group_sums(const uint32_t* __restrict__ bitmap, uint32_t words_per_sample,
-                                                         uint32_t n_parts, const EdgePos_t* __restrict__ row_ptr,
-                                                         uint64_t* __restrict__ group_through,
-                                                         uint64_t* __restrict__ part_total,
-                                                         uint32_t* __restrict__ marked) {
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t part = blockIdx.x * (256 / kWave) + (threadIdx.x >> 6);  // over all samples
-  if (part >= n_parts) return;  // a whole wavefront
+// The degrees of a part's 16,384 vertices do not depend on the sample, so a workgroup keeps
+// them in LDS and runs its samples past them: fetching the row extents of every marked vertex
+// of every sample from the caches instead (2.0e9 gathers a pass at full size, a lane waiting
+// for each) took as long as the marking itself.
+constexpr uint32_t kSumThreads = 1024;
+constexpr uint32_t kSumSamplesPerBlock = 128;
+constexpr uint32_t kGroupVertices = kGroupWords * 32u;
+constexpr uint32_t kGroupPitch = kGroupVertices + 1u;  // lanes walk different groups: the odd pitch spreads them over the banks
+
+// One workgroup per (part, block of 128 samples), a wavefront per sample, a lane per group:
+// group_through[(s * parts + part) * 64 + g] = degree^2 of the marked vertices of groups 0..g
+// of the part; part_total[s * parts + part]; marked[s] += marked vertices.  Workgroups of the
+// low parts (where the hubs of a skewed graph sit, marked in nearly every sample) come first.
+__global__ __launch_bounds__(kSumThreads) void bitmap_group_sums(const uint32_t* __restrict__ bitmap,
+                                                                 uint32_t words_per_sample, uint32_t n_samples,
+                                                                 uint32_t n_vertices,
+                                                                 const EdgePos_t* __restrict__ row_ptr,
+                                                                 uint64_t* __restrict__ group_through,
+                                                                 uint64_t* __restrict__ part_total,
+                                                                 uint32_t* __restrict__ marked) {
+  __shared__ uint32_t s_degree[kGroupsPerPart * kGroupPitch];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t parts_per_sample = words_per_sample / kPartWords;
-  const uint32_t s = part / parts_per_sample;
-  const uint32_t first_word = (part - s * parts_per_sample) * kPartWords + lane * kGroupWords;
-  const uint4* words = (const uint4*)(bitmap + (size_t)s * words_per_sample + first_word);
-  const uint4 a = words[0], b = words[1];
-  const uint32_t w[kGroupWords] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-  uint64_t sum = 0;
-  uint32_t count = 0;
+  const uint32_t sample_blocks = (n_samples + kSumSamplesPerBlock - 1) / kSumSamplesPerBlock;
+  const uint32_t part = blockIdx.x / sample_blocks;
+  const uint32_t first_sample = (blockIdx.x - part * sample_blocks) * kSumSamplesPerBlock;
+  const uint32_t first_vertex = part * (kPartWords * 32u);
+  for (uint32_t i = threadIdx.x; i < kPartWords * 32u; i += kSumThreads) {
+    const uint32_t v = first_vertex + i;
+    s_degree[(i / kGroupVertices) * kGroupPitch + i % kGroupVertices] =
+        v < n_vertices ? (uint32_t)(row_ptr[v + 1] - row_ptr[v]) : 0u;
+  }
+  __syncthreads();
+  const uint32_t end_sample = first_sample + kSumSamplesPerBlock < n_samples ? first_sample + kSumSamplesPerBlock : n_samples;
+  const uint32_t* mine = s_degree + lane * kGroupPitch;
+  for (uint32_t s = first_sample + wave; s < end_sample; s += kSumThreads / kWave) {
+    const uint4* words = (const uint4*)(bitmap + (size_t)s * words_per_sample + (size_t)part * kPartWords + lane * kGroupWords);
+    const uint4 a = words[0], b = words[1];
+    const uint64_t w[kGroupWords / 2] = {a.x | ((uint64_t)a.y << 32), a.z | ((uint64_t)a.w << 32),
+                                         b.x | ((uint64_t)b.y << 32), b.z | ((uint64_t)b.w << 32)};
+    uint64_t sum = 0;
+    uint32_t count = 0;
 #pragma unroll
-  for (uint32_t k = 0; k < kGroupWords; ++k) {
-    uint32_t bits = w[k];
-    count += __popc(bits);
-    const uint32_t base = (first_word + k) * 32u;
-    while (bits) {
-      // four row extents are fetched before the first is used: one at a time, a lane spent
-      // its time waiting for each in turn
-      uint32_t v[4];
-      bool has[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        has[q] = bits != 0;
-        v[q] = base + (has[q] ? (uint32_t)__ffs((int)bits) - 1u : 0u);
-        bits &= bits - 1u;  // 0 stays 0
-      }
-      EdgePos_t from[4], to[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        from[q] = has[q] ? row_ptr[v[q]] : 0;
-        to[q] = has[q] ? row_ptr[v[q] + 1] : 0;
-      }
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint64_t d = (uint64_t)(to[q] - from[q]);
-        sum += d * d;
+    for (uint32_t k = 0; k < kGroupWords / 2; ++k) {
+      uint64_t bits = w[k];
+      count += (uint32_t)__popcll(bits);
+      const uint32_t* from = mine + k * 64u;
+      while (bits) {
+        // two lookups under way per round
+        const uint32_t i0 = (uint32_t)__ffsll((unsigned long long)bits) - 1u;
+        bits &= bits - 1ull;
+        const bool second = bits != 0;
+        const uint32_t i1 = second ? (uint32_t)__ffsll((unsigned long long)bits) - 1u : i0;
+        bits &= bits - 1ull;  // 0 stays 0
+        const uint64_t d0 = from[i0];
+        const uint64_t d1 = second ? from[i1] : 0u;
+        sum += d0 * d0 + d1 * d1;
       }
     }
-  }
-  const uint64_t through = wave_inclusive_scan_u64(sum);
-  group_through[(size_t)part * kGroupsPerPart + lane] = through;
-  if (lane == 63) part_total[part] = through;
+    const uint64_t through = wave_inclusive_scan_u64(sum);
+    const size_t at = (size_t)s * parts_per_sample + part;
+    group_through[at * kGroupsPerPart + lane] = through;
+    if (lane == 63) part_total[at] = through;
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) count += __shfl_xor(count, d, kWave);
-  if (lane == 0 && count) atomicAdd(&marked[s], count);
+    for (int d = 32; d > 0; d >>= 1) count += __shfl_xor(count, d, kWave);
+    if (lane == 0 && count) atomicAdd(&marked[s], count);
+  }
 }
 
 // One wavefront per sample: part_before[s * (parts + 1) + p] = degree^2 of the marked vertices
@@ -1275,8 +1289,9 @@ class LayerEngine : public EngineBase {
         dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u);
     tock();
     ND_HIP_TRY(hipMemsetAsync(d_marked_, 0, sizeof(uint32_t) * (size_t)n, stream_));
-    bitmap_group_sums<<<dim3((unsigned)((n_parts + 3) / 4)), dim3(256), 0, stream_>>>(
-        d_bitmap_, bitmap_words_, (uint32_t)n_parts, dgraph_.row_ptr(), d_group_through_, d_part_total_, d_marked_);
+    const uint32_t sample_blocks = (n + kSumSamplesPerBlock - 1) / kSumSamplesPerBlock;
+    bitmap_group_sums<<<dim3(parts_per_sample * sample_blocks), dim3(kSumThreads), 0, stream_>>>(
+        d_bitmap_, bitmap_words_, n, (uint32_t)invalid_, dgraph_.row_ptr(), d_group_through_, d_part_total_, d_marked_);
     sample_part_sums<<<dim3(n), dim3(64), 0, stream_>>>(d_part_total_, parts_per_sample, d_part_before_);
     std::vector<uint32_t> marked(n);
     ND_HIP_TRY(hipMemcpyAsync(marked.data(), d_marked_, sizeof(uint32_t) * n, hipMemcpyDeviceToHost, stream_));
