@@ -237,6 +237,7 @@ def main():
         result["config"]["neighbourhood_entries"] = entries
         result["config"]["distinct_pairs"] = distinct
         result["config"]["chunks"] = sampler.counter(2)
+        result["config"]["hub_bitmaps"] = sampler.counter(3)
         result["config"]["neighbourhood_entries_per_s"] = entries / (ms_per_step / 1000.0)
         # dominant kernel: collective_mark_binned walks every entry of every collective
         # neighbourhood once.  Minimal traffic: the entry's vertex id (4 B; + 4 B weight for

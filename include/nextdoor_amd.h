@@ -134,7 +134,8 @@ int nd_sampler_distinct(nd_sampler* s);
 int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length);
 /* Sizes the last run worked on, for traffic accounting.  Layer-wise apps: which 0 = entries
  * of all collective neighbourhoods built, 1 = distinct (sample, vertex) pairs found,
- * 2 = chunks of samples processed; other apps return 0. */
+ * 2 = chunks of samples processed, 3 = ready-made stretch bitmaps of the graph's hubs (built
+ * by nd_sampler_set_graph for the FastGCN importance form); other apps return 0. */
 int64_t nd_sampler_counter(const nd_sampler* s, int which);
 /* The validators the reference's apps pass to nextdoor() as checkResultsFunc
  * (src/check_results.cu): checkSampledVerticesResult (162-299) for the per-transit apps and

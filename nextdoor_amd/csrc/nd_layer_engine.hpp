@@ -36,6 +36,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <string>
 #include <type_traits>
 #include <vector>
@@ -270,6 +271,7 @@ __device__ __forceinline__ void segmented_row_step(uint32_t& closed, unsigned lo
 constexpr uint32_t kBinThreads = 1024;
 constexpr uint32_t kBinWaves = kBinThreads / 64;
 constexpr uint32_t kBinAhead = 4;             // entries a lane fetches before it works on the first
+constexpr EdgePos_t kShortRest = 16;          // edges left of an adjacency that are stepped through one by one
 // consecutive stretches of a sample one workgroup takes (FastGCN form: few, large stretches per
 // sample, and the low ones hold most entries; LADIES form: hundreds of small ones)
 constexpr uint32_t kBinsPerGroupBits = 8;
@@ -277,12 +279,33 @@ constexpr uint32_t kBinsPerGroupSums = 16;
 constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
+// Dense pieces (FastGCN form).  What a hub contributes to a stretch can be thousands of entries
+// (a layer drawn by degree^2 sits on the hubs: 144 K entries per transit at full size), and it
+// is the same for every sample that holds the hub.  Where a vertex has kDensePieceEntries or
+// more edges into one stretch, the stretch's bitmap of that vertex is built once per graph
+// (1536 words); a sample then ORs the piece into the stretch on its way out of LDS instead
+// of marking the entries one by one.  hub_row[v] = row of v in piece_of or -1;
+// piece_of[row * stretches + stretch] = piece index or kNoPiece.
+constexpr uint32_t kDensePieceEntries = 512;
+constexpr size_t kDensePieceBudgetBytes = (size_t)2 << 30;
+constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
+struct DensePieces {
+  const int32_t* hub_row = nullptr;  // nullptr: the graph has none
+  const uint32_t* piece_of = nullptr;
+  const uint32_t* words = nullptr;
+};
+
+// 32-bit words of one sample's presence map: a bit per vertex, padded to whole tiles.
+inline uint32_t bitmap_words_for(uint32_t n_vertices) {
+  return ((n_vertices + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
+}
+
 template <bool kWithImportance>
 __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
-    unsigned long long* __restrict__ sums, uint32_t keys_per_sample) {
+    unsigned long long* __restrict__ sums, uint32_t keys_per_sample, DensePieces dense) {
   constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
   constexpr uint32_t kBinVertices = kBinWords * 32u;
   // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
@@ -296,6 +319,8 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // 1 / (the weights of its transit added up)
   __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
   __shared__ uint32_t s_ranges;                        // sub-ranges kept
+  __shared__ uint32_t s_piece[kWithImportance ? 1 : kMaxLayerTransits];  // dense pieces of the stretch
+  __shared__ uint32_t s_pieces[2];                     // how many; stretches alternate between the two counters
   // A workgroup takes kBinsPerGroup consecutive stretches of one sample, one after the other:
   // where a transit's sub-range ends in one stretch it begins in the next, and the end is
   // then only a short gallop away instead of a search of the whole adjacency.
@@ -310,10 +335,17 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   // tv.count <= kBinThreads: lane i keeps transit i's adjacency and how far the stretches
   // before this one reach into it
   EdgePos_t my_end = 0, my_reach = 0;
+  uint32_t my_next = 0xFFFFFFFFu;  // destination of edge my_reach; none left: above every vertex
   float my_row_sum = 1.0f;
+  int32_t my_hub = -1;
+  if (!kWithImportance) {
+    if (threadIdx.x < 2) s_pieces[threadIdx.x] = 0;
+    __syncthreads();
+  }
   if (threadIdx.x < tv.count) {
     const int32_t t = transits[threadIdx.x];
     if (t != invalid && t != -1) {
+      if (!kWithImportance && dense.hub_row) my_hub = dense.hub_row[t];
       my_end = csr.row_ptr[t + 1];
       EdgePos_t lo = csr.row_ptr[t], hi = my_end;  // first edge whose destination is in the first stretch or above
       const uint32_t v_first = first_bin * kBinVertices;
@@ -322,35 +354,63 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
         if ((uint32_t)csr.edges[mid] < v_first) lo = mid + 1; else hi = mid;
       }
       my_reach = lo;
+      if (lo < my_end) my_next = (uint32_t)csr.edges[lo];
       if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
   }
   for (uint32_t bin = first_bin; bin < first_bin + kBinsPerGroup && bin < bins_per_sample; ++bin) {
   const uint32_t v_lo = bin * kBinVertices;
+  const uint32_t parity = (bin - first_bin) & 1u;
   for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
   if (kWithImportance)
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
   if (threadIdx.x < tv.count) {
     const EdgePos_t my_from = my_reach;
-    // first edge at or after my_from whose destination is >= v_lo + kBinVertices: gallop, then bisect
-    EdgePos_t lo = my_from, width = 64;
-    while (lo < my_end) {
-      const EdgePos_t probe = lo + width < my_end ? lo + width : my_end;
-      if ((uint32_t)csr.edges[probe - 1] >= v_lo + kBinVertices) break;
-      lo = probe;
-      width <<= 1;
+    const uint32_t v_hi = v_lo + kBinVertices;
+    // first edge at or after my_from whose destination is >= v_hi.  The workgroup waits for
+    // the slowest of these searches in every stretch, and each probe is a trip to the caches:
+    // nothing is fetched where the next edge already lies beyond the stretch (a short
+    // adjacency misses most stretches), a short rest is stepped through edge by edge, a long
+    // one galloped and bisected.
+    if (my_next < v_hi) {
+      EdgePos_t lo = my_from;
+      if (my_end - my_from <= kShortRest) {
+        do {
+          ++lo;
+          my_next = lo < my_end ? (uint32_t)csr.edges[lo] : 0xFFFFFFFFu;
+        } while (my_next < v_hi);
+      } else {
+        EdgePos_t width = 64;
+        while (lo < my_end) {
+          const EdgePos_t probe = lo + width < my_end ? lo + width : my_end;
+          if ((uint32_t)csr.edges[probe - 1] >= v_hi) break;
+          lo = probe;
+          width <<= 1;
+        }
+        EdgePos_t hi = lo + width < my_end ? lo + width : my_end;
+        while (lo < hi) {
+          const EdgePos_t mid = lo + (hi - lo) / 2;
+          if ((uint32_t)csr.edges[mid] < v_hi) lo = mid + 1; else hi = mid;
+        }
+        my_next = lo < my_end ? (uint32_t)csr.edges[lo] : 0xFFFFFFFFu;
+      }
+      my_reach = lo;
     }
-    EdgePos_t hi = lo + width < my_end ? lo + width : my_end;
-    while (lo < hi) {
-      const EdgePos_t mid = lo + (hi - lo) / 2;
-      if ((uint32_t)csr.edges[mid] < v_lo + kBinVertices) lo = mid + 1; else hi = mid;
+    uint32_t length = (uint32_t)(my_reach - my_from);
+    if (!kWithImportance && my_hub >= 0 && length != 0) {
+      const uint32_t piece = dense.piece_of[(size_t)my_hub * bins_per_sample + bin];
+      if (piece != kNoPiece) {  // these entries reach the stretch as a ready-made bitmap
+        s_piece[atomicAdd(&s_pieces[parity], 1u)] = piece;
+        length = 0;
+      }
     }
-    my_reach = lo;
-    s_length[threadIdx.x] = (uint32_t)(my_reach - my_from);
+    s_length[threadIdx.x] = length;
     s_edge[threadIdx.x] = my_from;  // by transit for now
     if (kWithImportance) s_row_sum[threadIdx.x] = my_row_sum;
   }
   __syncthreads();
+  // the other counter is the next stretch's: the stretch before has been written out
+  if (!kWithImportance && threadIdx.x == 0) s_pieces[parity ^ 1u] = 0;
   // wave 0: drop the empty sub-ranges, turn lengths into starts (the tables are rewritten in
   // place: an entry moves down or stays, and a round only writes below what it has read)
   if (wave == 0) {
@@ -509,14 +569,26 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   } else {
     const uint32_t first_word = bin * kBinWords;
     uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
-    for (uint32_t i = threadIdx.x; i < kBinWords && first_word + i < words_per_sample; i += kBinThreads) {
-      uint32_t word = 0;
+    const uint32_t n_pieces = s_pieces[parity];
+    // two words per lane (stretches and bitmaps hold even numbers of words): eight bytes per
+    // load of a piece, several pieces under way
+    const uint32_t i = 2u * threadIdx.x;
+    if (i < kBinWords && first_word + i < words_per_sample) {
+      uint2 words = make_uint2(0u, 0u);
 #pragma unroll
       for (uint32_t q = 0; q < 8; ++q) {  // 32 bytes, each 0 or 1 -> 32 bits
-        const uint32_t four = s_bits[i * 8u + q];
-        word |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
+        const uint32_t four = s_bits[i * 8u + q], next_four = s_bits[i * 8u + 8u + q];
+        words.x |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
+        words.y |= ((next_four & 1u) | ((next_four >> 7) & 2u) | ((next_four >> 14) & 4u) | ((next_four >> 21) & 8u))
+                   << (4u * q);
       }
-      out[i] = word;
+#pragma unroll 8
+      for (uint32_t p = 0; p < n_pieces; ++p) {
+        const uint2 piece = *(const uint2*)(dense.words + (size_t)s_piece[p] * kBinWords + i);
+        words.x |= piece.x;
+        words.y |= piece.y;
+      }
+      *(uint2*)(out + i) = words;
     }
   }
   __syncthreads();  // the next stretch clears what this one has just read
@@ -968,8 +1040,75 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_row_sums_, sizeof(float) * V));
       ND_HIP_TRY(hipMemcpy(d_row_sums_, sums.data(), sizeof(float) * V, hipMemcpyHostToDevice));
     }
+    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+      const int rc = build_dense_pieces(graph);
+      if (rc != 0) return rc;
+    }
     graph_ = graph;
     return 0;
+  }
+
+  // The stretch bitmaps of the vertices with many edges into one stretch (see DensePieces).
+  int build_dense_pieces(const CSR* graph) {
+    release_dense_pieces();
+    uint32_t threshold = kDensePieceEntries;
+    if (const char* env = getenv("ND_DENSE_PIECE_ENTRIES")) {  // 0: no pieces; small: to exercise them on small graphs
+      const long long v = atoll(env);
+      if (v <= 0) return 0;
+      threshold = (uint32_t)v;
+    }
+    constexpr uint32_t stretch = kBinWordsBits * 32u;
+    const uint32_t V = (uint32_t)graph->get_n_vertices();
+    const uint32_t stretches = (bitmap_words_for(V) + kBinWordsBits - 1) / kBinWordsBits;
+    const size_t most_pieces = kDensePieceBudgetBytes / (sizeof(uint32_t) * kBinWordsBits);
+    std::vector<int32_t> hub_row(V, -1);
+    std::vector<uint32_t> piece_of, words;
+    size_t n_hubs = 0, n_pieces = 0;
+    for (uint32_t v = 0; v < V; ++v) {
+      const int32_t* first = graph->col.data() + graph->row_ptr[v];
+      const int32_t* last = graph->col.data() + graph->row_ptr[v + 1];
+      if ((size_t)(last - first) < threshold) continue;
+      while (first < last) {  // one sub-range of the sorted adjacency per stretch
+        const uint32_t b = (uint32_t)*first / stretch;
+        const uint32_t limit = (b + 1) * stretch;
+        const int32_t* stop = std::partition_point(first, last, [limit](int32_t c) { return (uint32_t)c < limit; });
+        if ((size_t)(stop - first) >= threshold && n_pieces < most_pieces) {
+          if (hub_row[v] < 0) {
+            hub_row[v] = (int32_t)n_hubs++;
+            piece_of.resize(n_hubs * stretches, kNoPiece);
+          }
+          piece_of[(size_t)hub_row[v] * stretches + b] = (uint32_t)n_pieces;
+          words.resize((n_pieces + 1) * kBinWordsBits, 0u);
+          uint32_t* w = words.data() + n_pieces * kBinWordsBits;
+          for (const int32_t* c = first; c < stop; ++c) {
+            const uint32_t local = (uint32_t)*c - b * stretch;
+            w[local >> 5] |= 1u << (local & 31u);
+          }
+          ++n_pieces;
+        }
+        first = stop;
+      }
+    }
+    if (n_pieces == 0) return 0;
+    ND_HIP_TRY(hipMalloc(&d_hub_row_, sizeof(int32_t) * V));
+    ND_HIP_TRY(hipMalloc(&d_piece_of_, sizeof(uint32_t) * piece_of.size()));
+    ND_HIP_TRY(hipMalloc(&d_piece_words_, sizeof(uint32_t) * words.size()));
+    ND_HIP_TRY(hipMemcpy(d_hub_row_, hub_row.data(), sizeof(int32_t) * V, hipMemcpyHostToDevice));
+    ND_HIP_TRY(hipMemcpy(d_piece_of_, piece_of.data(), sizeof(uint32_t) * piece_of.size(), hipMemcpyHostToDevice));
+    ND_HIP_TRY(hipMemcpy(d_piece_words_, words.data(), sizeof(uint32_t) * words.size(), hipMemcpyHostToDevice));
+    dense_.hub_row = d_hub_row_;
+    dense_.piece_of = d_piece_of_;
+    dense_.words = d_piece_words_;
+    dense_pieces_ = n_pieces;
+    return 0;
+  }
+
+  void release_dense_pieces() {
+    release(d_hub_row_);
+    release(d_piece_of_);
+    release(d_piece_words_);
+    dense_ = DensePieces();
+    dense_pieces_ = 0;
   }
 
   int alloc(uint64_t seed) override {
@@ -1023,9 +1162,7 @@ class LayerEngine : public EngineBase {
       if (v > 0) chunk_entries_ = bitmap_chunk_entries_ = (uint64_t)v;
     }
     // one byte per vertex for the LADIES form, one bit for the FastGCN form
-    const uint32_t per_word = 32u;
-    bitmap_words_ = (((uint32_t)invalid_ + per_word - 1u) / per_word + kBitmapTileWords - 1) / kBitmapTileWords *
-                    kBitmapTileWords;
+    bitmap_words_ = bitmap_words_for((uint32_t)invalid_);
     // bytes a sample of a chunk holds: its bitmap (FastGCN form) or one key per vertex, padded
     // to whole stretches (LADIES form)
     uint64_t bytes_per_sample = (uint64_t)bitmap_words_ * sizeof(uint32_t);
@@ -1159,12 +1296,14 @@ class LayerEngine : public EngineBase {
 
   // sizes of the last run, for the algorithmic-bytes figure
   int64_t counter(int which) const override {
-    return which == 0 ? (int64_t)neighborhood_total_ : which == 1 ? (int64_t)distinct_total_ : (int64_t)chunks_run_;
+    return which == 0 ? (int64_t)neighborhood_total_ : which == 1 ? (int64_t)distinct_total_
+           : which == 2 ? (int64_t)chunks_run_ : which == 3 ? (int64_t)dense_pieces_ : 0;
   }
 
   void free_device() override {
     free_run_buffers();
     release(d_row_sums_);
+    release_dense_pieces();
     dgraph_.release();
     graph_ = nullptr;
   }
@@ -1286,7 +1425,7 @@ class LayerEngine : public EngineBase {
     }
     tick();
     collective_mark_binned<false><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u);
+        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u, dense_);
     tock();
     ND_HIP_TRY(hipMemsetAsync(d_marked_, 0, sizeof(uint32_t) * (size_t)n, stream_));
     const uint32_t sample_blocks = (n + kSumSamplesPerBlock - 1) / kSumSamplesPerBlock;
@@ -1315,7 +1454,7 @@ class LayerEngine : public EngineBase {
     }
     tick();
     collective_mark_binned<true><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample);
+        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, DensePieces());
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
     const dim3 tiles(tiles_per_sample, n);
@@ -1445,6 +1584,11 @@ class LayerEngine : public EngineBase {
   const CSR* graph_ = nullptr;
   DeviceGraph dgraph_;
   float* d_row_sums_ = nullptr;
+  int32_t* d_hub_row_ = nullptr;       // dense pieces of the graph (FastGCN form)
+  uint32_t* d_piece_of_ = nullptr;
+  uint32_t* d_piece_words_ = nullptr;
+  DensePieces dense_;
+  size_t dense_pieces_ = 0;
   std::vector<SampleType> samples_;
   std::vector<uint32_t> h_sizes_;
   int64_t n_samples_ = 0;

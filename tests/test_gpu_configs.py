@@ -130,7 +130,9 @@ def test_config4_fastgcn_importance_rmat22(oracle, monkeypatch):
     og = graphs.oracle_view(g)
     d = desc_of(oracle, s, oracle.FASTGCN_IMPORTANCE)
     compare_ranges(oracle.sample_fastgcn_importance, d, og, s, got, 48)
-    print("config 4: neighbourhood entries", s.counter(0), "distinct", s.counter(1), flush=True)
+    print("config 4: neighbourhood entries", s.counter(0), "distinct", s.counter(1), "hub bitmaps", s.counter(3),
+          flush=True)
+    assert s.counter(3) > 0  # the hubs of this graph go through the ready-made bitmaps
     s.close()
 
 
