@@ -300,6 +300,73 @@ inline uint32_t bitmap_words_for(uint32_t n_vertices) {
   return ((n_vertices + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
 }
 
+// First edge of the sorted adjacency [from, end) whose destination is >= v_hi, given that the
+// destination of `from` is below it; *next = that edge's destination (0xFFFFFFFF: none left).
+// A workgroup waits for the slowest of these searches and each probe is a trip to the caches:
+// a short rest is stepped through edge by edge, a long one galloped and bisected.
+__device__ __forceinline__ EdgePos_t first_edge_at_or_above(const VertexID* __restrict__ edges, EdgePos_t from,
+                                                            EdgePos_t end, uint32_t v_hi, uint32_t* next) {
+  EdgePos_t lo = from;
+  if (end - from <= kShortRest) {
+    uint32_t dst;
+    do {
+      ++lo;
+      dst = lo < end ? (uint32_t)edges[lo] : 0xFFFFFFFFu;
+    } while (dst < v_hi);
+    *next = dst;
+    return lo;
+  }
+  EdgePos_t width = 64;
+  while (lo < end) {
+    const EdgePos_t probe = lo + width < end ? lo + width : end;
+    if ((uint32_t)edges[probe - 1] >= v_hi) break;
+    lo = probe;
+    width <<= 1;
+  }
+  EdgePos_t hi = lo + width < end ? lo + width : end;
+  while (lo < hi) {
+    const EdgePos_t mid = lo + (hi - lo) / 2;
+    if ((uint32_t)edges[mid] < v_hi) lo = mid + 1; else hi = mid;
+  }
+  *next = lo < end ? (uint32_t)edges[lo] : 0xFFFFFFFFu;
+  return lo;
+}
+
+// One wavefront: drops the empty sub-ranges of the per-transit tables (length, first edge,
+// row sum) and turns lengths into starts: starts[k] = first entry of kept sub-range k,
+// starts[kept] = all entries; *ranges = kept.  The tables are rewritten in place: an entry
+// moves down or stays, and a round only writes below what it has read.
+template <bool kWithImportance>
+__device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint32_t lane, const uint32_t* lengths,
+                                                      EdgePos_t* edge, float* row_sum, uint32_t* starts,
+                                                      uint32_t* ranges) {
+  uint32_t kept = 0, entries = 0;
+  for (uint32_t c = 0; c < n_transits; c += 64) {
+    const uint32_t i = c + lane;
+    const uint32_t len = i < n_transits ? lengths[i] : 0u;
+    const EdgePos_t first = i < n_transits ? edge[i] : 0;
+    const float sum = kWithImportance && i < n_transits ? row_sum[i] : 1.0f;
+    const uint64_t holds = __ballot(len != 0);
+    const uint32_t through = wave_inclusive_scan(len);
+    if (len != 0) {
+      const uint32_t k = kept + (uint32_t)__popcll(holds & ((1ull << lane) - 1ull));
+      starts[k] = entries + through - len;
+      edge[k] = first;
+      if (kWithImportance) row_sum[k] = sum;
+    }
+    kept += (uint32_t)__popcll(holds);
+    entries += __shfl(through, 63, kWave);
+  }
+  if (lane == 0) {
+    starts[kept] = entries;
+    *ranges = kept;
+  }
+}
+
+// A sample without hubs among its transits and with at most this many entries in a
+// workgroup's stretches (a layer whose transits are drawn uniformly) marks them all at once.
+constexpr uint32_t kSparseGroupEntries = 32768;
+
 template <bool kWithImportance>
 __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
@@ -310,7 +377,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   constexpr uint32_t kBinVertices = kBinWords * 32u;
   // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
   // packed into bits on the way out; LADIES form: bits and 64-bit sums, LDS atomics
-  __shared__ uint32_t s_bits[kWithImportance ? kBinWords : kBinVertices / 4u];
+  __shared__ __align__(16) uint32_t s_bits[kWithImportance ? kBinWords : kBinVertices / 4u];
   __shared__ unsigned long long s_acc[kWithImportance ? kBinVerticesSums : 1];
   uint8_t* s_bytes = (uint8_t*)s_bits;
   // the sub-ranges that hold entries, in transit order
@@ -338,14 +405,23 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   uint32_t my_next = 0xFFFFFFFFu;  // destination of edge my_reach; none left: above every vertex
   float my_row_sum = 1.0f;
   int32_t my_hub = -1;
+  int32_t my_transit = -1;
+  if (threadIdx.x < tv.count) {
+    my_transit = transits[threadIdx.x];
+    if (my_transit == invalid) my_transit = -1;
+    if (!kWithImportance && my_transit != -1 && dense.hub_row) my_hub = dense.hub_row[my_transit];
+  }
+  bool hubs_among_transits = false;
   if (!kWithImportance) {
+    // the byte map starts out clear and every stretch leaves it clear: what it reads on the
+    // way out it sets back to zero, so no stretch spends a pass on clearing
+    for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
     if (threadIdx.x < 2) s_pieces[threadIdx.x] = 0;
-    __syncthreads();
+    hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
   }
   if (threadIdx.x < tv.count) {
-    const int32_t t = transits[threadIdx.x];
-    if (t != invalid && t != -1) {
-      if (!kWithImportance && dense.hub_row) my_hub = dense.hub_row[t];
+    const int32_t t = my_transit;
+    if (t != -1) {
       my_end = csr.row_ptr[t + 1];
       EdgePos_t lo = csr.row_ptr[t], hi = my_end;  // first edge whose destination is in the first stretch or above
       const uint32_t v_first = first_bin * kBinVertices;
@@ -358,44 +434,58 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
       if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
   }
+  if (!kWithImportance && !hubs_among_transits) {
+    // The stretches of the workgroup as one: a bit per vertex fits the same LDS, and the few
+    // entries can afford LDS atomics.  Per stretch, the searches, the table and the way out
+    // are chains of dependent trips (to the caches, to LDS, through barriers) that cost the
+    // same however few entries there are: 3.5 ms a layer at full size for 2 K entries a sample.
+    const uint32_t group_bins = first_bin + kBinsPerGroup < bins_per_sample ? kBinsPerGroup : bins_per_sample - first_bin;
+    const uint32_t v_lo = first_bin * kBinVertices, v_hi = v_lo + group_bins * kBinVertices;
+    if (threadIdx.x < tv.count) {
+      uint32_t unused;
+      const EdgePos_t stop =
+          my_next < v_hi ? first_edge_at_or_above(csr.edges, my_reach, my_end, v_hi, &unused) : my_reach;
+      s_length[threadIdx.x] = (uint32_t)(stop - my_reach);
+      s_edge[threadIdx.x] = my_reach;
+    }
+    __syncthreads();
+    if (wave == 0) keep_filled_subranges<false>(tv.count, lane, s_length, s_edge, nullptr, s_start, &s_ranges);
+    __syncthreads();
+    const uint32_t ranges = s_ranges;
+    const uint32_t size = s_start[ranges];
+    if (size <= kSparseGroupEntries) {
+      for (uint32_t e = threadIdx.x; e < size; e += kBinThreads) {
+        uint32_t lo = 0, hi = ranges;  // the sub-range that holds entry e
+        while (hi - lo > 1) {
+          const uint32_t mid = lo + (hi - lo) / 2;
+          if (s_start[mid] <= e) lo = mid; else hi = mid;
+        }
+        const uint32_t local = (uint32_t)csr.edges[s_edge[lo] + (EdgePos_t)(e - s_start[lo])] - v_lo;
+        atomicOr(&s_bits[local >> 5], 1u << (local & 31u));
+      }
+      __syncthreads();
+      const uint32_t first_word = first_bin * kBinWords;
+      uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
+      for (uint32_t i = threadIdx.x; i < group_bins * kBinWords && first_word + i < words_per_sample; i += kBinThreads)
+        out[i] = s_bits[i];
+      return;
+    }
+    // too many entries for that: stretch by stretch (nothing has been marked, and the tables
+    // are next written after every lane has read the size above)
+  }
   for (uint32_t bin = first_bin; bin < first_bin + kBinsPerGroup && bin < bins_per_sample; ++bin) {
   const uint32_t v_lo = bin * kBinVertices;
   const uint32_t parity = (bin - first_bin) & 1u;
-  for (uint32_t i = threadIdx.x; i < (kWithImportance ? kBinWords : kBinVertices / 4u); i += kBinThreads) s_bits[i] = 0;
-  if (kWithImportance)
+  if (kWithImportance) {
+    for (uint32_t i = threadIdx.x; i < kBinWords; i += kBinThreads) s_bits[i] = 0;
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
+  }
   if (threadIdx.x < tv.count) {
     const EdgePos_t my_from = my_reach;
     const uint32_t v_hi = v_lo + kBinVertices;
-    // first edge at or after my_from whose destination is >= v_hi.  The workgroup waits for
-    // the slowest of these searches in every stretch, and each probe is a trip to the caches:
     // nothing is fetched where the next edge already lies beyond the stretch (a short
-    // adjacency misses most stretches), a short rest is stepped through edge by edge, a long
-    // one galloped and bisected.
-    if (my_next < v_hi) {
-      EdgePos_t lo = my_from;
-      if (my_end - my_from <= kShortRest) {
-        do {
-          ++lo;
-          my_next = lo < my_end ? (uint32_t)csr.edges[lo] : 0xFFFFFFFFu;
-        } while (my_next < v_hi);
-      } else {
-        EdgePos_t width = 64;
-        while (lo < my_end) {
-          const EdgePos_t probe = lo + width < my_end ? lo + width : my_end;
-          if ((uint32_t)csr.edges[probe - 1] >= v_hi) break;
-          lo = probe;
-          width <<= 1;
-        }
-        EdgePos_t hi = lo + width < my_end ? lo + width : my_end;
-        while (lo < hi) {
-          const EdgePos_t mid = lo + (hi - lo) / 2;
-          if ((uint32_t)csr.edges[mid] < v_hi) lo = mid + 1; else hi = mid;
-        }
-        my_next = lo < my_end ? (uint32_t)csr.edges[lo] : 0xFFFFFFFFu;
-      }
-      my_reach = lo;
-    }
+    // adjacency misses most stretches)
+    if (my_next < v_hi) my_reach = first_edge_at_or_above(csr.edges, my_from, my_end, v_hi, &my_next);
     uint32_t length = (uint32_t)(my_reach - my_from);
     if (!kWithImportance && my_hub >= 0 && length != 0) {
       const uint32_t piece = dense.piece_of[(size_t)my_hub * bins_per_sample + bin];
@@ -411,31 +501,8 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __syncthreads();
   // the other counter is the next stretch's: the stretch before has been written out
   if (!kWithImportance && threadIdx.x == 0) s_pieces[parity ^ 1u] = 0;
-  // wave 0: drop the empty sub-ranges, turn lengths into starts (the tables are rewritten in
-  // place: an entry moves down or stays, and a round only writes below what it has read)
-  if (wave == 0) {
-    uint32_t kept = 0, entries = 0;
-    for (uint32_t c = 0; c < tv.count; c += 64) {
-      const uint32_t i = c + lane;
-      const uint32_t len = i < tv.count ? s_length[i] : 0u;
-      const EdgePos_t edge = i < tv.count ? s_edge[i] : 0;
-      const float row_sum = kWithImportance && i < tv.count ? s_row_sum[i] : 1.0f;
-      const uint64_t holds = __ballot(len != 0);
-      const uint32_t through = wave_inclusive_scan(len);
-      if (len != 0) {
-        const uint32_t k = kept + (uint32_t)__popcll(holds & ((1ull << lane) - 1ull));
-        s_start[k] = entries + through - len;
-        s_edge[k] = edge;
-        if (kWithImportance) s_row_sum[k] = row_sum;
-      }
-      kept += (uint32_t)__popcll(holds);
-      entries += __shfl(through, 63, kWave);
-    }
-    if (lane == 0) {
-      s_start[kept] = entries;
-      s_ranges = kept;
-    }
-  }
+  if (wave == 0)
+    keep_filled_subranges<kWithImportance>(tv.count, lane, s_length, s_edge, s_row_sum, s_start, &s_ranges);
   __syncthreads();
   const uint32_t ranges = s_ranges;
   const uint32_t size = s_start[ranges];
@@ -575,12 +642,23 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     const uint32_t i = 2u * threadIdx.x;
     if (i < kBinWords && first_word + i < words_per_sample) {
       uint2 words = make_uint2(0u, 0u);
+      if (size != 0) {  // 2 x 32 bytes, each 0 or 1 -> 2 x 32 bits
+        uint4* bytes = (uint4*)s_bits + i * 2u;
+        const uint4 q0 = bytes[0], q1 = bytes[1], q2 = bytes[2], q3 = bytes[3];
+        const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+        bytes[0] = zero;
+        bytes[1] = zero;
+        bytes[2] = zero;
+        bytes[3] = zero;
+        const uint32_t low[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const uint32_t high[8] = {q2.x, q2.y, q2.z, q2.w, q3.x, q3.y, q3.z, q3.w};
 #pragma unroll
-      for (uint32_t q = 0; q < 8; ++q) {  // 32 bytes, each 0 or 1 -> 32 bits
-        const uint32_t four = s_bits[i * 8u + q], next_four = s_bits[i * 8u + 8u + q];
-        words.x |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
-        words.y |= ((next_four & 1u) | ((next_four >> 7) & 2u) | ((next_four >> 14) & 4u) | ((next_four >> 21) & 8u))
-                   << (4u * q);
+        for (uint32_t q = 0; q < 8; ++q) {
+          const uint32_t four = low[q], next_four = high[q];
+          words.x |= ((four & 1u) | ((four >> 7) & 2u) | ((four >> 14) & 4u) | ((four >> 21) & 8u)) << (4u * q);
+          words.y |= ((next_four & 1u) | ((next_four >> 7) & 2u) | ((next_four >> 14) & 4u) | ((next_four >> 21) & 8u))
+                     << (4u * q);
+        }
       }
 #pragma unroll 8
       for (uint32_t p = 0; p < n_pieces; ++p) {
