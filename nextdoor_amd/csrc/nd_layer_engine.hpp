@@ -287,12 +287,14 @@ constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit su
 // of marking the entries one by one.  hub_row[v] = row of v in piece_of or -1;
 // piece_of[row * stretches + stretch] = piece index or kNoPiece.
 constexpr uint32_t kDensePieceEntries = 512;
+constexpr uint32_t kDensePieceEntriesSums = 4096;  // LADIES form: a piece is 6144 64-bit sums
 constexpr size_t kDensePieceBudgetBytes = (size_t)2 << 30;
 constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
 struct DensePieces {
   const int32_t* hub_row = nullptr;  // nullptr: the graph has none
   const uint32_t* piece_of = nullptr;
-  const uint32_t* words = nullptr;
+  const uint32_t* words = nullptr;            // FastGCN form: 1536 words of bits per piece
+  const unsigned long long* sums = nullptr;  // LADIES form: 6144 importance sums per piece (kAbsentSum: no edge)
 };
 
 // 32-bit words of one sample's presence map: a bit per vertex, padded to whole tiles.
@@ -386,7 +388,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // 1 / (the weights of its transit added up)
   __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
   __shared__ uint32_t s_ranges;                        // sub-ranges kept
-  __shared__ uint32_t s_piece[kWithImportance ? 1 : kMaxLayerTransits];  // dense pieces of the stretch
+  __shared__ uint32_t s_piece[kMaxLayerTransits];      // dense pieces of the stretch
   __shared__ uint32_t s_pieces[2];                     // how many; stretches alternate between the two counters
   // A workgroup takes kBinsPerGroup consecutive stretches of one sample, one after the other:
   // where a transit's sub-range ends in one stretch it begins in the next, and the end is
@@ -409,10 +411,13 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   if (threadIdx.x < tv.count) {
     my_transit = transits[threadIdx.x];
     if (my_transit == invalid) my_transit = -1;
-    if (!kWithImportance && my_transit != -1 && dense.hub_row) my_hub = dense.hub_row[my_transit];
+    if (my_transit != -1 && dense.hub_row) my_hub = dense.hub_row[my_transit];
   }
   bool hubs_among_transits = false;
-  if (!kWithImportance) {
+  if (kWithImportance) {
+    if (threadIdx.x < 2) s_pieces[threadIdx.x] = 0;
+    __syncthreads();
+  } else {
     // the byte map starts out clear and every stretch leaves it clear: what it reads on the
     // way out it sets back to zero, so no stretch spends a pass on clearing
     for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     // adjacency misses most stretches)
     if (my_next < v_hi) my_reach = first_edge_at_or_above(csr.edges, my_from, my_end, v_hi, &my_next);
     uint32_t length = (uint32_t)(my_reach - my_from);
-    if (!kWithImportance && my_hub >= 0 && length != 0) {
+    if (my_hub >= 0 && length != 0) {
       const uint32_t piece = dense.piece_of[(size_t)my_hub * bins_per_sample + bin];
       if (piece != kNoPiece) {  // these entries reach the stretch as a ready-made bitmap
         s_piece[atomicAdd(&s_pieces[parity], 1u)] = piece;
@@ -500,7 +505,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   }
   __syncthreads();
   // the other counter is the next stretch's: the stretch before has been written out
-  if (!kWithImportance && threadIdx.x == 0) s_pieces[parity ^ 1u] = 0;
+  if (threadIdx.x == 0) s_pieces[parity ^ 1u] = 0;
   if (wave == 0)
     keep_filled_subranges<kWithImportance>(tv.count, lane, s_length, s_edge, s_row_sum, s_start, &s_ranges);
   __syncthreads();
@@ -631,8 +636,20 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     // streaming of the other workgroup of the compute unit, the same arithmetic took 100 ms
     // instead of 13.)
     unsigned long long* out = sums + (size_t)s * keys_per_sample + v_lo;
-    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads)
-      __builtin_nontemporal_store(((s_bits[i >> 5] >> (i & 31u)) & 1u) ? s_acc[i] : kAbsentSum, &out[i]);
+    const uint32_t n_pieces = s_pieces[parity];
+    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) {
+      bool present = ((s_bits[i >> 5] >> (i & 31u)) & 1u) != 0;
+      unsigned long long sum = s_acc[i];  // 0 where nothing was added
+#pragma unroll 4
+      for (uint32_t p = 0; p < n_pieces; ++p) {  // integer sums: the order of the additions does not matter
+        const unsigned long long ready = dense.sums[(size_t)s_piece[p] * kBinVerticesSums + i];
+        if (ready != kAbsentSum) {
+          sum += ready;
+          present = true;
+        }
+      }
+      __builtin_nontemporal_store(present ? sum : kAbsentSum, &out[i]);
+    }
   } else {
     const uint32_t first_word = bin * kBinWords;
     uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
@@ -1117,33 +1134,41 @@ class LayerEngine : public EngineBase {
       }
       ND_HIP_TRY(hipMalloc(&d_row_sums_, sizeof(float) * V));
       ND_HIP_TRY(hipMemcpy(d_row_sums_, sums.data(), sizeof(float) * V, hipMemcpyHostToDevice));
+      const int rc = build_dense_pieces(graph, sums.data());
+      if (rc != 0) return rc;
     }
     if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
-      const int rc = build_dense_pieces(graph);
+      const int rc = build_dense_pieces(graph, nullptr);
       if (rc != 0) return rc;
     }
     graph_ = graph;
     return 0;
   }
 
-  // The stretch bitmaps of the vertices with many edges into one stretch (see DensePieces).
-  int build_dense_pieces(const CSR* graph) {
+  // What the vertices with many edges into one stretch contribute to it, built once per graph
+  // (see DensePieces).  inverse_row_sums: the LADIES form's 1 / rowsum per vertex, else nullptr.
+  int build_dense_pieces(const CSR* graph, const float* inverse_row_sums) {
     release_dense_pieces();
-    uint32_t threshold = kDensePieceEntries;
+    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
+    uint32_t threshold = ladies ? kDensePieceEntriesSums : kDensePieceEntries;
     if (const char* env = getenv("ND_DENSE_PIECE_ENTRIES")) {  // 0: no pieces; small: to exercise them on small graphs
       const long long v = atoll(env);
       if (v <= 0) return 0;
       threshold = (uint32_t)v;
     }
-    constexpr uint32_t stretch = kBinWordsBits * 32u;
+    constexpr uint32_t stretch_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
+    constexpr uint32_t stretch = stretch_words * 32u;
+    // a piece: a bit per vertex of the stretch, or a 64-bit importance sum (kAbsentSum: no edge)
+    constexpr size_t piece_words = ladies ? (size_t)stretch * 2u : (size_t)stretch_words;
     const uint32_t V = (uint32_t)graph->get_n_vertices();
-    const uint32_t stretches = (bitmap_words_for(V) + kBinWordsBits - 1) / kBinWordsBits;
-    const size_t most_pieces = kDensePieceBudgetBytes / (sizeof(uint32_t) * kBinWordsBits);
+    const uint32_t stretches = (bitmap_words_for(V) + stretch_words - 1) / stretch_words;
+    const size_t most_pieces = kDensePieceBudgetBytes / (sizeof(uint32_t) * piece_words);
     std::vector<int32_t> hub_row(V, -1);
     std::vector<uint32_t> piece_of, words;
     size_t n_hubs = 0, n_pieces = 0;
     for (uint32_t v = 0; v < V; ++v) {
-      const int32_t* first = graph->col.data() + graph->row_ptr[v];
+      const int32_t* const row = graph->col.data() + graph->row_ptr[v];
+      const int32_t* first = row;
       const int32_t* last = graph->col.data() + graph->row_ptr[v + 1];
       if ((size_t)(last - first) < threshold) continue;
       while (first < last) {  // one sub-range of the sorted adjacency per stretch
@@ -1156,11 +1181,21 @@ class LayerEngine : public EngineBase {
             piece_of.resize(n_hubs * stretches, kNoPiece);
           }
           piece_of[(size_t)hub_row[v] * stretches + b] = (uint32_t)n_pieces;
-          words.resize((n_pieces + 1) * kBinWordsBits, 0u);
-          uint32_t* w = words.data() + n_pieces * kBinWordsBits;
+          words.resize((n_pieces + 1) * piece_words, ladies ? 0xFFFFFFFFu : 0u);
+          uint32_t* w = words.data() + n_pieces * piece_words;
           for (const int32_t* c = first; c < stop; ++c) {
             const uint32_t local = (uint32_t)*c - b * stretch;
-            w[local >> 5] |= 1u << (local & 31u);
+            if (ladies) {
+              // the term the marking kernel adds for this edge, in the same arithmetic
+              const float p = graph->weight[(size_t)graph->row_ptr[v] + (size_t)(c - row)] * inverse_row_sums[v];
+              unsigned long long sum;
+              memcpy(&sum, w + 2u * local, sizeof(sum));
+              if (sum == kAbsentSum) sum = 0;
+              sum += importance_term_fixed(p * p);
+              memcpy(w + 2u * local, &sum, sizeof(sum));
+            } else {
+              w[local >> 5] |= 1u << (local & 31u);
+            }
           }
           ++n_pieces;
         }
@@ -1177,6 +1212,7 @@ class LayerEngine : public EngineBase {
     dense_.hub_row = d_hub_row_;
     dense_.piece_of = d_piece_of_;
     dense_.words = d_piece_words_;
+    dense_.sums = (const unsigned long long*)d_piece_words_;
     dense_pieces_ = n_pieces;
     return 0;
   }
@@ -1532,7 +1568,7 @@ class LayerEngine : public EngineBase {
     }
     tick();
     collective_mark_binned<true><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, DensePieces());
+        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, dense_);
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
     const dim3 tiles(tiles_per_sample, n);

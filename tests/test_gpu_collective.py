@@ -96,17 +96,21 @@ def test_fastgcn_importance_matches_oracle(oracle, app, gname):
     s.close()
 
 
-@pytest.mark.parametrize("app", ["FastGCNImportance2x8", "FastGCNImportance3x16"])
-def test_fastgcn_importance_with_ready_made_hub_bitmaps(oracle, app, monkeypatch):
-    """Vertices with many edges into one stretch of the vertex range contribute a bitmap built
-    once per graph instead of their entries: same samples, with or without."""
+@pytest.mark.parametrize("app", ["FastGCNImportance2x8", "FastGCNImportance3x16", "LADIESImportance2x8",
+                                 "LADIESImportance3x16"])
+def test_importance_sampling_with_ready_made_hub_pieces(oracle, app, monkeypatch):
+    """Vertices with many edges into one stretch of the vertex range contribute a piece built
+    once per graph (a bitmap, or the importance sums) instead of their entries: same samples,
+    with or without."""
     g = graphs.random_graph(n=2000, mean_degree=12, seed=2, hub=5)
     og = graphs.oracle_view(g)
     monkeypatch.setenv("ND_DENSE_PIECE_ENTRIES", "0")
     s = nd.Sampler(app, g, seed=SEED)
     assert s.counter(3) == 0
-    d = layer_desc(oracle, s, oracle.FASTGCN_IMPORTANCE)
-    want = oracle.sample_fastgcn_importance(og, d, SEED, s.initial_contents)
+    ladies = app.startswith("LADIES")
+    d = layer_desc(oracle, s, oracle.LADIES_IMPORTANCE if ladies else oracle.FASTGCN_IMPORTANCE)
+    want = (oracle.sample_ladies_importance if ladies else oracle.sample_fastgcn_importance)(
+        og, d, SEED, s.initial_contents)
     s.do_transit_parallel(True)
     assert np.array_equal(s.final_samples(), want)
     s.close()

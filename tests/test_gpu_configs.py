@@ -145,7 +145,9 @@ def test_config5_ladies_importance_chung_lu(oracle, monkeypatch):
     print("config 5: sampling", flush=True)
     s.do_transit_parallel(True)
     got = s.final_samples()
-    print("config 5: neighbourhood entries", s.counter(0), "distinct", s.counter(1), "chunks", s.counter(2), flush=True)
+    print("config 5: neighbourhood entries", s.counter(0), "distinct", s.counter(1), "chunks", s.counter(2),
+          "hub pieces", s.counter(3), flush=True)
+    assert s.counter(3) > 0  # the hubs of this graph contribute ready-made importance sums
     og = graphs.oracle_view(g)
     d = desc_of(oracle, s, oracle.LADIES_IMPORTANCE)
     print("config 5: oracle ranges", flush=True)
