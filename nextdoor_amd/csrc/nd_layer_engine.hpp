@@ -336,32 +336,42 @@ __device__ __forceinline__ EdgePos_t first_edge_at_or_above(const VertexID* __re
 
 // One wavefront: drops the empty sub-ranges of the per-transit tables (length, first edge,
 // row sum) and turns lengths into starts: starts[k] = first entry of kept sub-range k,
-// starts[kept] = all entries; *ranges = kept.  The tables are rewritten in place: an entry
-// moves down or stays, and a round only writes below what it has read.
+// starts[kept] = all entries; *ranges = kept.  A length with kPieceFlag set stands for a
+// transit whose entries reach the stretch as a ready-made piece: no sub-range, and the piece
+// index joins the list that takes the place of the lengths, *pieces = how many.  The tables
+// are rewritten in place: an entry moves down or stays, and a round only writes below what it
+// has read.
+constexpr uint32_t kPieceFlag = 0x80000000u;
 template <bool kWithImportance>
-__device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint32_t lane, const uint32_t* lengths,
+__device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint32_t lane, uint32_t* lengths,
                                                       EdgePos_t* edge, float* row_sum, uint32_t* starts,
-                                                      uint32_t* ranges) {
-  uint32_t kept = 0, entries = 0;
+                                                      uint32_t* ranges, uint32_t* pieces) {
+  uint32_t kept = 0, entries = 0, listed = 0;
   for (uint32_t c = 0; c < n_transits; c += 64) {
     const uint32_t i = c + lane;
-    const uint32_t len = i < n_transits ? lengths[i] : 0u;
+    const uint32_t raw = i < n_transits ? lengths[i] : 0u;
+    const bool is_piece = (raw & kPieceFlag) != 0;
+    const uint32_t len = is_piece ? 0u : raw;
     const EdgePos_t first = i < n_transits ? edge[i] : 0;
     const float sum = kWithImportance && i < n_transits ? row_sum[i] : 1.0f;
-    const uint64_t holds = __ballot(len != 0);
+    const uint64_t holds = __ballot(len != 0), ready = __ballot(is_piece);
+    const uint64_t below = (1ull << lane) - 1ull;
     const uint32_t through = wave_inclusive_scan(len);
     if (len != 0) {
-      const uint32_t k = kept + (uint32_t)__popcll(holds & ((1ull << lane) - 1ull));
+      const uint32_t k = kept + (uint32_t)__popcll(holds & below);
       starts[k] = entries + through - len;
       edge[k] = first;
       if (kWithImportance) row_sum[k] = sum;
     }
+    if (is_piece) lengths[listed + (uint32_t)__popcll(ready & below)] = raw & ~kPieceFlag;
     kept += (uint32_t)__popcll(holds);
+    listed += (uint32_t)__popcll(ready);
     entries += __shfl(through, 63, kWave);
   }
   if (lane == 0) {
     starts[kept] = entries;
     *ranges = kept;
+    *pieces = listed;
   }
 }
 
@@ -369,8 +379,11 @@ __device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint3
 // workgroup's stretches (a layer whose transits are drawn uniformly) marks them all at once.
 constexpr uint32_t kSparseGroupEntries = 32768;
 
+// Two workgroups share a compute unit (8 wavefronts per SIMD): at most 64 registers per lane
+// and (measured) 66 KB of LDS per workgroup - with 70 KB only one workgroup is resident and
+// the LADIES form takes 1.6 times as long.
 template <bool kWithImportance>
-__global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
+__global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
@@ -386,10 +399,9 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // first entry of sub-range k among the stretch's entries
   __shared__ EdgePos_t s_edge[kMaxLayerTransits];      // its first edge
   __shared__ float s_row_sum[kWithImportance ? kMaxLayerTransits : 1];  // 1 / (the weights of its transit added up)
-  __shared__ uint32_t s_length[kMaxLayerTransits];     // scratch: length of every transit's sub-range
+  __shared__ uint32_t s_length[kMaxLayerTransits];     // length of every transit's sub-range, then the stretch's dense pieces
   __shared__ uint32_t s_ranges;                        // sub-ranges kept
-  __shared__ uint32_t s_piece[kMaxLayerTransits];      // dense pieces of the stretch
-  __shared__ uint32_t s_pieces[2];                     // how many; stretches alternate between the two counters
+  __shared__ uint32_t s_pieces;                        // dense pieces listed
   // A workgroup takes kBinsPerGroup consecutive stretches of one sample, one after the other:
   // where a transit's sub-range ends in one stretch it begins in the next, and the end is
   // then only a short gallop away instead of a search of the whole adjacency.
@@ -414,14 +426,10 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     if (my_transit != -1 && dense.hub_row) my_hub = dense.hub_row[my_transit];
   }
   bool hubs_among_transits = false;
-  if (kWithImportance) {
-    if (threadIdx.x < 2) s_pieces[threadIdx.x] = 0;
-    __syncthreads();
-  } else {
+  if (!kWithImportance) {
     // the byte map starts out clear and every stretch leaves it clear: what it reads on the
     // way out it sets back to zero, so no stretch spends a pass on clearing
     for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
-    if (threadIdx.x < 2) s_pieces[threadIdx.x] = 0;
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
   }
   if (threadIdx.x < tv.count) {
@@ -454,7 +462,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
       s_edge[threadIdx.x] = my_reach;
     }
     __syncthreads();
-    if (wave == 0) keep_filled_subranges<false>(tv.count, lane, s_length, s_edge, nullptr, s_start, &s_ranges);
+    if (wave == 0) keep_filled_subranges<false>(tv.count, lane, s_length, s_edge, nullptr, s_start, &s_ranges, &s_pieces);
     __syncthreads();
     const uint32_t ranges = s_ranges;
     const uint32_t size = s_start[ranges];
@@ -480,7 +488,6 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   }
   for (uint32_t bin = first_bin; bin < first_bin + kBinsPerGroup && bin < bins_per_sample; ++bin) {
   const uint32_t v_lo = bin * kBinVertices;
-  const uint32_t parity = (bin - first_bin) & 1u;
   if (kWithImportance) {
     for (uint32_t i = threadIdx.x; i < kBinWords; i += kBinThreads) s_bits[i] = 0;
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) s_acc[i] = 0;
@@ -494,20 +501,15 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     uint32_t length = (uint32_t)(my_reach - my_from);
     if (my_hub >= 0 && length != 0) {
       const uint32_t piece = dense.piece_of[(size_t)my_hub * bins_per_sample + bin];
-      if (piece != kNoPiece) {  // these entries reach the stretch as a ready-made bitmap
-        s_piece[atomicAdd(&s_pieces[parity], 1u)] = piece;
-        length = 0;
-      }
+      if (piece != kNoPiece) length = kPieceFlag | piece;  // these entries reach the stretch ready-made
     }
     s_length[threadIdx.x] = length;
     s_edge[threadIdx.x] = my_from;  // by transit for now
     if (kWithImportance) s_row_sum[threadIdx.x] = my_row_sum;
   }
   __syncthreads();
-  // the other counter is the next stretch's: the stretch before has been written out
-  if (threadIdx.x == 0) s_pieces[parity ^ 1u] = 0;
   if (wave == 0)
-    keep_filled_subranges<kWithImportance>(tv.count, lane, s_length, s_edge, s_row_sum, s_start, &s_ranges);
+    keep_filled_subranges<kWithImportance>(tv.count, lane, s_length, s_edge, s_row_sum, s_start, &s_ranges, &s_pieces);
   __syncthreads();
   const uint32_t ranges = s_ranges;
   const uint32_t size = s_start[ranges];
@@ -636,13 +638,13 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
     // streaming of the other workgroup of the compute unit, the same arithmetic took 100 ms
     // instead of 13.)
     unsigned long long* out = sums + (size_t)s * keys_per_sample + v_lo;
-    const uint32_t n_pieces = s_pieces[parity];
+    const uint32_t n_pieces = s_pieces;
     for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) {
       bool present = ((s_bits[i >> 5] >> (i & 31u)) & 1u) != 0;
       unsigned long long sum = s_acc[i];  // 0 where nothing was added
 #pragma unroll 4
       for (uint32_t p = 0; p < n_pieces; ++p) {  // integer sums: the order of the additions does not matter
-        const unsigned long long ready = dense.sums[(size_t)s_piece[p] * kBinVerticesSums + i];
+        const unsigned long long ready = dense.sums[(size_t)s_length[p] * kBinVerticesSums + i];
         if (ready != kAbsentSum) {
           sum += ready;
           present = true;
@@ -653,7 +655,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
   } else {
     const uint32_t first_word = bin * kBinWords;
     uint32_t* out = bitmap + (size_t)s * words_per_sample + first_word;
-    const uint32_t n_pieces = s_pieces[parity];
+    const uint32_t n_pieces = s_pieces;
     // two words per lane (stretches and bitmaps hold even numbers of words): eight bytes per
     // load of a piece, several pieces under way
     const uint32_t i = 2u * threadIdx.x;
@@ -679,7 +681,7 @@ __global__ __launch_bounds__(kBinThreads) void collective_mark_binned(
       }
 #pragma unroll 8
       for (uint32_t p = 0; p < n_pieces; ++p) {
-        const uint2 piece = *(const uint2*)(dense.words + (size_t)s_piece[p] * kBinWords + i);
+        const uint2 piece = *(const uint2*)(dense.words + (size_t)s_length[p] * kBinWords + i);
         words.x |= piece.x;
         words.y |= piece.y;
       }
