@@ -287,7 +287,7 @@ constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit su
 // of marking the entries one by one.  hub_row[v] = row of v in piece_of or -1;
 // piece_of[row * stretches + stretch] = piece index or kNoPiece.
 constexpr uint32_t kDensePieceEntries = 512;
-constexpr uint32_t kDensePieceEntriesSums = 4096;  // LADIES form: a piece is 6144 64-bit sums
+constexpr uint32_t kDensePieceEntriesSums = 2048;  // LADIES form: a piece is 6144 64-bit sums
 constexpr size_t kDensePieceBudgetBytes = (size_t)2 << 30;
 constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
 struct DensePieces {
