@@ -297,6 +297,19 @@ struct DensePieces {
   const unsigned long long* sums = nullptr;  // LADIES form: 6144 importance sums per piece (kAbsentSum: no edge)
 };
 
+// LADIES form, layers whose samples hold few vertices: the marking kernel turns the sums into
+// sampling keys itself where a stretch leaves LDS and writes those (4 bytes per vertex and
+// sample instead of 8, and the selection's first pass reads 4 instead of 8 and writes nothing).
+// keys == nullptr: the sums are written and the selection forms the keys (dense layers: the key
+// arithmetic of 2.5e9 present vertices next to the streaming took 100 ms instead of 13).
+struct KeysOnTheWayOut {
+  uint32_t* keys = nullptr;
+  uint64_t seed = 0;
+  uint64_t first_sample = 0;
+  uint32_t step = 0;
+  uint32_t n_vertices = 0;
+};
+
 // 32-bit words of one sample's presence map: a bit per vertex, padded to whole tiles.
 inline uint32_t bitmap_words_for(uint32_t n_vertices) {
   return ((n_vertices + 31u) / 32u + kBitmapTileWords - 1) / kBitmapTileWords * kBitmapTileWords;
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
-    unsigned long long* __restrict__ sums, uint32_t keys_per_sample, DensePieces dense) {
+    unsigned long long* __restrict__ sums, uint32_t keys_per_sample, DensePieces dense, KeysOnTheWayOut keys_out) {
   constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
   constexpr uint32_t kBinVertices = kBinWords * 32u;
   // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
@@ -650,7 +663,15 @@ __global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
           present = true;
         }
       }
-      __builtin_nontemporal_store(present ? sum : kAbsentSum, &out[i]);
+      if (keys_out.keys) {
+        const uint32_t v = v_lo + i;
+        keys_out.keys[(size_t)s * keys_per_sample + v] =
+            present ? ladies_key_bits(sum, (keys_out.first_sample + s) * (uint64_t)keys_out.n_vertices + v,
+                                      keys_out.step, keys_out.seed)
+                    : kAbsentKey;
+      } else {
+        __builtin_nontemporal_store(present ? sum : kAbsentSum, &out[i]);
+      }
     }
   } else {
     const uint32_t first_word = bin * kBinWords;
@@ -888,12 +909,27 @@ __global__ __launch_bounds__(256) void select_histogram(const unsigned long long
   if (threadIdx.x == 0) s_present = 0;
   const uint32_t s = blockIdx.y;
   uint32_t* mine = keys + (size_t)s * keys_per_sample;
-  const unsigned long long* my_sums = sums + (size_t)s * keys_per_sample;
+  const unsigned long long* my_sums = sums ? sums + (size_t)s * keys_per_sample : nullptr;
   const uint32_t tile_begin = blockIdx.x * kSelectTile;
   const uint32_t want8 = level == 1 ? prefix8[s] : 0u;
   __syncthreads();
   uint32_t seen = 0;
-  if (level == 0) {
+  if (level == 0 && sums == nullptr) {  // the marking has left keys, not sums
+    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
+      uint32_t batch[8];
+#pragma unroll
+      for (uint32_t k = 0; k < 8; ++k) {
+        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < 8; ++k)
+        if (batch[k] != kAbsentKey) {
+          ++seen;
+          atomicAdd(&s_hist[batch[k] >> 24], 1u);
+        }
+    }
+  } else if (level == 0) {
     for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 4) {
       unsigned long long batch[4];  // four loads under way before the arithmetic starts
 #pragma unroll
@@ -1455,7 +1491,7 @@ class LayerEngine : public EngineBase {
     TransitView tv = all;
     tv.base = all.base + (size_t)s0 * all.stride;
     if (form != apps::kConcatenated) {
-      if (build_distinct_by_bitmap(step, s0, tv, n) != 0) return -1;
+      if (build_distinct_by_bitmap(step, s0, tv, n, total) != 0) return -1;
     } else {
       // work items of the build: long neighbourhoods are spread over several workgroups
       uint64_t n_items = 0;
@@ -1510,7 +1546,7 @@ class LayerEngine : public EngineBase {
   }
 
   // What next() of the importance forms is handed, for every sample of the chunk.
-  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n) {
+  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint64_t total) {
     constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
@@ -1518,7 +1554,7 @@ class LayerEngine : public EngineBase {
     const uint32_t groups = (bins + per_group - 1) / per_group;
     if ((uint64_t)n * groups >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
     if constexpr (ladies) {
-      return rank_by_keys(step, s0, tv, n, bins, groups);
+      return rank_by_keys(step, s0, tv, n, bins, groups, total);
     } else {
       return list_distinct(tv, n, bins, groups);
     }
@@ -1541,7 +1577,7 @@ class LayerEngine : public EngineBase {
     }
     tick();
     collective_mark_binned<false><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u, dense_);
+        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u, dense_, KeysOnTheWayOut());
     tock();
     ND_HIP_TRY(hipMemsetAsync(d_marked_, 0, sizeof(uint32_t) * (size_t)n, stream_));
     const uint32_t sample_blocks = (n + kSumSamplesPerBlock - 1) / kSumSamplesPerBlock;
@@ -1559,7 +1595,8 @@ class LayerEngine : public EngineBase {
   // vertices that can be among its first `wanted` in key order are picked by a radix select on
   // the upper 16 bits of the key and ordered by descending key.  The distinct pairs of a
   // sample (2.4 M per batch at full size) are never listed.
-  int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
+  int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups,
+                   uint64_t total) {
     const uint32_t keys_per_sample = bins * kBinVerticesSums;
     const uint32_t tiles_per_sample = (keys_per_sample + kSelectTile - 1) / kSelectTile;
     if (n > bitmap_samples_) {
@@ -1568,9 +1605,18 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_sums_dense_, sizeof(unsigned long long) * (size_t)n * keys_per_sample));
       bitmap_samples_ = n;
     }
+    // a layer that can fill at most one position in 16 forms its keys in the marking kernel
+    KeysOnTheWayOut keys_out;
+    if (total * 16 < (uint64_t)n * keys_per_sample) {
+      keys_out.keys = d_keys_dense_;
+      keys_out.seed = seed_;
+      keys_out.first_sample = s0;
+      keys_out.step = (uint32_t)step;
+      keys_out.n_vertices = (uint32_t)invalid_;
+    }
     tick();
     collective_mark_binned<true><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, dense_);
+        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, dense_, keys_out);
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
     const dim3 tiles(tiles_per_sample, n);
@@ -1578,7 +1624,8 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipMemsetAsync(d_select_present_, 0, sizeof(uint32_t) * (size_t)n, stream_));
     for (int level = 0; level < 2; ++level) {
       ND_HIP_TRY(hipMemsetAsync(d_select_hist_, 0, sizeof(uint32_t) * 256 * (size_t)n, stream_));
-      select_histogram<<<tiles, dim3(256), 0, stream_>>>(d_sums_dense_, d_keys_dense_, keys_per_sample, level,
+      select_histogram<<<tiles, dim3(256), 0, stream_>>>(keys_out.keys ? nullptr : d_sums_dense_, d_keys_dense_,
+                                                         keys_per_sample, level,
                                                          (uint32_t)invalid_, seed_, (uint64_t)s0, (uint32_t)step,
                                                          d_select_prefix_, d_select_hist_, d_select_present_);
       select_pick<<<dim3(sample_blocks), dim3(256), 0, stream_>>>(d_select_hist_, n, level, wanted, d_select_prefix_,
