@@ -391,6 +391,7 @@ __device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint3
 // A sample without hubs among its transits and with at most this many entries in a
 // workgroup's stretches (a layer whose transits are drawn uniformly) marks them all at once.
 constexpr uint32_t kSparseGroupEntries = 32768;
+constexpr uint32_t kSparseGroupEntriesSums = 2048;  // LADIES form: sums in an LDS table of twice as many slots
 
 // Two workgroups share a compute unit (8 wavefronts per SIMD): at most 64 registers per lane
 // and (measured) 66 KB of LDS per workgroup - with 70 KB only one workgroup is resident and
@@ -444,6 +445,8 @@ __global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
     // way out it sets back to zero, so no stretch spends a pass on clearing
     for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
+  } else if (keys_out.keys) {
+    hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
   }
   if (threadIdx.x < tv.count) {
     const int32_t t = my_transit;
@@ -459,6 +462,70 @@ __global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
       if (lo < my_end) my_next = (uint32_t)csr.edges[lo];
       if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
+  }
+  if (kWithImportance && keys_out.keys && !hubs_among_transits) {
+    // LADIES form, a sample without hubs in a layer that fills few positions: the stretches
+    // of the workgroup as one.  At most kSparseGroupEntriesSums entries: their sums are
+    // gathered in an LDS table hashed by vertex (in the room of the per-vertex sums), the
+    // keys of the whole range are written as absent, and the table's vertices then get theirs.
+    // Stretch by stretch, 16 chains of searches, tables and barriers cost a workgroup 130 us
+    // for a few hundred entries.
+    const uint32_t group_bins = first_bin + kBinsPerGroup < bins_per_sample ? kBinsPerGroup : bins_per_sample - first_bin;
+    const uint32_t v_lo = first_bin * kBinVertices, v_hi = v_lo + group_bins * kBinVertices;
+    if (threadIdx.x < tv.count) {
+      uint32_t unused;
+      const EdgePos_t stop =
+          my_next < v_hi ? first_edge_at_or_above(csr.edges, my_reach, my_end, v_hi, &unused) : my_reach;
+      s_length[threadIdx.x] = (uint32_t)(stop - my_reach);
+      s_edge[threadIdx.x] = my_reach;
+      s_row_sum[threadIdx.x] = my_row_sum;
+    }
+    __syncthreads();
+    if (wave == 0) keep_filled_subranges<true>(tv.count, lane, s_length, s_edge, s_row_sum, s_start, &s_ranges, &s_pieces);
+    __syncthreads();
+    const uint32_t ranges = s_ranges;
+    const uint32_t size = s_start[ranges];
+    if (size <= kSparseGroupEntriesSums) {
+      constexpr uint32_t kSlots = 2u * kSparseGroupEntriesSums;  // a power of two
+      unsigned long long* slot_sum = s_acc;
+      uint32_t* slot_vertex = (uint32_t*)(s_acc + kSlots);
+      for (uint32_t i = threadIdx.x; i < kSlots; i += kBinThreads) {
+        slot_vertex[i] = 0xFFFFFFFFu;
+        slot_sum[i] = 0;
+      }
+      uint32_t* out_keys = keys_out.keys + (size_t)s * keys_per_sample + v_lo;
+      for (uint32_t i = threadIdx.x; i < group_bins * kBinVertices; i += kBinThreads) out_keys[i] = kAbsentKey;
+      __syncthreads();
+      for (uint32_t e = threadIdx.x; e < size; e += kBinThreads) {
+        uint32_t lo = 0, hi = ranges;  // the sub-range that holds entry e
+        while (hi - lo > 1) {
+          const uint32_t mid = lo + (hi - lo) / 2;
+          if (s_start[mid] <= e) lo = mid; else hi = mid;
+        }
+        const EdgePos_t src = s_edge[lo] + (EdgePos_t)(e - s_start[lo]);
+        const uint32_t local = (uint32_t)csr.edges[src] - v_lo;
+        const float p = csr.weights[src] * s_row_sum[lo];
+        const unsigned long long term = importance_term_fixed(p * p);
+        uint32_t slot = (local * 2654435761u) >> 20 & (kSlots - 1u);
+        for (;;) {  // at most half of the slots are ever taken
+          const uint32_t before = atomicCAS(&slot_vertex[slot], 0xFFFFFFFFu, local);
+          if (before == 0xFFFFFFFFu || before == local) break;
+          slot = (slot + 1u) & (kSlots - 1u);
+        }
+        if (term != 0) atomicAdd(&slot_sum[slot], term);
+      }
+      __syncthreads();  // the table is complete, and the absent keys have been written
+      for (uint32_t i = threadIdx.x; i < kSlots; i += kBinThreads) {
+        const uint32_t local = slot_vertex[i];
+        if (local == 0xFFFFFFFFu) continue;
+        const uint32_t v = v_lo + local;
+        out_keys[local] = ladies_key_bits(slot_sum[i], (keys_out.first_sample + s) * (uint64_t)keys_out.n_vertices + v,
+                                          keys_out.step, keys_out.seed);
+      }
+      return;
+    }
+    // too many entries for that: stretch by stretch (the tables are next written after every
+    // lane has read the size above)
   }
   if (!kWithImportance && !hubs_among_transits) {
     // The stretches of the workgroup as one: a bit per vertex fits the same LDS, and the few
