@@ -393,11 +393,11 @@ __device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint3
 constexpr uint32_t kSparseGroupEntries = 32768;
 constexpr uint32_t kSparseGroupEntriesSums = 2048;  // LADIES form: sums in an LDS table of twice as many slots
 
-// Two workgroups share a compute unit (8 wavefronts per SIMD): at most 64 registers per lane
-// and (measured) 66 KB of LDS per workgroup - with 70 KB only one workgroup is resident and
-// the LADIES form takes 1.6 times as long.
+// Two workgroups share a compute unit (8 wavefronts per SIMD) as long as a lane needs at most
+// 56 registers: measured, the LADIES form takes 1.6 times as long with 58 (one workgroup
+// resident) as with 56, whatever the LDS size between 62 and 70 KB.
 template <bool kWithImportance>
-__global__ __launch_bounds__(kBinThreads, 8) void collective_mark_binned(
+__global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
