@@ -279,12 +279,15 @@ constexpr uint32_t kBinsPerGroupSums = 16;
 constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
-// Dense pieces (FastGCN form).  What a hub contributes to a stretch can be thousands of entries
-// (a layer drawn by degree^2 sits on the hubs: 144 K entries per transit at full size), and it
-// is the same for every sample that holds the hub.  Where a vertex has kDensePieceEntries or
-// more edges into one stretch, the stretch's bitmap of that vertex is built once per graph
-// (1536 words); a sample then ORs the piece into the stretch on its way out of LDS instead
-// of marking the entries one by one.  hub_row[v] = row of v in piece_of or -1;
+// Dense pieces.  What a hub contributes to a stretch can be thousands of entries (a layer
+// drawn by degree^2 sits on the hubs: 144 K entries per transit at FastGCN's full size), and
+// it is the same for every sample that holds the hub.  Where a vertex has kDensePieceEntries
+// (LADIES form: kDensePieceEntriesSums) or more edges into one stretch, the stretch's piece of
+// that vertex is built once per graph - FastGCN form: its bitmap (1536 words); LADIES form:
+// the importance sum of every vertex of the stretch (6144 64-bit integers, kAbsentSum where
+// there is no edge; the sums are integers, so adding a piece gives the bits that adding its
+// edges one by one gives) - and a sample ORs / adds the piece on the stretch's way out of LDS
+// instead of going through the entries.  hub_row[v] = row of v in piece_of or -1;
 // piece_of[row * stretches + stretch] = piece index or kNoPiece.
 constexpr uint32_t kDensePieceEntries = 512;
 constexpr uint32_t kDensePieceEntriesSums = 2048;  // LADIES form: a piece is 6144 64-bit sums
