@@ -98,6 +98,19 @@ def main():
         out["apps"][app] = {"initial": imp_roots.tolist(), "final": final.reshape(-1).tolist(),
                             "shape": list(final.shape)}
 
+    # edge-list apps: batches of 5 consecutive vertices; two clusters of 3
+    n = ob.subgraph_num_samples(g, 5, 1500000)
+    verts = ob.mvs_vertices(g, n, 5)
+    rows, cols, start = ob.sample_mvs(g, verts)
+    out["apps"]["MVS5"] = {"initial": verts.reshape(-1).tolist(), "rows": rows.tolist(), "cols": cols.tolist(),
+                           "list_start": start.tolist()}
+    n = ob.subgraph_num_samples(g, 6, 2000000)
+    verts = ob.clustergcn_vertices(g, n, 3, 2)
+    final, rows, cols, start = ob.sample_clustergcn(g, verts)
+    out["apps"]["ClusterGCN3x2"] = {"initial": verts.reshape(-1).tolist(), "final": final.reshape(-1).tolist(),
+                                    "shape": list(final.shape), "rows": rows.tolist(), "cols": cols.tolist(),
+                                    "list_start": start.tolist()}
+
     with open(os.path.join(HERE, "sampler_vectors.json"), "w") as f:
         json.dump(out, f, separators=(",", ":"))
     print("wrote", os.path.join(HERE, "sampler_vectors.json"), os.path.getsize(os.path.join(HERE, "sampler_vectors.json")),
