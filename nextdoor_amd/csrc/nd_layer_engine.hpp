@@ -1253,86 +1253,6 @@ class LayerEngine : public EngineBase {
     return 0;
   }
 
-  // What the vertices with many edges into one stretch contribute to it, built once per graph
-  // (see DensePieces).  inverse_row_sums: the LADIES form's 1 / rowsum per vertex, else nullptr.
-  int build_dense_pieces(const CSR* graph, const float* inverse_row_sums) {
-    release_dense_pieces();
-    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
-    uint32_t threshold = ladies ? kDensePieceEntriesSums : kDensePieceEntries;
-    if (const char* env = getenv("ND_DENSE_PIECE_ENTRIES")) {  // 0: no pieces; small: to exercise them on small graphs
-      const long long v = atoll(env);
-      if (v <= 0) return 0;
-      threshold = (uint32_t)v;
-    }
-    constexpr uint32_t stretch_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
-    constexpr uint32_t stretch = stretch_words * 32u;
-    // a piece: a bit per vertex of the stretch, or a 64-bit importance sum (kAbsentSum: no edge)
-    constexpr size_t piece_words = ladies ? (size_t)stretch * 2u : (size_t)stretch_words;
-    const uint32_t V = (uint32_t)graph->get_n_vertices();
-    const uint32_t stretches = (bitmap_words_for(V) + stretch_words - 1) / stretch_words;
-    const size_t most_pieces = kDensePieceBudgetBytes / (sizeof(uint32_t) * piece_words);
-    std::vector<int32_t> hub_row(V, -1);
-    std::vector<uint32_t> piece_of, words;
-    size_t n_hubs = 0, n_pieces = 0;
-    for (uint32_t v = 0; v < V; ++v) {
-      const int32_t* const row = graph->col.data() + graph->row_ptr[v];
-      const int32_t* first = row;
-      const int32_t* last = graph->col.data() + graph->row_ptr[v + 1];
-      if ((size_t)(last - first) < threshold) continue;
-      while (first < last) {  // one sub-range of the sorted adjacency per stretch
-        const uint32_t b = (uint32_t)*first / stretch;
-        const uint32_t limit = (b + 1) * stretch;
-        const int32_t* stop = std::partition_point(first, last, [limit](int32_t c) { return (uint32_t)c < limit; });
-        if ((size_t)(stop - first) >= threshold && n_pieces < most_pieces) {
-          if (hub_row[v] < 0) {
-            hub_row[v] = (int32_t)n_hubs++;
-            piece_of.resize(n_hubs * stretches, kNoPiece);
-          }
-          piece_of[(size_t)hub_row[v] * stretches + b] = (uint32_t)n_pieces;
-          words.resize((n_pieces + 1) * piece_words, ladies ? 0xFFFFFFFFu : 0u);
-          uint32_t* w = words.data() + n_pieces * piece_words;
-          for (const int32_t* c = first; c < stop; ++c) {
-            const uint32_t local = (uint32_t)*c - b * stretch;
-            if (ladies) {
-              // the term the marking kernel adds for this edge, in the same arithmetic
-              const float p = graph->weight[(size_t)graph->row_ptr[v] + (size_t)(c - row)] * inverse_row_sums[v];
-              unsigned long long sum;
-              memcpy(&sum, w + 2u * local, sizeof(sum));
-              if (sum == kAbsentSum) sum = 0;
-              sum += importance_term_fixed(p * p);
-              memcpy(w + 2u * local, &sum, sizeof(sum));
-            } else {
-              w[local >> 5] |= 1u << (local & 31u);
-            }
-          }
-          ++n_pieces;
-        }
-        first = stop;
-      }
-    }
-    if (n_pieces == 0) return 0;
-    ND_HIP_TRY(hipMalloc(&d_hub_row_, sizeof(int32_t) * V));
-    ND_HIP_TRY(hipMalloc(&d_piece_of_, sizeof(uint32_t) * piece_of.size()));
-    ND_HIP_TRY(hipMalloc(&d_piece_words_, sizeof(uint32_t) * words.size()));
-    ND_HIP_TRY(hipMemcpy(d_hub_row_, hub_row.data(), sizeof(int32_t) * V, hipMemcpyHostToDevice));
-    ND_HIP_TRY(hipMemcpy(d_piece_of_, piece_of.data(), sizeof(uint32_t) * piece_of.size(), hipMemcpyHostToDevice));
-    ND_HIP_TRY(hipMemcpy(d_piece_words_, words.data(), sizeof(uint32_t) * words.size(), hipMemcpyHostToDevice));
-    dense_.hub_row = d_hub_row_;
-    dense_.piece_of = d_piece_of_;
-    dense_.words = d_piece_words_;
-    dense_.sums = (const unsigned long long*)d_piece_words_;
-    dense_pieces_ = n_pieces;
-    return 0;
-  }
-
-  void release_dense_pieces() {
-    release(d_hub_row_);
-    release(d_piece_of_);
-    release(d_piece_words_);
-    dense_ = DensePieces();
-    dense_pieces_ = 0;
-  }
-
   int alloc(uint64_t seed) override {
     if (!graph_) { last_error = "alloc before set_graph"; return -1; }
     free_run_buffers();
@@ -1536,6 +1456,87 @@ class LayerEngine : public EngineBase {
     if (p) (void)hipFree(p);
     p = nullptr;
   }
+
+  // What the vertices with many edges into one stretch contribute to it, built once per graph
+  // (see DensePieces).  inverse_row_sums: the LADIES form's 1 / rowsum per vertex, else nullptr.
+  int build_dense_pieces(const CSR* graph, const float* inverse_row_sums) {
+    release_dense_pieces();
+    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
+    uint32_t threshold = ladies ? kDensePieceEntriesSums : kDensePieceEntries;
+    if (const char* env = getenv("ND_DENSE_PIECE_ENTRIES")) {  // 0: no pieces; small: to exercise them on small graphs
+      const long long v = atoll(env);
+      if (v <= 0) return 0;
+      threshold = (uint32_t)v;
+    }
+    constexpr uint32_t stretch_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
+    constexpr uint32_t stretch = stretch_words * 32u;
+    // a piece: a bit per vertex of the stretch, or a 64-bit importance sum (kAbsentSum: no edge)
+    constexpr size_t piece_words = ladies ? (size_t)stretch * 2u : (size_t)stretch_words;
+    const uint32_t V = (uint32_t)graph->get_n_vertices();
+    const uint32_t stretches = (bitmap_words_for(V) + stretch_words - 1) / stretch_words;
+    const size_t most_pieces = kDensePieceBudgetBytes / (sizeof(uint32_t) * piece_words);
+    std::vector<int32_t> hub_row(V, -1);
+    std::vector<uint32_t> piece_of, words;
+    size_t n_hubs = 0, n_pieces = 0;
+    for (uint32_t v = 0; v < V; ++v) {
+      const int32_t* const row = graph->col.data() + graph->row_ptr[v];
+      const int32_t* first = row;
+      const int32_t* last = graph->col.data() + graph->row_ptr[v + 1];
+      if ((size_t)(last - first) < threshold) continue;
+      while (first < last) {  // one sub-range of the sorted adjacency per stretch
+        const uint32_t b = (uint32_t)*first / stretch;
+        const uint32_t limit = (b + 1) * stretch;
+        const int32_t* stop = std::partition_point(first, last, [limit](int32_t c) { return (uint32_t)c < limit; });
+        if ((size_t)(stop - first) >= threshold && n_pieces < most_pieces) {
+          if (hub_row[v] < 0) {
+            hub_row[v] = (int32_t)n_hubs++;
+            piece_of.resize(n_hubs * stretches, kNoPiece);
+          }
+          piece_of[(size_t)hub_row[v] * stretches + b] = (uint32_t)n_pieces;
+          words.resize((n_pieces + 1) * piece_words, ladies ? 0xFFFFFFFFu : 0u);
+          uint32_t* w = words.data() + n_pieces * piece_words;
+          for (const int32_t* c = first; c < stop; ++c) {
+            const uint32_t local = (uint32_t)*c - b * stretch;
+            if (ladies) {
+              // the term the marking kernel adds for this edge, in the same arithmetic
+              const float p = graph->weight[(size_t)graph->row_ptr[v] + (size_t)(c - row)] * inverse_row_sums[v];
+              unsigned long long sum;
+              memcpy(&sum, w + 2u * local, sizeof(sum));
+              if (sum == kAbsentSum) sum = 0;
+              sum += importance_term_fixed(p * p);
+              memcpy(w + 2u * local, &sum, sizeof(sum));
+            } else {
+              w[local >> 5] |= 1u << (local & 31u);
+            }
+          }
+          ++n_pieces;
+        }
+        first = stop;
+      }
+    }
+    if (n_pieces == 0) return 0;
+    ND_HIP_TRY(hipMalloc(&d_hub_row_, sizeof(int32_t) * V));
+    ND_HIP_TRY(hipMalloc(&d_piece_of_, sizeof(uint32_t) * piece_of.size()));
+    ND_HIP_TRY(hipMalloc(&d_piece_words_, sizeof(uint32_t) * words.size()));
+    ND_HIP_TRY(hipMemcpy(d_hub_row_, hub_row.data(), sizeof(int32_t) * V, hipMemcpyHostToDevice));
+    ND_HIP_TRY(hipMemcpy(d_piece_of_, piece_of.data(), sizeof(uint32_t) * piece_of.size(), hipMemcpyHostToDevice));
+    ND_HIP_TRY(hipMemcpy(d_piece_words_, words.data(), sizeof(uint32_t) * words.size(), hipMemcpyHostToDevice));
+    dense_.hub_row = d_hub_row_;
+    dense_.piece_of = d_piece_of_;
+    dense_.words = d_piece_words_;
+    dense_.sums = (const unsigned long long*)d_piece_words_;
+    dense_pieces_ = n_pieces;
+    return 0;
+  }
+
+  void release_dense_pieces() {
+    release(d_hub_row_);
+    release(d_piece_of_);
+    release(d_piece_words_);
+    dense_ = DensePieces();
+    dense_pieces_ = 0;
+  }
+
 
   // events around the neighbourhood kernel when profiling is on
   void tick() {
