@@ -126,6 +126,27 @@ def test_importance_sampling_with_ready_made_hub_pieces(oracle, app, monkeypatch
         s.close()
 
 
+@pytest.mark.parametrize("app", ["FastGCNImportance3x16", "LADIESImportance3x16"])
+@pytest.mark.parametrize("pieces", ["default", "8"])
+def test_importance_sampling_over_several_stretches(oracle, app, pieces, monkeypatch):
+    """130,000 vertices: three stretches of the FastGCN form, 22 of the LADIES form (two
+    workgroups per sample), a hub with edges into all of them."""
+    if pieces != "default":
+        monkeypatch.setenv("ND_DENSE_PIECE_ENTRIES", pieces)
+    g = graphs.random_graph(n=130000, mean_degree=3, seed=5, hub=8, isolated_every=6)
+    og = graphs.oracle_view(g)
+    s = nd.Sampler(app, g, seed=SEED)
+    ladies = app.startswith("LADIES")
+    d = layer_desc(oracle, s, oracle.LADIES_IMPORTANCE if ladies else oracle.FASTGCN_IMPORTANCE)
+    want = (oracle.sample_ladies_importance if ladies else oracle.sample_fastgcn_importance)(
+        og, d, SEED, s.initial_contents)
+    print("app", app, "pieces", pieces, "built", s.counter(3), flush=True)
+    assert s.counter(3) > 0
+    s.do_transit_parallel(True)
+    assert np.array_equal(s.final_samples(), want)
+    s.close()
+
+
 def test_distinct_is_refused_for_layer_apps():
     g = graphs.random_graph(n=100, mean_degree=4, seed=1)
     s = nd.Sampler("LayerLiteral2x8", g, seed=SEED)
