@@ -952,132 +952,109 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
 // ---- the best m keys of every sample, without sorting everything ----
 //
 // Only the first stepSize ranked vertices of a sample are ever read, out of up to millions of
-// distinct ones.  A two-level radix select on the upper 16 bits of the sort key finds, per
-// sample, the smallest 16-bit prefix T such that at least m keys have a prefix <= T; the
-// entries with a prefix <= T (m and a few more) are copied out in order and only those are
-// sorted.  Entries are grouped by sample, so a workgroup counts into an LDS histogram for the
-// sample its tile begins with and falls back to global atomics for the few entries beyond.
+// distinct ones.  A radix select on the upper 14 bits of the sort key finds, per sample, the
+// smallest prefix T such that at least m keys have a prefix <= T; the entries with a prefix
+// <= T (m and some more) are copied out and only those are sorted.
 // The keys of a chunk are dense: keys[s * keys_per_sample + v] for every vertex v (kAbsentKey
 // where sample s does not hold v), so position tells sample and vertex and no list of the
-// distinct pairs is ever written.  A workgroup takes kSelectTile consecutive vertices of one
-// sample: blockIdx.x = tile of the sample, blockIdx.y = sample.
+// distinct pairs is ever written.  The copying takes kSelectTile consecutive vertices of one
+// sample per workgroup: blockIdx.x = tile of the sample, blockIdx.y = sample.
 constexpr uint32_t kSelectPerLane = 32;
 constexpr uint32_t kSelectTile = 256 * kSelectPerLane;
 
-// level 0: forms the keys - keys[s][v] from sums[s][v], Philox slot (first_sample + s) * |V| + v -
-// and counts hist[s][key >> 24] over the sample's present keys, present[s] = how many there
-// are; level 1: hist[s][(key >> 16) & 255] over the keys whose upper 8 bits equal prefix8[s]
-__global__ __launch_bounds__(256) void select_histogram(const unsigned long long* __restrict__ sums,
-                                                        uint32_t* __restrict__ keys, uint32_t keys_per_sample,
-                                                        int level, uint32_t n_vertices, uint64_t seed,
-                                                        uint64_t first_sample, uint32_t step,
-                                                        const uint32_t* __restrict__ prefix8,
-                                                        uint32_t* __restrict__ hist, uint32_t* __restrict__ present) {
-  __shared__ uint32_t s_hist[256];
-  __shared__ uint32_t s_present;
-  s_hist[threadIdx.x] = 0;
-  if (threadIdx.x == 0) s_present = 0;
-  const uint32_t s = blockIdx.y;
-  uint32_t* mine = keys + (size_t)s * keys_per_sample;
-  const unsigned long long* my_sums = sums ? sums + (size_t)s * keys_per_sample : nullptr;
-  const uint32_t tile_begin = blockIdx.x * kSelectTile;
-  const uint32_t want8 = level == 1 ? prefix8[s] : 0u;
+// One workgroup per sample, one pass over its keys: forms them where the marking has left sums
+// (keys[s][v] from sums[s][v], Philox slot (first_sample + s) * |V| + v; sums == nullptr: the
+// keys are there already), counts the present ones by their upper kSelectBits bits in an LDS
+// histogram and picks the bin that holds the wanted-th smallest key: threshold[s] = that bin,
+// kept[s] = keys up to and including it (a sample with fewer keys than wanted keeps them all),
+// present[s] = all its keys.  A sample's whole histogram stays in the workgroup: no atomic
+// reaches memory, and no second pass over the keys refines the threshold (two levels of 8 bits,
+// counted by a workgroup per tile of 8192 keys, read every key twice).
+constexpr uint32_t kSelectBits = 14;
+constexpr uint32_t kSelectBins = 1u << kSelectBits;
+constexpr uint32_t kSelectThreads = 1024;
+__global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(56))) void select_threshold(
+    const unsigned long long* __restrict__ sums, uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+    uint32_t n_vertices, uint64_t seed, uint64_t first_sample, uint32_t step, uint32_t wanted,
+    uint32_t* __restrict__ threshold, uint32_t* __restrict__ kept, uint32_t* __restrict__ present) {
+  __shared__ uint32_t s_hist[kSelectBins];
+  __shared__ uint32_t s_wave_total[kSelectThreads / 64];
+  const uint32_t s = blockIdx.x;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  for (uint32_t i = threadIdx.x; i < kSelectBins; i += kSelectThreads) s_hist[i] = 0;
   __syncthreads();
-  uint32_t seen = 0;
-  if (level == 0 && sums == nullptr) {  // the marking has left keys, not sums
-    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
-      uint32_t batch[8];
-#pragma unroll
-      for (uint32_t k = 0; k < 8; ++k) {
-        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
-        batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
-      }
-#pragma unroll
-      for (uint32_t k = 0; k < 8; ++k)
-        if (batch[k] != kAbsentKey) {
-          ++seen;
-          atomicAdd(&s_hist[batch[k] >> 24], 1u);
-        }
-    }
-  } else if (level == 0) {
-    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 4) {
+  uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  if (sums) {
+    const unsigned long long* my_sums = sums + (size_t)s * keys_per_sample;
+    for (uint32_t v0 = 0; v0 < keys_per_sample; v0 += 4 * kSelectThreads) {
       unsigned long long batch[4];  // four loads under way before the arithmetic starts
 #pragma unroll
       for (uint32_t k = 0; k < 4; ++k) {
-        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
         batch[k] = v < keys_per_sample ? my_sums[v] : kAbsentSum;
       }
 #pragma unroll
       for (uint32_t k = 0; k < 4; ++k) {
-        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
         if (v >= keys_per_sample) continue;
         uint32_t key = kAbsentKey;
         if (batch[k] != kAbsentSum) {
           key = ladies_key_bits(batch[k], (first_sample + s) * (uint64_t)n_vertices + v, step, seed);
-          ++seen;
-          atomicAdd(&s_hist[key >> 24], 1u);
+          atomicAdd(&s_hist[key >> (32u - kSelectBits)], 1u);
         }
         mine[v] = key;
       }
     }
   } else {
-    for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
+    for (uint32_t v0 = 0; v0 < keys_per_sample; v0 += 8 * kSelectThreads) {
       uint32_t batch[8];
 #pragma unroll
       for (uint32_t k = 0; k < 8; ++k) {
-        const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
+        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
         batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
       }
 #pragma unroll
       for (uint32_t k = 0; k < 8; ++k)
-        if (batch[k] != kAbsentKey && (batch[k] >> 24) == want8) atomicAdd(&s_hist[(batch[k] >> 16) & 255u], 1u);
+        if (batch[k] != kAbsentKey) atomicAdd(&s_hist[batch[k] >> (32u - kSelectBits)], 1u);
     }
   }
-  if (level == 0 && seen) atomicAdd(&s_present, seen);
   __syncthreads();
-  const uint32_t c = s_hist[threadIdx.x];
-  if (c) atomicAdd(&hist[(size_t)s * 256 + threadIdx.x], c);
-  if (level == 0 && threadIdx.x == 0 && s_present) atomicAdd(&present[s], s_present);
-}
-
-// One lane per sample walks its 256 bins.  level 0: prefix8[s] = bin holding the need-th
-// smallest key, need[s] = what is still needed inside that bin, kept[s] = keys in the bins
-// before it.  level 1: threshold16[s] = (prefix8 << 8) | bin, kept[s] += keys up to and
-// including that bin.  A sample with fewer keys than needed keeps everything.
-__global__ void select_pick(const uint32_t* __restrict__ hist, uint32_t n_samples, int level, uint32_t wanted,
-                            uint32_t* __restrict__ prefix8, uint32_t* __restrict__ need,
-                            uint32_t* __restrict__ kept, uint32_t* __restrict__ threshold16) {
-  const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
-  if (s >= n_samples) return;
-  const uint32_t* h = hist + (size_t)s * 256;
-  const uint32_t target = level == 0 ? wanted : need[s];
-  uint32_t before = 0, bin = 0;
-  for (; bin < 256; ++bin) {
-    const uint32_t c = h[bin];
-    if (before + c >= target) break;
-    before += c;
+  // lane t owns bins [16 t, 16 t + 16): the bin in which the running count reaches `wanted`
+  constexpr uint32_t kOwn = kSelectBins / kSelectThreads;
+  uint32_t own = 0;
+#pragma unroll
+  for (uint32_t b = 0; b < kOwn; ++b) own += s_hist[threadIdx.x * kOwn + b];
+  const uint32_t through_wave = wave_inclusive_scan(own);
+  if (lane == 63) s_wave_total[wave] = through_wave;
+  __syncthreads();
+  uint32_t before = through_wave - own, total = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < kSelectThreads / 64; ++w) {
+    const uint32_t t = s_wave_total[w];
+    if (w < wave) before += t;
+    total += t;
   }
-  if (level == 0) {
-    if (bin == 256) {  // fewer keys than wanted: everything stays
-      prefix8[s] = 255;
-      need[s] = 0xFFFFFFFFu;
-      kept[s] = before - h[255];
-    } else {
-      prefix8[s] = bin;
-      need[s] = target - before;
-      kept[s] = before;
+  if (threadIdx.x == 0) present[s] = total;
+  if (total < wanted) {  // everything stays
+    if (threadIdx.x == 0) {
+      threshold[s] = kSelectBins - 1u;
+      kept[s] = total;
     }
-  } else {
-    if (bin == 256) bin = 255;
-    threshold16[s] = (prefix8[s] << 8) | bin;
-    uint32_t through = 0;
-    for (uint32_t b = 0; b <= bin; ++b) through += h[b];
-    kept[s] += through;
+  } else if (before < wanted && before + own >= wanted) {  // exactly one lane
+    uint32_t running = before;
+    for (uint32_t b = 0; b < kOwn; ++b) {
+      running += s_hist[threadIdx.x * kOwn + b];
+      if (running >= wanted) {
+        threshold[s] = threadIdx.x * kOwn + b;
+        kept[s] = running;
+        break;
+      }
+    }
   }
 }
 
-__device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold16) {
-  return key != kAbsentKey && (key >> 16) <= threshold16;
+__device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold) {
+  return key != kAbsentKey && (key >> (32u - kSelectBits)) <= threshold;
 }
 
 // Copies the kept entries of sample s into its stretch [ranked_start[s], ranked_start[s + 1]) of
@@ -1085,13 +1062,13 @@ __device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold16)
 // the entries of a round with one atomic; a few hundred of a sample's millions of keys stay,
 // so most rounds claim nothing).  The sorts that follow fix the order.
 __global__ __launch_bounds__(256) void select_collect(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
-                                                      const uint32_t* __restrict__ threshold16,
+                                                      const uint32_t* __restrict__ threshold_of,
                                                       const uint32_t* __restrict__ ranked_start,
                                                       uint32_t* __restrict__ claimed, uint32_t* __restrict__ kept_key,
                                                       uint32_t* __restrict__ kept_sample, int32_t* __restrict__ kept_id) {
   const uint32_t s = blockIdx.y;
   const uint32_t* mine = keys + (size_t)s * keys_per_sample;
-  const uint32_t threshold = threshold16[s];
+  const uint32_t threshold = threshold_of[s];
   const uint32_t first = ranked_start[s];
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t tile_begin = blockIdx.x * kSelectTile;
@@ -1346,11 +1323,8 @@ class LayerEngine : public EngineBase {
     if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
       const size_t per_sample = sizeof(uint32_t) * ((size_t)n_samples_ + 1);
       ND_HIP_TRY(hipMalloc(&d_ranked_start_, per_sample));
-      ND_HIP_TRY(hipMalloc(&d_select_prefix_, per_sample));
-      ND_HIP_TRY(hipMalloc(&d_select_need_, per_sample));
       ND_HIP_TRY(hipMalloc(&d_select_kept_, per_sample));
       ND_HIP_TRY(hipMalloc(&d_select_threshold_, per_sample));
-      ND_HIP_TRY(hipMalloc(&d_select_hist_, sizeof(uint32_t) * 256 * (size_t)n_samples_));
       ND_HIP_TRY(hipMalloc(&d_select_present_, per_sample));
     }
     return 0;
@@ -1691,17 +1665,9 @@ class LayerEngine : public EngineBase {
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
     const dim3 tiles(tiles_per_sample, n);
-    const unsigned sample_blocks = (n + 255) / 256;
-    ND_HIP_TRY(hipMemsetAsync(d_select_present_, 0, sizeof(uint32_t) * (size_t)n, stream_));
-    for (int level = 0; level < 2; ++level) {
-      ND_HIP_TRY(hipMemsetAsync(d_select_hist_, 0, sizeof(uint32_t) * 256 * (size_t)n, stream_));
-      select_histogram<<<tiles, dim3(256), 0, stream_>>>(keys_out.keys ? nullptr : d_sums_dense_, d_keys_dense_,
-                                                         keys_per_sample, level,
-                                                         (uint32_t)invalid_, seed_, (uint64_t)s0, (uint32_t)step,
-                                                         d_select_prefix_, d_select_hist_, d_select_present_);
-      select_pick<<<dim3(sample_blocks), dim3(256), 0, stream_>>>(d_select_hist_, n, level, wanted, d_select_prefix_,
-                                                                  d_select_need_, d_select_kept_, d_select_threshold_);
-    }
+    select_threshold<<<dim3(n), dim3(kSelectThreads), 0, stream_>>>(
+        keys_out.keys ? nullptr : d_sums_dense_, d_keys_dense_, keys_per_sample, (uint32_t)invalid_, seed_, (uint64_t)s0,
+        (uint32_t)step, wanted, d_select_threshold_, d_select_kept_, d_select_present_);
     // where every sample's ranked list starts: exclusive scan of the kept counts
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
     ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
@@ -1801,8 +1767,8 @@ class LayerEngine : public EngineBase {
     release(d_initial_); release(d_samples_); release(d_samples_init_); release(d_final_);
     release(d_sizes_); release(d_offsets_); release(d_row_offsets_); release(d_small_scratch_);
     release(d_item_count_); release(d_item_start_);
-    release(d_ranked_start_); release(d_select_prefix_); release(d_select_need_); release(d_select_kept_);
-    release(d_select_threshold_); release(d_select_hist_); release(d_select_present_);
+    release(d_ranked_start_); release(d_select_kept_);
+    release(d_select_threshold_); release(d_select_present_);
     release_neighborhood_buffers();
     if (allocated_) {
       (void)hipEventDestroy(ev_begin_);
@@ -1854,8 +1820,7 @@ class LayerEngine : public EngineBase {
   uint32_t *d_sizes_ = nullptr, *d_offsets_ = nullptr, *d_row_offsets_ = nullptr, *d_small_scratch_ = nullptr;
   uint32_t *d_item_count_ = nullptr, *d_item_start_ = nullptr;
   // LADIES form: the selection of the best keys per sample
-  uint32_t *d_ranked_start_ = nullptr, *d_select_prefix_ = nullptr, *d_select_need_ = nullptr;
-  uint32_t *d_select_kept_ = nullptr, *d_select_threshold_ = nullptr, *d_select_hist_ = nullptr;
+  uint32_t *d_ranked_start_ = nullptr, *d_select_kept_ = nullptr, *d_select_threshold_ = nullptr;
   uint32_t* d_select_present_ = nullptr;  // present[s]: distinct vertices of sample s's neighbourhood
   uint32_t *d_kept_key_ = nullptr, *d_kept_sample_ = nullptr;
   int32_t* d_kept_id_ = nullptr;
