@@ -1638,7 +1638,7 @@ class LayerEngine : public EngineBase {
 
   // LADIES form: the marking leaves one sampling key per (sample, vertex); per sample, the
   // vertices that can be among its first `wanted` in key order are picked by a radix select on
-  // the upper 16 bits of the key and ordered by descending key.  The distinct pairs of a
+  // the upper 14 bits of the key and ordered by descending key.  The distinct pairs of a
   // sample (2.4 M per batch at full size) are never listed.
   int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups,
                    uint64_t total) {
