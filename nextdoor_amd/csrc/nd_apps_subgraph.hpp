@@ -70,7 +70,7 @@ struct MVSSamplingAppT : nd::apps::SubgraphCommon<kBatch> {
   __host__ __device__ int stepSize(int) { return kBatch; }
 
   template <typename SampleType, typename EdgeArray, typename WeightArray>
-  __device__ inline VertexID next(int, CSRPartition*, const VertexID* transits, const VertexID, SampleType* sample,
+  __device__ __forceinline__ VertexID next(int, CSRPartition*, const VertexID* transits, const VertexID, SampleType* sample,
                                   const float, EdgeArray& transitEdges, WeightArray&, const EdgePos_t numEdges,
                                   const VertexID_t neighbrID, curandState*) {
     const VertexID_t row = transits[0];
@@ -116,7 +116,7 @@ struct SubGraphSamplingAppT : nd::apps::SubgraphCommon<kClusterVertices * kClust
   __host__ __device__ int stepSize(int k) { return k == 0 ? 1 : kVertices; }
 
   template <typename SampleType, typename EdgeArray, typename WeightArray>
-  __device__ inline VertexID next(int step, CSRPartition*, const VertexID* transits, const VertexID,
+  __device__ __forceinline__ VertexID next(int step, CSRPartition*, const VertexID* transits, const VertexID,
                                   SampleType* sample, const float, EdgeArray& transitEdges, WeightArray&,
                                   const EdgePos_t numEdges, const VertexID_t neighbrID, curandState*) {
     const VertexID_t v1 = transits[0];

@@ -44,23 +44,36 @@ struct WritingSink {
   // nothing the app reads lives in the lists: loads may be moved ahead of these stores
   VertexID_t* __restrict__ rows;  // start of the unit's stretch
   VertexID_t* __restrict__ cols;
-  OrderPointer order;             // 64 entries (count << 8 | lane), ascending
-  uint64_t with_edge;             // lanes that have an edge of index n
+  OrderPointer order;             // 64 entries (count << 8 | lane), ascending; unused when no lane has more than kEarly edges
+  uint32_t early_at;              // where the lane's next edge of index < kEarly goes: known before next() runs
+  uint32_t early_steps;           // then 8 bits each: from edge 0 to edge 1, 1 to 2, 2 to 3 (one running value:
+                                  // a choice among four members would keep the whole object in memory)
+  uint64_t with_edge = ~0ull;     // from index kEarly on: lanes that have an edge of index n
   uint64_t below_me;
-  uint32_t before = 0;            // edges of the unit with index < n
+  uint32_t before = 0;            // from index kEarly on: edges of the unit with index < n
   uint32_t retired = 0;           // entries of `order` already taken out of with_edge
   uint32_t n = 0;
+  static constexpr uint32_t kEarly = 4;
   __device__ __forceinline__ void put(VertexID_t row, VertexID_t col) {
-    while (retired < 64) {
-      const uint64_t entry = order[retired];
-      if ((uint32_t)(entry >> 8) > n) break;
-      with_edge &= ~(1ull << (entry & 63u));
-      ++retired;
+    uint32_t at;
+    if (n < kEarly) {
+      // most lanes list a few edges: no trip to the table for those (a lane used to walk the
+      // table entry by entry, one LDS latency each, past every lane without edges)
+      at = early_at;
+      early_at += early_steps & 0xFFu;
+      early_steps >>= 8;
+    } else {
+      while (retired < 64) {
+        const uint64_t entry = order[retired];
+        if ((uint32_t)(entry >> 8) > n) break;
+        with_edge &= ~(1ull << (entry & 63u));
+        ++retired;
+      }
+      at = before + (uint32_t)__popcll(with_edge & below_me);
+      before += (uint32_t)__popcll(with_edge);
     }
-    const uint32_t at = before + (uint32_t)__popcll(with_edge & below_me);
     rows[at] = row;
     cols[at] = col;
-    before += (uint32_t)__popcll(with_edge);
     ++n;
   }
 };
@@ -170,12 +183,23 @@ __global__ __launch_bounds__(kSubgraphThreads) void subgraph_step_kernel(Subgrap
   for (int d = 32; d > 0; d >>= 1) before += __shfl_xor(before, d, 64);
   WritingSink sink;
   uint32_t first_edge = live ? P.list_start[s] + before : 0u;  // of the unit
-  if (__ballot(count > 1) == 0) {
-    // at most one edge per lane: lane order, no table needed
-    first_edge += wave_inclusive_scan(count) - count;  // of this lane
-    sink.order = nullptr;
-    sink.retired = 64;
-    sink.with_edge = 1ull << lane;
+  {
+    const uint64_t below = (1ull << lane) - 1ull;
+    const uint64_t have0 = __ballot(count > 0), have1 = __ballot(count > 1), have2 = __ballot(count > 2),
+                   have3 = __ballot(count > 3);
+    uint32_t through = (uint32_t)__popcll(have0);
+    const uint32_t at0 = (uint32_t)__popcll(have0 & below);
+    const uint32_t at1 = through + (uint32_t)__popcll(have1 & below);
+    through += (uint32_t)__popcll(have1);
+    const uint32_t at2 = through + (uint32_t)__popcll(have2 & below);
+    through += (uint32_t)__popcll(have2);
+    const uint32_t at3 = through + (uint32_t)__popcll(have3 & below);
+    sink.early_at = at0;
+    sink.early_steps = (at1 - at0) | ((at2 - at1) << 8) | ((at3 - at2) << 16);  // each at most 128
+    sink.before = through + (uint32_t)__popcll(have3);
+  }
+  if (__ballot(count > WritingSink::kEarly) == 0) {
+    sink.order = nullptr;  // never read
   } else {
     // the unit's lanes by ascending (count, lane): a lane's place is the number of lanes
     // before it.  Only this wavefront reads its table, and a wavefront's LDS accesses are
@@ -190,7 +214,6 @@ __global__ __launch_bounds__(kSubgraphThreads) void subgraph_step_kernel(Subgrap
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     sink.order = (WritingSink::OrderPointer)s_order[wave];
-    sink.with_edge = ~0ull;
   }
   if (count != 0) {
     curandState rng;
