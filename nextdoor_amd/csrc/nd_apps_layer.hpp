@@ -140,8 +140,8 @@ struct FastGCNImportanceAppT : nd::apps::LayerCommon<kLayers, kBatch, kNumSample
 // LADIES-style layer-dependent importance sampling WITHOUT replacement.  With U the
 // previous layer, importance(v) = sum over edges u -> v, u in U, of (w_uv * (1 / rowsum(u)))^2 (the inverse rounded to float once per row).
 // The engine computes it over the collective neighbourhood, draws one Efraimidis-Spirakis
-// key log2(uniform) / importance per distinct vertex (uniform from Philox at slot
-// sample * |V| + v) and hands next() the vertices in descending key order: the first
+// key log2(uniform) / importance per distinct vertex (uniform from Philox, four consecutive
+// vertices of a sample to a block) and hands next() the vertices in descending key order: the first
 // stepSize(k) of them are a weighted sample without replacement, in selection order.
 template <int kLayers, int kBatch, int kNumSamples>
 struct LadiesImportanceAppT : FastGCNImportanceAppT<kLayers, kBatch, kNumSamples> {

@@ -204,25 +204,44 @@ __host__ __device__ __forceinline__ float det_log2(float x) {
   return (float)e + ln_m * 1.44269502f;
 }
 
-// Efraimidis-Spirakis key of (sample, vertex): log2(u) / importance with u from Philox at slot
-// sample * |V| + vertex and importance the fixed-point sum of the vertex's terms (the common
-// 2^53 scale does not change the order of the keys); as sortable bits, inverted so that an
-// ascending sort yields descending keys.  No key is 0xFFFFFFFF (it would be a negative NaN):
-// kAbsentKey marks the vertices a sample's neighbourhood does not hold.
+// Efraimidis-Spirakis key of (sample, vertex): log2(u) / importance, importance the fixed-point
+// sum of the vertex's terms (the common 2^53 scale does not change the order of the keys), u
+// from Philox: the pair's index is P = sample * (|V| rounded up to a multiple of 4) + vertex,
+// its uniform comes from word P & 3 of the block with counter P >> 2 - four consecutive
+// vertices of a sample share a block, so a lane that handles four of them pays for one (the
+// ten rounds of multiplications are what the key pass of a dense layer is bound by).  As
+// sortable bits, inverted so that an ascending sort yields descending keys.  No key is
+// 0xFFFFFFFF (it would be a negative NaN): kAbsentKey marks the vertices a sample's
+// neighbourhood does not hold.
 constexpr uint32_t kAbsentKey = 0xFFFFFFFFu;
 // importance sums stay below 2^63 (at most 1024 transits, each adding at most 2^53)
 constexpr unsigned long long kAbsentSum = ~0ull;
-__device__ __forceinline__ uint32_t ladies_key_bits(unsigned long long importance_fixed, uint64_t slot, uint32_t step,
-                                                    uint64_t seed) {
+__host__ __device__ __forceinline__ uint64_t ladies_pair_index(uint64_t sample, uint32_t n_vertices, uint32_t v) {
+  return sample * (uint64_t)((n_vertices + 3u) & ~3u) + v;
+}
+__device__ __forceinline__ PhiloxBlock ladies_block(uint64_t pair, uint32_t step, uint64_t seed) {
+  const uint64_t block = pair >> 2;
+  return philox4x32_10((uint32_t)block, (uint32_t)(block >> 32), step, 0, (uint32_t)seed, (uint32_t)(seed >> 32));
+}
+__device__ __forceinline__ uint32_t ladies_key_from_word(unsigned long long importance_fixed, uint32_t word) {
   const float importance = (float)importance_fixed;
-  const PhiloxBlock blk = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, 0, (uint32_t)seed,
-                                        (uint32_t)(seed >> 32));
-  const float u = ((float)(blk.w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+  const float u = ((float)(word >> 8) + 0.5f) * 5.9604644775390625e-08f;
   float key = -__builtin_inff();
   if (importance > 0.0f) key = det_log2(u) / importance;
   uint32_t b = __float_as_uint(key);
   b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
   return ~b;
+}
+// one pair on its own
+__device__ __forceinline__ uint32_t ladies_key_bits(unsigned long long importance_fixed, uint64_t pair, uint32_t step,
+                                                    uint64_t seed) {
+  const PhiloxBlock blk = ladies_block(pair, step, seed);
+  const uint32_t which = (uint32_t)pair & 3u;
+  uint32_t word = blk.w[0];
+  word = which == 1 ? blk.w[1] : word;
+  word = which == 2 ? blk.w[2] : word;
+  word = which == 3 ? blk.w[3] : word;
+  return ladies_key_from_word(importance_fixed, word);
 }
 
 // ---- wave-wide data movement on the VALU (DPP), no LDS traffic ----
@@ -522,7 +541,7 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
         const uint32_t local = slot_vertex[i];
         if (local == 0xFFFFFFFFu) continue;
         const uint32_t v = v_lo + local;
-        out_keys[local] = ladies_key_bits(slot_sum[i], (keys_out.first_sample + s) * (uint64_t)keys_out.n_vertices + v,
+        out_keys[local] = ladies_key_bits(slot_sum[i], ladies_pair_index(keys_out.first_sample + s, keys_out.n_vertices, v),
                                           keys_out.step, keys_out.seed);
       }
       return;
@@ -736,7 +755,7 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
       if (keys_out.keys) {
         const uint32_t v = v_lo + i;
         keys_out.keys[(size_t)s * keys_per_sample + v] =
-            present ? ladies_key_bits(sum, (keys_out.first_sample + s) * (uint64_t)keys_out.n_vertices + v,
+            present ? ladies_key_bits(sum, ladies_pair_index(keys_out.first_sample + s, keys_out.n_vertices, v),
                                       keys_out.step, keys_out.seed)
                     : kAbsentKey;
       } else {
@@ -985,24 +1004,36 @@ __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(5
   __syncthreads();
   uint32_t* mine = keys + (size_t)s * keys_per_sample;
   if (sums) {
-    const unsigned long long* my_sums = sums + (size_t)s * keys_per_sample;
-    for (uint32_t v0 = 0; v0 < keys_per_sample; v0 += 4 * kSelectThreads) {
-      unsigned long long batch[4];  // four loads under way before the arithmetic starts
+    // a lane takes four consecutive vertices: their keys come from one Philox block
+    // (keys_per_sample is a multiple of 4, and so is the pair index of the sample's vertex 0)
+    const ulonglong2* my_sums = (const ulonglong2*)(sums + (size_t)s * keys_per_sample);
+    uint4* my_keys = (uint4*)mine;
+    for (uint32_t q0 = 0; q0 < keys_per_sample / 4u; q0 += 2 * kSelectThreads) {
+      ulonglong2 low[2], high[2];  // two quads under way before the arithmetic starts
 #pragma unroll
-      for (uint32_t k = 0; k < 4; ++k) {
-        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
-        batch[k] = v < keys_per_sample ? my_sums[v] : kAbsentSum;
+      for (uint32_t k = 0; k < 2; ++k) {
+        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
+        const bool inside = q < keys_per_sample / 4u;
+        low[k] = inside ? my_sums[2u * q] : make_ulonglong2(kAbsentSum, kAbsentSum);
+        high[k] = inside ? my_sums[2u * q + 1u] : make_ulonglong2(kAbsentSum, kAbsentSum);
       }
 #pragma unroll
-      for (uint32_t k = 0; k < 4; ++k) {
-        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
-        if (v >= keys_per_sample) continue;
-        uint32_t key = kAbsentKey;
-        if (batch[k] != kAbsentSum) {
-          key = ladies_key_bits(batch[k], (first_sample + s) * (uint64_t)n_vertices + v, step, seed);
-          atomicAdd(&s_hist[key >> (32u - kSelectBits)], 1u);
+      for (uint32_t k = 0; k < 2; ++k) {
+        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
+        if (q >= keys_per_sample / 4u) continue;
+        const unsigned long long four[4] = {low[k].x, low[k].y, high[k].x, high[k].y};
+        uint32_t key[4] = {kAbsentKey, kAbsentKey, kAbsentKey, kAbsentKey};
+        if ((four[0] & four[1] & four[2] & four[3]) != kAbsentSum) {
+          const PhiloxBlock blk = ladies_block(ladies_pair_index(first_sample + s, n_vertices, 4u * q), step, seed);
+#pragma unroll
+          for (uint32_t i = 0; i < 4; ++i) {
+            if (four[i] != kAbsentSum) {
+              key[i] = ladies_key_from_word(four[i], blk.w[i]);
+              atomicAdd(&s_hist[key[i] >> (32u - kSelectBits)], 1u);
+            }
+          }
         }
-        mine[v] = key;
+        my_keys[q] = make_uint4(key[0], key[1], key[2], key[3]);
       }
     }
   } else {

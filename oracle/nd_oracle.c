@@ -833,10 +833,14 @@ int ndo_sample_ladies_importance(const ndo_graph* g, const ndo_app_desc* app, ui
         const float imp = (float)imp_fixed;
         const int32_t v = occ[i].vertex;
         uint32_t ctr[4], key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)}, w[4];
-        const uint64_t slot = (uint64_t)(first_sample + s) * (uint64_t)g->n_vertices + (uint64_t)v;
-        ctr[0] = (uint32_t)slot; ctr[1] = (uint32_t)(slot >> 32); ctr[2] = (uint32_t)k; ctr[3] = 0;
+        /* four vertices share a Philox block: pair index P = sample * (|V| rounded up to a
+         * multiple of 4) + v, block P >> 2, word P & 3 */
+        const uint64_t padded_vertices = ((uint64_t)g->n_vertices + 3u) & ~(uint64_t)3;
+        const uint64_t pair = (uint64_t)(first_sample + s) * padded_vertices + (uint64_t)v;
+        const uint64_t block = pair >> 2;
+        ctr[0] = (uint32_t)block; ctr[1] = (uint32_t)(block >> 32); ctr[2] = (uint32_t)k; ctr[3] = 0;
         ndo_philox4x32_10(ctr, key, w);
-        const float u01 = ((float)(w[0] >> 8) + 0.5f) * 5.9604644775390625e-08f;
+        const float u01 = ((float)(w[pair & 3u] >> 8) + 0.5f) * 5.9604644775390625e-08f;
         float keyf;
         if (imp > 0.0f) keyf = ndo_det_log2(u01) / imp;
         else keyf = -__builtin_inff();

@@ -223,7 +223,9 @@ int ndo_sample_fastgcn_importance(const ndo_graph* g, const ndo_app_desc* app, u
  * of the additions), converted to float: the squared column norm of the row-normalised
  * adjacency restricted to the frontier, times 2^53.  m_k vertices are drawn WITHOUT replacement with probability
  * proportional to importance by Efraimidis-Spirakis keys: key(v) = log2(u_v) / importance(v),
- * u_v = ((word >> 8) + 0.5) * 2^-24 from Philox at slot (first_sample + s) * |V| + v, layer k;
+ * u_v = ((word >> 8) + 0.5) * 2^-24, word = word (P & 3) of the Philox block with counter
+ * (P >> 2, layer k, 0), P = (first_sample + s) * (|V| rounded up to a multiple of 4) + v (four
+ * consecutive vertices of a sample share a block);
  * log2 is ndo_det_log2 (single IEEE operations only, so the GPU reproduces it bit for bit).
  * The result is the m_k largest keys in descending key order, ties by ascending vertex id;
  * fewer than m_k distinct vertices leave INVALID.  pinned by brute-force probability

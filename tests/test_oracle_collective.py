@@ -137,7 +137,9 @@ def test_ladies_importance_definition_on_a_tiny_graph(oracle):
     for s in range(50):
         keys = {}
         for v in (2, 3, 4):
-            word = oracle.philox(((s * n + v) & 0xffffffff, (s * n + v) >> 32, 0, 0), (SEED, 0))[0]
+            # pair index P = sample * (|V| rounded up to a multiple of 4) + v: word P & 3 of block P >> 2
+            pair = s * ((n + 3) // 4 * 4) + v
+            word = oracle.philox(((pair >> 2) & 0xffffffff, (pair >> 2) >> 32, 0, 0), (SEED, 0))[pair & 3]
             u = np.float32((np.float32(word >> 8) + np.float32(0.5)) * np.float32(2.0 ** -24))
             keys[v] = np.float32(oracle.lib().ndo_det_log2(float(u))) / imp[v]
         order = sorted(keys, key=lambda v: (-keys[v], v))
