@@ -976,10 +976,7 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
 // <= T (m and some more) are copied out and only those are sorted.
 // The keys of a chunk are dense: keys[s * keys_per_sample + v] for every vertex v (kAbsentKey
 // where sample s does not hold v), so position tells sample and vertex and no list of the
-// distinct pairs is ever written.  The copying takes kSelectTile consecutive vertices of one
-// sample per workgroup: blockIdx.x = tile of the sample, blockIdx.y = sample.
-constexpr uint32_t kSelectPerLane = 32;
-constexpr uint32_t kSelectTile = 256 * kSelectPerLane;
+// distinct pairs is ever written.
 
 // One workgroup per sample, one pass over its keys: forms them where the marking has left sums
 // (keys[s][v] from sums[s][v], Philox slot (first_sample + s) * |V| + v; sums == nullptr: the
@@ -992,10 +989,36 @@ constexpr uint32_t kSelectTile = 256 * kSelectPerLane;
 constexpr uint32_t kSelectBits = 14;
 constexpr uint32_t kSelectBins = 1u << kSelectBits;
 constexpr uint32_t kSelectThreads = 1024;
+// The pass also notes, for every stretch of 256 consecutive keys (what a wavefront handles at a
+// time, four keys per lane), the smallest prefix in it: the copying of the kept entries then
+// reads only the stretches that hold one (a few hundred of a sample's 12,000).
+constexpr uint32_t kCollectStretch = 256;
+__device__ __forceinline__ void note_best_of_stretch(const uint32_t (&key)[4], uint32_t quad, uint32_t lane,
+                                                     uint16_t* __restrict__ best_of) {
+  uint32_t a = key[0] < key[1] ? key[0] : key[1], b = key[2] < key[3] ? key[2] : key[3];
+  uint32_t best = (a < b ? a : b) >> (32u - kSelectBits);  // kAbsentKey: the largest prefix
+  // minimum of the wavefront into lane 63, on the VALU (DPP): along the rows of 16 lanes, then
+  // the last lane of a row into the next row, then lane 31 into the upper half
+  const uint32_t none = 0xFFFFFFFFu;
+  uint32_t other = row_shift_up<1>(none, best);
+  best = other < best ? other : best;
+  other = row_shift_up<2>(none, best);
+  best = other < best ? other : best;
+  other = row_shift_up<4>(none, best);
+  best = other < best ? other : best;
+  other = row_shift_up<8>(none, best);
+  best = other < best ? other : best;
+  other = (uint32_t)__builtin_amdgcn_update_dpp((int)none, (int)best, 0x142, 0xA, 0xF, false);  // row_bcast:15
+  best = other < best ? other : best;
+  other = (uint32_t)__builtin_amdgcn_update_dpp((int)none, (int)best, 0x143, 0xC, 0xF, false);  // row_bcast:31
+  best = other < best ? other : best;
+  if (lane == 63) best_of[quad / 64u] = (uint16_t)best;
+}
 __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(56))) void select_threshold(
     const unsigned long long* __restrict__ sums, uint32_t* __restrict__ keys, uint32_t keys_per_sample,
     uint32_t n_vertices, uint64_t seed, uint64_t first_sample, uint32_t step, uint32_t wanted,
-    uint32_t* __restrict__ threshold, uint32_t* __restrict__ kept, uint32_t* __restrict__ present) {
+    uint32_t* __restrict__ threshold, uint32_t* __restrict__ kept, uint32_t* __restrict__ present,
+    uint16_t* __restrict__ stretch_best) {
   __shared__ uint32_t s_hist[kSelectBins];
   __shared__ uint32_t s_wave_total[kSelectThreads / 64];
   const uint32_t s = blockIdx.x;
@@ -1003,6 +1026,7 @@ __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(5
   for (uint32_t i = threadIdx.x; i < kSelectBins; i += kSelectThreads) s_hist[i] = 0;
   __syncthreads();
   uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  uint16_t* my_best = stretch_best + (size_t)s * (keys_per_sample / kCollectStretch);
   if (sums) {
     // a lane takes four consecutive vertices: their keys come from one Philox block
     // (keys_per_sample is a multiple of 4, and so is the pair index of the sample's vertex 0)
@@ -1034,19 +1058,28 @@ __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(5
           }
         }
         my_keys[q] = make_uint4(key[0], key[1], key[2], key[3]);
+        note_best_of_stretch(key, q, lane, my_best);
       }
     }
   } else {
-    for (uint32_t v0 = 0; v0 < keys_per_sample; v0 += 8 * kSelectThreads) {
-      uint32_t batch[8];
+    const uint4* my_keys = (const uint4*)mine;
+    for (uint32_t q0 = 0; q0 < keys_per_sample / 4u; q0 += 4 * kSelectThreads) {
+      uint4 batch[4];
 #pragma unroll
-      for (uint32_t k = 0; k < 8; ++k) {
-        const uint32_t v = v0 + k * kSelectThreads + threadIdx.x;
-        batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
+        batch[k] = q < keys_per_sample / 4u ? my_keys[q] : make_uint4(kAbsentKey, kAbsentKey, kAbsentKey, kAbsentKey);
       }
 #pragma unroll
-      for (uint32_t k = 0; k < 8; ++k)
-        if (batch[k] != kAbsentKey) atomicAdd(&s_hist[batch[k] >> (32u - kSelectBits)], 1u);
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
+        if (q >= keys_per_sample / 4u) continue;  // whole wavefronts: the sample holds a multiple of 256 keys
+        const uint32_t key[4] = {batch[k].x, batch[k].y, batch[k].z, batch[k].w};
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i)
+          if (key[i] != kAbsentKey) atomicAdd(&s_hist[key[i] >> (32u - kSelectBits)], 1u);
+        note_best_of_stretch(key, q, lane, my_best);
+      }
     }
   }
   __syncthreads();
@@ -1088,43 +1121,50 @@ __device__ __forceinline__ bool select_keeps(uint32_t key, uint32_t threshold) {
   return key != kAbsentKey && (key >> (32u - kSelectBits)) <= threshold;
 }
 
-// Copies the kept entries of sample s into its stretch [ranked_start[s], ranked_start[s + 1]) of
+// Copies the kept entries of sample s into its part [ranked_start[s], ranked_start[s + 1]) of
 // kept_key / kept_id, in whatever order the wavefronts get there (a wavefront claims room for
-// the entries of a round with one atomic; a few hundred of a sample's millions of keys stay,
-// so most rounds claim nothing).  The sorts that follow fix the order.
-__global__ __launch_bounds__(256) void select_collect(const uint32_t* __restrict__ keys, uint32_t keys_per_sample,
+// the entries of a round with one atomic).  A few hundred of a sample's millions of keys stay:
+// one workgroup per sample, whose wavefronts look at the best prefix of each stretch of 256 keys
+// first and read only those that hold a kept key.  The sorts that follow fix the order.
+__global__ __launch_bounds__(kSelectThreads) void select_collect(const uint32_t* __restrict__ keys,
+                                                                 uint32_t keys_per_sample,
+                                                                 const uint16_t* __restrict__ stretch_best,
                                                       const uint32_t* __restrict__ threshold_of,
                                                       const uint32_t* __restrict__ ranked_start,
                                                       uint32_t* __restrict__ claimed, uint32_t* __restrict__ kept_key,
                                                       uint32_t* __restrict__ kept_sample, int32_t* __restrict__ kept_id) {
-  const uint32_t s = blockIdx.y;
+  const uint32_t s = blockIdx.x;
   const uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  const uint32_t stretches = keys_per_sample / kCollectStretch;
+  const uint16_t* best_of = stretch_best + (size_t)s * stretches;
   const uint32_t threshold = threshold_of[s];
   const uint32_t first = ranked_start[s];
-  const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t tile_begin = blockIdx.x * kSelectTile;
-  for (uint32_t k0 = 0; k0 < kSelectPerLane; k0 += 8) {
-    uint32_t batch[8];  // eight loads under way before the first is looked at
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  // a wavefront looks at 64 stretches at a time: lane i knows whether stretch i holds a kept key
+  for (uint32_t stretch_begin = wave * 64u; stretch_begin < stretches; stretch_begin += (kSelectThreads / 64u) * 64u) {
+    const uint32_t my_stretch = stretch_begin + lane;
+    const bool holds = my_stretch < stretches && best_of[my_stretch] <= threshold;
+    uint64_t todo = __ballot(holds);
+    while (todo) {  // the same for every lane
+      const uint32_t stretch = stretch_begin + (uint32_t)__ffsll((long long)todo) - 1u;
+      todo &= todo - 1ull;
+      const uint32_t v0 = stretch * kCollectStretch + lane * 4u;
+      const uint4 four = *(const uint4*)(mine + v0);
+      const uint32_t key[4] = {four.x, four.y, four.z, four.w};
 #pragma unroll
-    for (uint32_t k = 0; k < 8; ++k) {
-      const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
-      batch[k] = v < keys_per_sample ? mine[v] : kAbsentKey;
-    }
-#pragma unroll
-    for (uint32_t k = 0; k < 8; ++k) {
-      const uint32_t v = tile_begin + (k0 + k) * 256 + threadIdx.x;
-      const uint32_t key = batch[k];
-      const bool stays = select_keeps(key, threshold);
-      const uint64_t mask = __ballot(stays);
-      if (mask == 0) continue;  // the same for every lane of the wavefront
-      uint32_t base = 0;
-      if (lane == (uint32_t)__ffsll((long long)mask) - 1u) base = atomicAdd(&claimed[s], (uint32_t)__popcll(mask));
-      base = __shfl(base, __ffsll((long long)mask) - 1, kWave);
-      if (stays) {
-        const uint32_t at = first + base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-        kept_key[at] = key;
-        kept_sample[at] = s;
-        kept_id[at] = (int32_t)v;
+      for (uint32_t i = 0; i < 4; ++i) {
+        const bool stays = select_keeps(key[i], threshold);
+        const uint64_t mask = __ballot(stays);
+        if (mask == 0) continue;
+        uint32_t base = 0;
+        if (lane == (uint32_t)__ffsll((long long)mask) - 1u) base = atomicAdd(&claimed[s], (uint32_t)__popcll(mask));
+        base = __shfl(base, __ffsll((long long)mask) - 1, kWave);
+        if (stays) {
+          const uint32_t at = first + base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+          kept_key[at] = key[i];
+          kept_sample[at] = s;
+          kept_id[at] = (int32_t)(v0 + i);
+        }
       }
     }
   }
@@ -1674,10 +1714,10 @@ class LayerEngine : public EngineBase {
   int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups,
                    uint64_t total) {
     const uint32_t keys_per_sample = bins * kBinVerticesSums;
-    const uint32_t tiles_per_sample = (keys_per_sample + kSelectTile - 1) / kSelectTile;
     if (n > bitmap_samples_) {
-      release(d_keys_dense_); release(d_sums_dense_);
+      release(d_keys_dense_); release(d_sums_dense_); release(d_stretch_best_);
       ND_HIP_TRY(hipMalloc(&d_keys_dense_, sizeof(uint32_t) * (size_t)n * keys_per_sample));
+      ND_HIP_TRY(hipMalloc(&d_stretch_best_, sizeof(uint16_t) * (size_t)n * (keys_per_sample / kCollectStretch)));
       ND_HIP_TRY(hipMalloc(&d_sums_dense_, sizeof(unsigned long long) * (size_t)n * keys_per_sample));
       bitmap_samples_ = n;
     }
@@ -1695,10 +1735,9 @@ class LayerEngine : public EngineBase {
         dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, dense_, keys_out);
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
-    const dim3 tiles(tiles_per_sample, n);
     select_threshold<<<dim3(n), dim3(kSelectThreads), 0, stream_>>>(
         keys_out.keys ? nullptr : d_sums_dense_, d_keys_dense_, keys_per_sample, (uint32_t)invalid_, seed_, (uint64_t)s0,
-        (uint32_t)step, wanted, d_select_threshold_, d_select_kept_, d_select_present_);
+        (uint32_t)step, wanted, d_select_threshold_, d_select_kept_, d_select_present_, d_stretch_best_);
     // where every sample's ranked list starts: exclusive scan of the kept counts
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
     ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
@@ -1711,7 +1750,7 @@ class LayerEngine : public EngineBase {
     for (uint32_t c : present) distinct_total_ += c;
     if (ensure_distinct_capacity(n_kept) != 0) return -1;
     ND_HIP_TRY(hipMemsetAsync(d_select_present_, 0, sizeof(uint32_t) * (size_t)n, stream_));  // now: room claimed
-    select_collect<<<tiles, dim3(256), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_select_threshold_,
+    select_collect<<<dim3(n), dim3(kSelectThreads), 0, stream_>>>(d_keys_dense_, keys_per_sample, d_stretch_best_, d_select_threshold_,
                                                      d_ranked_start_, d_select_present_, d_kept_key_, d_kept_sample_,
                                                      d_kept_id_);
     // order the kept vertices of every sample by descending key, equal keys by ascending
@@ -1787,7 +1826,7 @@ class LayerEngine : public EngineBase {
 
   void release_neighborhood_buffers() {
     release(d_nbr_cols_); release(d_nbr_weights_);
-    release(d_bitmap_); release(d_keys_dense_); release(d_sums_dense_);
+    release(d_bitmap_); release(d_keys_dense_); release(d_sums_dense_); release(d_stretch_best_);
     release(d_group_through_); release(d_part_total_); release(d_part_before_); release(d_marked_);
     release_distinct_buffers();
     capacity_ = 0;
@@ -1838,6 +1877,7 @@ class LayerEngine : public EngineBase {
   // LADIES form: importance sums and sampling keys, [sample][vertex, padded to whole stretches]
   unsigned long long* d_sums_dense_ = nullptr;
   uint32_t* d_keys_dense_ = nullptr;
+  uint16_t* d_stretch_best_ = nullptr;  // LADIES form: best key prefix of every 256 keys of every sample
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
   uint64_t chunk_entries_ = kLayerChunkEntries;
   bool progress_ = false;
