@@ -32,12 +32,12 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
     "fastgcn_importance_rmat22": 6.025e9,    # collective_mark_binned, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 6.79e10,  # collective_mark_binned, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 6.775e10,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
     "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 17.9e9, "ladies_importance_chunglu3m": 212.1e9,
+    "fastgcn_importance_rmat22": 17.9e9, "ladies_importance_chunglu3m": 187.6e9,
 }
 
 WORKLOADS = {
