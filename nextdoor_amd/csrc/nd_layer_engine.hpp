@@ -319,11 +319,11 @@ struct DensePieces {
   const unsigned long long* sums = nullptr;  // LADIES form: 6144 importance sums per piece (kAbsentSum: no edge)
 };
 
-// LADIES form, layers whose samples hold few vertices: the marking kernel turns the sums into
-// sampling keys itself where a stretch leaves LDS and writes those (4 bytes per vertex and
-// sample instead of 8, and the selection's first pass reads 4 instead of 8 and writes nothing).
-// keys == nullptr: the sums are written and the selection forms the keys (dense layers: the key
-// arithmetic of 2.5e9 present vertices next to the streaming took 100 ms instead of 13).
+// LADIES form: the marking kernel turns the importance sums into sampling keys itself where a
+// stretch leaves LDS (a lane takes four consecutive vertices and pays for one Philox block) and
+// writes those, 4 bytes per vertex and sample.  Writing the sums instead and forming the keys in
+// the selection's pass cost 8 + 8 + 4 bytes per vertex and sample of traffic, and 3.4 ms more
+// per pass at full size.
 struct KeysOnTheWayOut {
   uint32_t* keys = nullptr;
   uint64_t seed = 0;
@@ -423,13 +423,13 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
     uint32_t* __restrict__ bitmap,
     uint32_t words_per_sample, const float* __restrict__ inverse_row_sums,
-    unsigned long long* __restrict__ sums, uint32_t keys_per_sample, DensePieces dense, KeysOnTheWayOut keys_out) {
+    uint32_t keys_per_sample, DensePieces dense, KeysOnTheWayOut keys_out) {
   constexpr uint32_t kBinWords = kWithImportance ? kBinVerticesSums / 32u : kBinWordsBits;
   constexpr uint32_t kBinVertices = kBinWords * 32u;
   // FastGCN form: a byte per vertex, set with plain LDS stores (every writer stores 1) and
   // packed into bits on the way out; LADIES form: bits and 64-bit sums, LDS atomics
   __shared__ __align__(16) uint32_t s_bits[kWithImportance ? kBinWords : kBinVertices / 4u];
-  __shared__ unsigned long long s_acc[kWithImportance ? kBinVerticesSums : 1];
+  __shared__ __align__(16) unsigned long long s_acc[kWithImportance ? kBinVerticesSums : 1];
   uint8_t* s_bytes = (uint8_t*)s_bits;
   // the sub-ranges that hold entries, in transit order
   __shared__ uint32_t s_start[kMaxLayerTransits + 1];  // first entry of sub-range k among the stretch's entries
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
     // way out it sets back to zero, so no stretch spends a pass on clearing
     for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
-  } else if (keys_out.keys) {
+  } else {
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
   }
   if (threadIdx.x < tv.count) {
@@ -485,9 +485,8 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
       if (kWithImportance) my_row_sum = inverse_row_sums[t];
     }
   }
-  if (kWithImportance && keys_out.keys && !hubs_among_transits) {
-    // LADIES form, a sample without hubs in a layer that fills few positions: the stretches
-    // of the workgroup as one.  At most kSparseGroupEntriesSums entries: their sums are
+  if (kWithImportance && !hubs_among_transits) {
+    // LADIES form, a sample without hubs: the stretches of the workgroup as one.  At most kSparseGroupEntriesSums entries: their sums are
     // gathered in an LDS table hashed by vertex (in the room of the per-vertex sums), the
     // keys of the whole range are written as absent, and the table's vertices then get theirs.
     // Stretch by stretch, 16 chains of searches, tables and barriers cost a workgroup 130 us
@@ -734,33 +733,38 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
   }
   __syncthreads();
   if (kWithImportance) {
-    // LADIES form: what leaves the workgroup is the importance sum of every vertex of the
-    // stretch (kAbsentSum where the neighbourhood does not hold the vertex); no bitmap.  (The
-    // sampling keys are formed by the first pass of the selection: done here, next to the
-    // streaming of the other workgroup of the compute unit, the same arithmetic took 100 ms
-    // instead of 13.)
-    unsigned long long* out = sums + (size_t)s * keys_per_sample + v_lo;
+    // LADIES form: what leaves the workgroup is the sampling key of every vertex of the
+    // stretch (kAbsentKey where the neighbourhood does not hold the vertex); no bitmap.
+    // A lane takes four consecutive vertices: 16-byte accesses to LDS, to the pieces and to
+    // the output, and one Philox block where it forms keys.
     const uint32_t n_pieces = s_pieces;
-    for (uint32_t i = threadIdx.x; i < kBinVerticesSums; i += kBinThreads) {
-      bool present = ((s_bits[i >> 5] >> (i & 31u)) & 1u) != 0;
-      unsigned long long sum = s_acc[i];  // 0 where nothing was added
+    for (uint32_t q = threadIdx.x; q < kBinVerticesSums / 4u; q += kBinThreads) {
+      const uint32_t i = 4u * q;
+      const uint32_t bits = (s_bits[i >> 5] >> (i & 31u)) & 15u;
+      const ulonglong2 low = ((const ulonglong2*)s_acc)[2u * q], high = ((const ulonglong2*)s_acc)[2u * q + 1u];
+      unsigned long long sum[4] = {low.x, low.y, high.x, high.y};  // 0 where nothing was added
+      bool present[4] = {(bits & 1u) != 0, (bits & 2u) != 0, (bits & 4u) != 0, (bits & 8u) != 0};
 #pragma unroll 4
       for (uint32_t p = 0; p < n_pieces; ++p) {  // integer sums: the order of the additions does not matter
-        const unsigned long long ready = dense.sums[(size_t)s_length[p] * kBinVerticesSums + i];
-        if (ready != kAbsentSum) {
-          sum += ready;
-          present = true;
-        }
+        const ulonglong2* piece = (const ulonglong2*)(dense.sums + (size_t)s_length[p] * kBinVerticesSums + i);
+        const ulonglong2 a = piece[0], b = piece[1];
+        const unsigned long long ready[4] = {a.x, a.y, b.x, b.y};
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+          if (ready[k] != kAbsentSum) {
+            sum[k] += ready[k];
+            present[k] = true;
+          }
       }
-      if (keys_out.keys) {
-        const uint32_t v = v_lo + i;
-        keys_out.keys[(size_t)s * keys_per_sample + v] =
-            present ? ladies_key_bits(sum, ladies_pair_index(keys_out.first_sample + s, keys_out.n_vertices, v),
-                                      keys_out.step, keys_out.seed)
-                    : kAbsentKey;
-      } else {
-        __builtin_nontemporal_store(present ? sum : kAbsentSum, &out[i]);
+      uint32_t key[4] = {kAbsentKey, kAbsentKey, kAbsentKey, kAbsentKey};
+      if (present[0] || present[1] || present[2] || present[3]) {
+        const PhiloxBlock blk = ladies_block(ladies_pair_index(keys_out.first_sample + s, keys_out.n_vertices, v_lo + i),
+                                             keys_out.step, keys_out.seed);
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k)
+          if (present[k]) key[k] = ladies_key_from_word(sum[k], blk.w[k]);
       }
+      *(uint4*)(keys_out.keys + (size_t)s * keys_per_sample + v_lo + i) = make_uint4(key[0], key[1], key[2], key[3]);
     }
   } else {
     const uint32_t first_word = bin * kBinWords;
@@ -978,9 +982,8 @@ __global__ void fill_u32(uint32_t* dst, size_t n, uint32_t value) {
 // where sample s does not hold v), so position tells sample and vertex and no list of the
 // distinct pairs is ever written.
 
-// One workgroup per sample, one pass over its keys: forms them where the marking has left sums
-// (keys[s][v] from sums[s][v], Philox slot (first_sample + s) * |V| + v; sums == nullptr: the
-// keys are there already), counts the present ones by their upper kSelectBits bits in an LDS
+// One workgroup per sample, one pass over its keys: counts the present ones by their upper
+// kSelectBits bits in an LDS
 // histogram and picks the bin that holds the wanted-th smallest key: threshold[s] = that bin,
 // kept[s] = keys up to and including it (a sample with fewer keys than wanted keeps them all),
 // present[s] = all its keys.  A sample's whole histogram stays in the workgroup: no atomic
@@ -1015,8 +1018,7 @@ __device__ __forceinline__ void note_best_of_stretch(const uint32_t (&key)[4], u
   if (lane == 63) best_of[quad / 64u] = (uint16_t)best;
 }
 __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(56))) void select_threshold(
-    const unsigned long long* __restrict__ sums, uint32_t* __restrict__ keys, uint32_t keys_per_sample,
-    uint32_t n_vertices, uint64_t seed, uint64_t first_sample, uint32_t step, uint32_t wanted,
+    const uint32_t* __restrict__ keys, uint32_t keys_per_sample, uint32_t wanted,
     uint32_t* __restrict__ threshold, uint32_t* __restrict__ kept, uint32_t* __restrict__ present,
     uint16_t* __restrict__ stretch_best) {
   __shared__ uint32_t s_hist[kSelectBins];
@@ -1025,43 +1027,9 @@ __global__ __launch_bounds__(kSelectThreads, 8) __attribute__((amdgpu_num_vgpr(5
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   for (uint32_t i = threadIdx.x; i < kSelectBins; i += kSelectThreads) s_hist[i] = 0;
   __syncthreads();
-  uint32_t* mine = keys + (size_t)s * keys_per_sample;
+  const uint32_t* mine = keys + (size_t)s * keys_per_sample;
   uint16_t* my_best = stretch_best + (size_t)s * (keys_per_sample / kCollectStretch);
-  if (sums) {
-    // a lane takes four consecutive vertices: their keys come from one Philox block
-    // (keys_per_sample is a multiple of 4, and so is the pair index of the sample's vertex 0)
-    const ulonglong2* my_sums = (const ulonglong2*)(sums + (size_t)s * keys_per_sample);
-    uint4* my_keys = (uint4*)mine;
-    for (uint32_t q0 = 0; q0 < keys_per_sample / 4u; q0 += 2 * kSelectThreads) {
-      ulonglong2 low[2], high[2];  // two quads under way before the arithmetic starts
-#pragma unroll
-      for (uint32_t k = 0; k < 2; ++k) {
-        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
-        const bool inside = q < keys_per_sample / 4u;
-        low[k] = inside ? my_sums[2u * q] : make_ulonglong2(kAbsentSum, kAbsentSum);
-        high[k] = inside ? my_sums[2u * q + 1u] : make_ulonglong2(kAbsentSum, kAbsentSum);
-      }
-#pragma unroll
-      for (uint32_t k = 0; k < 2; ++k) {
-        const uint32_t q = q0 + k * kSelectThreads + threadIdx.x;
-        if (q >= keys_per_sample / 4u) continue;
-        const unsigned long long four[4] = {low[k].x, low[k].y, high[k].x, high[k].y};
-        uint32_t key[4] = {kAbsentKey, kAbsentKey, kAbsentKey, kAbsentKey};
-        if ((four[0] & four[1] & four[2] & four[3]) != kAbsentSum) {
-          const PhiloxBlock blk = ladies_block(ladies_pair_index(first_sample + s, n_vertices, 4u * q), step, seed);
-#pragma unroll
-          for (uint32_t i = 0; i < 4; ++i) {
-            if (four[i] != kAbsentSum) {
-              key[i] = ladies_key_from_word(four[i], blk.w[i]);
-              atomicAdd(&s_hist[key[i] >> (32u - kSelectBits)], 1u);
-            }
-          }
-        }
-        my_keys[q] = make_uint4(key[0], key[1], key[2], key[3]);
-        note_best_of_stretch(key, q, lane, my_best);
-      }
-    }
-  } else {
+  {
     const uint4* my_keys = (const uint4*)mine;
     for (uint32_t q0 = 0; q0 < keys_per_sample / 4u; q0 += 4 * kSelectThreads) {
       uint4 batch[4];
@@ -1358,8 +1326,7 @@ class LayerEngine : public EngineBase {
     uint64_t bytes_per_sample = (uint64_t)bitmap_words_ * sizeof(uint32_t);
     if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
       const uint32_t bin_words = kBinVerticesSums / 32u;
-      bytes_per_sample = (uint64_t)((bitmap_words_ + bin_words - 1) / bin_words) * kBinVerticesSums *
-                         (sizeof(uint32_t) + sizeof(unsigned long long));
+      bytes_per_sample = (uint64_t)((bitmap_words_ + bin_words - 1) / bin_words) * kBinVerticesSums * sizeof(uint32_t);
     }
     const uint64_t fit = kBitmapBudgetBytes / bytes_per_sample;
     bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
@@ -1607,7 +1574,7 @@ class LayerEngine : public EngineBase {
     TransitView tv = all;
     tv.base = all.base + (size_t)s0 * all.stride;
     if (form != apps::kConcatenated) {
-      if (build_distinct_by_bitmap(step, s0, tv, n, total) != 0) return -1;
+      if (build_distinct_by_bitmap(step, s0, tv, n) != 0) return -1;
     } else {
       // work items of the build: long neighbourhoods are spread over several workgroups
       uint64_t n_items = 0;
@@ -1662,7 +1629,7 @@ class LayerEngine : public EngineBase {
   }
 
   // What next() of the importance forms is handed, for every sample of the chunk.
-  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint64_t total) {
+  int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n) {
     constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
@@ -1670,7 +1637,7 @@ class LayerEngine : public EngineBase {
     const uint32_t groups = (bins + per_group - 1) / per_group;
     if ((uint64_t)n * groups >= (1ull << 31)) { last_error = "a chunk needs 2^31 or more workgroups"; return -1; }
     if constexpr (ladies) {
-      return rank_by_keys(step, s0, tv, n, bins, groups, total);
+      return rank_by_keys(step, s0, tv, n, bins, groups);
     } else {
       return list_distinct(tv, n, bins, groups);
     }
@@ -1693,7 +1660,7 @@ class LayerEngine : public EngineBase {
     }
     tick();
     collective_mark_binned<false><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, nullptr, 0u, dense_, KeysOnTheWayOut());
+        dgraph_.view, tv, invalid_, n, bins, d_bitmap_, bitmap_words_, nullptr, 0u, dense_, KeysOnTheWayOut());
     tock();
     ND_HIP_TRY(hipMemsetAsync(d_marked_, 0, sizeof(uint32_t) * (size_t)n, stream_));
     const uint32_t sample_blocks = (n + kSumSamplesPerBlock - 1) / kSumSamplesPerBlock;
@@ -1711,33 +1678,28 @@ class LayerEngine : public EngineBase {
   // vertices that can be among its first `wanted` in key order are picked by a radix select on
   // the upper 14 bits of the key and ordered by descending key.  The distinct pairs of a
   // sample (2.4 M per batch at full size) are never listed.
-  int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups,
-                   uint64_t total) {
+  int rank_by_keys(int step, uint32_t s0, const TransitView& tv, uint32_t n, uint32_t bins, uint32_t groups) {
     const uint32_t keys_per_sample = bins * kBinVerticesSums;
     if (n > bitmap_samples_) {
-      release(d_keys_dense_); release(d_sums_dense_); release(d_stretch_best_);
+      release(d_keys_dense_); release(d_stretch_best_);
       ND_HIP_TRY(hipMalloc(&d_keys_dense_, sizeof(uint32_t) * (size_t)n * keys_per_sample));
       ND_HIP_TRY(hipMalloc(&d_stretch_best_, sizeof(uint16_t) * (size_t)n * (keys_per_sample / kCollectStretch)));
-      ND_HIP_TRY(hipMalloc(&d_sums_dense_, sizeof(unsigned long long) * (size_t)n * keys_per_sample));
       bitmap_samples_ = n;
     }
-    // a layer that can fill at most one position in 16 forms its keys in the marking kernel
     KeysOnTheWayOut keys_out;
-    if (total * 16 < (uint64_t)n * keys_per_sample) {
-      keys_out.keys = d_keys_dense_;
-      keys_out.seed = seed_;
-      keys_out.first_sample = s0;
-      keys_out.step = (uint32_t)step;
-      keys_out.n_vertices = (uint32_t)invalid_;
-    }
+    keys_out.keys = d_keys_dense_;
+    keys_out.seed = seed_;
+    keys_out.first_sample = s0;
+    keys_out.step = (uint32_t)step;
+    keys_out.n_vertices = (uint32_t)invalid_;
     tick();
     collective_mark_binned<true><<<dim3(n * groups), dim3(kBinThreads), 0, stream_>>>(
-        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, d_sums_dense_, keys_per_sample, dense_, keys_out);
+        dgraph_.view, tv, invalid_, n, bins, nullptr, 0u, d_row_sums_, keys_per_sample, dense_, keys_out);
     tock();
     const uint32_t wanted = (uint32_t)App().stepSize(step);
-    select_threshold<<<dim3(n), dim3(kSelectThreads), 0, stream_>>>(
-        keys_out.keys ? nullptr : d_sums_dense_, d_keys_dense_, keys_per_sample, (uint32_t)invalid_, seed_, (uint64_t)s0,
-        (uint32_t)step, wanted, d_select_threshold_, d_select_kept_, d_select_present_, d_stretch_best_);
+    select_threshold<<<dim3(n), dim3(kSelectThreads), 0, stream_>>>(d_keys_dense_, keys_per_sample, wanted,
+                                                                    d_select_threshold_, d_select_kept_,
+                                                                    d_select_present_, d_stretch_best_);
     // where every sample's ranked list starts: exclusive scan of the kept counts
     fill_u32<<<dim3(1), dim3(1), 0, stream_>>>(d_select_kept_ + n, 1, 0u);
     ND_HIP_TRY(exclusive_scan_u32(d_select_kept_, d_ranked_start_, (size_t)n + 1, d_small_scratch_, stream_));
@@ -1826,7 +1788,7 @@ class LayerEngine : public EngineBase {
 
   void release_neighborhood_buffers() {
     release(d_nbr_cols_); release(d_nbr_weights_);
-    release(d_bitmap_); release(d_keys_dense_); release(d_sums_dense_); release(d_stretch_best_);
+    release(d_bitmap_); release(d_keys_dense_); release(d_stretch_best_);
     release(d_group_through_); release(d_part_total_); release(d_part_before_); release(d_marked_);
     release_distinct_buffers();
     capacity_ = 0;
@@ -1875,7 +1837,6 @@ class LayerEngine : public EngineBase {
   size_t distinct_capacity_ = 0;
   uint32_t* d_bitmap_ = nullptr;
   // LADIES form: importance sums and sampling keys, [sample][vertex, padded to whole stretches]
-  unsigned long long* d_sums_dense_ = nullptr;
   uint32_t* d_keys_dense_ = nullptr;
   uint16_t* d_stretch_best_ = nullptr;  // LADIES form: best key prefix of every 256 keys of every sample
   uint64_t neighborhood_total_ = 0, distinct_total_ = 0, chunks_run_ = 0;
