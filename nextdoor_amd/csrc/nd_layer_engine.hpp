@@ -23,7 +23,8 @@
 //    and a draw searches those sums.
 //  * For kRankedByLadiesImportance each entry also carries (weight * (1 / rowsum(transit)))^2;
 //    the terms of a vertex are summed as 2^53 fixed-point integers (in LDS) into one sum per
-//    (sample, vertex), its Efraimidis-Spirakis key is formed from the sum, a radix select keeps
+//    (sample, vertex), its Efraimidis-Spirakis key is formed from the sum as it leaves LDS (the
+//    only thing stored per sample and vertex), a radix select keeps
 //    the few entries that can be among a sample's first picks, and stable sorts order those by
 //    descending key.
 //  * Samples are processed in chunks whose concatenated neighbourhoods fit a fixed budget
@@ -169,8 +170,9 @@ __host__ __device__ __forceinline__ unsigned long long importance_term_fixed(flo
 // 2.0e9 distinct pairs at FastGCN's full size).  FastGCN form: the result is a bitmap per
 // sample (words_per_sample 32-bit words, a multiple of the tile below).  LADIES form
 // (kWithImportance): every entry also adds (weight * inverse_row_sum[transit])^2, as a 2^53
-// fixed-point integer, to the 64-bit sum of (sample, vertex); the result is that sum for every
-// vertex of every sample, kAbsentSum where the sample's neighbourhood does not hold the vertex.
+// fixed-point integer, to the 64-bit sum of (sample, vertex) in LDS; the result is the sampling
+// key formed from that sum for every vertex of every sample, kAbsentKey where the sample's
+// neighbourhood does not hold the vertex.
 constexpr uint32_t kBitmapTileWords = 2048;  // bitmaps are padded to whole tiles of 65536 vertices (4 parts)
 
 // log2 of a positive normal float from exponent extraction and an atanh series; every step
