@@ -417,9 +417,10 @@ __device__ __forceinline__ void keep_filled_subranges(uint32_t n_transits, uint3
 constexpr uint32_t kSparseGroupEntries = 32768;
 constexpr uint32_t kSparseGroupEntriesSums = 2048;  // LADIES form: sums in an LDS table of twice as many slots
 
-// Two workgroups share a compute unit (8 wavefronts per SIMD) as long as a lane needs at most
-// 56 registers: measured, the LADIES form takes 1.6 times as long with 58 (one workgroup
-// resident) as with 56, whatever the LDS size between 62 and 70 KB.
+// Two workgroups of 16 wavefronts share a compute unit only at 8 wavefronts per SIMD, which the
+// kernel's attributes ask the compiler for.  Measured without them: 63 (LADIES form) and 66
+// registers per lane, 7 wavefronts per SIMD, one workgroup resident, and the LADIES form takes
+// 1.6 times as long; the LDS size (tried: 62 to 70 KB) makes no difference.
 template <bool kWithImportance>
 __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))) void collective_mark_binned(
     CSRPartition csr, TransitView tv, int32_t invalid, uint32_t n_samples, uint32_t bins_per_sample,
