@@ -469,7 +469,20 @@ __global__ __launch_bounds__(kBinThreads, 8) __attribute__((amdgpu_num_vgpr(56))
     // the byte map starts out clear and every stretch leaves it clear: what it reads on the
     // way out it sets back to zero, so no stretch spends a pass on clearing
     for (uint32_t i = threadIdx.x; i < kBinVertices / 4u; i += kBinThreads) s_bits[i] = 0;
+    if (threadIdx.x < tv.count) s_start[threadIdx.x] = (uint32_t)my_transit;  // the table is free until the first stretch
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
+    // A vertex marks the same bits however often it is among the transits, and a layer drawn
+    // with replacement by degree^2 repeats its hubs: 29 distinct transits of 64 at full size,
+    // four fifths of all entries belong to repeats.  Only a vertex's first occurrence counts.
+    if (my_transit != -1) {
+      bool repeated = false;
+      for (uint32_t j = 0; j < threadIdx.x; ++j) repeated |= s_start[j] == (uint32_t)my_transit;
+      if (repeated) {
+        my_transit = -1;
+        my_hub = -1;
+      }
+    }
+    __syncthreads();  // the table is written next
   } else {
     hubs_among_transits = __syncthreads_or(my_hub >= 0) != 0;
   }
