@@ -139,7 +139,7 @@ def marking_bytes_per_pass(graph, sampler, final, ladies):
     for LADIES); with more, the stretch's ready-made piece (a bit per vertex, or a 64-bit sum
     per vertex).  Every layer writes its whole per-sample map (bits, or 32-bit sampling keys).
     FastGCN: a vertex that is among a sample's transits more than once counts once."""
-    stretch = 6144 if ladies else 49152
+    stretch = 6144 if ladies else 65536
     threshold = int(os.environ.get("ND_DENSE_PIECE_ENTRIES", 2048 if ladies else 512))
     piece_bytes = stretch * 8 if ladies else stretch // 8
     entry_bytes = 8 if ladies else 4

@@ -297,14 +297,14 @@ constexpr EdgePos_t kShortRest = 16;          // edges left of an adjacency that
 // sample, and the low ones hold most entries; LADIES form: hundreds of small ones)
 constexpr uint32_t kBinsPerGroupBits = 8;
 constexpr uint32_t kBinsPerGroupSums = 16;
-constexpr uint32_t kBinWordsBits = 1536;      // FastGCN form: 49,152 vertices, one byte each in LDS (48 KB)
+constexpr uint32_t kBinWordsBits = 2048;      // FastGCN form: 65,536 vertices, one byte each in LDS (64 KB)
 constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
 
 // Dense pieces.  What a hub contributes to a stretch can be thousands of entries (a layer
 // drawn by degree^2 sits on the hubs: 144 K entries per transit at FastGCN's full size), and
 // it is the same for every sample that holds the hub.  Where a vertex has kDensePieceEntries
 // (LADIES form: kDensePieceEntriesSums) or more edges into one stretch, the stretch's piece of
-// that vertex is built once per graph - FastGCN form: its bitmap (1536 words); LADIES form:
+// that vertex is built once per graph - FastGCN form: its bitmap (2048 words); LADIES form:
 // the importance sum of every vertex of the stretch (6144 64-bit integers, kAbsentSum where
 // there is no edge; the sums are integers, so adding a piece gives the bits that adding its
 // edges one by one gives) - and a sample ORs / adds the piece on the stretch's way out of LDS
@@ -317,7 +317,7 @@ constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
 struct DensePieces {
   const int32_t* hub_row = nullptr;  // nullptr: the graph has none
   const uint32_t* piece_of = nullptr;
-  const uint32_t* words = nullptr;            // FastGCN form: 1536 words of bits per piece
+  const uint32_t* words = nullptr;            // FastGCN form: 2048 words of bits per piece
   const unsigned long long* sums = nullptr;  // LADIES form: 6144 importance sums per piece (kAbsentSum: no edge)
 };
 
