@@ -31,13 +31,13 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "weighted_node2vec_rmat22": 1.246e9,     # step_flat_kernel
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
-    "fastgcn_importance_rmat22": 6.431e9,    # collective_mark_binned, average over its 2 launches per pass
+    "fastgcn_importance_rmat22": 5.273e9,    # collective_mark_binned, average over its 2 launches per pass
     "ladies_importance_chunglu3m": 6.507e10,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
     "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 18.7e9, "ladies_importance_chunglu3m": 156.8e9,
+    "fastgcn_importance_rmat22": 16.4e9, "ladies_importance_chunglu3m": 156.8e9,
 }
 
 WORKLOADS = {
@@ -140,7 +140,7 @@ def marking_bytes_per_pass(graph, sampler, final, ladies):
     per vertex).  Every layer writes its whole per-sample map (bits, or 32-bit sampling keys).
     FastGCN: a vertex that is among a sample's transits more than once counts once."""
     stretch = 6144 if ladies else 65536
-    threshold = int(os.environ.get("ND_DENSE_PIECE_ENTRIES", 2048 if ladies else 512))
+    threshold = int(os.environ.get("ND_DENSE_PIECE_ENTRIES", 2048 if ladies else 1024))
     piece_bytes = stretch * 8 if ladies else stretch // 8
     entry_bytes = 8 if ladies else 4
     rp, col = np.asarray(graph.row_ptr), np.asarray(graph.col)

@@ -310,7 +310,7 @@ constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit su
 // edges one by one gives) - and a sample ORs / adds the piece on the stretch's way out of LDS
 // instead of going through the entries.  hub_row[v] = row of v in piece_of or -1;
 // piece_of[row * stretches + stretch] = piece index or kNoPiece.
-constexpr uint32_t kDensePieceEntries = 512;
+constexpr uint32_t kDensePieceEntries = 1024;
 constexpr uint32_t kDensePieceEntriesSums = 2048;  // LADIES form: a piece is 6144 64-bit sums
 constexpr size_t kDensePieceBudgetBytes = (size_t)2 << 30;
 constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
