@@ -32,12 +32,12 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
     "fastgcn_importance_rmat22": 5.273e9,    # collective_mark_binned, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 6.507e10,  # collective_mark_binned, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 6.71e10,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
     "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 16.4e9, "ladies_importance_chunglu3m": 156.8e9,
+    "fastgcn_importance_rmat22": 16.4e9, "ladies_importance_chunglu3m": 160.8e9,
 }
 
 WORKLOADS = {
@@ -139,7 +139,7 @@ def marking_bytes_per_pass(graph, sampler, final, ladies):
     for LADIES); with more, the stretch's ready-made piece (a bit per vertex, or a 64-bit sum
     per vertex).  Every layer writes its whole per-sample map (bits, or 32-bit sampling keys).
     FastGCN: a vertex that is among a sample's transits more than once counts once."""
-    stretch = 6144 if ladies else 65536
+    stretch = 7168 if ladies else 65536
     threshold = int(os.environ.get("ND_DENSE_PIECE_ENTRIES", 2048 if ladies else 1024))
     piece_bytes = stretch * 8 if ladies else stretch // 8
     entry_bytes = 8 if ladies else 4
@@ -169,7 +169,7 @@ def marking_bytes_per_pass(graph, sampler, final, ladies):
         pieces += int(c) * int(ready.sum())
         entries += int(c) * int(per_stretch[~ready].sum())
     words = ((graph.n_vertices + 31) // 32 + 2047) // 2048 * 2048  # a bit per vertex, padded to 2048 words
-    per_sample_out = (words + 191) // 192 * 6144 * 4 if ladies else words * 4  # LADIES: a 32-bit key per vertex
+    per_sample_out = (words + 223) // 224 * 7168 * 4 if ladies else words * 4  # LADIES: a 32-bit key per vertex
     written = sampler.steps * n_samples * per_sample_out
     return entries * entry_bytes + pieces * piece_bytes + written, entries, pieces
 

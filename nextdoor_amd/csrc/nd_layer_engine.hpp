@@ -298,27 +298,27 @@ constexpr EdgePos_t kShortRest = 16;          // edges left of an adjacency that
 constexpr uint32_t kBinsPerGroupBits = 8;
 constexpr uint32_t kBinsPerGroupSums = 16;
 constexpr uint32_t kBinWordsBits = 2048;      // FastGCN form: 65,536 vertices, one byte each in LDS (64 KB)
-constexpr uint32_t kBinVerticesSums = 6144;   // LADIES form: 48 KB of 64-bit sums + 768 B of bits
+constexpr uint32_t kBinVerticesSums = 7168;   // LADIES form: 56 KB of 64-bit sums + 896 B of bits
 
 // Dense pieces.  What a hub contributes to a stretch can be thousands of entries (a layer
 // drawn by degree^2 sits on the hubs: 144 K entries per transit at FastGCN's full size), and
 // it is the same for every sample that holds the hub.  Where a vertex has kDensePieceEntries
 // (LADIES form: kDensePieceEntriesSums) or more edges into one stretch, the stretch's piece of
 // that vertex is built once per graph - FastGCN form: its bitmap (2048 words); LADIES form:
-// the importance sum of every vertex of the stretch (6144 64-bit integers, kAbsentSum where
+// the importance sum of every vertex of the stretch (7168 64-bit integers, kAbsentSum where
 // there is no edge; the sums are integers, so adding a piece gives the bits that adding its
 // edges one by one gives) - and a sample ORs / adds the piece on the stretch's way out of LDS
 // instead of going through the entries.  hub_row[v] = row of v in piece_of or -1;
 // piece_of[row * stretches + stretch] = piece index or kNoPiece.
 constexpr uint32_t kDensePieceEntries = 1024;
-constexpr uint32_t kDensePieceEntriesSums = 2048;  // LADIES form: a piece is 6144 64-bit sums
+constexpr uint32_t kDensePieceEntriesSums = 2048;  // LADIES form: a piece is 7168 64-bit sums
 constexpr size_t kDensePieceBudgetBytes = (size_t)2 << 30;
 constexpr uint32_t kNoPiece = 0xFFFFFFFFu;
 struct DensePieces {
   const int32_t* hub_row = nullptr;  // nullptr: the graph has none
   const uint32_t* piece_of = nullptr;
   const uint32_t* words = nullptr;            // FastGCN form: 2048 words of bits per piece
-  const unsigned long long* sums = nullptr;  // LADIES form: 6144 importance sums per piece (kAbsentSum: no edge)
+  const unsigned long long* sums = nullptr;  // LADIES form: 7168 importance sums per piece (kAbsentSum: no edge)
 };
 
 // LADIES form: the marking kernel turns the importance sums into sampling keys itself where a

@@ -129,7 +129,7 @@ def test_importance_sampling_with_ready_made_hub_pieces(oracle, app, monkeypatch
 @pytest.mark.parametrize("app", ["FastGCNImportance3x16", "LADIESImportance3x16"])
 @pytest.mark.parametrize("pieces", ["default", "8", "0"])
 def test_importance_sampling_over_several_stretches(oracle, app, pieces, monkeypatch):
-    """130,000 vertices: two stretches of the FastGCN form, 22 of the LADIES form (two
+    """130,000 vertices: two stretches of the FastGCN form, 19 of the LADIES form (two
     workgroups per sample), a hub with edges into all of them."""
     if pieces != "default":
         monkeypatch.setenv("ND_DENSE_PIECE_ENTRIES", pieces)
