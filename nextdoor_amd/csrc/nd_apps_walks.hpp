@@ -161,11 +161,12 @@ struct Node2VecAppT : Sizing {
   }
 };
 
-// Weighted second-order walk (p = 2, q = 0.5).  Bias of candidate v reached over edge x
-// from transit u, with t the vertex visited before u:
+// Weighted second-order walk, p = kPNum / kPDen and q = kQNum / kQDen (default p = 2,
+// q = 0.5).  Bias of candidate v reached over edge x from transit u, with t the vertex
+// visited before u:
 //   h = p if v == t, 1/q if v is adjacent to t, else 1   (h = 1 at step 0: no t yet)
 // accepted when uniform * max_weight(u) * max(p, 1/q, 1) < h * weight(x).
-template <int kWalkLength>
+template <int kWalkLength, int kPNum = 2, int kPDen = 1, int kQNum = 1, int kQDen = 2>
 struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
   static constexpr bool kUsesEdgeWeights = true;
   static constexpr bool kUsesEdgeLookup = true;
@@ -180,7 +181,7 @@ struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
       sample->t = *transits;
       return transitEdges[0];
     }
-    const float p = 2.0f, q = 0.5f;
+    const float p = (float)kPNum / (float)kPDen, q = (float)kQNum / (float)kQDen;
     const float h_max = fmaxf(fmaxf(p, 1 / q), 1.0f), h_min = fminf(fminf(p, 1 / q), 1.0f);
     const float envelope = max_weight * h_max;
     VertexID prev = -1;  // read from the sample only when a decision depends on it

@@ -89,6 +89,9 @@ const AppEntry kApps[] = {
     // short variants for quick checks
     {"UniformRandomWalk8", make_engine<UniformRandomWalkSample, UniformRandomWalkAppT<8>>},
     {"WeightedNode2Vec8", make_engine<Node2VecSample, WeightedNode2VecAppT<8>>},
+    // the same walk with p = 4, q = 0.5 and with p = 0.5, q = 4: the three biases p, 1/q and 1 all differ
+    {"WeightedNode2Vec8P4Q05", make_engine<Node2VecSample, WeightedNode2VecAppT<8, 4, 1, 1, 2>>},
+    {"WeightedNode2Vec8P05Q4", make_engine<Node2VecSample, WeightedNode2VecAppT<8, 1, 2, 4, 1>>},
     {"KHop3x2", make_engine<KHopSample, KHopAppT<3, 2>>},
     {"KHop4x3x2", make_engine<KHopSample, KHopAppT<4, 3, 2>>},
     {"KHop40x30", make_engine<KHopSample, KHopAppT<40, 30>>},

@@ -10,8 +10,10 @@
  * Parity status of each function is stated next to its declaration:
  *   "pinned by ..."     - an independent check exists in tests/ (KAT, closed form,
  *                         brute force, special case reducing to a library routine)
- *   "parity unpinned"   - semantics are this repo's own definition; the reference
- *                         holds no vector or test for it.
+ *   "parity unpinned"   - no independent check pins the function.
+ * A sampler that is this repository's own definition (the reference has no such app) says
+ * so; what pins it is then its stated mathematical definition: a draw-by-draw evaluation
+ * written apart from this file, and the distribution it must produce.
  */
 #ifndef ND_ORACLE_H
 #define ND_ORACLE_H
@@ -30,7 +32,8 @@ enum ndo_app_kind {
   NDO_DEEPWALK = 1,          /* src/apps/randomwalks/randomWalks.cu:65-91   */
   NDO_PPR = 2,               /* src/apps/randomwalks/randomWalks.cu:93-125  */
   NDO_NODE2VEC = 3,          /* src/apps/randomwalks/randomWalks.cu:132-173 */
-  NDO_WEIGHTED_NODE2VEC = 4, /* this repo's weighted variant; parity unpinned */
+  NDO_WEIGHTED_NODE2VEC = 4, /* this repo's weighted variant (no counterpart in the reference);
+                                pinned by a draw-by-draw trace and chi-square over all three biases */
   NDO_KHOP = 5,              /* src/apps/khop/khop.cu:10-23                 */
   NDO_LAYER_LITERAL = 6,     /* src/apps/fastgcn/fastgcnSampling.cu:23-47 and
                                 src/apps/ladies/ladiessampling.cu:23-47 (identical bodies) */
@@ -99,8 +102,9 @@ int ndo_max_bits(int32_t n_vertices);                                /* nextdoor
  * state_t (may be NULL): Node2VecSample::t per sample after the last step.
  * Uniform/k-hop: pinned by closed forms on path/star/complete graphs;
  * DeepWalk: pinned by equal-weight reduction + chi-square; Node2Vec literal: pinned by
- * hand-traced cases; weighted node2vec: parity unpinned (own definition) beyond
- * distribution checks. */
+ * hand-traced cases; weighted node2vec (own definition): pinned by a draw-by-draw trace at
+ * (p, q) = (4, 0.5), (0.5, 4), (2, 0.5) that visits the return, adjacent and far branch, and by
+ * chi-square against bias * weight where p, 1/q and 1 all differ. */
 int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t seed,
                           int64_t n_samples, int64_t first_sample,
                           const int32_t* initial, int32_t* final_samples,

@@ -48,8 +48,8 @@ def make_graph():
     return row_ptr, col, w
 
 
-def desc(kind, steps, sizes, initial_size=1):
-    return ob.app_desc(kind, steps, sizes, initial_size=initial_size)
+def desc(kind, steps, sizes, initial_size=1, p=2.0, q=0.5):
+    return ob.app_desc(kind, steps, sizes, initial_size=initial_size, p=p, q=q)
 
 
 def main():
@@ -59,8 +59,8 @@ def main():
     ids = np.arange(V, dtype=np.int32)
     out = {"seed": SEED, "graph": {"row_ptr": row_ptr, "col": col, "weight": w}, "apps": {}}
 
-    def individual(app, kind, steps, sizes, with_state=False):
-        d = desc(kind, steps, sizes)
+    def individual(app, kind, steps, sizes, with_state=False, p=2.0, q=0.5):
+        d = desc(kind, steps, sizes, p=p, q=q)
         final, state = ob.sample_individual(g, d, SEED, ids)
         entry = {"initial": ids.tolist(), "final": final.reshape(-1).tolist(), "shape": list(final.shape)}
         if with_state:
@@ -69,6 +69,8 @@ def main():
 
     individual("UniformRandomWalk8", ob.UNIFORM_WALK, 8, 1)
     individual("WeightedNode2Vec8", ob.WEIGHTED_NODE2VEC, 8, 1, with_state=True)
+    individual("WeightedNode2Vec8P4Q05", ob.WEIGHTED_NODE2VEC, 8, 1, with_state=True, p=4.0, q=0.5)
+    individual("WeightedNode2Vec8P05Q4", ob.WEIGHTED_NODE2VEC, 8, 1, with_state=True, p=0.5, q=4.0)
     individual("DeepWalkPerVertex", ob.DEEPWALK, 100, 1)
     individual("PPRPerVertex", ob.PPR, 100, 1)
     individual("Node2VecPerVertex", ob.NODE2VEC, 100, 1, with_state=True)

@@ -37,7 +37,7 @@ def test_oracle_still_produces_the_committed_vectors(oracle, tmp_path, monkeypat
     assert fresh == load("sampler_vectors.json")
 
 
-APPS = ["UniformRandomWalk8", "WeightedNode2Vec8", "DeepWalkPerVertex", "PPRPerVertex", "Node2VecPerVertex",
+APPS = ["UniformRandomWalk8", "WeightedNode2Vec8", "WeightedNode2Vec8P4Q05", "WeightedNode2Vec8P05Q4", "DeepWalkPerVertex", "PPRPerVertex", "Node2VecPerVertex",
         "KHop3x2", "KHop4x3x2", "MultiRW4x6", "LayerLiteral2x8", "FastGCNImportance2x8", "LADIESImportance2x8",
         "MVS5", "ClusterGCN3x2"]
 

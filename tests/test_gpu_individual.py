@@ -12,10 +12,15 @@ pytestmark = pytest.mark.gpu
 SEED = 42
 
 
-def desc_for(oracle, sampler, kind):
+# return and in-out parameters of the registered weighted node2vec instances (default 2, 0.5)
+P_AND_Q = {"WeightedNode2Vec8P4Q05": (4.0, 0.5), "WeightedNode2Vec8P05Q4": (0.5, 4.0)}
+
+
+def desc_for(oracle, sampler, kind, app=None):
     steps = sampler.steps
+    p, q = P_AND_Q.get(app, (2.0, 0.5))
     return oracle.app_desc(kind, steps, [sampler.step_size(k) for k in range(steps)],
-                           initial_size=sampler.initial_sample_size)
+                           initial_size=sampler.initial_sample_size, p=p, q=q)
 
 
 def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True), inversion_period=1):
@@ -23,7 +28,7 @@ def run_and_compare(oracle, app, kind, g, check_state=False, modes=(False, True)
     s = nd.Sampler(app, g, seed=SEED)
     s.set_inversion_period(inversion_period)
     try:
-        d = desc_for(oracle, s, kind)
+        d = desc_for(oracle, s, kind, app)
         roots = s.initial_contents
         assert s.invalid_vertex == g.n_vertices
         want, want_state = oracle.sample_individual(og, d, SEED, roots)
@@ -147,6 +152,8 @@ def test_command_line_runs_checks_and_prints(oracle, tmp_path):
 GRAPHS = {
     "sparse": dict(n=300, mean_degree=3, seed=1, isolated_every=7),
     "dense_hub": dict(n=2000, mean_degree=12, seed=2, hub=5),
+    # a tenth of all vertex pairs joined: a candidate is often a neighbour of the previous vertex
+    "triangles": dict(n=160, mean_degree=16, seed=5, hub=7),
 }
 
 
@@ -157,12 +164,26 @@ GRAPHS = {
     ("PPRPerVertex", "PPR", False),
     ("Node2VecPerVertex", "NODE2VEC", True),
     ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+    ("WeightedNode2Vec8P4Q05", "WEIGHTED_NODE2VEC", True),
+    ("WeightedNode2Vec8P05Q4", "WEIGHTED_NODE2VEC", True),
     ("KHop", "KHOP", False),
     ("KHop4x3x2", "KHOP", False),
 ])
 def test_app_matches_oracle(oracle, app, kind_name, state, gname):
     g = graphs.random_graph(**GRAPHS[gname])
     run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+
+
+def test_weighted_node2vec_instances_differ_where_the_biases_do(oracle):
+    # p = 4, q = 0.5 against p = 0.5, q = 4 on a graph full of triangles: were the bias of a
+    # candidate adjacent to the previous vertex mixed up with p or with 1, the two instances (or
+    # one of them and the oracle) would agree where they must not
+    g = graphs.random_graph(**GRAPHS["triangles"])
+    a = run_and_compare(oracle, "WeightedNode2Vec8P4Q05", oracle.WEIGHTED_NODE2VEC, g, check_state=True)
+    b = run_and_compare(oracle, "WeightedNode2Vec8P05Q4", oracle.WEIGHTED_NODE2VEC, g, check_state=True)
+    c = run_and_compare(oracle, "WeightedNode2Vec8", oracle.WEIGHTED_NODE2VEC, g, check_state=True)
+    assert np.array_equal(a[:, 0], b[:, 0]) and np.array_equal(a[:, 0], c[:, 0])  # step 0 knows no p, q
+    assert (a[:, 1:] != b[:, 1:]).mean() > 0.2 and (a[:, 1:] != c[:, 1:]).mean() > 0.05
 
 
 def test_reference_sized_deepwalk_has_100_walks_per_vertex(oracle):

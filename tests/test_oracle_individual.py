@@ -240,6 +240,90 @@ def test_weighted_node2vec_distribution(oracle):
     assert chi2 < 20.5
 
 
+def weighted_node2vec_graph():
+    # node2vec_graph() with weights that are exact in float32 and all different per vertex
+    adj = node2vec_graph()
+    w = [[1.0, 2.5, 4.0], [3.0, 1.5, 2.0], [1.0, 2.0, 3.0, 4.0, 2.5], [4.5, 1.0, 3.5], [2.0], [1.5]]
+    return adj, w
+
+
+@pytest.mark.parametrize("p,q", [(4.0, 0.5), (0.5, 4.0), (2.0, 0.5)])
+def test_weighted_node2vec_trace(oracle, p, q):
+    # Draw-by-draw evaluation of the definition: candidate i uses draw 2i for the edge index and
+    # draw 2i + 1 for the height; h = p when the candidate IS the previous vertex, 1/q when it is
+    # another neighbour of the previous vertex, 1 otherwise (and at step 0); accepted when
+    # u * (max_weight * max(p, 1/q, 1)) < h * weight.  With p != 1/q != 1 the three branches give
+    # different outcomes, so none of them can be swapped for another unnoticed.
+    adj, w = weighted_node2vec_graph()
+    g = oracle.Graph.from_adjacency(adj, w)
+    n, steps = len(adj), 8
+    f32 = np.float32
+    inv_q = f32(1.0) / f32(q)
+    h_max = max(f32(p), inv_q, f32(1.0))
+    S = 40 * n  # 40 walks per root: enough draws to hit every branch many times
+    roots = np.arange(S) % n
+    final, state = oracle.sample_individual(g, oracle.app_desc(oracle.WEIGHTED_NODE2VEC, steps, 1, p=p, q=q), SEED,
+                                            roots)
+    seen = {"return": 0, "adjacent": 0, "far": 0, "rejected": 0}
+    for s in range(S):
+        cur, t = int(roots[s]), None
+        for k in range(steps):
+            nb = sorted(zip(adj[cur], w[cur]))
+            if len(nb) == 1:
+                nxt = nb[0][0]
+            else:
+                envelope = f32(max(x[1] for x in nb)) * h_max
+                draw = 0
+                while True:
+                    x = rint(oracle.uniform(SEED, s, k, draw), len(nb))
+                    y = f32(oracle.uniform(SEED, s, k, draw + 1)) * envelope
+                    draw += 2
+                    v, wx = nb[x][0], f32(nb[x][1])
+                    if k == 0:
+                        h, branch = f32(1.0), None
+                    elif v == t:
+                        h, branch = f32(p), "return"
+                    elif v in adj[t]:
+                        h, branch = inv_q, "adjacent"
+                    else:
+                        h, branch = f32(1.0), "far"
+                    if y < h * wx:
+                        nxt = v
+                        if branch:
+                            seen[branch] += 1
+                        break
+                    seen["rejected"] += 1
+            t, cur = cur, nxt
+            assert final[s, k] == cur, (s, k)
+        assert state[s] == t
+    assert min(seen.values()) > 50, seen
+
+
+@pytest.mark.parametrize("p,q", [(4.0, 0.5), (0.5, 4.0)])
+def test_weighted_node2vec_distribution_over_all_three_biases(oracle, p, q):
+    # walks 0 -> 2 -> ?: the previous vertex is t = 0 and the candidates of 2 are 0 (== t: bias p),
+    # 1 and 3 (neighbours of 0, not 0 itself: bias 1/q), 4 and 5 (bias 1); P(v) ~ bias * weight
+    adj, w = weighted_node2vec_graph()
+    g = oracle.Graph.from_adjacency(adj, w)
+    S = 240000
+    final, _ = oracle.sample_individual(g, oracle.app_desc(oracle.WEIGHTED_NODE2VEC, 2, 1, p=p, q=q), SEED,
+                                        np.zeros(S, np.int32))
+    second = final[final[:, 0] == 2, 1]  # the draws of step 1 are independent of those of step 0
+    assert len(second) > S // 5
+    bias = np.array([p, 1 / q, 1 / q, 1.0, 1.0]) * np.array(w[2])
+    counts = np.array([(second == v).sum() for v in (0, 1, 3, 4, 5)], dtype=float)
+    assert counts.sum() == len(second)
+    expected = len(second) * bias / bias.sum()
+    chi2 = ((counts - expected) ** 2 / expected).sum()
+    assert chi2 < 20.5  # 4 dof, p ~ 4e-4
+    # and the bias of the adjacent candidates is not the one of the other branches: with h = p
+    # or h = 1 in their place the expected counts would be off by far more than the threshold
+    for wrong in (p, 1.0):
+        alt = np.array([p, wrong, wrong, 1.0, 1.0]) * np.array(w[2])
+        alt = len(second) * alt / alt.sum()
+        assert ((counts - alt) ** 2 / alt).sum() > 1000
+
+
 def test_weighted_node2vec_step0_is_a_weighted_pick(oracle):
     adj = [[1, 2, 3, 4], [0], [0], [0], [0]]
     w = [[1.0, 2.0, 3.0, 4.0], [1.0], [1.0], [1.0], [1.0]]
