@@ -183,6 +183,18 @@ int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, in
  * (key, value) by the low key_bits bits.  vals == NULL: value = index. */
 int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_bits, int32_t* keys_out,
                   int32_t* vals_out);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): nd_sort_pairs on
+ * DEVICE arrays, enqueued on `stream` (a hipStream_t; NULL = the default stream) without
+ * waiting for it, with all working memory in a fixed array inside the library
+ * (ND_SORT_PAIRS_NOALLOC_MAX pairs at most: 8.5 MiB per GPU, held until the process ends).
+ * Calls no hipMalloc / hipFree / memset.  d_vals == NULL: value = index.  The output arrays
+ * must not be the input arrays.  More than ND_SORT_PAIRS_NOALLOC_MAX pairs: returns -2.  All
+ * calls on one GPU share the working array: calls that overlap on one GPU (two streams, two
+ * host threads) race; calls on one stream are ordered by the stream. */
+#define ND_SORT_PAIRS_NOALLOC_MAX 1048576
+int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t n, int key_bits, int32_t* d_keys_out,
+                          int32_t* d_vals_out, void* stream);
 /* invalidVertexStartPos + DeviceRunLengthEncode::Encode + DeviceScan::ExclusiveSum
  * (src/nextdoor.cu:1804-1836, 2535-2545, 2560-2567) over a sorted key array. */
 int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,

@@ -22,7 +22,7 @@ from . import _capi
 from ._capi import NextDoorError, check, lib
 
 __all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
-           "sort_pairs", "unique_transits", "collective_neighborhood", "check_sampled_vertices"]
+           "sort_pairs", "sort_pairs_noalloc", "unique_transits", "collective_neighborhood", "check_sampled_vertices"]
 
 
 def app_names():
@@ -323,6 +323,16 @@ def sort_pairs(keys, vals, key_bits):
     check(lib().nd_sort_pairs(_ptr(keys, C.c_int32), None if v is None else _ptr(v, C.c_int32), len(keys), key_bits,
                               _ptr(ko, C.c_int32), _ptr(vo, C.c_int32)))
     return ko, vo
+
+
+SORT_PAIRS_NOALLOC_MAX = 1 << 20  # ND_SORT_PAIRS_NOALLOC_MAX of include/nextdoor_amd.h
+
+
+def sort_pairs_noalloc(d_keys, d_vals, n, key_bits, d_keys_out, d_vals_out, stream=0):
+    """nd_sort_pairs_noalloc: the sort on DEVICE arrays given as addresses (integers; d_vals 0 =
+    value is the index), enqueued on `stream` (a hipStream_t as an integer, 0 = default stream)
+    with all working memory inside the library; allocates nothing and does not wait."""
+    check(lib().nd_sort_pairs_noalloc(d_keys, d_vals or None, n, key_bits, d_keys_out, d_vals_out, stream or None))
 
 
 def unique_transits(sorted_keys, invalid):

@@ -5,6 +5,7 @@
 
 #include <exception>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -147,6 +148,45 @@ __global__ void philox_fill_kernel(uint64_t seed, uint32_t step, uint64_t first_
 __global__ void run_counts_kernel(const uint32_t* run_start, const nd::RunsMeta* meta, uint32_t* counts) {
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r < meta->n_runs) counts[r] = run_start[r + 1] - run_start[r];
+}
+
+// Working memory of nd_sort_pairs_noalloc: one ping-pong side of the sort (keys, values), the
+// digit table and the digit totals, for at most ND_SORT_PAIRS_NOALLOC_MAX pairs.  Every GPU the
+// library runs on holds its own copy of the array, at its own address, until the process ends.
+constexpr size_t kNoAllocMaxPairs = ND_SORT_PAIRS_NOALLOC_MAX;
+constexpr size_t kNoAllocTiles = (kNoAllocMaxPairs + (size_t)nd::kSortThreads * nd::kSortItemsSmall - 1) /
+                                 ((size_t)nd::kSortThreads * nd::kSortItemsSmall);
+constexpr size_t kNoAllocKeysAt = 0;
+constexpr size_t kNoAllocValsAt = kNoAllocKeysAt + kNoAllocMaxPairs;
+constexpr size_t kNoAllocHistAt = kNoAllocValsAt + kNoAllocMaxPairs;
+constexpr size_t kNoAllocTotalsAt = kNoAllocHistAt + (size_t)nd::kRadix * kNoAllocTiles;
+constexpr size_t kNoAllocWords = kNoAllocTotalsAt + nd::kRadix;
+static_assert(kNoAllocMaxPairs < nd::kSortLargeFrom, "the digit table is sized for the small sort tile");
+
+static __device__ __align__(256) uint32_t scratch[kNoAllocWords];
+
+// Address of `scratch` on each device.  In host code the array's name is only a stand-in for
+// the symbol, not a device address: the address is asked for once per device, with that device
+// current, and everything below uses the pointer.
+constexpr int kMaxDevices = 64;
+uint32_t* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+hipError_t scratch_on_current_device(uint32_t** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = (uint32_t*)p;
+  }
+  *out = g_scratch_ptr[device];
+  return hipSuccess;
 }
 
 #define CAPI_HIP(expr)                                                                        \
@@ -531,7 +571,7 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
     if (n == 0) return 0;
     if (n >= (int64_t)1 << 31) return fail("too many pairs");
     const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);
-    DeviceBuffer k_in, v_in, k_a, v_a, k_b, v_b, hist, scratch;
+    DeviceBuffer k_in, v_in, k_a, v_a, k_b, v_b, hist, totals;
     const size_t bytes = sizeof(uint32_t) * (size_t)n;
     CAPI_HIP(k_in.alloc(bytes));
     CAPI_HIP(k_a.alloc(bytes));
@@ -539,7 +579,7 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
     CAPI_HIP(k_b.alloc(bytes));
     CAPI_HIP(v_b.alloc(bytes));
     CAPI_HIP(hist.alloc(sizeof(uint32_t) * plan.hist_elems));
-    CAPI_HIP(scratch.alloc(sizeof(uint32_t) * plan.scratch_elems));
+    CAPI_HIP(totals.alloc(sizeof(uint32_t) * plan.scratch_elems));
     CAPI_HIP(hipMemcpy(k_in.p, keys, bytes, hipMemcpyHostToDevice));
     if (vals) {
       CAPI_HIP(v_in.alloc(bytes));
@@ -548,10 +588,43 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
     uint32_t *k_sorted = nullptr, *v_sorted = nullptr;
     CAPI_HIP(nd::radix_sort_pairs(plan, k_in.as<uint32_t>(), vals ? v_in.as<uint32_t>() : nullptr, k_a.as<uint32_t>(),
                                   v_a.as<uint32_t>(), k_b.as<uint32_t>(), v_b.as<uint32_t>(), hist.as<uint32_t>(),
-                                  scratch.as<uint32_t>(), 0, &k_sorted, &v_sorted));
+                                  totals.as<uint32_t>(), 0, &k_sorted, &v_sorted));
     CAPI_HIP(hipDeviceSynchronize());
     CAPI_HIP(hipMemcpy(keys_out, k_sorted, bytes, hipMemcpyDeviceToHost));
     CAPI_HIP(hipMemcpy(vals_out, v_sorted, bytes, hipMemcpyDeviceToHost));
+    return 0;
+  });
+}
+
+int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t n, int key_bits, int32_t* d_keys_out,
+                          int32_t* d_vals_out, void* stream) {
+  return guarded([&]() -> int {
+    if (n < 0 || key_bits < 1 || key_bits > 32 || (n > 0 && (!d_keys || !d_keys_out || !d_vals_out)))
+      return fail("bad argument");
+    if ((uint64_t)n > kNoAllocMaxPairs)
+      return fail("nd_sort_pairs_noalloc sorts at most " + std::to_string(kNoAllocMaxPairs) + " pairs, " +
+                  std::to_string(n) + " given (use nd_sort_pairs)", -2);
+    if (n == 0) return 0;
+    if (d_keys_out == d_keys || (d_vals && d_vals_out == d_vals)) return fail("the sort is not in place");
+    uint32_t* work = nullptr;
+    CAPI_HIP(scratch_on_current_device(&work));
+    const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);
+    // the digit passes alternate between the caller's output arrays and the scratch side, in
+    // the order that makes the last pass land in the output arrays
+    const bool first_to_out = plan.passes % 2 == 1;
+    nd::SortJob job;
+    job.keys_in = (const uint32_t*)d_keys;
+    job.vals_in = (const uint32_t*)d_vals;
+    job.keys_a = first_to_out ? (uint32_t*)d_keys_out : work + kNoAllocKeysAt;
+    job.vals_a = first_to_out ? (uint32_t*)d_vals_out : work + kNoAllocValsAt;
+    job.keys_b = first_to_out ? work + kNoAllocKeysAt : (uint32_t*)d_keys_out;
+    job.vals_b = first_to_out ? work + kNoAllocValsAt : (uint32_t*)d_vals_out;
+    // every word of the digit table and the totals that a pass reads, the pass has written
+    // before: nothing of the previous call's contents is used and nothing needs clearing
+    job.hist = work + kNoAllocHistAt;
+    job.scratch = work + kNoAllocTotalsAt;
+    CAPI_HIP(nd::radix_sort(plan, job, (hipStream_t)stream));
+    if (job.keys_sorted != (uint32_t*)d_keys_out) return fail("internal error: result outside the output arrays");
     return 0;
   });
 }
@@ -565,16 +638,16 @@ int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, i
     *n_valid = 0;
     if (n == 0) return 0;
     const size_t bytes = sizeof(uint32_t) * (size_t)n;
-    DeviceBuffer keys, run_key, run_start, run_count, meta, scratch;
+    DeviceBuffer keys, run_key, run_start, run_count, meta, scan_tmp;
     CAPI_HIP(keys.alloc(bytes));
     CAPI_HIP(run_key.alloc(bytes));
     CAPI_HIP(run_start.alloc(bytes + sizeof(uint32_t)));
     CAPI_HIP(run_count.alloc(bytes));
     CAPI_HIP(meta.alloc(sizeof(nd::RunsMeta)));
-    CAPI_HIP(scratch.alloc(sizeof(uint32_t) * nd::runs_scratch_elems((size_t)n)));
+    CAPI_HIP(scan_tmp.alloc(sizeof(uint32_t) * nd::runs_scratch_elems((size_t)n)));
     CAPI_HIP(hipMemcpy(keys.p, sorted_keys, bytes, hipMemcpyHostToDevice));
     CAPI_HIP(nd::find_transit_runs(keys.as<uint32_t>(), (size_t)n, (uint32_t)invalid, run_key.as<uint32_t>(),
-                                   run_start.as<uint32_t>(), meta.as<nd::RunsMeta>(), scratch.as<uint32_t>(), 0));
+                                   run_start.as<uint32_t>(), meta.as<nd::RunsMeta>(), scan_tmp.as<uint32_t>(), 0));
     run_counts_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(run_start.as<uint32_t>(),
                                                                              meta.as<nd::RunsMeta>(),
                                                                              run_count.as<uint32_t>());
