@@ -134,10 +134,16 @@ int nd_sampler_get_adjacency(nd_sampler* s, const int32_t** rows, const int32_t*
  * nd_sampler_do_transit_parallel; nd_sampler_get_final_samples then returns the packed rows. */
 int nd_sampler_distinct(nd_sampler* s);
 int nd_sampler_get_distinct_counts(const nd_sampler* s, const int32_t** data, int64_t* length);
-/* Sizes the last run worked on, for traffic accounting.  Layer-wise apps: which 0 = entries
- * of all collective neighbourhoods built, 1 = distinct (sample, vertex) pairs found,
- * 2 = chunks of samples processed, 3 = ready-made stretch bitmaps of the graph's hubs (built
- * by nd_sampler_set_graph for the FastGCN importance form); other apps return 0. */
+/* Sizes the last run worked on.  Layer-wise apps: which 0 = entries of all collective
+ * neighbourhoods built, 1 = distinct (sample, vertex) pairs found, 2 = chunks of samples
+ * processed, 3 = ready-made stretch bitmaps of the graph's hubs (built by nd_sampler_set_graph for
+ * the FastGCN importance form).  Per-transit apps, after a load-balanced pass, the pairs per
+ * kernel class summed over its steps (what the reference's printKernelTypes shows,
+ * src/nextdoor.cu:2117-2189): 0 = pairs the classifications looked at, 1 = of these, pairs on
+ * transits the workgroup kernel served as one work item, 2 = pairs on transits split over several
+ * work items (grid-wide), 3 = pairs in runs long enough for the workgroup kernel that stayed with
+ * the flat kernel because of the transit's degree, 4 = work items; the flat kernel served
+ * 0 minus 1 minus 2.  Edge-list apps: 0 = edges listed. */
 int64_t nd_sampler_counter(const nd_sampler* s, int which);
 /* The validators the reference's apps pass to nextdoor() as checkResultsFunc
  * (src/check_results.cu): checkSampledVerticesResult (162-299) for the per-transit apps and
@@ -199,6 +205,23 @@ int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t 
  * (src/nextdoor.cu:1804-1836, 2535-2545, 2560-2567) over a sorted key array. */
 int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
                        int32_t* offsets, int64_t* n_runs, int64_t* n_valid);
+
+/* partitionTransitsInKernels with its thresholds (src/nextdoor.cu:1520-1802, src/utils.hpp:491-497)
+ * over a sorted key array, as the engine runs it between the inversion and the step kernels:
+ * degrees[v] = edges of vertex v; a run of `count` equal keys goes to the workgroup kernel when
+ * count * step_size >= thresholds[0], the transit has edges and staging its adjacency pays (at
+ * most thresholds[2] edges unless partial_cache != 0, which stages the first thresholds[2] and
+ * reads the rest from memory; and no more than 32 staged edges per output); such a run is cut
+ * into work items of at most thresholds[1] / step_size pairs: items[2 i] = first pair,
+ * items[2 i + 1] = pairs, in no particular order; taken[v] = 1 for the transits so served (the flat
+ * kernel skips their pairs).  *n_items = items wanted (those beyond `capacity` are not written and
+ * their transit is then not marked).  counters: 0 pairs looked at, 1 pairs in single-item runs,
+ * 2 pairs in runs cut into several items (grid-wide), 3 pairs in runs long enough but refused for
+ * their degree, 4 items.  pairs_per_lane: 1 or 16, the two launch shapes the engine uses. */
+int nd_load_balancing_thresholds(int32_t thresholds[3]);
+int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,
+                     int partial_cache, int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items,
+                     uint8_t* taken, int64_t counters[5]);
 
 /* collectiveNeighbrsSize + collectiveNeighborhood (src/nextdoor.cu:1206-1283) for n_samples
  * samples of transits_per_sample transits each (transits[s * transits_per_sample + i]):

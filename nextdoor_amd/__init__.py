@@ -22,7 +22,7 @@ from . import _capi
 from ._capi import NextDoorError, check, lib
 
 __all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
-           "sort_pairs", "sort_pairs_noalloc", "unique_transits", "collective_neighborhood", "check_sampled_vertices"]
+           "sort_pairs", "sort_pairs_noalloc", "unique_transits", "classify_runs", "load_balancing_thresholds", "collective_neighborhood", "check_sampled_vertices"]
 
 
 def app_names():
@@ -323,6 +323,27 @@ def sort_pairs(keys, vals, key_bits):
     check(lib().nd_sort_pairs(_ptr(keys, C.c_int32), None if v is None else _ptr(v, C.c_int32), len(keys), key_bits,
                               _ptr(ko, C.c_int32), _ptr(vo, C.c_int32)))
     return ko, vo
+
+
+def load_balancing_thresholds():
+    """(outputs a transit needs for the workgroup kernel, outputs per work item, edges the LDS cache holds)"""
+    out = np.zeros(3, np.int32)
+    check(lib().nd_load_balancing_thresholds(_ptr(out, C.c_int32)))
+    return tuple(int(x) for x in out)
+
+
+def classify_runs(sorted_keys, degrees, step_size, partial_cache=True, pairs_per_lane=1, capacity=None):
+    """The load-balancing classification over a sorted key array: (items [k, 2] = first pair and
+    pairs of every work item, items wanted, taken [n_vertices], counters [5])."""
+    keys, degrees = _as(sorted_keys, np.int32), _as(degrees, np.int32)
+    capacity = capacity or max(len(keys), 1)
+    items = np.zeros((capacity, 2), np.int32)
+    taken = np.zeros(len(degrees), np.uint8)
+    counters, wanted = np.zeros(5, np.int64), C.c_int64()
+    check(lib().nd_classify_runs(_ptr(keys, C.c_int32), len(keys), _ptr(degrees, C.c_int32), len(degrees), step_size,
+                                 int(partial_cache), pairs_per_lane, _ptr(items, C.c_int32), capacity,
+                                 C.byref(wanted), _ptr(taken, C.c_uint8), _ptr(counters, C.c_int64)))
+    return items[:min(wanted.value, capacity)], wanted.value, taken, counters
 
 
 SORT_PAIRS_NOALLOC_MAX = 1 << 20  # ND_SORT_PAIRS_NOALLOC_MAX of include/nextdoor_amd.h

@@ -67,6 +67,9 @@ SIGNATURES = {
     "nd_philox_fill_uniform": (C.c_int, [C.c_uint64, C.c_uint32, C.c_uint64, C.c_int64, C.c_int, c_f32p]),
     "nd_sort_pairs": (C.c_int, [c_i32p, c_i32p, C.c_int64, C.c_int, c_i32p, c_i32p]),
     "nd_sort_pairs_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nd_load_balancing_thresholds": (C.c_int, [c_i32p]),
+    "nd_classify_runs": (C.c_int, [c_i32p, C.c_int64, c_i32p, C.c_int32, C.c_int, C.c_int, C.c_int, c_i32p, C.c_int64,
+                                   c_i64p, C.POINTER(C.c_uint8), c_i64p]),
     "nd_collective_neighborhood": (C.c_int, [C.c_void_p, c_i32p, C.c_int64, C.c_int32, C.c_int32, c_i32p, c_i32p, c_i32p,
                                              c_f32p, C.c_int64, c_i32p]),
     "nd_unique_transits": (C.c_int, [c_i32p, C.c_int64, C.c_int32, c_i32p, c_i32p, c_i32p, c_i64p, c_i64p]),

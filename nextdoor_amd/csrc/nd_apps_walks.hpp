@@ -57,6 +57,17 @@ struct OneWalkPerVertex : WalkCommon<kWalkLength> {
   }
 };
 
+// Several walks rooted at every vertex: sample i starts at vertex i mod |V|.
+template <int kWalkLength, int kWalksPerVertex>
+struct WalksPerVertex : WalkCommon<kWalkLength> {
+  __host__ __device__ EdgePos_t numSamples(CSR* graph) { return kWalksPerVertex * graph->get_n_vertices(); }
+
+  template <class SampleType>
+  __host__ std::vector<VertexID_t> initialSample(int sampleIdx, CSR* graph, SampleType&) {
+    return std::vector<VertexID_t>(1, sampleIdx % graph->get_n_vertices());
+  }
+};
+
 // The reference's RandomWalkApp sizing (randomWalks.cu:23-37): small graphs get 100
 // walks per vertex, roots wrap around the vertex range.
 template <int kWalkLength>
@@ -166,10 +177,16 @@ struct Node2VecAppT : Sizing {
 // visited before u:
 //   h = p if v == t, 1/q if v is adjacent to t, else 1   (h = 1 at step 0: no t yet)
 // accepted when uniform * max_weight(u) * max(p, 1/q, 1) < h * weight(x).
-template <int kWalkLength, int kPNum = 2, int kPDen = 1, int kQNum = 1, int kQDen = 2>
-struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
+template <int kWalkLength, int kPNum = 2, int kPDen = 1, int kQNum = 1, int kQDen = 2,
+          class Sizing = nd::apps::OneWalkPerVertex<kWalkLength>>
+struct WeightedNode2VecAppT : Sizing {
   static constexpr bool kUsesEdgeWeights = true;
   static constexpr bool kUsesEdgeLookup = true;
+
+  __host__ __device__ static float return_bias() { return (float)kPNum / (float)kPDen; }        // p
+  __host__ __device__ static float adjacent_bias() { return 1 / ((float)kQNum / (float)kQDen); }  // 1/q
+  __host__ __device__ static float largest_bias() { return fmaxf(fmaxf(return_bias(), adjacent_bias()), 1.0f); }
+  __host__ __device__ static float smallest_bias() { return fminf(fminf(return_bias(), adjacent_bias()), 1.0f); }
 
   template <typename SampleType, typename EdgeArray, typename WeightArray>
   __device__ inline VertexID next(int step, CSRPartition* csr, const VertexID* transits, const VertexID,
@@ -181,29 +198,30 @@ struct WeightedNode2VecAppT : nd::apps::OneWalkPerVertex<kWalkLength> {
       sample->t = *transits;
       return transitEdges[0];
     }
-    const float p = (float)kPNum / (float)kPDen, q = (float)kQNum / (float)kQDen;
-    const float h_max = fmaxf(fmaxf(p, 1 / q), 1.0f), h_min = fminf(fminf(p, 1 / q), 1.0f);
-    const float envelope = max_weight * h_max;
+    const float envelope = max_weight * largest_bias();
     VertexID prev = -1;  // read from the sample only when a decision depends on it
-    // h is one of {p, 1/q, 1}: a height below h_min * w is accepted and one not below
-    // h_max * w rejected whatever h is, so only the band in between needs the adjacency test
-    auto accepts = [&](VertexID v, float wx, float y) -> bool {
-      if (step == 0) return y < wx;  // no previous vertex yet: h = 1
-      if (y < h_min * wx) return true;
-      if (!(y < h_max * wx)) return false;
-      if (prev < 0) prev = sample->t;
-      float h = 1.0f;
-      if (v == prev) h = p;
-      else if (csr->has_edge_logn(prev, v)) h = 1 / q;
-      return y < h * wx;
-    };
     // candidate i consumes draws 2i (edge index) and 2i+1 (height)
     for (;;) {
       const EdgePos_t x = RandNumGen::rand_int(state, numEdges);
       const float y = curand_uniform(state) * envelope;
       const VertexID v = transitEdges[x];
       const float wx = transitEdgeWeights[x];
-      if (accepts(v, wx, y)) {
+      bool accepted;
+      if (step == 0) {
+        accepted = y < wx;  // no previous vertex yet: bias 1
+      } else if (y < smallest_bias() * wx) {
+        accepted = true;    // the bias is one of {p, 1/q, 1}: below the smallest, accepted whatever it is
+      } else if (!(y < largest_bias() * wx)) {
+        accepted = false;   // not below the largest: rejected whatever it is
+      } else {
+        // only in the band between does the candidate's relation to the previous vertex matter
+        if (prev < 0) prev = sample->t;
+        float h = 1.0f;
+        if (v == prev) h = return_bias();
+        else if (csr->has_edge_logn(prev, v)) h = adjacent_bias();
+        accepted = y < h * wx;
+      }
+      if (accepted) {
         sample->t = *transits;
         return v;
       }

@@ -87,6 +87,9 @@ const AppEntry kApps[] = {
     {"PPRPerVertex", make_engine<DummySample, PPRPerVertexApp>},
     {"Node2VecPerVertex", make_engine<Node2VecSample, Node2VecPerVertexApp>},
     {"WeightedNode2Vec", make_engine<Node2VecSample, WeightedNode2VecApp>},
+    // four weighted second-order walks per vertex
+    {"WeightedNode2Vec4PerVertex",
+     make_engine<Node2VecSample, WeightedNode2VecAppT<100, 2, 1, 1, 2, nd::apps::WalksPerVertex<100, 4>>>},
     // short variants for quick checks
     {"UniformRandomWalk8", make_engine<UniformRandomWalkSample, UniformRandomWalkAppT<8>>},
     {"WeightedNode2Vec8", make_engine<Node2VecSample, WeightedNode2VecAppT<8>>},
@@ -625,6 +628,92 @@ int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t 
     job.scratch = work + kNoAllocTotalsAt;
     CAPI_HIP(nd::radix_sort(plan, job, (hipStream_t)stream));
     if (job.keys_sorted != (uint32_t*)d_keys_out) return fail("internal error: result outside the output arrays");
+    return 0;
+  });
+}
+
+int nd_load_balancing_thresholds(int32_t out[3]) {
+  if (!out) return fail("null argument");
+  out[0] = (int32_t)nd::kWorkgroupWork;
+  out[1] = (int32_t)nd::kChunkOutputs;
+  out[2] = (int32_t)nd::kCacheEdges;
+  return 0;
+}
+
+int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,
+                     int partial_cache, int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items,
+                     uint8_t* taken, int64_t counters[5]) {
+  return guarded([&]() -> int {
+    if (n < 0 || n_vertices < 1 || step_size < 1 || capacity < 1 || !degrees || !items || !n_items || !taken ||
+        !counters || (n > 0 && !sorted_keys) || n >= (1ll << 31) || capacity >= (1ll << 31) ||
+        (pairs_per_lane != 1 && pairs_per_lane != nd::kClassifyItemsLarge))
+      return fail("bad argument");
+    for (int64_t i = 0; i < n; ++i)
+      if (sorted_keys[i] < 0 || sorted_keys[i] >= n_vertices || (i > 0 && sorted_keys[i] < sorted_keys[i - 1]))
+        return fail("keys must be vertices in ascending order");
+    std::vector<EdgePos_t> row_ptr((size_t)n_vertices + 1, 0);
+    for (int32_t v = 0; v < n_vertices; ++v) {
+      if (degrees[v] < 0) return fail("negative degree");
+      row_ptr[(size_t)v + 1] = row_ptr[v] + degrees[v];
+    }
+    *n_items = 0;
+    for (int i = 0; i < 5; ++i) counters[i] = 0;
+    memset(taken, 0, (size_t)n_vertices);
+    if (n == 0) return 0;
+    DeviceBuffer d_keys, d_n, d_meta, d_rows, d_items, d_taken, d_balance;
+    constexpr size_t kFoundWords = nd::kMaxSteps + 2;
+    CAPI_HIP(d_keys.alloc(sizeof(uint32_t) * (size_t)n));
+    CAPI_HIP(d_n.alloc(sizeof(uint32_t)));
+    CAPI_HIP(d_meta.alloc(sizeof(nd::RunsMeta) * 2));
+    CAPI_HIP(d_rows.alloc(sizeof(EdgePos_t) * row_ptr.size()));
+    CAPI_HIP(d_items.alloc(sizeof(uint32_t) * 2 * (size_t)capacity));
+    CAPI_HIP(d_taken.alloc((size_t)n_vertices));
+    constexpr size_t kCounterBytes = sizeof(nd::ClassCounters) * nd::kCounterCopies;
+    CAPI_HIP(d_balance.alloc(sizeof(uint32_t) * kFoundWords + kCounterBytes));
+    const uint32_t n32 = (uint32_t)n;
+    CAPI_HIP(hipMemcpy(d_keys.p, sorted_keys, sizeof(uint32_t) * (size_t)n, hipMemcpyHostToDevice));
+    CAPI_HIP(hipMemcpy(d_n.p, &n32, sizeof(n32), hipMemcpyHostToDevice));
+    CAPI_HIP(hipMemcpy(d_rows.p, row_ptr.data(), sizeof(EdgePos_t) * row_ptr.size(), hipMemcpyHostToDevice));
+    CAPI_HIP(hipMemset(d_meta.p, 0, sizeof(nd::RunsMeta) * 2));
+    CAPI_HIP(hipMemset(d_taken.p, 0, (size_t)n_vertices));
+    CAPI_HIP(hipMemset(d_balance.p, 0, sizeof(uint32_t) * kFoundWords + kCounterBytes));
+    nd::RunsMeta* meta = d_meta.as<nd::RunsMeta>();
+    nd::ClassCounters* d_counters = (nd::ClassCounters*)(d_balance.as<uint32_t>() + kFoundWords);
+    if (pairs_per_lane == 1) {
+      nd::classify_run_tails<1><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(
+          d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
+          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint8_t>(), d_counters, partial_cache ? 1u : 0u,
+          d_balance.as<uint32_t>(), 1u);
+    } else {
+      const int64_t per_block = 256 * nd::kClassifyItemsLarge;
+      nd::classify_run_tails<nd::kClassifyItemsLarge><<<dim3((unsigned)((n + per_block - 1) / per_block)), dim3(256), 0, 0>>>(
+          d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
+          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint8_t>(), d_counters, partial_cache ? 1u : 0u,
+          d_balance.as<uint32_t>(), 1u);
+    }
+    CAPI_HIP(hipGetLastError());
+    CAPI_HIP(hipDeviceSynchronize());
+    nd::RunsMeta h;
+    nd::ClassCounters copies[nd::kCounterCopies], c = nd::ClassCounters();
+    CAPI_HIP(hipMemcpy(&h, meta, sizeof(h), hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(copies, d_counters, sizeof(copies), hipMemcpyDeviceToHost));
+    for (const nd::ClassCounters& one : copies) {
+      c.sorted_pairs += one.sorted_pairs;
+      c.workgroup_pairs += one.workgroup_pairs;
+      c.split_pairs += one.split_pairs;
+      c.refused_pairs += one.refused_pairs;
+      c.work_items += one.work_items;
+    }
+    // the kernel counts every item it wants; those beyond the capacity were not written
+    *n_items = h.n_chunks;
+    const int64_t written = h.n_chunks < capacity ? (int64_t)h.n_chunks : capacity;
+    CAPI_HIP(hipMemcpy(items, d_items.p, sizeof(uint32_t) * 2 * (size_t)written, hipMemcpyDeviceToHost));
+    CAPI_HIP(hipMemcpy(taken, d_taken.p, (size_t)n_vertices, hipMemcpyDeviceToHost));
+    counters[0] = (int64_t)c.sorted_pairs;
+    counters[1] = (int64_t)c.workgroup_pairs;
+    counters[2] = (int64_t)c.split_pairs;
+    counters[3] = (int64_t)c.refused_pairs;
+    counters[4] = (int64_t)c.work_items;
     return 0;
   });
 }

@@ -87,33 +87,43 @@ class CSRPartition {
   __host__ __device__ __forceinline__ const CSR::Edge* get_edges(VertexID v) const { return edges + row_ptr[v]; }
   __host__ __device__ __forceinline__ const float* get_weights(VertexID v) const { return weights + row_ptr[v]; }
 
-  // Optional exact edge index: open-addressing table of (src << 32 | dst) keys over all
-  // edges, at most half full, empty slots all-ones.  Built by the engine for apps that
-  // declare kUsesEdgeLookup; nullptr otherwise.
+  // Optional exact edge index over all edges, built by the engine for apps that declare
+  // kUsesEdgeLookup; nullptr otherwise.  Keys are (src << 32 | dst), empty slots all-ones.
+  // The table is made of buckets of kEdgeBucket consecutive keys (32 bytes, aligned: one
+  // bucket is fetched with two 16-byte loads, i.e. one memory round trip); a key lives in the
+  // first bucket, counted from the one its hash names, that had room when it was inserted, and
+  // a bucket fills from its first slot on.  With at most a quarter of the slots in use a
+  // bucket holds one key on average and overflows into its neighbour for one key in some
+  // hundreds: the answer nearly always takes ONE round trip, found or not.  (A table of
+  // single keys, half full, needs 1.5 dependent round trips for a key that is there and 2.5
+  // for one that is not - and a wavefront waits for its slowest lane.)
+  static constexpr uint32_t kEdgeBucket = 4;
   const unsigned long long* edge_table;
-  uint32_t edge_table_mask;
+  uint32_t edge_table_mask;  // number of buckets - 1 (a power of two)
 
-  __host__ __device__ __forceinline__ static uint32_t edge_hash(unsigned long long key) {
-    key ^= key >> 33;
-    key *= 0xff51afd7ed558ccdull;
-    key ^= key >> 33;
-    key *= 0xc4ceb9fe1a85ec53ull;
-    key ^= key >> 33;
-    return (uint32_t)key;
+  __host__ __device__ __forceinline__ static uint32_t edge_hash(uint32_t src, uint32_t dst) {
+    uint32_t h = src * 0x9E3779B1u ^ dst * 0x85EBCA77u;
+    h ^= h >> 15;
+    h *= 0x2C1B3C6Du;
+    h ^= h >> 12;
+    h *= 0x297A2D39u;
+    h ^= h >> 15;
+    return h;
   }
 
   // Is dst in the adjacency of src?  The reference answers with a binary search of the
   // sorted adjacency (src/csr.hpp:342-359); with the edge index present the same answer
-  // comes from one or two probes of the table instead of log2(degree) dependent loads.
+  // comes from the key's bucket instead of log2(degree) dependent loads.
   __host__ __device__ __forceinline__ bool has_edge_logn(VertexID src, VertexID dst) const {
     if (edge_table != nullptr) {
       const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)dst;
-      uint32_t h = edge_hash(key) & edge_table_mask;
+      uint32_t bucket = edge_hash((uint32_t)src, (uint32_t)dst) & edge_table_mask;
       for (;;) {
-        const unsigned long long k = edge_table[h];
-        if (k == key) return true;
-        if (k == ~0ull) return false;
-        h = (h + 1) & edge_table_mask;
+        const ulonglong2* keys = (const ulonglong2*)(edge_table + (size_t)bucket * kEdgeBucket);
+        const ulonglong2 first = keys[0], second = keys[1];
+        if (first.x == key || first.y == key || second.x == key || second.y == key) return true;
+        if (second.y == ~0ull) return false;  // the bucket has room: the key was never pushed past it
+        bucket = (bucket + 1) & edge_table_mask;
       }
     }
     EdgePos_t l = row_ptr[src];

@@ -25,16 +25,23 @@ __device__ __forceinline__ VertexID source_of_edge(const EdgePos_t* row_ptr, Ver
   return lo;
 }
 
-__global__ void build_edge_table(CSRPartition csr, unsigned long long* table, uint32_t mask) {
+// One lane per edge: the key goes into the first free slot of the first bucket with room,
+// counted from the bucket its hash names.  Slots of a bucket are tried in order, so a bucket
+// fills from its first slot on; a duplicate edge finds its key on the way and stops.
+__global__ void build_edge_table(CSRPartition csr, unsigned long long* table, uint32_t bucket_mask) {
   const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= (size_t)csr.n_edges) return;
   const VertexID src = source_of_edge(csr.row_ptr, csr.n_vertices, (EdgePos_t)e);
-  const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)csr.edges[e];
-  uint32_t h = CSRPartition::edge_hash(key) & mask;
+  const VertexID dst = csr.edges[e];
+  const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)dst;
+  uint32_t bucket = CSRPartition::edge_hash((uint32_t)src, (uint32_t)dst) & bucket_mask;
   for (;;) {
-    const unsigned long long seen = atomicCAS(&table[h], ~0ull, key);
-    if (seen == ~0ull || seen == key) return;  // inserted, or a duplicate edge already there
-    h = (h + 1) & mask;
+    unsigned long long* slots = table + (size_t)bucket * CSRPartition::kEdgeBucket;
+    for (uint32_t i = 0; i < CSRPartition::kEdgeBucket; ++i) {
+      const unsigned long long seen = atomicCAS(&slots[i], ~0ull, key);
+      if (seen == ~0ull || seen == key) return;  // inserted, or a duplicate edge already there
+    }
+    bucket = (bucket + 1) & bucket_mask;
   }
 }
 
@@ -88,14 +95,15 @@ class DeviceGraph {
       ND_GRAPH_TRY(hipGetLastError());
     }
     if (want_edge_table) {
-      size_t slots = 16;  // power of two, at most half full
-      while (slots < 2 * E) slots <<= 1;
+      size_t slots = 16;  // power of two, at most a quarter full
+      while (slots < 4 * E) slots <<= 1;
+      const size_t buckets = slots / CSRPartition::kEdgeBucket;
       ND_GRAPH_TRY(hipMalloc(&edge_table_, sizeof(unsigned long long) * slots));
       ND_GRAPH_TRY(hipMemset(edge_table_, 0xFF, sizeof(unsigned long long) * slots));
-      if (E) build_edge_table<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(view, edge_table_, (uint32_t)(slots - 1));
+      if (E) build_edge_table<<<dim3((unsigned)((E + 255) / 256)), dim3(256)>>>(view, edge_table_, (uint32_t)(buckets - 1));
       ND_GRAPH_TRY(hipGetLastError());
       view.edge_table = edge_table_;
-      view.edge_table_mask = (uint32_t)(slots - 1);
+      view.edge_table_mask = (uint32_t)(buckets - 1);
     }
     ND_GRAPH_TRY(hipDeviceSynchronize());
 #undef ND_GRAPH_TRY

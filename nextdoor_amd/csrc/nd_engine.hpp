@@ -27,6 +27,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <chrono>
 #include <memory>
@@ -532,6 +533,21 @@ __device__ __forceinline__ uint32_t run_start(const uint32_t* __restrict__ keys,
   return lo;
 }
 
+// Pairs per kernel class, summed over the load-balanced steps of a pass (what the reference's
+// printKernelTypes shows per step, src/nextdoor.cu:2117-2189).
+struct ClassCounters {
+  unsigned long long sorted_pairs;     // pairs the inversions kept and the classification looked at
+  unsigned long long workgroup_pairs;  // on transits served by the workgroup kernel as one work item
+  unsigned long long split_pairs;      // on transits split over several work items (grid-wide)
+  unsigned long long refused_pairs;    // in runs long enough for the workgroup kernel that stay with the flat
+                                       // kernel because of the transit's degree
+  unsigned long long work_items;       // work items handed to the workgroup kernel
+};
+// The counters are kept in kCounterCopies copies, a wavefront adding to copy (its number mod
+// kCounterCopies), and summed on the host: atomics on one address are served one after the
+// other, and a k-hop step has more than 10^5 qualifying runs.
+constexpr uint32_t kCounterCopies = 64;
+
 constexpr uint32_t kDirectSegment = 16;  // ids: segments this long are written straight into the result rows
 // Consecutive pairs per lane of classify_run_tails: many for large maps (fewer atomics),
 // one for small ones (the launch is latency bound: 3.4 vs 1.8 ms over the 99 steps of 4.2 M walks).
@@ -540,10 +556,15 @@ constexpr uint32_t kClassifyLargeFrom = 16u << 20;  // pairs
 
 // Is pair i the last of a run that the workgroup kernel should take?  Gives the run and the
 // number of work items it needs.
+// partial_cache: a transit whose adjacency is longer than the LDS cache may go to the workgroup
+// kernel too, with its first kCacheEdges edges in LDS and the rest read from memory (the
+// reference's CachedArray, src/nextdoor.cu:76-124).  refused_out (nullable): set to the run's
+// length when the run is long enough but stays with the flat kernel because of the degree.
 __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict__ keys, uint32_t i, uint32_t n,
                                                       const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
-                                                      uint32_t* transit_out, uint32_t* start_out, uint32_t* count_out,
-                                                      uint32_t* n_items_out) {
+                                                      bool partial_cache, uint32_t* transit_out, uint32_t* start_out,
+                                                      uint32_t* count_out, uint32_t* n_items_out,
+                                                      uint32_t* refused_out = nullptr) {
   const uint32_t transit = keys[i];
   if (i + 1 != n && keys[i + 1] == transit) return false;  // not the last pair of its run
   // pairs a run needs for the workgroup kernel; a shorter run is ruled out with one read
@@ -554,7 +575,12 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
   const uint64_t work = (uint64_t)count * step_size;
   if (work < kWorkgroupWork) return false;
   const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
-  if (degree == 0 || degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) return false;
+  if (degree == 0) return false;
+  const uint32_t staged = degree < (uint32_t)kCacheEdges ? degree : (uint32_t)kCacheEdges;
+  if ((degree > (uint32_t)kCacheEdges && !partial_cache) || (uint64_t)staged > 32ull * work) {
+    if (refused_out) *refused_out = count;
+    return false;
+  }
   uint32_t pairs_per_chunk = kChunkOutputs / step_size;
   if (pairs_per_chunk == 0) pairs_per_chunk = 1;
   *transit_out = transit;
@@ -570,27 +596,60 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
 // order in the list is irrelevant to the results.  The list is sized so that every claim
 // fits (see Engine::alloc); should one not fit, the transit is left to the flat kernel and
 // the entries that did fit are processed twice with identical results.
+// When the classification of the step before found nothing for the workgroup kernel (or did not
+// look), this one only looks every kQuietLookEvery-th step: on a map where no transit carries
+// enough pairs, as with one walk per vertex of a large graph, most launches end at once.
+// found_by_step[k] != 0: step k's classification found a run; cleared before every pass.  What
+// a step's classification decides never changes a result, only which kernel draws it.
+constexpr uint32_t kQuietLookEvery = 4;
+
 template <int kClassifyItems>
 __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __restrict__ keys,
                                                           const uint32_t* __restrict__ n_dev, RunsMeta* meta,
                                                           RunsMeta* meta_of_next_step,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                           uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
-                                                          uint8_t* __restrict__ skip_flag) {
+                                                          uint8_t* __restrict__ skip_flag,
+                                                          ClassCounters* __restrict__ counters, uint32_t partial_cache,
+                                                          uint32_t* __restrict__ found_by_step, uint32_t step) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t s_base;
   const uint32_t n = *n_dev;
   // the work-item counters alternate between steps: this launch clears the one the next
   // step will count into (its last reader, the previous step's workgroup kernel, is done)
   if (blockIdx.x == 0 && threadIdx.x == 0) meta_of_next_step->n_chunks = 0;
+  if (step > 1 && found_by_step[step - 1] == 0 && step % kQuietLookEvery != 0) return;
+  if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&counters->sorted_pairs, (unsigned long long)n);
   const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
   uint32_t transit, start, count, n_items;
   uint32_t mine = 0;
+  uint32_t single_pairs = 0, split_pairs = 0, refused_pairs = 0;
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
-    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count,
-                                       &n_items))
+    uint32_t refused = 0;
+    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, partial_cache != 0, &transit, &start,
+                                       &count, &n_items, &refused)) {
       mine += n_items;
+      if (n_items > 1) split_pairs += count; else single_pairs += count;
+    }
+    refused_pairs += refused;
+  }
+  {
+    // the wavefront's counts, added by one lane to the wavefront's copy of the counters
+    uint32_t items = mine;
+    for (int d = 1; d < kWave; d <<= 1) {
+      single_pairs += __shfl_xor(single_pairs, d, kWave);
+      split_pairs += __shfl_xor(split_pairs, d, kWave);
+      refused_pairs += __shfl_xor(refused_pairs, d, kWave);
+      items += __shfl_xor(items, d, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      ClassCounters* mine_c = counters + ((blockIdx.x * (256 / kWave) + threadIdx.x / kWave) % kCounterCopies);
+      if (single_pairs) atomicAdd(&mine_c->workgroup_pairs, (unsigned long long)single_pairs);
+      if (split_pairs) atomicAdd(&mine_c->split_pairs, (unsigned long long)split_pairs);
+      if (refused_pairs) atomicAdd(&mine_c->refused_pairs, (unsigned long long)refused_pairs);
+      if (items) atomicAdd(&mine_c->work_items, (unsigned long long)items);
+    }
   }
   uint32_t base;
   if (kClassifyItems == 1) {
@@ -616,7 +675,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
     const uint64_t i = first + k;
     // one pair per lane: the run found above is still in the registers
     if (kClassifyItems > 1 && !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size,
-                                                               &transit, &start, &count, &n_items)))
+                                                               partial_cache != 0, &transit, &start, &count, &n_items)))
       continue;
     const bool fits = base + n_items <= chunk_capacity;
     for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
@@ -624,7 +683,10 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
       chunks[2 * (base + g)] = start + off;
       chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
     }
-    if (fits) skip_flag[transit] = 1;
+    if (fits) {
+      skip_flag[transit] = 1;
+      found_by_step[step] = 1;  // the next step looks again
+    }
     base += n_items;
   }
 }
@@ -926,6 +988,10 @@ class Engine : public EngineBase {
     }
     ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta) * 2));
     ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta) * 2));
+    ND_HIP_TRY(hipMalloc(&d_balance_, sizeof(uint32_t) * kBalanceWords));
+    ND_HIP_TRY(hipMemset(d_balance_, 0, sizeof(uint32_t) * kBalanceWords));
+    class_counters_ = ClassCounters();
+    idle_passes_ = 0;
     balanced_steps_ = 0;
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
     ND_HIP_TRY(hipMalloc(&d_skip_flag_, (size_t)invalid_ + 1));
@@ -965,15 +1031,62 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
+    if (balanced_this_pass_) {
+      // after the pass and outside its timed region: what the classifications counted
+      ClassCounters copies[kCounterCopies];
+      ND_HIP_TRY(hipMemcpy(copies, counters_dev(), sizeof(copies), hipMemcpyDeviceToHost));
+      class_counters_ = ClassCounters();
+      for (const ClassCounters& c : copies) {
+        class_counters_.sorted_pairs += c.sorted_pairs;
+        class_counters_.workgroup_pairs += c.workgroup_pairs;
+        class_counters_.split_pairs += c.split_pairs;
+        class_counters_.refused_pairs += c.refused_pairs;
+        class_counters_.work_items += c.work_items;
+      }
+      idle_passes_ = class_counters_.work_items == 0 && class_counters_.sorted_pairs != 0 ? 1 : 0;
+    }
     return 0;
+  }
+
+  // Per-transit apps: 0 = pairs the classifications of the last load-balanced pass looked at,
+  // 1 = of these, pairs on transits the workgroup kernel served as one work item, 2 = pairs on
+  // transits split over several work items (grid-wide), 3 = pairs in runs long enough for the
+  // workgroup kernel that stayed with the flat kernel because of the transit's degree,
+  // 4 = work items; the flat kernel served 0 minus 1 minus 2.
+  int64_t counter(int which) const override {
+    switch (which) {
+      case 0: return (int64_t)class_counters_.sorted_pairs;
+      case 1: return (int64_t)class_counters_.workgroup_pairs;
+      case 2: return (int64_t)class_counters_.split_pairs;
+      case 3: return (int64_t)class_counters_.refused_pairs;
+      case 4: return (int64_t)class_counters_.work_items;
+      default: return 0;
+    }
   }
 
   // Every launch of one pass, in order, on stream_; no host wait in between.
   int enqueue_pass(int mode) {
-    const bool balance = mode == kTransitParallelLoadBalanced;
     App app;
     const int n_steps = app.steps();
     const size_t F = (size_t)final_sample_size();
+    // With few walks per vertex hardly any two walks share a transit: the sorted order then
+    // saves less in the step kernels (shared lines) than the inversion costs.
+    int sort_period = inversion_period;
+    if (sort_period <= 0)
+      sort_period = (double)n_samples_ < kWalksPerVertexForInversion * (double)invalid_ ? kSparseInversionPeriod : 1;
+    const bool sample_parallel = mode == kSampleParallel;
+    if (sample_parallel && sort_period <= 1) sort_period = kSparseInversionPeriod;
+    // A pass whose classifications found nothing at all for the workgroup kernel is followed by
+    // passes that do not classify (nor launch the workgroup kernel); every kIdleLookEvery-th
+    // pass looks again.  Results do not depend on it.
+    bool balance = mode == kTransitParallelLoadBalanced && n_steps > 1 && !(walk_mode_ && sort_period > 1);
+    if (balance && !wants_launch_graph() && idle_passes_ > 0 && idle_passes_ % kIdleLookEvery != 0) {
+      balance = false;
+      idle_passes_++;
+    }
+    balanced_this_pass_ = balance;
+    if (balance)
+      fill_i32<<<dim3((kBalanceWords + 255) / 256), dim3(256), 0, stream_>>>((int32_t*)d_balance_, kBalanceWords, 0);
     // pairs whose transit is INVALID are dropped by the inversion and never reach a step
     // kernel: their outputs keep this fill
     {
@@ -985,13 +1098,6 @@ class Engine : public EngineBase {
     uint32_t transits_per_sample = (uint32_t)init_size_;
     const uint32_t* live_last = nullptr;  // pairs the last inversion kept (device count)
     int sorts_done = 0;
-    // With few walks per vertex hardly any two walks share a transit: the sorted order then
-    // saves less in the step kernels (shared lines) than the inversion costs.
-    int sort_period = inversion_period;
-    if (sort_period <= 0)
-      sort_period = (double)n_samples_ < kWalksPerVertexForInversion * (double)invalid_ ? kSparseInversionPeriod : 1;
-    const bool sample_parallel = mode == kSampleParallel;
-    if (sample_parallel && sort_period <= 1) sort_period = kSparseInversionPeriod;
     const int32_t* transits = d_initial_;  // (sample -> transit) map entering the step
     KeyLayout transits_layout;             // and how it is laid out
     for (int step = 0; step < n_steps; ++step) {
@@ -1109,11 +1215,11 @@ class Engine : public EngineBase {
             const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
             classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
                 sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                d_skip_flag_);
+                d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
           } else {
             classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
                 sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                d_skip_flag_);
+                d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
           }
           tock(&times.load_balancing);
           tick();
@@ -1271,6 +1377,22 @@ class Engine : public EngineBase {
   }
 
  private:
+  // d_balance_: found_by_step[kMaxSteps + 1], then the ClassCounters (8-byte aligned)
+  static constexpr int kBalanceWords =
+      kMaxSteps + 2 + (int)(kCounterCopies * sizeof(ClassCounters) / sizeof(uint32_t));
+  static constexpr int kIdleLookEvery = 8;
+  ClassCounters* counters_dev() const { return (ClassCounters*)(d_balance_ + kMaxSteps + 2); }
+  // Transits whose adjacency is longer than the LDS cache stay with the flat kernel unless
+  // ND_HUB_CACHE=1 sends them to the workgroup kernel with the first kCacheEdges edges staged
+  // (the reference's CachedArray, src/nextdoor.cu:76-124).  Off because it loses: draws are
+  // uniform over the adjacency, so a hub of 10^5 edges finds a tenth of them in LDS, and on 4.2 M
+  // weighted walks the pass takes 57.7 ms with it against 37.2 ms without (the workgroup kernel
+  // then serves 9 % of the pairs in 20.7 ms); two-hop sampling gains 3 % (8.23 against 8.46 ms).
+  static bool partial_hub_cache() {
+    static const bool on = getenv("ND_HUB_CACHE") && atoi(getenv("ND_HUB_CACHE")) != 0;
+    return on;
+  }
+
   void launch_flat(const StepParams& P, unsigned flat_grid, const uint8_t* skip_flag) {
     if (P.step_size == 1)
       step_flat_kernel<SampleType, App, true><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
@@ -1328,6 +1450,7 @@ class Engine : public EngineBase {
     release(d_aux_a_);
     release(d_aux_b_);
     release(d_meta_);
+    release(d_balance_);
     release(d_chunks_);
     release(d_skip_flag_);
     release(d_distinct_counts_);
@@ -1374,6 +1497,10 @@ class Engine : public EngineBase {
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;          // two work-item counters, alternating between load-balanced steps
+  uint32_t* d_balance_ = nullptr;       // which steps' classifications found a run; the pass's ClassCounters
+  ClassCounters class_counters_{};      // of the last load-balanced pass
+  int idle_passes_ = 0;                 // passes since one whose classifications found nothing (0: none)
+  bool balanced_this_pass_ = false;
   struct RecordedPass {
     int mode = 0, inversion_period = 0, parity = 0;
     uint64_t balanced_steps = 0;  // load-balanced steps of the pass

@@ -66,7 +66,11 @@ ND_HD float u32_to_unit_float(uint32_t word) {
 struct RandState {
   uint32_t slot_lo, slot_hi, step, draw;
   uint32_t key0, key1;
-  PhiloxBlock cache;
+  // The words of the current Philox block that have not been drawn yet, next one first.  A
+  // draw takes word0 and moves the others up: no word is ever picked by an index, so the state
+  // stays in registers (an array indexed by the draw number, or selects among its members,
+  // end up as a memory object with a computed address).
+  uint32_t word0, word1, word2, word3;
 
   ND_HD void reset(uint64_t seed, uint64_t slot, uint32_t step_) {
     slot_lo = (uint32_t)slot;
@@ -75,17 +79,22 @@ struct RandState {
     draw = 0;
     key0 = (uint32_t)seed;
     key1 = (uint32_t)(seed >> 32);
+    word0 = word1 = word2 = word3 = 0;
   }
 
   ND_HD uint32_t next_word() {
-    const uint32_t lane = draw & 3u;
-    if (lane == 0) cache = philox4x32_10(slot_lo, slot_hi, step, draw >> 2, key0, key1);
+    if ((draw & 3u) == 0) {
+      const PhiloxBlock b = philox4x32_10(slot_lo, slot_hi, step, draw >> 2, key0, key1);
+      word0 = b.w[0];
+      word1 = b.w[1];
+      word2 = b.w[2];
+      word3 = b.w[3];
+    }
     ++draw;
-    // select without dynamic register indexing
-    uint32_t word = cache.w[0];
-    word = lane == 1 ? cache.w[1] : word;
-    word = lane == 2 ? cache.w[2] : word;
-    word = lane == 3 ? cache.w[3] : word;
+    const uint32_t word = word0;
+    word0 = word1;
+    word1 = word2;
+    word2 = word3;
     return word;
   }
 

@@ -222,6 +222,8 @@ static int32_t next_individual(const ndo_graph* g, const ndo_app_desc* app, int 
       const float p = app->p, q = app->q;
       float hmax = p > 1.0f / q ? p : 1.0f / q;
       if (hmax < 1.0f) hmax = 1.0f;
+      float hmin = p < 1.0f / q ? p : 1.0f / q;
+      if (hmin > 1.0f) hmin = 1.0f;
       const float envelope = max_w * hmax;
       for (;;) {
         int32_t x = next_int(rc, n);
@@ -230,6 +232,7 @@ static int32_t next_individual(const ndo_graph* g, const ndo_app_desc* app, int 
         if (st) { st->edge_reads++; st->weight_reads++; }
         float y = next_uniform(rc) * envelope;
         float h;
+        if (st && step > 0 && !(y < hmin * wx) && y < hmax * wx) st->band_tests++;  /* statistics only */
         if (step == 0) h = 1.0f;
         else {
           int32_t t = *t_state;
@@ -310,6 +313,7 @@ int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t 
       stats->valid_outputs += per_thread[i].valid_outputs;
       stats->edge_reads += per_thread[i].edge_reads;
       stats->weight_reads += per_thread[i].weight_reads;
+      stats->band_tests += per_thread[i].band_tests;
     }
   }
   free(per_thread);

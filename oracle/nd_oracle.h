@@ -65,6 +65,9 @@ typedef struct {
   int64_t valid_outputs;  /* output slots != INVALID (reference: totalSampledVertices, nextdoor.cu:3284-3299) */
   int64_t edge_reads;     /* neighbour-id loads */
   int64_t weight_reads;   /* edge-weight loads */
+  int64_t band_tests;     /* weighted node2vec: candidates whose acceptance depends on the bias, i.e.
+                             min(p, 1/q, 1) * w <= height < max(p, 1/q, 1) * w at a step after the first:
+                             the adjacency tests a sampler needs that only tests when the answer matters */
 } ndo_stats;
 
 /* ---- random numbers (replaces cuRAND XORWOW; rand_num_gen.cuh:117-122) ---- */

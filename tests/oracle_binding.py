@@ -29,7 +29,8 @@ class AppDesc(C.Structure):
 
 class Stats(C.Structure):
     _fields_ = [("next_calls", C.c_int64), ("draws", C.c_int64), ("search_probes", C.c_int64),
-                ("valid_outputs", C.c_int64), ("edge_reads", C.c_int64), ("weight_reads", C.c_int64)]
+                ("valid_outputs", C.c_int64), ("edge_reads", C.c_int64), ("weight_reads", C.c_int64),
+                ("band_tests", C.c_int64)]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}

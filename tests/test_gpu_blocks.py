@@ -64,3 +64,70 @@ def test_unique_transits_matches_oracle(oracle, n, frac_invalid):
     wu, wc, wo, w_valid = oracle.unique_transits(keys, invalid)
     assert n_valid == w_valid
     assert np.array_equal(u, wu) and np.array_equal(c, wc) and np.array_equal(o, wo)
+
+
+def brute_force_classes(keys, degrees, step_size, partial_cache, thresholds):
+    """Which runs the workgroup kernel takes, by the stated rule, and how they are cut."""
+    need_work, per_item_outputs, cache_edges = thresholds
+    per_item = max(per_item_outputs // step_size, 1)
+    transits, starts, counts = np.unique(keys, return_index=True, return_counts=True)
+    taken, n_items, single, split, refused = {}, 0, 0, 0, 0
+    for t, first, count in zip(transits, starts, counts):
+        work = int(count) * step_size
+        if work < need_work or degrees[t] == 0:
+            continue
+        staged = min(int(degrees[t]), cache_edges)
+        if (degrees[t] > cache_edges and not partial_cache) or staged > 32 * work:
+            refused += int(count)
+            continue
+        k = -(-int(count) // per_item)
+        taken[int(t)] = (int(first), int(count))
+        n_items += k
+        if k > 1:
+            split += int(count)
+        else:
+            single += int(count)
+    return taken, n_items, single, split, refused, per_item
+
+
+@pytest.mark.parametrize("pairs_per_lane", [1, 16])
+@pytest.mark.parametrize("step_size,partial_cache", [(1, True), (1, False), (10, True), (25, False), (3000, True)])
+def test_run_classification_covers_every_pair_of_a_taken_transit_once(step_size, partial_cache, pairs_per_lane):
+    # the binning of transits into kernel classes (src/nextdoor.cu:1520-1802; the reference asserts
+    # the same covering at :1745-1749) against a brute-force partition of the sorted map
+    rng = np.random.default_rng(11 + step_size)
+    thresholds = nd.load_balancing_thresholds()
+    n_vertices = 5000
+    degrees = rng.integers(0, 40, n_vertices).astype(np.int32)
+    degrees[rng.integers(0, n_vertices, 60)] = rng.integers(5000, 30000, 60)  # adjacencies around and beyond the cache
+    degrees[rng.integers(0, n_vertices, 40)] = 0
+    # short runs everywhere, some long ones (a few beyond one work item), one at each end of the map
+    counts = rng.integers(0, 4, n_vertices)
+    long_ones = rng.integers(0, n_vertices, 80)
+    counts[long_ones] = rng.integers(20, 700, 80)
+    counts[rng.integers(0, n_vertices, 6)] = rng.integers(2500, 9000, 6)
+    counts[0], counts[n_vertices - 1] = 300, 2100
+    keys = np.repeat(np.arange(n_vertices, dtype=np.int32), counts)
+    print("classify n", len(keys), "step size", step_size, "partial", partial_cache, "lane", pairs_per_lane, flush=True)
+    items, wanted, taken, counters = nd.classify_runs(keys, degrees, step_size, partial_cache, pairs_per_lane)
+    want_taken, want_items, single, split, refused, per_item = brute_force_classes(keys, degrees, step_size,
+                                                                                   partial_cache, thresholds)
+    assert wanted == want_items == len(items)
+    assert sorted(np.flatnonzero(taken).tolist()) == sorted(want_taken)
+    assert counters.tolist() == [len(keys), single, split, refused, want_items]
+    covered = np.zeros(len(keys), np.int32)
+    for first, count in items:
+        assert 1 <= count <= per_item
+        assert len(set(keys[first:first + count].tolist())) == 1  # an item never straddles two transits
+        covered[first:first + count] += 1
+    for t, (first, count) in want_taken.items():
+        assert np.all(covered[first:first + count] == 1)
+    assert covered.sum() == sum(c for _, c in want_taken.values())  # nothing else is covered
+
+
+def test_run_classification_of_a_map_without_long_runs_and_of_an_empty_map():
+    degrees = np.full(100, 5, np.int32)
+    items, wanted, taken, counters = nd.classify_runs(np.arange(100, dtype=np.int32), degrees, 1)
+    assert wanted == 0 and not taken.any() and counters.tolist() == [100, 0, 0, 0, 0]
+    items, wanted, taken, counters = nd.classify_runs(np.zeros(0, np.int32), degrees, 1)
+    assert wanted == 0 and not taken.any()
