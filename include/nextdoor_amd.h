@@ -30,6 +30,16 @@ const char* nd_last_error(void);
 int nd_num_apps(void);
 const char* nd_app_name(int index);
 
+/* Adds an application to the registry, so that nd_sampler_create(name) finds it.  The reference
+ * has no registry: every application is a translation unit that instantiates the engine on its
+ * <SampleType, App> (src/apps/khop/main.cu:1-21, src/tests/testBase.h:14-24).  Here such a
+ * translation unit - the App struct, nd_app_registry.hpp and ND_REGISTER_APP - is compiled with
+ * hipcc into a shared object of its own, and loading it calls this.  make(name) returns a new
+ * nd::EngineBase* (nd_engine.hpp) for the application; engine_abi must be ND_ENGINE_ABI of the
+ * headers the caller was built from.  Returns 0, or a negative value (name taken, ABI mismatch). */
+#define ND_ENGINE_ABI 2
+int nd_register_app(const char* name, void* (*make)(const char* name), int engine_abi);
+
 /* ---- graphs ------------------------------------------------------------------------ */
 
 /* loadGraph(graph, file, type, format), src/nextdoor.cu:1845-1891.

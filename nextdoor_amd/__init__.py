@@ -21,13 +21,32 @@ import numpy as np
 from . import _capi
 from ._capi import NextDoorError, check, lib
 
-__all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "philox_fill_uniform",
-           "sort_pairs", "sort_pairs_noalloc", "unique_transits", "classify_runs", "load_balancing_thresholds", "collective_neighborhood", "check_sampled_vertices"]
+__all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "load_app_library",
+           "philox_fill_uniform", "sort_pairs", "sort_pairs_noalloc", "unique_transits", "classify_runs", "load_balancing_thresholds", "collective_neighborhood", "check_sampled_vertices"]
 
 
 def app_names():
     L = lib()
     return [L.nd_app_name(i).decode() for i in range(L.nd_num_apps())]
+
+
+_app_libraries = {}
+
+
+def load_app_library(path):
+    """Loads a shared object of applications that were compiled apart from the library (an App
+    struct on the contract plus ``ND_REGISTER_APP(name, SampleType, App)``, built by hipcc and
+    linked against libnextdoor_amd.so).  Its apps register themselves while it loads; returns
+    the names that appeared.  The counterpart of compiling one's own app binary against the
+    reference (src/apps/*/main.cu)."""
+    import os
+    L = lib()  # the library first: the registrations call into it
+    before = set(app_names())
+    real = os.path.realpath(path)
+    if real not in _app_libraries:
+        _app_libraries[real] = C.CDLL(real, mode=C.RTLD_GLOBAL)
+    del L
+    return sorted(set(app_names()) - before)
 
 
 def check_sampled_vertices(graph, step_sizes, initial, final_samples, invalid=None, collective=False):

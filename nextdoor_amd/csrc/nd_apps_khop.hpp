@@ -50,3 +50,8 @@ typedef KHopAppT<25, 10> KHopApp;
 // src/apps/layer/layerSampling.cu:1-81: the same sampler with fan-outs 10 and 25
 class LayerSample {};
 typedef KHopAppT<10, 25> LayerSamplingApp;
+
+ND_APP_REGISTERED_AS(KHopApp, "KHop")
+ND_APP_REGISTERED_AS(LayerSamplingApp, "Layer")
+typedef KHopAppT<3, 2> KHop3x2App;
+ND_APP_REGISTERED_AS(KHop3x2App, "KHop3x2")

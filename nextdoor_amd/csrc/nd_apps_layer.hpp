@@ -39,6 +39,14 @@ namespace apps {
 //                  adjacency restricted to the transits); no weights
 enum NeighborhoodForm { kConcatenated = 0, kDistinctByDegreeSquared = 1, kRankedByLadiesImportance = 2 };
 
+// The form an App's next() takes the collective neighbourhood in: App::kNeighborhoodForm, or the
+// concatenation for an App that does not say (the reference's layer-wise apps, whose next() is
+// handed the concatenated adjacencies and never looks at them: fastgcnSampling.cu:23-47).
+template <class App, class = void>
+struct neighborhood_form_of { static constexpr int value = kConcatenated; };
+template <class App>
+struct neighborhood_form_of<App, decltype((void)App::kNeighborhoodForm)> { static constexpr int value = App::kNeighborhoodForm; };
+
 template <int kLayers, int kBatch, int kNumSamples>
 struct LayerCommon {
   __host__ __device__ int steps() { return kLayers; }
@@ -157,8 +165,14 @@ struct LadiesImportanceAppT : FastGCNImportanceAppT<kLayers, kBatch, kNumSamples
 
 class LayerNoState {};
 
-// The reference's names and sizes.
+// The reference's names and sizes (left out with ND_NO_REFERENCE_APP_NAMES, for a translation
+// unit that brings the reference's own structs of these names).
+#ifndef ND_NO_REFERENCE_APP_NAMES
 typedef LayerSampleT<5, 64> FastGCNSample;
 typedef LayerSamplingAppT<5, 64, 10000> FastGCNSamplingApp;
 typedef LayerSampleT<5, 64> ImportanceSample;
 typedef LayerSamplingAppT<5, 64, 10000> ImportanceSampleApp;
+
+// FastGCNSamplingApp and ImportanceSampleApp are one type, as the reference's two apps are one text
+ND_APP_REGISTERED_AS(FastGCNSamplingApp, "FastGCN")
+#endif

@@ -73,3 +73,5 @@ struct MultiRWAppT {
 // The reference's sizes: 100 walkers, 100 steps (multiRW.cu:3, 14).
 typedef MultiRWSampleT<100> MultiRWSample;
 typedef MultiRWAppT<100, 100> MultiRWApp;
+
+ND_APP_REGISTERED_AS(MultiRWApp, "MultiRW")

@@ -35,6 +35,7 @@ namespace apps {
 
 template <int kVertices>
 struct SubgraphCommon {
+  static constexpr bool kListsEdges = true;  // next() hands edges to sample->emit: the edge-list engine
   __host__ __device__ int samplingType() { return SamplingType::IndividualNeighborhood; }
   __host__ __device__ OutputFormat outputFormat() { return AdjacencyMatrix; }
   __host__ __device__ EdgePos_t initialSampleSize(CSR*) { return kVertices; }
@@ -152,3 +153,6 @@ typedef SubgraphSampleT<32> MVSSample;
 typedef MVSSamplingAppT<32> MVSSamplingApp;
 typedef SubgraphSampleT<32> SubGraphSample;
 typedef SubGraphSamplingAppT<16, 2> SubGraphSamplingAppI;
+
+ND_APP_REGISTERED_AS(MVSSamplingApp, "MVS")
+ND_APP_REGISTERED_AS(SubGraphSamplingAppI, "ClusterGCN")

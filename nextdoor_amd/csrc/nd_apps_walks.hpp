@@ -240,3 +240,13 @@ typedef WeightedNode2VecAppT<100> WeightedNode2VecApp;
 typedef DeepWalkAppT<nd::apps::OneWalkPerVertex<100>> DeepWalkPerVertexApp;
 typedef Node2VecAppT<nd::apps::OneWalkPerVertex<100>> Node2VecPerVertexApp;
 typedef PPRAppT<nd::apps::OneWalkPerVertex<100>> PPRPerVertexApp;
+
+ND_APP_REGISTERED_AS(UniformRandomWalkApp, "UniformRandomWalk")
+ND_APP_REGISTERED_AS(DeepWalkApp, "DeepWalk")
+ND_APP_REGISTERED_AS(PPRApp, "PPR")
+ND_APP_REGISTERED_AS(Node2VecApp, "Node2Vec")
+ND_APP_REGISTERED_AS(WeightedNode2VecApp, "WeightedNode2Vec")
+ND_APP_REGISTERED_AS(DeepWalkPerVertexApp, "DeepWalkPerVertex")
+ND_APP_REGISTERED_AS(Node2VecPerVertexApp, "Node2VecPerVertex")
+ND_APP_REGISTERED_AS(PPRPerVertexApp, "PPRPerVertex")
+ND_APP_REGISTERED_AS(UniformRandomWalkAppT<8>, "UniformRandomWalk8")

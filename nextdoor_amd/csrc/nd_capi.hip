@@ -3,6 +3,7 @@
 
 #include <string.h>
 
+#include <deque>
 #include <exception>
 #include <memory>
 #include <mutex>
@@ -15,16 +16,10 @@
 #include "nd_apps_subgraph.hpp"
 #include "nd_apps_layer.hpp"
 #include "nd_apps_walks.hpp"
-#include "nd_engine.hpp"
-#include "nd_sharded_engine.hpp"
-#include "nd_layer_engine.hpp"
-#include "nd_subgraph_engine.hpp"
+#include "nd_app_registry.hpp"
 #include "nd_graph.hpp"
 #include "nd_check.hpp"
 
-struct nd_graph {
-  CSR csr;
-};
 
 struct nd_sampler {
   std::unique_ptr<nd::EngineBase> engine;
@@ -57,22 +52,20 @@ int guarded(Body body) {
 
 struct AppEntry {
   const char* name;
-  nd::EngineBase* (*make)(const char*);
+  void* (*make)(const char*);
 };
 
 template <class SampleType, class App>
-nd::EngineBase* make_engine(const char* name) {
-  return new nd::ShardedEngine<SampleType, App>(name);
+void* make_engine(const char* name) {
+  return nd::make_app_engine<SampleType, App>(name);
 }
-
 template <class SampleType, class App>
-nd::EngineBase* make_subgraph_engine(const char* name) {
-  return new nd::SubgraphEngine<SampleType, App>(name);
+void* make_subgraph_engine(const char* name) {
+  return nd::make_app_engine<SampleType, App>(name);
 }
-
 template <class SampleType, class App>
-nd::EngineBase* make_layer_engine(const char* name) {
-  return new nd::LayerEngine<SampleType, App>(name);
+void* make_layer_engine(const char* name) {
+  return nd::make_app_engine<SampleType, App>(name);
 }
 
 // name -> instantiation.  The first block carries the reference's app names and sizes.
@@ -127,7 +120,31 @@ const AppEntry kApps[] = {
     {"LADIESImportance2x8", make_layer_engine<LayerNoState, LadiesImportanceAppT<2, 8, 100>>},
     {"LADIESImportance3x16", make_layer_engine<LayerNoState, LadiesImportanceAppT<3, 16, 300>>},
 };
-constexpr int kNumApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
+constexpr int kNumBuiltInApps = (int)(sizeof(kApps) / sizeof(kApps[0]));
+
+// Applications added with nd_register_app, after the built-in ones.  A function-local static:
+// registrations run from the static initialisers of other shared objects, in no set order.
+struct RegisteredApp {
+  std::string name;
+  void* (*make)(const char*);
+};
+std::deque<RegisteredApp>& registered_apps() {
+  static std::deque<RegisteredApp> apps;  // deque: names handed out stay where they are
+  return apps;
+}
+std::mutex& registry_mutex() {
+  static std::mutex m;
+  return m;
+}
+
+bool find_app(const char* name, AppEntry* out) {
+  for (int i = 0; i < kNumBuiltInApps; ++i)
+    if (strcmp(kApps[i].name, name) == 0) { *out = kApps[i]; return true; }
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  for (const RegisteredApp& a : registered_apps())
+    if (a.name == name) { *out = AppEntry{a.name.c_str(), a.make}; return true; }
+  return false;
+}
 
 nd_sampler* g_module_sampler = nullptr;
 nd_graph* g_module_graph = nullptr;
@@ -204,8 +221,30 @@ extern "C" {
 
 const char* nd_last_error(void) { return g_error.c_str(); }
 
-int nd_num_apps(void) { return kNumApps; }
-const char* nd_app_name(int index) { return index >= 0 && index < kNumApps ? kApps[index].name : nullptr; }
+int nd_num_apps(void) {
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  return kNumBuiltInApps + (int)registered_apps().size();
+}
+const char* nd_app_name(int index) {
+  if (index >= 0 && index < kNumBuiltInApps) return kApps[index].name;
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  const int i = index - kNumBuiltInApps;
+  return i >= 0 && i < (int)registered_apps().size() ? registered_apps()[(size_t)i].name.c_str() : nullptr;
+}
+
+int nd_register_app(const char* name, void* (*make)(const char* name), int engine_abi) {
+  return guarded([&]() -> int {
+    if (!name || !*name || !make) return fail("null argument");
+    if (engine_abi != ND_ENGINE_ABI)
+      return fail(std::string("app '") + name + "' was built against engine ABI " + std::to_string(engine_abi) +
+                  ", the library has " + std::to_string(ND_ENGINE_ABI), -2);
+    AppEntry taken;
+    if (find_app(name, &taken)) return fail(std::string("an app named '") + name + "' is already registered", -3);
+    std::lock_guard<std::mutex> lock(registry_mutex());
+    registered_apps().push_back(RegisteredApp{name, make});
+    return 0;
+  });
+}
 
 // ---- graphs ---------------------------------------------------------------------------
 
@@ -214,7 +253,7 @@ int nd_graph_load(const char* path, const char* graph_type, const char* graph_fo
     if (!out) return fail("null out");
     std::unique_ptr<nd_graph> g(new nd_graph);
     std::string err;
-    if (nd::load_graph_file(g->csr, path, graph_type, graph_format, &err) != 0) return fail(err);
+    if (nd::load_graph_file(*g, path, graph_type, graph_format, &err) != 0) return fail(err);
     *out = g.release();
     return 0;
   });
@@ -226,7 +265,7 @@ int nd_graph_from_edges(int32_t n_vertices, int64_t n_edges, const int32_t* src,
     if (!out || n_edges < 0 || (n_edges > 0 && (!src || !dst))) return fail("bad argument");
     std::unique_ptr<nd_graph> g(new nd_graph);
     std::string err;
-    if (nd::csr_from_edges(g->csr, n_vertices, (size_t)n_edges, src, dst, weight, &err) != 0) return fail(err);
+    if (nd::csr_from_edges(*g, n_vertices, (size_t)n_edges, src, dst, weight, &err) != 0) return fail(err);
     *out = g.release();
     return 0;
   });
@@ -238,7 +277,7 @@ int nd_graph_from_csr(int32_t n_vertices, int64_t n_edges, const int32_t* row_pt
     if (!out || !row_ptr || (n_edges > 0 && !col)) return fail("bad argument");
     std::unique_ptr<nd_graph> g(new nd_graph);
     std::string err;
-    if (nd::csr_from_arrays(g->csr, n_vertices, n_edges, row_ptr, col, weight, &err) != 0) return fail(err);
+    if (nd::csr_from_arrays(*g, n_vertices, n_edges, row_ptr, col, weight, &err) != 0) return fail(err);
     *out = g.release();
     return 0;
   });
@@ -250,7 +289,7 @@ int nd_graph_rmat(int scale, int edge_factor, double a, double b, double c, uint
     if (!out) return fail("null out");
     std::unique_ptr<nd_graph> g(new nd_graph);
     std::string err;
-    if (nd::generate_rmat(g->csr, scale, edge_factor, a, b, c, seed, symmetrise != 0, &err) != 0) return fail(err);
+    if (nd::generate_rmat(*g, scale, edge_factor, a, b, c, seed, symmetrise != 0, &err) != 0) return fail(err);
     *out = g.release();
     return 0;
   });
@@ -261,18 +300,18 @@ int nd_graph_chung_lu(int32_t n_vertices, int64_t n_edges, double exponent, uint
     if (!out) return fail("null out");
     std::unique_ptr<nd_graph> g(new nd_graph);
     std::string err;
-    if (nd::generate_chung_lu(g->csr, n_vertices, n_edges, exponent, seed, &err) != 0) return fail(err);
+    if (nd::generate_chung_lu(*g, n_vertices, n_edges, exponent, seed, &err) != 0) return fail(err);
     *out = g.release();
     return 0;
   });
 }
 
-int32_t nd_graph_num_vertices(const nd_graph* g) { return g ? g->csr.get_n_vertices() : 0; }
-int64_t nd_graph_num_edges(const nd_graph* g) { return g ? (int64_t)g->csr.col.size() : 0; }
-const int32_t* nd_graph_row_ptr(const nd_graph* g) { return g ? g->csr.row_ptr.data() : nullptr; }
-const int32_t* nd_graph_col(const nd_graph* g) { return g ? g->csr.col.data() : nullptr; }
-const float* nd_graph_weight(const nd_graph* g) { return g ? g->csr.weight.data() : nullptr; }
-const float* nd_graph_max_weight(const nd_graph* g) { return g ? g->csr.max_weight.data() : nullptr; }
+int32_t nd_graph_num_vertices(const nd_graph* g) { return g ? g->get_n_vertices() : 0; }
+int64_t nd_graph_num_edges(const nd_graph* g) { return g ? (int64_t)g->col.size() : 0; }
+const int32_t* nd_graph_row_ptr(const nd_graph* g) { return g ? g->row_ptr.data() : nullptr; }
+const int32_t* nd_graph_col(const nd_graph* g) { return g ? g->col.data() : nullptr; }
+const float* nd_graph_weight(const nd_graph* g) { return g ? g->weight.data() : nullptr; }
+const float* nd_graph_max_weight(const nd_graph* g) { return g ? g->max_weight.data() : nullptr; }
 void nd_graph_free(nd_graph* g) { delete g; }
 
 // ---- sampler --------------------------------------------------------------------------
@@ -280,15 +319,12 @@ void nd_graph_free(nd_graph* g) { delete g; }
 int nd_sampler_create(const char* app_name, nd_sampler** out) {
   return guarded([&]() -> int {
     if (!app_name || !out) return fail("null argument");
-    for (int i = 0; i < kNumApps; ++i) {
-      if (strcmp(kApps[i].name, app_name) == 0) {
-        nd_sampler* s = new nd_sampler;
-        s->engine.reset(kApps[i].make(kApps[i].name));
-        *out = s;
-        return 0;
-      }
-    }
-    return fail(std::string("unknown app '") + app_name + "'");
+    AppEntry app;
+    if (!find_app(app_name, &app)) return fail(std::string("unknown app '") + app_name + "'");
+    nd_sampler* s = new nd_sampler;
+    s->engine.reset((nd::EngineBase*)app.make(app.name));
+    *out = s;
+    return 0;
   });
 }
 
@@ -298,7 +334,7 @@ int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g) {
     int n_devices = 0;
     if (hipGetDeviceCount(&n_devices) != hipSuccess || n_devices < 1) return fail("no HIP device available");
     s->graph = g;
-    const int rc = s->engine->set_graph(&g->csr);
+    const int rc = s->engine->set_graph(g);
     return rc == 0 ? 0 : fail(s->engine->last_error, rc);
   });
 }
@@ -444,7 +480,7 @@ int nd_check_sampled_vertices(const nd_graph* g, int n_steps, const int32_t* ste
     shape.initial_size = initial_size;
     shape.collective = collective != 0;
     std::string report;
-    if (nd::check_sampled_vertices(g->csr, shape, n_samples, initial, final_samples, invalid, &report)) return 1;
+    if (nd::check_sampled_vertices(*g, shape, n_samples, initial, final_samples, invalid, &report)) return 1;
     g_error = report;
     return 0;
   });
@@ -472,7 +508,7 @@ int nd_sampler_check_results(nd_sampler* s, int* ok) {
     if (e.lists_edges()) {
       const int rc2 = e.fetch_adjacency();
       if (rc2 != 0) return fail(e.last_error, rc2);
-      pass = nd::check_subgraph_edge_lists(s->graph->csr, e.num_samples(), shape.initial_size, e.initialContents.data(),
+      pass = nd::check_subgraph_edge_lists(*s->graph, e.num_samples(), shape.initial_size, e.initialContents.data(),
                                            e.hListStart.data(), e.hListRows.data(), e.hListCols.data(), &report);
       *ok = pass ? 1 : 0;
       if (!pass) g_error = report;
@@ -484,12 +520,12 @@ int nd_sampler_check_results(nd_sampler* s, int* ok) {
       std::vector<int32_t> states((size_t)e.num_samples() * matrix_ints);
       const int rc2 = e.fetch_sample_states(states.data(), states.size() * sizeof(int32_t));
       if (rc2 != 0) return fail(e.last_error, rc2);
-      pass = nd::check_layer_adjacency_matrix(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+      pass = nd::check_layer_adjacency_matrix(*s->graph, shape, e.num_samples(), e.initialContents.data(),
                                               e.hFinalSamples.data(), states.data() + layers,
                                               states.data() + layers + layers * cells, matrix_ints, e.invalid_vertex(),
                                               &report);
     } else {
-      pass = nd::check_sampled_vertices(s->graph->csr, shape, e.num_samples(), e.initialContents.data(),
+      pass = nd::check_sampled_vertices(*s->graph, shape, e.num_samples(), e.initialContents.data(),
                                         e.hFinalSamples.data(), e.invalid_vertex(), &report);
     }
     *ok = pass ? 1 : 0;
@@ -768,14 +804,14 @@ int nd_collective_neighborhood(const nd_graph* g, const int32_t* transits, int64
     for (size_t i = 0; i < n_tr; ++i) {
       const int32_t t = transits[i];
       if (t == invalid || t == -1) continue;
-      if (!g->csr.has_vertex(t)) return fail("transit " + std::to_string(t) + " is not a vertex of the graph");
-      entries += (uint64_t)g->csr.n_edges_for_vertex(t);
+      if (!g->has_vertex(t)) return fail("transit " + std::to_string(t) + " is not a vertex of the graph");
+      entries += (uint64_t)g->n_edges_for_vertex(t);
     }
     if (entries >= (1ull << 31)) return fail("collective neighbourhoods of more than 2^31 entries");
     if ((int64_t)entries > capacity) return fail("collective neighbourhood larger than the capacity given");
     nd::DeviceGraph dg;
     std::string err;
-    if (!dg.upload(&g->csr, false, false, &err)) return fail(err);
+    if (!dg.upload(g, false, false, &err)) return fail(err);
     DeviceBuffer d_tr, d_sizes, d_offsets, d_scratch, d_cols, d_weights, d_rows;
     CAPI_HIP(d_tr.alloc(sizeof(int32_t) * n_tr));
     CAPI_HIP(d_sizes.alloc(sizeof(uint32_t) * ((size_t)S + 1)));

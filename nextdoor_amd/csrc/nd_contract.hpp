@@ -10,9 +10,27 @@
 // CSRPartition, SamplingType / OutputFormat, RandNumGen::rand_int, utils::binarySearch and
 // the random-state handle.  The handle is the engine's own Philox cursor (nd::RandState);
 // it only carries the name the app signature spells.  No vendor RNG library is involved.
+//
+// Device translation units (hipcc) see the real qualifiers.  A host-only translation unit
+// (g++: the host API header, checkers that call an App's next() in a plain CPU loop) sees
+// __host__ / __device__ / __forceinline__ as empty words, so the same App source compiles as
+// ordinary C++.
 #pragma once
 
+#if defined(__HIPCC__)
 #include <hip/hip_runtime.h>
+#else
+#include <math.h>
+#ifndef __host__
+#define __host__
+#endif
+#ifndef __device__
+#define __device__
+#endif
+#ifndef __forceinline__
+#define __forceinline__ inline
+#endif
+#endif
 #include <stdint.h>
 
 #include <algorithm>
@@ -98,6 +116,9 @@ class CSRPartition {
   // single keys, half full, needs 1.5 dependent round trips for a key that is there and 2.5
   // for one that is not - and a wavefront waits for its slowest lane.)
   static constexpr uint32_t kEdgeBucket = 4;
+  struct alignas(16) EdgeKeyPair {  // half a bucket: one 16-byte load
+    unsigned long long x, y;
+  };
   const unsigned long long* edge_table;
   uint32_t edge_table_mask;  // number of buckets - 1 (a power of two)
 
@@ -119,8 +140,8 @@ class CSRPartition {
       const unsigned long long key = ((unsigned long long)(uint32_t)src << 32) | (uint32_t)dst;
       uint32_t bucket = edge_hash((uint32_t)src, (uint32_t)dst) & edge_table_mask;
       for (;;) {
-        const ulonglong2* keys = (const ulonglong2*)(edge_table + (size_t)bucket * kEdgeBucket);
-        const ulonglong2 first = keys[0], second = keys[1];
+        const EdgeKeyPair* keys = (const EdgeKeyPair*)(edge_table + (size_t)bucket * kEdgeBucket);
+        const EdgeKeyPair first = keys[0], second = keys[1];
         if (first.x == key || first.y == key || second.x == key || second.y == key) return true;
         if (second.y == ~0ull) return false;  // the bucket has room: the key was never pushed past it
         bucket = (bucket + 1) & edge_table_mask;
@@ -175,6 +196,7 @@ namespace nd {
 // (the reference's CachedArray, src/nextdoor.cu:76-124, plays this role).
 // The LDS half is held as a pointer in the LDS address space, so reads of it are plain LDS
 // loads and no generic-pointer test is generated.
+#if defined(__HIPCC__)
 template <typename T>
 struct LdsBackedArray {
   typedef const __attribute__((address_space(3))) T* LdsPointer;
@@ -185,6 +207,7 @@ struct LdsBackedArray {
       : lds((LdsPointer)lds_array), global(global_array), cached(n_cached) {}
   __device__ __forceinline__ T operator[](EdgePos_t i) const { return i < cached ? lds[i] : global[i]; }
 };
+#endif
 
 // Optional compile-time hints an App may carry; absent members mean `false`.
 //   static constexpr bool kUsesEdgeWeights = true;  -> next() reads transitEdgeWeights: the
@@ -220,3 +243,21 @@ struct PairedEdgeWeights {
 };
 
 }  // namespace nd
+
+// Registry name of an App that is compiled into libnextdoor_amd.so (nullptr: it is not): how
+// the template spellings of the host API (include/libNextDoor_amd.hpp) find the library's
+// instantiation for an App type.  Declared next to the App with ND_APP_REGISTERED_AS.
+template <class App>
+struct NextDoorAppName {
+  static const char* name() { return nullptr; }
+};
+#define ND_APP_REGISTERED_AS(App, literal)             \
+  template <>                                           \
+  struct NextDoorAppName<App> {                         \
+    static const char* name() { return literal; }       \
+  };
+
+// The opaque graph handle of the C ABI (include/nextdoor_amd.h) is the host CSR above: C++
+// callers may use an nd_graph* as the CSR* the reference's host functions pass around
+// (loadGraph returns it, App::numSamples / initialSample receive it).
+struct nd_graph : CSR {};

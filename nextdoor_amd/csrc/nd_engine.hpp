@@ -286,25 +286,32 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
   const uint32_t transit_index = pair_slot - sample * P.transits_per_sample;
-  VertexID neighbor, next_transit;
-  if (state_fits_pair<SampleType>::value && P.state_travels) {
-    // the state travels with the pair: a register copy
-    SampleType state;
-    uint32_t bits = P.pair_state ? P.pair_state[pair] : ((const uint32_t*)P.samples)[sample];
-    __builtin_memcpy(&state, &bits, sizeof(uint32_t));
-    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                        edges, weights, &state, &next_transit);
-    __builtin_memcpy(&bits, &state, sizeof(uint32_t));
-    if (P.emit_state) P.emit_state[pair] = bits;
-    // a walk that ends here leaves the stream of pairs: its state goes home
-    if (P.is_last || next_transit == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
-  } else if (std::is_empty<SampleType>::value) {
-    SampleType no_state;
-    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                        edges, weights, &no_state, &next_transit);
-  } else {
-    neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                        edges, weights, (SampleType*)P.samples + sample, &next_transit);
+  VertexID neighbor = P.invalid, next_transit = P.invalid;
+  bool travelled = false;
+  if constexpr (state_fits_pair<SampleType>::value) {
+    if (P.state_travels) {
+      // the state travels with the pair: a register copy
+      SampleType state;
+      uint32_t bits = P.pair_state ? P.pair_state[pair] : ((const uint32_t*)P.samples)[sample];
+      __builtin_memcpy(&state, &bits, sizeof(uint32_t));
+      neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                          edges, weights, &state, &next_transit);
+      __builtin_memcpy(&bits, &state, sizeof(uint32_t));
+      if (P.emit_state) P.emit_state[pair] = bits;
+      // a walk that ends here leaves the stream of pairs: its state goes home
+      if (P.is_last || next_transit == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
+      travelled = true;
+    }
+  }
+  if (!travelled) {
+    if constexpr (std::is_empty<SampleType>::value) {
+      SampleType no_state;
+      neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                          edges, weights, &no_state, &next_transit);
+    } else {
+      neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
+                                          edges, weights, (SampleType*)P.samples + sample, &next_transit);
+    }
   }
   const uint32_t per_sample = P.transits_per_sample * P.step_size;
   P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;

@@ -36,6 +36,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include <algorithm>
 #include <string>
@@ -1199,7 +1200,7 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
   rng.reset(P.seed, (P.first_sample + s) * P.step_size + nbr, (uint32_t)P.step);
   const VertexID sample_id = (VertexID)(P.first_sample + s);
   VertexID neighbor = P.invalid;
-  if constexpr (App::kNeighborhoodForm == apps::kConcatenated) {
+  if constexpr (apps::neighborhood_form_of<App>::value == apps::kConcatenated) {
     // only the first transit decides whether next() runs (nextdoor.cu:1421)
     if (transits[0] != P.invalid && transits[0] != -1) {
       const uint32_t begin = P.offsets[ls];
@@ -1210,7 +1211,7 @@ __global__ __launch_bounds__(256) void layer_execute_kernel(LayerParams P) {
           (VertexID_t)nbr, &rng);
       neighbor = r == -1 ? P.invalid : r;
     }
-  } else if constexpr (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+  } else if constexpr (apps::neighborhood_form_of<App>::value == apps::kDistinctByDegreeSquared) {
     const uint32_t parts = P.words_per_sample / kPartWords;
     DistinctByDegreeSquared distinct{P.bitmap + (size_t)ls * P.words_per_sample,
                                      P.part_before + (size_t)ls * (parts + 1),
@@ -1263,7 +1264,7 @@ class LayerEngine : public EngineBase {
     graph_ = nullptr;
     release(d_row_sums_);
     if (!dgraph_.upload(graph, false, app_uses_edge_lookup<App>::value, &last_error)) return -1;
-    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+    if (apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance) {
       // 1 / (weights of every vertex summed in edge order, sequential float adds)
       const size_t V = (size_t)graph->get_n_vertices();
       std::vector<float> sums(V);
@@ -1277,7 +1278,7 @@ class LayerEngine : public EngineBase {
       const int rc = build_dense_pieces(graph, sums.data());
       if (rc != 0) return rc;
     }
-    if (App::kNeighborhoodForm == apps::kDistinctByDegreeSquared) {
+    if (apps::neighborhood_form_of<App>::value == apps::kDistinctByDegreeSquared) {
       const int rc = build_dense_pieces(graph, nullptr);
       if (rc != 0) return rc;
     }
@@ -1340,14 +1341,14 @@ class LayerEngine : public EngineBase {
     // bytes a sample of a chunk holds: its bitmap (FastGCN form) or one key per vertex, padded
     // to whole stretches (LADIES form)
     uint64_t bytes_per_sample = (uint64_t)bitmap_words_ * sizeof(uint32_t);
-    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+    if (apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance) {
       const uint32_t bin_words = kBinVerticesSums / 32u;
       bytes_per_sample = (uint64_t)((bitmap_words_ + bin_words - 1) / bin_words) * kBinVerticesSums * sizeof(uint32_t);
     }
     const uint64_t fit = kBitmapBudgetBytes / bytes_per_sample;
     bitmap_chunk_samples_ = fit < 1 ? 1u : fit > (uint64_t)n_samples_ ? (uint32_t)n_samples_ : (uint32_t)fit;
     // the selection kernels of the LADIES form index the samples of a chunk by blockIdx.y
-    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance && bitmap_chunk_samples_ > 65535u)
+    if (apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance && bitmap_chunk_samples_ > 65535u)
       bitmap_chunk_samples_ = 65535u;
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
@@ -1374,7 +1375,7 @@ class LayerEngine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_item_start_, sizeof(uint32_t) * ((size_t)n_samples_ + 1)));
     ND_HIP_TRY(hipMalloc(&d_row_offsets_, sizeof(uint32_t) * (size_t)n_samples_ * widest));
     ND_HIP_TRY(hipMalloc(&d_small_scratch_, sizeof(uint32_t) * scan_scratch_elems((size_t)n_samples_ + 1)));
-    if (App::kNeighborhoodForm == apps::kRankedByLadiesImportance) {
+    if (apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance) {
       const size_t per_sample = sizeof(uint32_t) * ((size_t)n_samples_ + 1);
       ND_HIP_TRY(hipMalloc(&d_ranked_start_, per_sample));
       ND_HIP_TRY(hipMalloc(&d_select_kept_, per_sample));
@@ -1417,7 +1418,7 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipStreamSynchronize(stream_));
       // chunk limits: entries of concatenation the work arrays hold, or (bitmap form) bitmaps
       // that fit the budget and a grid of marking work items that fits 31 bits
-      constexpr bool by_bitmap = App::kNeighborhoodForm != apps::kConcatenated;
+      constexpr bool by_bitmap = apps::neighborhood_form_of<App>::value != apps::kConcatenated;
       const uint64_t entry_budget = by_bitmap ? bitmap_chunk_entries_ : chunk_entries_;
       const uint32_t sample_budget = by_bitmap ? bitmap_chunk_samples_ : S;
       for (uint32_t s = 0; s < S; ++s)
@@ -1489,7 +1490,7 @@ class LayerEngine : public EngineBase {
   // (see DensePieces).  inverse_row_sums: the LADIES form's 1 / rowsum per vertex, else nullptr.
   int build_dense_pieces(const CSR* graph, const float* inverse_row_sums) {
     release_dense_pieces();
-    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
+    constexpr bool ladies = apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance;
     uint32_t threshold = ladies ? kDensePieceEntriesSums : kDensePieceEntries;
     if (const char* env = getenv("ND_DENSE_PIECE_ENTRIES")) {  // 0: no pieces; small: to exercise them on small graphs
       const long long v = atoll(env);
@@ -1586,7 +1587,7 @@ class LayerEngine : public EngineBase {
     App app;
     const uint32_t n = s1 - s0;
     const size_t F = (size_t)final_sample_size();
-    constexpr int form = App::kNeighborhoodForm;
+    constexpr int form = apps::neighborhood_form_of<App>::value;
     TransitView tv = all;
     tv.base = all.base + (size_t)s0 * all.stride;
     if (form != apps::kConcatenated) {
@@ -1646,7 +1647,7 @@ class LayerEngine : public EngineBase {
 
   // What next() of the importance forms is handed, for every sample of the chunk.
   int build_distinct_by_bitmap(int step, uint32_t s0, const TransitView& tv, uint32_t n) {
-    constexpr bool ladies = App::kNeighborhoodForm == apps::kRankedByLadiesImportance;
+    constexpr bool ladies = apps::neighborhood_form_of<App>::value == apps::kRankedByLadiesImportance;
     constexpr uint32_t bin_words = ladies ? kBinVerticesSums / 32u : kBinWordsBits;
     const uint32_t bins = (bitmap_words_ + bin_words - 1) / bin_words;
     constexpr uint32_t per_group = ladies ? kBinsPerGroupSums : kBinsPerGroupBits;
@@ -1761,7 +1762,7 @@ class LayerEngine : public EngineBase {
   // (FastGCN form) or the pairs the selection keeps (LADIES form).
   int ensure_distinct_capacity(uint32_t n_distinct) {
     if (n_distinct <= distinct_capacity_ && distinct_capacity_ > 0) return 0;
-    constexpr int form = App::kNeighborhoodForm;
+    constexpr int form = apps::neighborhood_form_of<App>::value;
     const size_t cap = (size_t)n_distinct + n_distinct / 8 + 1024;
     release_distinct_buffers();
     if (form == apps::kRankedByLadiesImportance) {

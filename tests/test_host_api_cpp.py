@@ -5,18 +5,8 @@ import subprocess
 
 import pytest
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SRC = os.path.join(ROOT, "tests", "cpp", "host_api_probe.cpp")
-EXE = os.path.join(ROOT, "tests", "cpp", "host_api_probe")
-
-
-def build_probe():
-    from nextdoor_amd.build import LIB_PATH
-    assert os.path.exists(LIB_PATH), "build the library first: python -m nextdoor_amd.build"
-    lib_dir = os.path.dirname(LIB_PATH)
-    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), SRC, "-o", EXE,
-           "-L", lib_dir, "-lnextdoor_amd", "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib"]
-    subprocess.run(cmd, check=True, capture_output=True, text=True)
+from tests.cpp import build_cpp
+from tests.cpp.build_cpp import HOST_PROBE as EXE, TEMPLATE_PROBE, build_host_probe as build_probe
 
 
 def write_graph(path):
@@ -47,3 +37,47 @@ def test_nextdoor_entry_runs_on_the_gpu(tmp_path):
     assert "final_size 8 values 96" in out.stdout
     assert "kernel types agree" in out.stdout
     assert "edge lists 300" in out.stdout  # MVS5: 20 batches of 5 vertices with 3 out-edges each
+    assert "reference-style tests pass" in out.stdout  # the testBase.h macro with the template spellings
+
+
+def test_caller_with_an_app_of_its_own_compiles():
+    """A translation unit in the reference's style - an App struct, then
+    appMain<SampleType, App>(argc, argv, checkSampledVerticesResult<SampleType, App>) - builds
+    with hipcc against the header; so does the testBase.h macro with the template spellings."""
+    exe = build_cpp.build_template_probe()
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)  # no graph: usage text, as src/main.cu:31-47
+    assert out.returncode == 0 and "--graph-file" in out.stdout
+
+
+def parse_samples(text):
+    rows = []
+    for line in text.splitlines():
+        if line.startswith("Contents of sample"):
+            rows.append([int(v) for v in line[line.index("[") + 1:line.index("]")].split(",") if v.strip()])
+    return rows
+
+
+@pytest.mark.gpu
+def test_caller_with_an_app_of_its_own_samples_what_the_oracle_does(tmp_path):
+    import numpy as np
+    from tests import oracle_binding as ob
+    assert os.path.exists(TEMPLATE_PROBE), "tests/cpp/template_api_probe is built by __graft_entry__.build()"
+    graph = tmp_path / "ring.txt"
+    write_graph(graph)
+    import nextdoor_amd as nd
+    from tests import graphs
+    loaded = nd.Graph.load(str(graph), "edge-list", "text")  # the same ingest, host only; owns the arrays below
+    og = graphs.oracle_view(loaded)
+    d = ob.app_desc(ob.UNIFORM_WALK, 6, [1] * 6)
+    want, _ = ob.sample_individual(og, d, 42, np.arange(12, dtype=np.int32))
+    for flags in (["-k", "TransitParallel", "-l"], ["-k", "TransitParallel"], ["-k", "SampleParallel"]):
+        print("template_api_probe", flags, flush=True)
+        out = subprocess.run([TEMPLATE_PROBE, "-g", str(graph), "-t", "edge-list", "-f", "text", "-n", "1", "-c", "-p"] + flags,
+                             capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert "Graph has 36 edges and 12 vertices" in out.stdout
+        assert np.array_equal(np.array(parse_samples(out.stdout), np.int32), want), out.stdout
+        assert "totalSampledVertices 72" in out.stdout
+    out = subprocess.run([TEMPLATE_PROBE, "--registry-app", str(graph)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.count("totalSampledVertices 108") == 2  # KHop3x2App: 12 samples x (3 + 6)
