@@ -212,7 +212,8 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
 int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t n, int key_bits, int32_t* d_keys_out,
                           int32_t* d_vals_out, void* stream);
 /* invalidVertexStartPos + DeviceRunLengthEncode::Encode + DeviceScan::ExclusiveSum
- * (src/nextdoor.cu:1804-1836, 2535-2545, 2560-2567) over a sorted key array. */
+ * (src/nextdoor.cu:1804-1836, 2535-2545, 2560-2567) over a sorted key array.  Stand-alone: the
+ * sampling pass classifies runs at their last pair (nd_classify_runs) and never lists them. */
 int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, int32_t* uniq, int32_t* counts,
                        int32_t* offsets, int64_t* n_runs, int64_t* n_valid);
 

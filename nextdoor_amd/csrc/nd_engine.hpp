@@ -855,6 +855,7 @@ class Engine : public EngineBase {
   // transferCSRToGPUs: the whole graph is resident on the device, plus the derived
   // structures the app asks for (interleaved edges, edge index).
   int set_graph(const CSR* graph) override {
+    free_run_buffers();  // sized against the previous graph: alloc() is due again
     graph_ = nullptr;
     dgraph_ = std::make_shared<DeviceGraph>();
     if (!dgraph_->upload(graph, app_uses_weights<App>::value, app_uses_edge_lookup<App>::value, &last_error)) return -1;
@@ -878,7 +879,8 @@ class Engine : public EngineBase {
   // Allocates for samples [first, first + count) of the app's samples (count < 0: all).
   // Sample indices, roots and random streams are those of the whole run, so the ranges of
   // several engines put together are the bytes one engine produces for everything.
-  int alloc_range(uint64_t seed, int64_t first, int64_t count) {
+  // host_rows false: the caller fetches the rows into memory of its own (fetch_final_samples_into).
+  int alloc_range(uint64_t seed, int64_t first, int64_t count, bool host_rows = true) {
     if (!graph_) { last_error = "alloc before set_graph"; return -1; }
     free_run_buffers();
     seed_ = seed;
@@ -948,7 +950,7 @@ class Engine : public EngineBase {
     max_pairs_ = (size_t)max_pairs;
     chunk_capacity_ = (uint32_t)chunk_cap;
     const size_t F = (size_t)final_sample_size();
-    hFinalSamples.assign((size_t)n_samples_ * F, invalid_);
+    if (host_rows) hFinalSamples.assign((size_t)n_samples_ * F, invalid_); else hFinalSamples.clear();
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
     ND_HIP_TRY(hipMalloc(&d_initial_, sizeof(VertexID_t) * initialContents.size()));
@@ -1461,13 +1463,13 @@ class Engine : public EngineBase {
     release(d_chunks_);
     release(d_skip_flag_);
     release(d_distinct_counts_);
-    if (allocated_) {
-      (void)hipEventDestroy(ev_a_);
-      (void)hipEventDestroy(ev_b_);
-      (void)hipEventDestroy(ev_begin_);
-      (void)hipEventDestroy(ev_end_);
-      (void)hipStreamDestroy(stream_);
+    // whatever exists, also after an alloc that failed half way
+    for (hipEvent_t* ev : {&ev_a_, &ev_b_, &ev_begin_, &ev_end_}) {
+      if (*ev) (void)hipEventDestroy(*ev);
+      *ev = nullptr;
     }
+    if (stream_) (void)hipStreamDestroy(stream_);
+    stream_ = nullptr;
     allocated_ = false;
   }
 

@@ -1261,6 +1261,7 @@ class LayerEngine : public EngineBase {
   }
 
   int set_graph(const CSR* graph) override {
+    free_run_buffers();  // sized against the previous graph: alloc() is due again
     graph_ = nullptr;
     release(d_row_sums_);
     if (!dgraph_.upload(graph, false, app_uses_edge_lookup<App>::value, &last_error)) return -1;
@@ -1819,13 +1820,13 @@ class LayerEngine : public EngineBase {
     release(d_ranked_start_); release(d_select_kept_);
     release(d_select_threshold_); release(d_select_present_);
     release_neighborhood_buffers();
-    if (allocated_) {
-      (void)hipEventDestroy(ev_begin_);
-      (void)hipEventDestroy(ev_end_);
-      (void)hipEventDestroy(ev_a_);
-      (void)hipEventDestroy(ev_b_);
-      (void)hipStreamDestroy(stream_);
+    // whatever exists, also after an alloc that failed half way
+    for (hipEvent_t* ev : {&ev_a_, &ev_b_, &ev_begin_, &ev_end_}) {
+      if (*ev) (void)hipEventDestroy(*ev);
+      *ev = nullptr;
     }
+    if (stream_) (void)hipStreamDestroy(stream_);
+    stream_ = nullptr;
     allocated_ = false;
   }
 

@@ -74,14 +74,12 @@ class ShardedEngine : public EngineBase {
     int64_t first = 0;
     for (int i = 0; i < n_parts; ++i) {
       const int64_t count = (n - first) / (n_parts - i);
-      const int rc = parts_[i]->alloc_range(seed, first, count);
+      const int rc = parts_[i]->alloc_range(seed, first, count, /*host_rows=*/false);  // the rows come home through ours
       if (rc != 0) return fail(i, rc);
       initialContents.insert(initialContents.end(), parts_[i]->initialContents.begin(),
                              parts_[i]->initialContents.end());
       first += count;
     }
-    if (n_parts > 1)
-      for (auto& p : parts_) p->hFinalSamples.clear();  // the rows come home through ours
     hFinalSamples.assign((size_t)n * (size_t)final_sample_size(), invalid_vertex());
     return 0;
   }

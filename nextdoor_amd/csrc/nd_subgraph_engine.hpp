@@ -283,6 +283,7 @@ class SubgraphEngine : public EngineBase {
   size_t sample_state_bytes() const override { return sizeof(SampleType) * (size_t)n_samples_; }
 
   int set_graph(const CSR* graph) override {
+    free_run_buffers();  // sized against the previous graph: alloc() is due again
     graph_ = nullptr;
     if (!dgraph_.upload(graph, false, false, &last_error)) return -1;
     graph_ = graph;
@@ -504,8 +505,8 @@ class SubgraphEngine : public EngineBase {
   }
 
   void free_run_buffers() {
-    if (!allocated_) return;
-    (void)hipStreamSynchronize(stream_);
+    // whatever exists, also after an alloc that failed half way
+    if (stream_) (void)hipStreamSynchronize(stream_);
     release(d_initial_);
     release(d_stored_);
     release(d_final_);
@@ -517,9 +518,12 @@ class SubgraphEngine : public EngineBase {
     release(d_rows_);
     release(d_cols_);
     list_capacity_ = 0;
-    (void)hipEventDestroy(ev_begin_);
-    (void)hipEventDestroy(ev_end_);
-    (void)hipStreamDestroy(stream_);
+    for (hipEvent_t* ev : {&ev_begin_, &ev_end_}) {
+      if (*ev) (void)hipEventDestroy(*ev);
+      *ev = nullptr;
+    }
+    if (stream_) (void)hipStreamDestroy(stream_);
+    stream_ = nullptr;
     allocated_ = false;
   }
 

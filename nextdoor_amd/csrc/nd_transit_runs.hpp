@@ -7,6 +7,11 @@
 // device->host copies in between, this does the same in three launches whose sizes are
 // known on the host up front; every count the later kernels need stays in device memory.
 //
+// A building block with an entry point and tests of its own (nd_unique_transits): the engine's
+// pass does not launch it.  The step loop needs no list of the unique transits - it finds each
+// run's extent at the run's last pair and classifies it there (classify_run_tails in
+// nd_engine.hpp); only RunsMeta below is shared with it.
+//
 // A run head is a position i with key[i] != INVALID and (i == 0 or key[i] != key[i-1]).
 // run r = the r-th head: run_key[r], run_start[r]; run_start[n_runs] = n_valid, so the
 // count of run r is run_start[r+1] - run_start[r] (the exclusive scan of the counts is

@@ -304,3 +304,30 @@ def test_two_sample_ranges_give_the_bytes_of_one(oracle, app, kind_name, state, 
     g = graphs.random_graph(n=1501, mean_degree=6, seed=17, hub=4, isolated_every=11)
     run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
     run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, inversion_period=0)
+
+
+@pytest.mark.parametrize("app", ["KHop", "FastGCN", "MVS5"])
+def test_a_new_graph_needs_a_new_alloc(oracle, app):
+    """transferCSRToGPUs on a sampler that already ran: the buffers of the old graph are gone,
+    sampling before the next allocNextDoorDataOnGPU is an error, and after it the samples are
+    those of the new graph."""
+    L = nd._capi.lib()
+    small = graphs.random_graph(n=200, mean_degree=6, seed=21)
+    large = graphs.random_graph(n=900, mean_degree=6, seed=22, hub=4)
+    s = nd.Sampler(app, large, seed=SEED)
+    try:
+        s.do_transit_parallel(True)
+        nd.check(L.nd_sampler_set_graph(s._h, small._h))
+        s.graph = small
+        with pytest.raises(nd.NextDoorError, match="alloc"):
+            s.do_transit_parallel(True)
+        nd.check(L.nd_sampler_alloc(s._h, SEED))
+        s.do_transit_parallel(True)
+        got = s.final_samples()
+        fresh = nd.Sampler(app, small, seed=SEED)
+        fresh.do_transit_parallel(True)
+        want = fresh.final_samples()
+        fresh.close()
+        assert got.shape == want.shape and np.array_equal(got, want)
+    finally:
+        s.close()
