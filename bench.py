@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
 # known size).  None where no such run has been recorded.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 1.246e9,     # step_flat_kernel
+    "weighted_node2vec_rmat22": 1.171e9,     # step_flat_kernel
     "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
     "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
     "fastgcn_importance_rmat22": 5.273e9,    # collective_mark_binned, average over its 2 launches per pass
@@ -36,8 +36,14 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
-    "weighted_node2vec_rmat22": 163.4e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
+    "weighted_node2vec_rmat22": 154.3e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
     "fastgcn_importance_rmat22": 16.4e9, "ladies_importance_chunglu3m": 160.8e9,
+}
+
+# Read requests one launch of the dominant kernel sends past L2 (rocprofv3 TCC_EA0_RDREQ_sum, every
+# one of them 128 bytes: profiles/step_kernels_<workload>_l2_requests.md).  None where not recorded.
+MEASURED_L2_MISS_REQUESTS_PER_LAUNCH = {
+    "weighted_node2vec_rmat22": 8.31e6,      # step_flat_kernel
 }
 
 WORKLOADS = {
@@ -407,6 +413,22 @@ def main():
                            "measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
         }
         result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
+        misses = MEASURED_L2_MISS_REQUESTS_PER_LAUNCH.get(args.workload)
+        if misses:
+            # The step kernel's reads are dependent random gathers; each one that misses L2 costs a
+            # 128-byte request whatever it uses.  The ceiling for such requests is measured here, on
+            # this GPU, over a table of the size of the graph's arrays (rounded down to a power of two).
+            graph_bytes = 4.0 * graph.n_vertices * 2 + graph.n_edges * (8.0 + 4.0 * 8.0)
+            table_bytes = 1 << (int(graph_bytes).bit_length() - 1)
+            ceiling = nd.measure_gather_rate(table_bytes)
+            flat_ms = prof["flat_kernel_ms"] / max(launches, 1)
+            result["roofline"]["l2_miss_path"] = {
+                "requests_per_launch": misses, "bytes_per_request": 128,
+                "achieved_requests_per_s": misses / (flat_ms / 1000.0),
+                "ceiling_requests_per_s": ceiling, "ceiling_table_bytes": table_bytes,
+                "frac_of_ceiling": misses / (flat_ms / 1000.0) / ceiling,
+                "ceiling_as_GBps": ceiling * 128 / 1e9,
+            }
     del final
     sampler.close()
     print(json.dumps(result))

@@ -234,6 +234,12 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
                      int partial_cache, int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items,
                      uint8_t* taken, int64_t counters[5]);
 
+/* Measurement, no counterpart in the reference: the rate (requests per second) at which this GPU
+ * serves independent random 8-byte reads over a table of table_bytes (a power of two, 4 KiB to
+ * 32 GiB; allocated and freed inside): 4 M lanes, 16 reads each, two in flight per lane.  The
+ * ceiling a gather-bound step kernel is priced against next to the HBM byte peak. */
+int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s);
+
 /* collectiveNeighbrsSize + collectiveNeighborhood (src/nextdoor.cu:1206-1283) for n_samples
  * samples of transits_per_sample transits each (transits[s * transits_per_sample + i]):
  * sizes[s] = sum of the degrees of the valid transits, offsets = their exclusive scan

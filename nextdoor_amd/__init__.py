@@ -22,7 +22,7 @@ from . import _capi
 from ._capi import NextDoorError, check, lib
 
 __all__ = ["Graph", "Sampler", "SamplingModule", "NextDoorError", "app_names", "load_app_library",
-           "philox_fill_uniform", "sort_pairs", "sort_pairs_noalloc", "unique_transits", "classify_runs", "load_balancing_thresholds", "collective_neighborhood", "check_sampled_vertices"]
+           "philox_fill_uniform", "sort_pairs", "sort_pairs_noalloc", "unique_transits", "classify_runs", "load_balancing_thresholds", "measure_gather_rate", "collective_neighborhood", "check_sampled_vertices"]
 
 
 def app_names():
@@ -373,6 +373,13 @@ def sort_pairs_noalloc(d_keys, d_vals, n, key_bits, d_keys_out, d_vals_out, stre
     value is the index), enqueued on `stream` (a hipStream_t as an integer, 0 = default stream)
     with all working memory inside the library; allocates nothing and does not wait."""
     check(lib().nd_sort_pairs_noalloc(d_keys, d_vals or None, n, key_bits, d_keys_out, d_vals_out, stream or None))
+
+
+def measure_gather_rate(table_bytes):
+    """Independent random 8-byte reads per second over a table of ``table_bytes`` (power of two)."""
+    rate = C.c_double()
+    check(lib().nd_measure_gather_rate(int(table_bytes), C.byref(rate)))
+    return rate.value
 
 
 def unique_transits(sorted_keys, invalid):

@@ -165,6 +165,32 @@ __global__ void philox_fill_kernel(uint64_t seed, uint32_t step, uint64_t first_
   for (int d = 0; d < draws_per_slot; ++d) out[slot * draws_per_slot + d] = rng.next_uniform();
 }
 
+__device__ __forceinline__ uint32_t probe_mix(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+// Every lane reads `reads` 8-byte words at hashed positions of a table of (mask + 1) words,
+// kInFlight of them issued before any is used.
+template <int kInFlight>
+__global__ __launch_bounds__(256) void gather_rate_kernel(const uint2* __restrict__ table, uint32_t mask,
+                                                         uint32_t rounds, uint32_t* sink) {
+  const uint32_t lane = blockIdx.x * 256 + threadIdx.x;
+  uint32_t acc = 0, at = probe_mix(lane * 2654435761u + 1u);
+  for (uint32_t r = 0; r < rounds; ++r) {
+    uint2 got[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      at = probe_mix(at + (uint32_t)k + r);
+      got[k] = table[at & mask];
+    }
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) acc += got[k].x ^ got[k].y;
+    at ^= acc & 1u;
+  }
+  sink[lane] = acc;
+}
+
 __global__ void run_counts_kernel(const uint32_t* run_start, const nd::RunsMeta* meta, uint32_t* counts) {
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r < meta->n_runs) counts[r] = run_start[r + 1] - run_start[r];
@@ -674,6 +700,41 @@ int nd_load_balancing_thresholds(int32_t out[3]) {
   out[1] = (int32_t)nd::kChunkOutputs;
   out[2] = (int32_t)nd::kCacheEdges;
   return 0;
+}
+
+// ---- measurement: what the memory system gives independent random 8-byte reads --------------
+
+int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
+  return guarded([&]() -> int {
+    if (!requests_per_s || table_bytes < 4096 || table_bytes > (1ll << 35) || (table_bytes & (table_bytes - 1)))
+      return fail("table_bytes must be a power of two between 4 KiB and 32 GiB");
+    constexpr uint32_t kLanes = 1u << 22, kRounds = 8;
+    constexpr int kInFlight = 2;
+    DeviceBuffer table, sink;
+    CAPI_HIP(table.alloc((size_t)table_bytes));
+    CAPI_HIP(sink.alloc(sizeof(uint32_t) * kLanes));
+    CAPI_HIP(hipMemset(table.p, 1, (size_t)table_bytes));
+    hipEvent_t begin = nullptr, end = nullptr;
+    CAPI_HIP(hipEventCreate(&begin));
+    hipError_t e = hipEventCreate(&end);
+    float best_ms = 0.0f;
+    for (int rep = 0; e == hipSuccess && rep < 3; ++rep) {  // the first launch warms the translation caches
+      e = hipEventRecord(begin, nullptr);
+      gather_rate_kernel<kInFlight><<<dim3(kLanes / 256), dim3(256)>>>(table.as<uint2>(), (uint32_t)(table_bytes / 8 - 1),
+                                                                       kRounds, sink.as<uint32_t>());
+      if (e == hipSuccess) e = hipGetLastError();
+      if (e == hipSuccess) e = hipEventRecord(end, nullptr);
+      if (e == hipSuccess) e = hipEventSynchronize(end);
+      float ms = 0.0f;
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, begin, end);
+      if (rep > 0 && (best_ms == 0.0f || ms < best_ms)) best_ms = ms;
+    }
+    (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    CAPI_HIP(e);
+    *requests_per_s = (double)kLanes * kRounds * kInFlight / ((double)best_ms / 1000.0);
+    return 0;
+  });
 }
 
 int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,

@@ -414,7 +414,7 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
   constexpr bool kTravels = state_fits_pair<SampleType>::value;
   SampleType local_state;
   SampleType* state = &local_state;
-  if (kTravels) {
+  if constexpr (kTravels) {
     const uint32_t bits = P.pair_state ? P.pair_state[i] : ((const uint32_t*)P.samples)[slot];
     __builtin_memcpy(&local_state, &bits, sizeof(uint32_t));
   } else if (!std::is_empty<SampleType>::value) {
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
     P.emit_keys[i] = (uint32_t)transit;
     P.emit_slots[i] = slot;
   }
-  if (kTravels) {
+  if constexpr (kTravels) {
     uint32_t bits;
     __builtin_memcpy(&bits, &local_state, sizeof(uint32_t));
     if (P.emit_state && !pass_over) P.emit_state[i] = bits;

@@ -131,3 +131,14 @@ def test_run_classification_of_a_map_without_long_runs_and_of_an_empty_map():
     assert wanted == 0 and not taken.any() and counters.tolist() == [100, 0, 0, 0, 0]
     items, wanted, taken, counters = nd.classify_runs(np.zeros(0, np.int32), degrees, 1)
     assert wanted == 0 and not taken.any()
+
+
+def test_gather_rate_measurement_orders_the_memory_levels():
+    """The measurement behind the bench's request ceiling: a table that fits L2 serves random
+    reads faster than one that does not, and bad sizes are refused."""
+    small = nd.measure_gather_rate(1 << 20)
+    large = nd.measure_gather_rate(1 << 30)
+    print("gather rates", small, large, flush=True)
+    assert small > large > 1e9
+    with pytest.raises(nd.NextDoorError):
+        nd.measure_gather_rate(3 << 20)
