@@ -1362,7 +1362,10 @@ class Engine : public EngineBase {
     }
     times.distinct = 0;
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
-    for (int k = 0; k < n_steps; ++k) {
+    const bool rows_at_once = launch_distinct_rows(d_final_, d_distinct_counts_, (uint32_t)n_samples_,
+                                                   (uint32_t)final_sample_size(), layout_.seg_base, layout_.seg_len,
+                                                   (uint32_t)n_steps, invalid_, !app.hasExplicitTransits(), stream_);
+    for (int k = 0; k < n_steps && !rows_at_once; ++k) {
       if (!launch_distinct_segment(d_final_, d_distinct_counts_, (uint32_t)n_samples_, (uint32_t)final_sample_size(),
                                    layout_.seg_base[k], layout_.seg_len[k], invalid_, (uint32_t)n_steps, (uint32_t)k,
                                    stream_)) {
