@@ -221,6 +221,16 @@ struct StepParams {
   uint32_t* emit_keys;           // next transit of each pair; nullptr: nothing is emitted
   uint32_t* emit_slots;          // its slot
   uint32_t* emit_state;          // its state after next()
+  // Small maps (see small_map_scan): a pair that goes on also takes its place among the pairs
+  // that will share its next transit - emit_ranks[pair] = its number among them, counted in
+  // emit_counts[next transit] - so that the next inversion needs no sort (nullptr: not in use).
+  // Transit v counts in the counters [emit_counter_base[v], emit_counter_base[v + 1]), a power
+  // of two of them, a pair counting in copy (its index & (copies - 1)): atomics on one address
+  // are served tens of nanoseconds apart, and a hub that takes thousands of walks per step would
+  // otherwise hold the step kernel up.  Most vertices have one counter.
+  uint32_t* emit_counts;
+  uint32_t* emit_ranks;
+  const uint32_t* emit_counter_base;
 };
 
 // A SampleType small enough to travel with its pair through the inversion.
@@ -318,6 +328,11 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
   if (P.emit_keys) {
     P.emit_keys[pair] = (uint32_t)next_transit;
     P.emit_slots[pair] = pair_slot;
+    if (P.emit_counts && next_transit != P.invalid) {
+      const uint32_t first = P.emit_counter_base[next_transit];
+      const uint32_t copies = P.emit_counter_base[next_transit + 1] - first;
+      P.emit_ranks[pair] = atomicAdd(&P.emit_counts[first + (pair & (copies - 1u))], 1u);
+    }
   }
 }
 
@@ -698,6 +713,155 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Inversion of a small map without a sort
+// ---------------------------------------------------------------------------------------
+// A digit pass of the radix sort is three dependent launches, and on a map of a few ten thousand
+// pairs every launch is a handful of microseconds of latency whatever it does: 57 K walks spend
+// 3.5 of their 4.8 ms per pass there.  For walks over at most kSmallMapPairs pairs and
+// kSmallMapVertices vertices the step kernels count, as they emit a pair, how many pairs went to
+// the same next transit before it (emit_ranks, emit_counts); two launches then place every pair:
+// small_map_scan turns the counts into starts inside chunks of 1024 counters and chunk totals;
+// small_map_place scans the (at most 1024) chunk totals once per workgroup in LDS - cheaper than
+// a third launch or a ticket that every chunk takes with an atomic on one address - and writes
+// pair i to start[transit] + rank and lets the pair with rank 0 classify
+// its run for the load-balancing classes, as classify_run_tails does from the run's tail.  The
+// order inside a run is the order the atomics were served in; results do not depend on it
+// (randomness is keyed by the slot).  The counters of a transit (StepParams::emit_counter_base)
+// are consecutive, so its run is still one stretch of the placed pairs.
+constexpr uint32_t kSmallMapPairs = 1u << 17;
+constexpr uint32_t kSmallMapCounters = 1u << 20;  // counters of all vertices at most
+constexpr uint32_t kSmallMapWalksPerCounter = 16;   // a vertex expected to take more walks per step gets copies
+constexpr uint32_t kSmallMapMaxCopies = 256;
+constexpr uint32_t kSmallMapChunk = 1024;  // counters per workgroup of small_map_scan; at most 1024 chunks
+
+__global__ __launch_bounds__(256) void small_map_scan(uint32_t* __restrict__ counts, uint32_t n_counters,
+                                                      uint32_t* __restrict__ local_start,
+                                                      uint32_t* __restrict__ chunk_total) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  const uint32_t first = blockIdx.x * kSmallMapChunk + threadIdx.x * 4u;
+  uint32_t c[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    c[k] = first + k < n_counters ? counts[first + k] : 0u;
+    if (c[k]) counts[first + k] = 0;  // ready for the pairs the coming step emits
+  }
+  uint32_t block_total;
+  uint32_t before = block_exclusive_scan_256(c[0] + c[1] + c[2] + c[3], s_wave, &block_total);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (first + k < n_counters) local_start[first + k] = before;
+    before += c[k];
+  }
+  if (threadIdx.x == 0) chunk_total[blockIdx.x] = block_total;
+}
+
+__global__ __launch_bounds__(256) void small_map_place(
+    const uint32_t* __restrict__ emit_keys, const uint32_t* __restrict__ emit_slots,
+    const uint32_t* __restrict__ emit_state, const uint32_t* __restrict__ emit_ranks, const uint32_t* __restrict__ n_in_dev,
+    uint32_t n_in_host, uint32_t invalid, const uint32_t* __restrict__ counter_base, const uint32_t* __restrict__ local_start,
+    const uint32_t* __restrict__ chunk_total, uint32_t n_chunks, uint32_t* __restrict__ live_out,
+    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ slots_out,
+    uint32_t* __restrict__ state_out,
+    // load balancing (classify == 0: none of it)
+    uint32_t classify, RunsMeta* meta, RunsMeta* meta_of_next_step, const EdgePos_t* __restrict__ row_ptr,
+    uint32_t step_size, uint32_t* __restrict__ chunks, uint32_t chunk_capacity, uint8_t* __restrict__ skip_flag,
+    ClassCounters* __restrict__ counters, uint32_t partial_cache) {
+  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  __shared__ uint32_t chunk_base[1024];
+  const uint32_t n_in = n_in_dev ? *n_in_dev : n_in_host;
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  {
+    // where every chunk starts among the placed pairs
+    uint32_t t[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t[k] = threadIdx.x * 4u + k < n_chunks ? chunk_total[threadIdx.x * 4u + k] : 0u;
+    uint32_t total;
+    uint32_t base = block_exclusive_scan_256(t[0] + t[1] + t[2] + t[3], s_wave, &total);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      chunk_base[threadIdx.x * 4u + k] = base;
+      base += t[k];
+    }
+    __syncthreads();
+    if (i == 0) {
+      *live_out = total;  // pairs that go on: what the step kernels of this step walk
+      if (classify) {
+        meta_of_next_step->n_chunks = 0;  // see classify_run_tails
+        atomicAdd(&counters->sorted_pairs, (unsigned long long)total);
+      }
+    }
+  }
+  uint32_t transit = invalid, start = 0, count = 0, n_items = 0, refused = 0;
+  bool head = false;
+  if (i < n_in) {
+    transit = emit_keys[i];
+    if (transit != invalid) {
+      const uint32_t rank = emit_ranks[i];
+      const uint32_t first_copy = counter_base[transit];
+      const uint32_t beyond = counter_base[transit + 1];  // the counter after the last one exists
+      const uint32_t mine = first_copy + (i & (beyond - first_copy - 1u));
+      const uint32_t pos = chunk_base[mine / kSmallMapChunk] + local_start[mine] + rank;
+      keys_out[pos] = transit;
+      slots_out[pos] = emit_slots[i];
+      if (state_out) state_out[pos] = emit_state[i];
+      if (rank == 0) {
+        // the first pair of the first copy that counted any is the first pair of the run
+        const uint32_t run_start = chunk_base[first_copy / kSmallMapChunk] + local_start[first_copy];
+        if (pos == run_start) {
+          head = true;
+          start = pos;
+          count = chunk_base[beyond / kSmallMapChunk] + local_start[beyond] - run_start;
+        }
+      }
+    }
+  }
+  if (!classify) return;
+  // the run's class, decided by its first pair (rules of workgroup_run_ends_at)
+  if (head) {
+    const uint64_t work = (uint64_t)count * step_size;
+    const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
+    if (work >= kWorkgroupWork && degree != 0) {
+      const uint32_t staged = degree < (uint32_t)kCacheEdges ? degree : (uint32_t)kCacheEdges;
+      if ((degree > (uint32_t)kCacheEdges && !partial_cache) || (uint64_t)staged > 32ull * work) {
+        refused = count;
+      } else {
+        uint32_t pairs_per_chunk = kChunkOutputs / step_size;
+        if (pairs_per_chunk == 0) pairs_per_chunk = 1;
+        n_items = (count + pairs_per_chunk - 1) / pairs_per_chunk;
+      }
+    }
+  }
+  uint32_t single_pairs = n_items == 1 ? count : 0, split_pairs = n_items > 1 ? count : 0, items = n_items;
+  for (int d = 1; d < kWave; d <<= 1) {
+    single_pairs += __shfl_xor(single_pairs, d, kWave);
+    split_pairs += __shfl_xor(split_pairs, d, kWave);
+    refused += __shfl_xor(refused, d, kWave);
+    items += __shfl_xor(items, d, kWave);
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    ClassCounters* mine_c = counters + ((blockIdx.x * (256 / kWave) + threadIdx.x / kWave) % kCounterCopies);
+    if (single_pairs) atomicAdd(&mine_c->workgroup_pairs, (unsigned long long)single_pairs);
+    if (split_pairs) atomicAdd(&mine_c->split_pairs, (unsigned long long)split_pairs);
+    if (refused) atomicAdd(&mine_c->refused_pairs, (unsigned long long)refused);
+    if (items) atomicAdd(&mine_c->work_items, (unsigned long long)items);
+  }
+  if (items == 0) return;  // the same for every lane of the wavefront
+  const uint32_t incl = wave_inclusive_scan(n_items);
+  uint32_t wave_base = 0;
+  if ((threadIdx.x & (kWave - 1)) == kWave - 1) wave_base = atomicAdd(&meta->n_chunks, incl);
+  const uint32_t base = __shfl(wave_base, kWave - 1, kWave) + incl - n_items;
+  if (n_items == 0) return;
+  uint32_t pairs_per_chunk = kChunkOutputs / step_size;
+  if (pairs_per_chunk == 0) pairs_per_chunk = 1;
+  for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
+    const uint32_t off = g * pairs_per_chunk;
+    chunks[2 * (base + g)] = start + off;
+    chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+  }
+  if (base + n_items <= chunk_capacity) skip_flag[transit] = 1;
+}
+
 __global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = value;
@@ -990,6 +1154,38 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_emit_keys_, sizeof(uint32_t) * max_pairs_));
       ND_HIP_TRY(hipMalloc(&d_emit_slots_, sizeof(uint32_t) * max_pairs_));
     }
+    // Counters per vertex for the small-map inversion: the walks that step onto a vertex are
+    // about its share of the edge ends; one counter per kSmallMapWalksPerCounter of them.
+    small_map_ = false;
+    if (walk_mode_ && max_pairs_ <= kSmallMapPairs && (uint64_t)invalid_ < kSmallMapCounters &&
+        !(getenv("ND_SMALL_MAP") && atoi(getenv("ND_SMALL_MAP")) == 0)) {
+      const size_t V = (size_t)graph_->get_n_vertices();
+      const double per_edge = graph_->col.empty() ? 0.0 : (double)max_pairs_ / (double)graph_->col.size();
+      std::vector<uint32_t> base(V + 1), edges_into(V, 0);
+      for (const CSR::Edge dst : graph_->col) edges_into[(size_t)dst]++;
+      uint64_t at = 0;
+      for (size_t v = 0; v < V; ++v) {
+        base[v] = (uint32_t)at;
+        const double walks = per_edge * (double)edges_into[v];
+        uint32_t copies = 1;
+        while (copies < kSmallMapMaxCopies && (double)(copies * kSmallMapWalksPerCounter) < walks) copies <<= 1;
+        at += copies;
+      }
+      base[V] = (uint32_t)at;
+      small_counters_ = (size_t)at + 1;  // one more, so that every run has an end to read
+      small_map_ = small_counters_ < kSmallMapCounters;
+      if (small_map_) {
+        ND_HIP_TRY(hipMalloc(&d_counter_base_, sizeof(uint32_t) * base.size()));
+        ND_HIP_TRY(hipMemcpy(d_counter_base_, base.data(), sizeof(uint32_t) * base.size(), hipMemcpyHostToDevice));
+      }
+    }
+    if (small_map_) {
+      // counters, their starts inside a chunk, chunk totals
+      const size_t counters = small_counters_, chunks = (counters + kSmallMapChunk - 1) / kSmallMapChunk;
+      ND_HIP_TRY(hipMalloc(&d_small_, sizeof(uint32_t) * (2 * counters + chunks)));
+      ND_HIP_TRY(hipMemset(d_small_, 0, sizeof(uint32_t) * (2 * counters + chunks)));
+      ND_HIP_TRY(hipMalloc(&d_emit_ranks_, sizeof(uint32_t) * max_pairs_));
+    }
     if (state_travels_) {
       ND_HIP_TRY(hipMalloc(&d_emit_state_, sizeof(uint32_t) * max_pairs_));
       ND_HIP_TRY(hipMalloc(&d_aux_a_, sizeof(uint32_t) * max_pairs_));
@@ -1141,6 +1337,11 @@ class Engine : public EngineBase {
       P.emit_keys = emits ? d_emit_keys_ : nullptr;
       P.emit_slots = emits ? d_emit_slots_ : nullptr;
       P.emit_state = emits && state_travels_ ? d_emit_state_ : nullptr;
+      // small maps inverted at every step: the emitting kernels count the pairs per next transit
+      const bool counted = small_map_ && sort_period == 1 && !sample_parallel;
+      P.emit_counts = emits && counted ? d_small_ : nullptr;
+      P.emit_ranks = emits && counted ? d_emit_ranks_ : nullptr;
+      P.emit_counter_base = d_counter_base_;
       uint32_t* live_now = d_live_ + (sorts_done & 1);  // pairs the inversion of this step keeps
       // lanes of the flat kernel per pair: one when the pairs alone fill the machine, else
       // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
@@ -1164,83 +1365,123 @@ class Engine : public EngineBase {
         // Walks that invert only now and then gain nothing from the transit order (few of them
         // share a transit, and the order is stale one step later): they only drop the walks
         // that have ended, keeping slot order, in which the writes of a step's results coalesce.
-        const bool compact_only = sample_parallel || (walk_mode_ && sort_period > 1);
-        const SortPlan plan = make_sort_plan(n_pairs, compact_only ? 0 : max_bits_);
-        SortJob job;
-        if (walk_mode_) {
-          job.keys_in = d_emit_keys_;
-          job.vals_in = d_emit_slots_;
-          job.aux_in = state_travels_ ? d_emit_state_ : nullptr;
-          job.n_in_dev = live_last;
-        } else {
-          job.keys_in = (const uint32_t*)transits;
-          job.keys_in_layout = transits_layout;
-        }
-        job.keys_a = d_keys_a_;
-        job.vals_a = d_vals_a_;
-        job.aux_a = d_aux_a_;
-        job.keys_b = d_keys_b_;
-        job.vals_b = d_vals_b_;
-        job.aux_b = d_aux_b_;
-        job.hist = d_hist_;
-        job.scratch = d_scratch_;
-        job.drop_key = (uint32_t)invalid_;
-        job.kept_dev = live_now;
-        tick();
-        ND_HIP_TRY(radix_sort(plan, job, stream_));
-        tock(&times.inversion);
-        times.sort_launches += plan.passes;
-        uint32_t* sorted_keys = job.keys_sorted;
-        P.pair_keys = sorted_keys;
-        P.pair_slots = job.vals_sorted;
-        P.pair_state = state_travels_ ? job.aux_sorted : nullptr;
-        P.live_pairs = live_now;
-        live_last = live_now;
-        sorts_done++;
-        if (compact_only && walk_mode_) {
-          // the walks keep their lanes until the next compaction
-          const int stretch = n_steps - step < sort_period ? n_steps - step : sort_period;
-          P.emit_keys = d_emit_keys_;
-          P.emit_slots = d_emit_slots_;
-          P.emit_state = state_travels_ ? d_emit_state_ : nullptr;
-          tick();
-          walk_stretch_kernel<SampleType, App><<<dim3((n_pairs + kFlatThreads - 1) / kFlatThreads), dim3(kFlatThreads), 0,
-                                                 stream_>>>(P, stretch, n_steps - 1, (size_t)n_samples_);
-          tock(&times.flat_kernel);
-          times.flat_launches++;
-          step += stretch - 1;
-        } else if (!balance || compact_only) {
-          tick();
-          launch_flat(P, flat_grid, nullptr);
-          tock(&times.flat_kernel);
-          times.flat_launches++;
-        } else {
-          tick();
-          const unsigned pair_blocks = (n_pairs + 255) / 256;
+        if (counted) {
+          // small map: the previous step's kernels have counted the pairs per transit
+          const uint32_t n_keys = (uint32_t)small_counters_;
+          const uint32_t n_chunks = (n_keys + kSmallMapChunk - 1) / kSmallMapChunk;
+          uint32_t* counts = d_small_;
+          uint32_t* local_start = counts + n_keys;
+          uint32_t* chunk_total = local_start + n_keys;
           RunsMeta* meta = d_meta_ + (balanced_steps_ & 1);
           RunsMeta* meta_next = d_meta_ + ((balanced_steps_ + 1) & 1);
-          balanced_steps_++;
-          if (n_pairs >= kClassifyLargeFrom) {
-            const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
-            classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
-          } else {
-            classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
-                sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
-          }
-          tock(&times.load_balancing);
+          if (balance) balanced_steps_++;
           tick();
-          launch_flat(P, flat_grid, d_skip_flag_);
+          small_map_scan<<<dim3(n_chunks), dim3(256), 0, stream_>>>(counts, n_keys, local_start, chunk_total);
+          small_map_place<<<dim3((n_pairs + 255) / 256), dim3(256), 0, stream_>>>(
+              d_emit_keys_, d_emit_slots_, state_travels_ ? d_emit_state_ : nullptr, d_emit_ranks_, live_last, n_pairs,
+              (uint32_t)invalid_, d_counter_base_, local_start, chunk_total, n_chunks, live_now,
+              d_keys_a_, d_vals_a_,
+              state_travels_ ? d_aux_a_ : nullptr, balance ? 1u : 0u, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_,
+              chunk_capacity_, d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u);
+          tock(&times.inversion);
+          times.sort_launches += 1;
+          P.pair_keys = d_keys_a_;
+          P.pair_slots = d_vals_a_;
+          P.pair_state = state_travels_ ? d_aux_a_ : nullptr;
+          P.live_pairs = live_now;
+          live_last = live_now;
+          sorts_done++;
+          tick();
+          launch_flat(P, flat_grid, balance ? d_skip_flag_ : nullptr);
           tock(&times.flat_kernel);
           times.flat_launches++;
+          if (balance) {
+            tick();
+            unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
+            step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
+                P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
+            tock(&times.workgroup_kernel);
+            times.workgroup_launches++;
+          }
+        } else {
+          const bool compact_only = sample_parallel || (walk_mode_ && sort_period > 1);
+          const SortPlan plan = make_sort_plan(n_pairs, compact_only ? 0 : max_bits_);
+          SortJob job;
+          if (walk_mode_) {
+            job.keys_in = d_emit_keys_;
+            job.vals_in = d_emit_slots_;
+            job.aux_in = state_travels_ ? d_emit_state_ : nullptr;
+            job.n_in_dev = live_last;
+          } else {
+            job.keys_in = (const uint32_t*)transits;
+            job.keys_in_layout = transits_layout;
+          }
+          job.keys_a = d_keys_a_;
+          job.vals_a = d_vals_a_;
+          job.aux_a = d_aux_a_;
+          job.keys_b = d_keys_b_;
+          job.vals_b = d_vals_b_;
+          job.aux_b = d_aux_b_;
+          job.hist = d_hist_;
+          job.scratch = d_scratch_;
+          job.drop_key = (uint32_t)invalid_;
+          job.kept_dev = live_now;
           tick();
-          unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
-          step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
-              P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
-          tock(&times.workgroup_kernel);
-          times.workgroup_launches++;
+          ND_HIP_TRY(radix_sort(plan, job, stream_));
+          tock(&times.inversion);
+          times.sort_launches += plan.passes;
+          uint32_t* sorted_keys = job.keys_sorted;
+          P.pair_keys = sorted_keys;
+          P.pair_slots = job.vals_sorted;
+          P.pair_state = state_travels_ ? job.aux_sorted : nullptr;
+          P.live_pairs = live_now;
+          live_last = live_now;
+          sorts_done++;
+          if (compact_only && walk_mode_) {
+            // the walks keep their lanes until the next compaction
+            const int stretch = n_steps - step < sort_period ? n_steps - step : sort_period;
+            P.emit_keys = d_emit_keys_;
+            P.emit_slots = d_emit_slots_;
+            P.emit_state = state_travels_ ? d_emit_state_ : nullptr;
+            tick();
+            walk_stretch_kernel<SampleType, App><<<dim3((n_pairs + kFlatThreads - 1) / kFlatThreads), dim3(kFlatThreads), 0,
+                                                   stream_>>>(P, stretch, n_steps - 1, (size_t)n_samples_);
+            tock(&times.flat_kernel);
+            times.flat_launches++;
+            step += stretch - 1;
+          } else if (!balance || compact_only) {
+            tick();
+            launch_flat(P, flat_grid, nullptr);
+            tock(&times.flat_kernel);
+            times.flat_launches++;
+          } else {
+            tick();
+            const unsigned pair_blocks = (n_pairs + 255) / 256;
+            RunsMeta* meta = d_meta_ + (balanced_steps_ & 1);
+            RunsMeta* meta_next = d_meta_ + ((balanced_steps_ + 1) & 1);
+            balanced_steps_++;
+            if (n_pairs >= kClassifyLargeFrom) {
+              const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
+              classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
+                  sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
+                  d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
+            } else {
+              classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
+                  sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
+                  d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
+            }
+            tock(&times.load_balancing);
+            tick();
+            launch_flat(P, flat_grid, d_skip_flag_);
+            tock(&times.flat_kernel);
+            times.flat_launches++;
+            tick();
+            unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
+            step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
+                P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
+            tock(&times.workgroup_kernel);
+            times.workgroup_launches++;
+          }
         }
       }
       ND_HIP_TRY(hipGetLastError());
@@ -1458,6 +1699,9 @@ class Engine : public EngineBase {
     release(d_live_);
     release(d_emit_keys_);
     release(d_emit_slots_);
+    release(d_emit_ranks_);
+    release(d_small_);
+    release(d_counter_base_);
     release(d_emit_state_);
     release(d_aux_a_);
     release(d_aux_b_);
@@ -1507,6 +1751,12 @@ class Engine : public EngineBase {
   uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
   bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false;
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
+  // small maps: the inversion without a sort (small_map_scan, small_map_place)
+  bool small_map_ = false;
+  size_t small_counters_ = 0;
+  uint32_t* d_counter_base_ = nullptr;  // first counter of every vertex
+  uint32_t* d_emit_ranks_ = nullptr;
+  uint32_t* d_small_ = nullptr;  // counters, their starts inside a chunk, chunk totals
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;          // two work-item counters, alternating between load-balanced steps
   uint32_t* d_balance_ = nullptr;       // which steps' classifications found a run; the pass's ClassCounters

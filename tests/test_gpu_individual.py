@@ -331,3 +331,26 @@ def test_a_new_graph_needs_a_new_alloc(oracle, app):
         assert got.shape == want.shape and np.array_equal(got, want)
     finally:
         s.close()
+
+
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("DeepWalk", "DEEPWALK", False),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+])
+def test_both_inversions_of_a_small_map_give_the_oracle_bytes(oracle, app, kind_name, state, monkeypatch):
+    """Walks over a small map are inverted without a sort (counts per next transit, taken while
+    the pairs are emitted); ND_SMALL_MAP=0 sends the same map through the radix sort.  Also the
+    largest map that still takes the first route, and a hub that gathers every walk."""
+    g = graphs.random_graph(n=3000, mean_degree=8, seed=23, hub=7, isolated_every=13)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+    monkeypatch.setenv("ND_SMALL_MAP", "0")
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+    monkeypatch.delenv("ND_SMALL_MAP")
+    if app == "UniformRandomWalk":
+        n = 1 << 17  # as many pairs as the small-map route takes; one more vertex takes the other route
+        for vertices in (n, n + 1):
+            src = np.arange(vertices)
+            big = nd.Graph.from_edges(np.concatenate([src, src]), np.concatenate([(src * 7 + 1) % vertices, src % 5]),
+                                      np.ones(2 * vertices, np.float32), n_vertices=vertices)
+            run_and_compare(oracle, app, getattr(oracle, kind_name), big, check_state=state, modes=(True,))
