@@ -29,15 +29,15 @@ HBM_PEAK_GBS = 8000.0
 # known size).  None where no such run has been recorded.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "weighted_node2vec_rmat22": 1.171e9,     # step_flat_kernel
-    "uniform_walk_chunglu57k": 4.26e6,       # step_flat_kernel
-    "khop_rmat21": 3.25e9,                   # step kernels of one hop (2 x flat 2.012e9 + workgroup 2.482e9, over 2 hops)
-    "fastgcn_importance_rmat22": 5.273e9,    # collective_mark_binned, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 6.71e10,  # collective_mark_binned, average over its 2 launches per pass
+    "uniform_walk_chunglu57k": 6.585e6,      # step_flat_kernel
+    "khop_rmat21": 3.265e9,                  # step kernels of one hop (2 x flat 2.024e9 + workgroup 2.482e9, over 2 hops)
+    "fastgcn_importance_rmat22": 5.28e9,     # collective_mark_binned, average over its 2 launches per pass
+    "ladies_importance_chunglu3m": 6.727e10,  # collective_mark_binned, average over its 2 launches per pass
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
-    "weighted_node2vec_rmat22": 154.3e9, "uniform_walk_chunglu57k": 0.93e9, "khop_rmat21": 14.65e9,
-    "fastgcn_importance_rmat22": 16.4e9, "ladies_importance_chunglu3m": 160.8e9,
+    "weighted_node2vec_rmat22": 154.3e9, "uniform_walk_chunglu57k": 1.36e9, "khop_rmat21": 13.54e9,
+    "fastgcn_importance_rmat22": 16.44e9, "ladies_importance_chunglu3m": 161.15e9,
 }
 
 # Read requests one launch of the dominant kernel sends past L2 (rocprofv3 TCC_EA0_RDREQ_sum, every
