@@ -347,9 +347,10 @@ int nd_sampler_create(const char* app_name, nd_sampler** out) {
     if (!app_name || !out) return fail("null argument");
     AppEntry app;
     if (!find_app(app_name, &app)) return fail(std::string("unknown app '") + app_name + "'");
-    nd_sampler* s = new nd_sampler;
+    std::unique_ptr<nd_sampler> s(new nd_sampler);
     s->engine.reset((nd::EngineBase*)app.make(app.name));
-    *out = s;
+    if (!s->engine) return fail(std::string("the factory of app '") + app_name + "' returned no engine");
+    *out = s.release();
     return 0;
   });
 }

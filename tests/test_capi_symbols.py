@@ -63,3 +63,42 @@ def test_bad_arguments_are_refused_before_anything_reaches_a_device():
         nextdoor_amd.Graph.from_csr([0, 2, 1, 3], [1, 2, 0])
     with pytest.raises(nextdoor_amd.NextDoorError, match="out of range"):
         nextdoor_amd.Graph.from_csr([0, 1, 2, 3], [1, 2, 9])
+
+
+def test_app_registration_refuses_what_it_cannot_run():
+    """nd_register_app, the door for apps built outside the library: another engine layout, a
+    name that is taken and missing arguments are refused with a message; a good registration
+    shows up in the list (its factory is never called here: no sampler is made)."""
+    import ctypes as C
+    import nextdoor_amd
+    from nextdoor_amd import _capi
+    L = _capi.lib()
+    maker_type = C.CFUNCTYPE(C.c_void_p, C.c_char_p)
+    maker = maker_type(lambda name: None)
+    keep_alive.append(maker)
+    fn = C.cast(maker, C.c_void_p)
+    abi = 2  # ND_ENGINE_ABI of include/nextdoor_amd.h
+    text = open(os.path.join(ROOT, "include", "nextdoor_amd.h")).read()
+    assert re.search(r"#define\s+ND_ENGINE_ABI\s+%d\b" % abi, text)
+    assert L.nd_register_app(b"HostSideProbeApp", fn, abi + 1) == -2
+    assert b"engine ABI" in L.nd_last_error()
+    assert L.nd_register_app(b"KHop", fn, abi) == -3
+    assert b"already registered" in L.nd_last_error()
+    assert L.nd_register_app(None, fn, abi) != 0 and L.nd_register_app(b"HostSideProbeApp", None, abi) != 0
+    assert "HostSideProbeApp" not in nextdoor_amd.app_names()
+    assert L.nd_register_app(b"HostSideProbeApp", fn, abi) == 0
+    assert "HostSideProbeApp" in nextdoor_amd.app_names()
+    assert L.nd_register_app(b"HostSideProbeApp", fn, abi) == -3
+
+
+keep_alive = []  # ctypes callbacks handed to the library must outlive the test
+
+
+def test_an_app_whose_factory_gives_nothing_is_an_error():
+    import nextdoor_amd
+    import pytest
+    if "HostSideProbeApp" not in nextdoor_amd.app_names():
+        test_app_registration_refuses_what_it_cannot_run()
+    g = nextdoor_amd.Graph.from_edges([0, 1], [1, 0])
+    with pytest.raises(nextdoor_amd.NextDoorError, match="returned no engine"):
+        nextdoor_amd.Sampler("HostSideProbeApp", g)
