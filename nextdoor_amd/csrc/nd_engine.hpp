@@ -209,6 +209,12 @@ struct StepParams {
                                  // inside the rows of the result (out_pitch = F).  It is also
                                  // the (sample -> transit) map of step k+1.
   uint32_t out_pitch;
+  // Walks whose transit is the previous step's result: the results of steps 2j and 2j + 1 of
+  // sample s share one 8-byte cell, pair_cells[(j * pair_cell_samples + s) * 2 + (step & 1)],
+  // and the odd step writes both at once (it knows the even step's result: it is its transit) -
+  // one scattered store per two steps instead of two.  nullptr: step_out as described above.
+  int32_t* pair_cells;
+  uint32_t pair_cell_samples;
   void* samples;                 // SampleType[S] or nullptr
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
   // Walks (one transit per sample, stepSize 1 everywhere): the step kernels also emit the
@@ -287,6 +293,23 @@ __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& c
   return neighbor;
 }
 
+// The result of a walk's step into the cells two steps share (StepParams::pair_cells).  An even
+// step leaves its result to the odd step that follows - a walk that ends at the even step has
+// INVALID there, which the cell holds already - unless it is the last step of all.
+__device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t sample, VertexID transit,
+                                                  VertexID neighbor, int step) {
+  int32_t* cell = P.pair_cells + ((size_t)(step >> 1) * P.pair_cell_samples + sample) * 2;
+  if (step & 1) {
+    *reinterpret_cast<int2*>(cell) = make_int2(transit, neighbor);
+  } else if (P.is_last) {
+    cell[0] = neighbor;
+  }
+}
+__device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t sample, VertexID transit,
+                                                  VertexID neighbor) {
+  store_walk_result(P, sample, transit, neighbor, P.step);
+}
+
 // pair: index of the pair in the order the step kernels walk them (sorted by transit, or
 // the raw map at step 0).
 template <class SampleType, class App, class EdgeArray, class WeightArray>
@@ -323,8 +346,12 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
                                           edges, weights, (SampleType*)P.samples + sample, &next_transit);
     }
   }
-  const uint32_t per_sample = P.transits_per_sample * P.step_size;
-  P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
+  if (P.pair_cells) {
+    store_walk_result(P, sample, transit, neighbor);
+  } else {
+    const uint32_t per_sample = P.transits_per_sample * P.step_size;
+    P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
+  }
   if (P.emit_keys) {
     P.emit_keys[pair] = (uint32_t)next_transit;
     P.emit_slots[pair] = pair_slot;
@@ -459,7 +486,14 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
       }
       neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
     }
-    P.step_out[(size_t)k * out_stride + slot] = neighbor;
+    if (P.pair_cells) {
+      // the last step of all, or of this walk, or of the stretch may be an even one
+      int32_t* cell = P.pair_cells + ((size_t)(step >> 1) * P.pair_cell_samples + slot) * 2;
+      if (step & 1) *reinterpret_cast<int2*>(cell) = make_int2(transit, neighbor);
+      else if (step == last_step) cell[0] = neighbor;
+    } else {
+      P.step_out[(size_t)k * out_stride + slot] = neighbor;
+    }
     transit = neighbor;
     if (explicit_transits && step != last_step) {
       if (n_edges == 0) rng.reset(P.seed, P.first_slot + slot, (uint32_t)step);
@@ -924,21 +958,31 @@ __global__ __launch_bounds__(256) void assemble_final_rows(const int32_t* __rest
   }
 }
 
-// The same for walks (every step contributes one id per sample: step_out[k * n_samples + s]),
+// The same for walks (every step contributes one id per sample: step_out[k * n_samples + s], or,
+// paired != 0, the 8-byte cells two steps share, see StepParams::pair_cells),
 // without the index arithmetic of the general case: a wavefront reads 64 consecutive samples
 // of one step, and the rows are written out with running (row, column) counters.
 __global__ __launch_bounds__(256) void assemble_walk_rows(const int32_t* __restrict__ step_out,
                                                           int32_t* __restrict__ final_samples, uint32_t n_samples,
                                                           uint32_t n_steps, uint32_t row_pitch,
-                                                          uint32_t samples_per_block) {
+                                                          uint32_t samples_per_block, uint32_t paired) {
   extern __shared__ int32_t s_rows[];
   const uint32_t s0 = blockIdx.x * samples_per_block;
   const uint32_t nb = n_samples - s0 < samples_per_block ? n_samples - s0 : samples_per_block;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   for (uint32_t first = 0; first < nb; first += 64u) {
     const uint32_t s = first + lane;
-    if (s < nb)
+    if (s >= nb) continue;
+    if (paired) {
+      const int2* cells = reinterpret_cast<const int2*>(step_out);
+      for (uint32_t j = wave; 2u * j < n_steps; j += 4u) {
+        const int2 c = cells[(size_t)j * n_samples + s0 + s];
+        s_rows[s * row_pitch + 2u * j] = c.x;
+        if (2u * j + 1u < n_steps) s_rows[s * row_pitch + 2u * j + 1u] = c.y;
+      }
+    } else {
       for (uint32_t k = wave; k < n_steps; k += 4u) s_rows[s * row_pitch + k] = step_out[(size_t)k * n_samples + s0 + s];
+    }
   }
   __syncthreads();
   int32_t* dst = final_samples + (size_t)s0 * n_steps;
@@ -1133,7 +1177,8 @@ class Engine : public EngineBase {
     // the result per output, so they go to one array per step and are regrouped at the end.
     rows_direct_ = true;
     for (int k = 0; k < n_steps; ++k) rows_direct_ = rows_direct_ && layout_.seg_len[k] >= kDirectSegment;
-    if (!rows_direct_) ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
+    // (one more column where the steps of a walk are odd in number: its results go in cells of two)
+    if (!rows_direct_) ND_HIP_TRY(hipMalloc(&d_step_out_, sizeof(VertexID_t) * (size_t)n_samples_ * (F + 1)));
     ND_HIP_TRY(hipMalloc(&d_keys_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_vals_a_, sizeof(uint32_t) * max_pairs_));
     ND_HIP_TRY(hipMalloc(&d_keys_b_, sizeof(uint32_t) * max_pairs_));
@@ -1216,6 +1261,8 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipFuncSetAttribute((const void*)assemble_walk_rows, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      65536));
     }
+    paired_results_ = walk_mode_ && !rows_direct_ && rows_per_block_ > 0 && !App().hasExplicitTransits() &&
+                      !(getenv("ND_PAIRED_RESULTS") && atoi(getenv("ND_PAIRED_RESULTS")) == 0);
     allocated_ = true;
     return 0;
   }
@@ -1295,7 +1342,7 @@ class Engine : public EngineBase {
     // pairs whose transit is INVALID are dropped by the inversion and never reach a step
     // kernel: their outputs keep this fill
     {
-      const size_t n_out = (size_t)n_samples_ * F;
+      const size_t n_out = (size_t)n_samples_ * (paired_results() ? (F + 1) / 2 * 2 : F);
       fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(
           rows_direct_ ? d_final_ : d_step_out_, n_out, invalid_);
     }
@@ -1329,6 +1376,8 @@ class Engine : public EngineBase {
         P.step_out = d_step_out_ + (size_t)n_samples_ * layout_.seg_base[step];
         P.out_pitch = layout_.seg_len[step];
       }
+      P.pair_cells = paired_results() ? d_step_out_ : nullptr;
+      P.pair_cell_samples = (uint32_t)n_samples_;
       P.samples = d_samples_;
       P.paired_edges = dgraph_->paired;
       const bool emits = walk_mode_ && step + 1 < n_steps;
@@ -1501,7 +1550,8 @@ class Engine : public EngineBase {
       const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
       assemble_walk_rows<<<dim3(blocks), dim3(256), lds, stream_>>>(d_step_out_, d_final_, (uint32_t)n_samples_,
-                                                                    (uint32_t)n_steps, row_pitch_, rows_per_block_);
+                                                                    (uint32_t)n_steps, row_pitch_, rows_per_block_,
+                                                                    paired_results() ? 1u : 0u);
     } else if (rows_per_block_ > 0) {
       const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
@@ -1646,6 +1696,10 @@ class Engine : public EngineBase {
     return on;
   }
 
+  // Walks write their results in cells of two steps (StepParams::pair_cells) where a step's
+  // transit is the previous step's result and the rows are regrouped by assemble_walk_rows.
+  bool paired_results() const { return paired_results_; }
+
   void launch_flat(const StepParams& P, unsigned flat_grid, const uint8_t* skip_flag) {
     if (P.step_size == 1)
       step_flat_kernel<SampleType, App, true><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
@@ -1735,6 +1789,7 @@ class Engine : public EngineBase {
   size_t max_pairs_ = 0;
   uint32_t chunk_capacity_ = 0;
   uint32_t row_pitch_ = 0, rows_per_block_ = 0;
+  bool paired_results_ = false;
   StepLayout layout_{};
   bool allocated_ = false;
 
