@@ -141,8 +141,13 @@ class CSRPartition {
       uint32_t bucket = edge_hash((uint32_t)src, (uint32_t)dst) & edge_table_mask;
       for (;;) {
         const EdgeKeyPair* keys = (const EdgeKeyPair*)(edge_table + (size_t)bucket * kEdgeBucket);
-        const EdgeKeyPair first = keys[0], second = keys[1];
-        if (first.x == key || first.y == key || second.x == key || second.y == key) return true;
+        // a bucket fills from its first slot on and holds one key on average: the first half
+        // decides 9 tests in 10, and the second half is then in the cache the first came through
+        const EdgeKeyPair first = keys[0];
+        if (first.x == key || first.y == key) return true;
+        if (first.y == ~0ull) return false;
+        const EdgeKeyPair second = keys[1];
+        if (second.x == key || second.y == key) return true;
         if (second.y == ~0ull) return false;  // the bucket has room: the key was never pushed past it
         bucket = (bucket + 1) & edge_table_mask;
       }
