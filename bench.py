@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
 # known size).  None where no such run has been recorded.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 1.115e9,     # step_flat_kernel
+    "weighted_node2vec_rmat22": 1.119e9,     # step_flat_kernel
     "uniform_walk_chunglu57k": 6.233e6,      # step_flat_kernel
     "khop_rmat21": 3.265e9,                  # step kernels of one hop (2 x flat 2.024e9 + workgroup 2.482e9, over 2 hops)
     "fastgcn_importance_rmat22": 5.28e9,     # collective_mark_binned, average over its 2 launches per pass
@@ -36,14 +36,14 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 }
 # HBM bytes of all kernels of one pass, same source.
 MEASURED_TRAFFIC_BYTES_PER_PASS = {
-    "weighted_node2vec_rmat22": 148.7e9, "uniform_walk_chunglu57k": 1.31e9, "khop_rmat21": 13.54e9,
+    "weighted_node2vec_rmat22": 149.1e9, "uniform_walk_chunglu57k": 1.31e9, "khop_rmat21": 13.54e9,
     "fastgcn_importance_rmat22": 16.44e9, "ladies_importance_chunglu3m": 161.15e9,
 }
 
 # Read requests one launch of the dominant kernel sends past L2 (rocprofv3 TCC_EA0_RDREQ_sum, every
 # one of them 128 bytes: profiles/step_kernels_<workload>_l2_requests.md).  None where not recorded.
 MEASURED_L2_MISS_REQUESTS_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 8.18e6,      # step_flat_kernel
+    "weighted_node2vec_rmat22": 8.21e6,      # step_flat_kernel
 }
 
 WORKLOADS = {
