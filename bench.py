@@ -413,6 +413,11 @@ def main():
                            "measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
         }
         result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
+        traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
+        if traffic:
+            # recorded counter traffic of one launch over this run's launch duration (flat kernel alone)
+            flat_launch_s = prof["flat_kernel_ms"] / max(launches, 1) / 1000.0
+            result["roofline"]["traffic_frac"] = traffic / flat_launch_s / 1e9 / HBM_PEAK_GBS
         misses = MEASURED_L2_MISS_REQUESTS_PER_LAUNCH.get(args.workload)
         if misses:
             # The step kernel's reads are dependent random gathers; each one that misses L2 costs a
