@@ -414,7 +414,7 @@ def main():
         }
         result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
         traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
-        if traffic:
+        if traffic and w["kind"] != "KHOP":  # walks: the recorded figure is the flat kernel's launch
             # recorded counter traffic of one launch over this run's launch duration (flat kernel alone)
             flat_launch_s = prof["flat_kernel_ms"] / max(launches, 1) / 1000.0
             result["roofline"]["traffic_frac"] = traffic / flat_launch_s / 1e9 / HBM_PEAK_GBS
