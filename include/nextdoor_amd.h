@@ -178,6 +178,11 @@ void nd_sampler_destroy(nd_sampler* s);
 /* initSampling(graph): binary edge-list path (nextDoorPythonModule.cu:40-52).  The
  * reference compiles one module per app; here the app is named.  seed as above. */
 int nd_init_sampling(const char* app_name, const char* graph_path, uint64_t seed);
+/* The same for a graph the caller already holds as CSR arrays (copied; sorted rows as in
+ * nd_graph_from_csr; weight == NULL: all 1).  No counterpart in the reference, whose module
+ * only reads files. */
+int nd_init_sampling_from_csr(const char* app_name, int32_t n_vertices, int64_t n_edges, const int32_t* row_ptr,
+                              const int32_t* col, const float* weight, uint64_t seed);
 /* sample() (nextDoorPythonModule.cu:54-58); runs the load-balanced transit-parallel engine. */
 int nd_sample(void);
 /* finalSampleLength() (nextDoorPythonModule.cu:75-81): total length of the final-samples vector. */

@@ -306,6 +306,14 @@ class SamplingModule:
     def initSampling(self, graph_path):
         check(lib().nd_init_sampling(self.app.encode(), str(graph_path).encode(), self.seed))
 
+    def initSamplingFromCSR(self, row_ptr, col, weight=None):
+        """The same from CSR arrays in memory (no counterpart in the reference's module)."""
+        row_ptr, col = _as(row_ptr, np.int32), _as(col, np.int32)
+        weight = None if weight is None else _as(weight, np.float32)
+        check(lib().nd_init_sampling_from_csr(self.app.encode(), len(row_ptr) - 1, len(col), _ptr(row_ptr, C.c_int32),
+                                              _ptr(col, C.c_int32),
+                                              None if weight is None else _ptr(weight, C.c_float), self.seed))
+
     def sample(self):
         check(lib().nd_sample())
 

@@ -61,6 +61,7 @@ SIGNATURES = {
     "nd_sampler_free_device": (None, [C.c_void_p]),
     "nd_sampler_destroy": (None, [C.c_void_p]),
     "nd_init_sampling": (C.c_int, [C.c_char_p, C.c_char_p, C.c_uint64]),
+    "nd_init_sampling_from_csr": (C.c_int, [C.c_char_p, C.c_int32, C.c_int64, c_i32p, c_i32p, c_f32p, C.c_uint64]),
     "nd_sample": (C.c_int, []),
     "nd_final_sample_length": (C.c_int64, []),
     "nd_final_samples_array": (c_i32p, []),

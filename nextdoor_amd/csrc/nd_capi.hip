@@ -593,6 +593,24 @@ int nd_init_sampling(const char* app_name, const char* graph_path, uint64_t seed
   });
 }
 
+int nd_init_sampling_from_csr(const char* app_name, int32_t n_vertices, int64_t n_edges, const int32_t* row_ptr,
+                              const int32_t* col, const float* weight, uint64_t seed) {
+  return guarded([&]() -> int {
+    nd_free_device_memory();
+    int rc = nd_graph_from_csr(n_vertices, n_edges, row_ptr, col, weight, &g_module_graph);
+    if (rc != 0) return rc;
+    rc = nd_sampler_create(app_name, &g_module_sampler);
+    if (rc == 0) rc = nd_sampler_set_graph(g_module_sampler, g_module_graph);
+    if (rc == 0) rc = nd_sampler_alloc(g_module_sampler, seed);
+    if (rc != 0) {
+      const std::string keep = g_error;
+      nd_free_device_memory();
+      g_error = keep;
+    }
+    return rc;
+  });
+}
+
 int nd_sample(void) {
   if (!g_module_sampler) return fail("sample() before initSampling()");
   return nd_sampler_do_transit_parallel(g_module_sampler, 1);

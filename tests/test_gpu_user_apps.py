@@ -97,6 +97,16 @@ def test_sampling_module_functions_end_to_end(tmp_path):
             got = module.finalSamplesArray()
             assert got.dtype == np.int32 and np.array_equal(got.reshape(-1, final), want)
         assert module.finalSamples()[:final] == want[0].tolist()
+    # the same sampler from CSR arrays in memory
+    app, kind, g = cases[0]
+    module = nd.SamplingModule(app, seed=SEED)
+    module.initSamplingFromCSR(g.row_ptr, g.col, g.weight)
+    module.sample()
+    reference = nd.Sampler(app, g, seed=SEED)
+    want, _ = ob.sample_individual(graphs.oracle_view(g), ob.app_desc(kind, reference.steps, [reference.step_size(k) for k in range(reference.steps)]),
+                                   SEED, reference.initial_contents.copy())
+    reference.close()
+    assert np.array_equal(module.finalSamplesArray().reshape(want.shape), want)
     module.freeDeviceMemory()
     assert module.finalSampleLength() == 0
     with pytest.raises(nd.NextDoorError, match="before initSampling"):
