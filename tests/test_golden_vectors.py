@@ -81,3 +81,53 @@ def test_library_produces_the_committed_vectors(app):
             assert st[:, 2 + 128:2 + 256].reshape(-1).tolist() == want["cols"]
     finally:
         s.close()
+
+
+# ---- vectors decided by the reference's own functor sources --------------------------------
+# tests/golden/reference_functor_vectors.json was written by make_reference_functor_vectors.py
+# from the reference's khop.cu / randomWalks.cu compiled on the CPU (see that script); neither
+# the reference tree nor that build is needed here.
+
+REFERENCE_APPS = {"KHop": "KHOP", "DeepWalk": "DEEPWALK", "PPR": "PPR", "Node2Vec": "NODE2VEC"}
+
+
+@pytest.mark.parametrize("app", sorted(REFERENCE_APPS))
+def test_oracle_produces_what_the_reference_functors_do(oracle, app):
+    fx = load("reference_functor_vectors.json")
+    gr, want = fx["graph"], fx["apps"][app]
+    g = oracle.Graph(gr["row_ptr"], gr["col"], gr["weight"])
+    d = oracle.app_desc(getattr(oracle, REFERENCE_APPS[app]), want["steps"], want["step_sizes"])
+    final, state = oracle.sample_individual(g, d, fx["seed"], np.array(want["initial"], np.int32))
+    assert list(final.shape) == want["shape"]
+    assert final.reshape(-1).tolist() == want["final"]
+    if "state_t" in want:
+        moved = final[:, 0] != g.n_vertices
+        assert np.array_equal(state[moved], np.array(want["state_t"], np.int32)[moved])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("app", sorted(REFERENCE_APPS))
+def test_library_produces_what_the_reference_functors_do(app):
+    """The registry apps under the reference's names and sizes: the first samples of a run are
+    the fixture's (a sample's values depend on its index and root only)."""
+    import nextdoor_amd as nd
+    fx = load("reference_functor_vectors.json")
+    gr, want = fx["graph"], fx["apps"][app]
+    g = nd.Graph.from_csr(gr["row_ptr"], gr["col"], np.array(gr["weight"], np.float32))
+    s = nd.Sampler(app, g, seed=fx["seed"])
+    try:
+        kept = want["shape"][0]
+        assert s.num_samples == want["samples_of_the_app"]
+        assert [s.step_size(k) for k in range(s.steps)] == want["step_sizes"]
+        assert s.initial_contents[:kept].tolist() == want["initial"]
+        for lb in (True, False):
+            print("app", app, "lb", lb, flush=True)
+            s.do_transit_parallel(load_balancing=lb)
+            got = s.final_samples()[:kept]
+            assert got.reshape(-1).tolist() == want["final"]
+            if "state_t" in want:
+                t = s.sample_states().view(np.int32)[:kept]
+                moved = got[:, 0] != g.n_vertices
+                assert np.array_equal(t[moved], np.array(want["state_t"], np.int32)[moved])
+    finally:
+        s.close()
