@@ -354,3 +354,47 @@ def test_both_inversions_of_a_small_map_give_the_oracle_bytes(oracle, app, kind_
             big = nd.Graph.from_edges(np.concatenate([src, src]), np.concatenate([(src * 7 + 1) % vertices, src % 5]),
                                       np.ones(2 * vertices, np.float32), n_vertices=vertices)
             run_and_compare(oracle, app, getattr(oracle, kind_name), big, check_state=state, modes=(True,))
+
+
+def test_small_map_inversion_classifies_every_run_by_the_rules(oracle):
+    """The placing launch of the small-map inversion decides the load-balancing class of every
+    run from the counts; what it reports (nd_sampler_counter) is what the rules give for the
+    transits the oracle's walks are on, step by step."""
+    work_from, item_outputs, cache_edges = nd.load_balancing_thresholds()
+    # a hub that fits the LDS cache, one that does not, and a sparse rest
+    n = 20000
+    rng = np.random.default_rng(31)
+    src = [rng.integers(0, n, 3 * n), np.full(4000, 7), rng.integers(0, n, 30000), np.full(9000, 11), rng.integers(0, n, 30000)]
+    dst = [rng.integers(0, n, 3 * n), rng.integers(0, n, 4000), np.full(30000, 7), rng.integers(0, n, 9000), np.full(30000, 11)]
+    g = nd.Graph.from_edges(np.concatenate(src), np.concatenate(dst), n_vertices=n)
+    degree = np.diff(g.row_ptr)
+    assert degree[7] < cache_edges < degree[11]
+    s = nd.Sampler("UniformRandomWalk8", g, seed=SEED)
+    try:
+        s.do_transit_parallel(load_balancing=True)
+        final = s.final_samples()
+        want, _ = oracle.sample_individual(graphs.oracle_view(g), oracle.app_desc(oracle.UNIFORM_WALK, 8, [1] * 8), SEED,
+                                           s.initial_contents)
+        assert np.array_equal(final, want)
+        looked = single = split = refused = items = 0
+        for k in range(1, 8):
+            transits = final[:, k - 1]
+            transits = transits[transits != n]
+            looked += len(transits)
+            vertices, counts = np.unique(transits, return_counts=True)
+            for v, c in zip(vertices.tolist(), counts.tolist()):
+                if c < work_from or degree[v] == 0:
+                    continue
+                if degree[v] > cache_edges or min(degree[v], cache_edges) > 32 * c:
+                    refused += c
+                    continue
+                n_items = -(-c // item_outputs)
+                items += n_items
+                if n_items > 1:
+                    split += c
+                else:
+                    single += c
+        assert single + split > 0 and refused > 0  # both hubs gather enough walks
+        assert [s.counter(i) for i in range(5)] == [looked, single, split, refused, items]
+    finally:
+        s.close()
