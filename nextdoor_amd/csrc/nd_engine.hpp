@@ -652,8 +652,9 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
 // order in the list is irrelevant to the results.  The list is sized so that every claim
 // fits (see Engine::alloc); should one not fit, the transit is left to the flat kernel and
 // the entries that did fit are processed twice with identical results.
-// When the classification of the step before found nothing for the workgroup kernel (or did not
-// look), this one only looks every kQuietLookEvery-th step: on a map where no transit carries
+// When the classifications of the two steps before found nothing for the workgroup kernel (or did
+// not look; two, because walks on a bipartite graph meet its hubs every other step), this one
+// only looks every kQuietLookEvery-th step: on a map where no transit carries
 // enough pairs, as with one walk per vertex of a large graph, most launches end at once.
 // found_by_step[k] != 0: step k's classification found a run; cleared before every pass.  What
 // a step's classification decides never changes a result, only which kernel draws it.
@@ -674,7 +675,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   // the work-item counters alternate between steps: this launch clears the one the next
   // step will count into (its last reader, the previous step's workgroup kernel, is done)
   if (blockIdx.x == 0 && threadIdx.x == 0) meta_of_next_step->n_chunks = 0;
-  if (step > 1 && found_by_step[step - 1] == 0 && step % kQuietLookEvery != 0) return;
+  if (step > 2 && found_by_step[step - 1] == 0 && found_by_step[step - 2] == 0 && step % kQuietLookEvery != 0) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&counters->sorted_pairs, (unsigned long long)n);
   const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
   uint32_t transit, start, count, n_items;
