@@ -92,7 +92,7 @@ inline const char* nextDoorRegistryName() {
 #if defined(__HIPCC__) && !defined(ND_HOST_API_ONLY)
   static const std::string name = [] {
     std::string n = std::string("app:") + typeid(App).name() + ":" + typeid(SampleType).name();
-    if (nd_register_app(n.c_str(), &nd::make_app_engine<SampleType, App>, ND_ENGINE_ABI) != 0)
+    if (nd_register_app(n.c_str(), &nd::make_app_engine<SampleType, App>, nd::engine_abi()) != 0)
       fprintf(stderr, "nextdoor: %s\n", nd_last_error());
     return n;
   }();
@@ -105,7 +105,25 @@ inline const char* nextDoorRegistryName() {
 template <class SampleType, typename App>
 struct NextDoorData : NextDoorDataByName {
   NextDoorData() : NextDoorDataByName(nextDoorRegistryName<SampleType, App>()) {}
+  // libNextDoor.hpp:16: one SampleType per sample.  After allocNextDoorDataOnGPU what
+  // initializeSample / initialSample left in it (src/nextdoor.cu:1955-1963), after
+  // getFinalSamples the state the sampling left on the device (src/nextdoor.cu:3226-3227);
+  // the reference's checkers read it (src/check_results.cu:55, src/tests/singleGPU/multirw.cu:21).
+  std::vector<SampleType> samples;
 };
+
+// Device -> data.samples.  False when the engine keeps a state of another size than
+// sizeof(SampleType) per sample (the caller's SampleType is not the engine's).
+template <class SampleType, typename App>
+inline bool fetchSampleStates(NextDoorData<SampleType, App>& data) {
+  if (!data.sampler) return false;
+  const int64_t n = nd_sampler_num_samples(data.sampler);
+  const int64_t bytes = nd_sampler_sample_state_bytes(data.sampler);
+  data.samples.assign((size_t)(n > 0 ? n : 0), SampleType());
+  if (bytes == 0) return true;  // a SampleType without members: nothing is kept on the device
+  if (bytes != (int64_t)sizeof(SampleType) * n) return false;
+  return nd_sampler_get_sample_states(data.sampler, (void*)data.samples.data(), bytes) == 0;
+}
 
 // loadGraph(graph, file, type, format), src/nextdoor.cu:1845-1891: nullptr on failure.
 inline CSR* loadGraph(Graph& graph, const char* graph_file, const char* graph_type, const char* graph_format) {
@@ -157,7 +175,7 @@ inline bool allocNextDoorDataOnGPU(CSR* csr, NextDoorDataByName& data) {
 }
 template <class SampleType, typename App>
 inline bool allocNextDoorDataOnGPU(CSR* csr, NextDoorData<SampleType, App>& data) {
-  return allocNextDoorDataOnGPU(csr, static_cast<NextDoorDataByName&>(data));
+  return allocNextDoorDataOnGPU(csr, static_cast<NextDoorDataByName&>(data)) && fetchSampleStates(data);
 }
 
 // doTransitParallelSampling(csr, data, enableLoadBalancing), src/nextdoor.cu:2191-3006: the
@@ -188,6 +206,14 @@ inline std::vector<VertexID_t>& getFinalSamples(NextDoorDataByName& data) {
   const VertexID_t* p = nullptr;
   int64_t n = 0;
   if (data.sampler && nd_sampler_get_final_samples(data.sampler, &p, &n) == 0) data.hFinalSamples.assign(p, p + n);
+  return data.hFinalSamples;
+}
+
+// ... and, with the template spelling, data.samples (src/nextdoor.cu:3226-3227).
+template <class SampleType, typename App>
+inline std::vector<VertexID_t>& getFinalSamples(NextDoorData<SampleType, App>& data) {
+  getFinalSamples(static_cast<NextDoorDataByName&>(data));
+  if (!fetchSampleStates(data)) fprintf(stderr, "getFinalSamples: %s\n", nd_last_error());
   return data.hFinalSamples;
 }
 

@@ -35,9 +35,13 @@ const char* nd_app_name(int index);
  * <SampleType, App> (src/apps/khop/main.cu:1-21, src/tests/testBase.h:14-24).  Here such a
  * translation unit - the App struct, nd_app_registry.hpp and ND_REGISTER_APP - is compiled with
  * hipcc into a shared object of its own, and loading it calls this.  make(name) returns a new
- * nd::EngineBase* (nd_engine.hpp) for the application; engine_abi must be ND_ENGINE_ABI of the
- * headers the caller was built from.  Returns 0, or a negative value (name taken, ABI mismatch). */
-#define ND_ENGINE_ABI 2
+ * nd::EngineBase* (nd_engine.hpp) for the application; engine_abi must be nd::engine_abi()
+ * (nd_app_registry.hpp) of the headers the caller was built from: ND_ENGINE_ABI, raised by hand
+ * with every change of the engine's interface, combined with the sizes of the structs the two
+ * sides share, so that a forgotten raise is caught as well.  nd_engine_abi() is the library's own
+ * value.  Returns 0, or a negative value (-2 ABI mismatch, -3 name taken). */
+#define ND_ENGINE_ABI 3
+int nd_engine_abi(void);
 int nd_register_app(const char* name, void* (*make)(const char* name), int engine_abi);
 
 /* ---- graphs ------------------------------------------------------------------------ */
@@ -226,8 +230,7 @@ int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, i
  * over a sorted key array, as the engine runs it between the inversion and the step kernels:
  * degrees[v] = edges of vertex v; a run of `count` equal keys goes to the workgroup kernel when
  * count * step_size >= thresholds[0], the transit has edges and staging its adjacency pays (at
- * most thresholds[2] edges unless partial_cache != 0, which stages the first thresholds[2] and
- * reads the rest from memory; and no more than 32 staged edges per output); such a run is cut
+ * most thresholds[2] edges, and no more than 32 staged edges per output); such a run is cut
  * into work items of at most thresholds[1] / step_size pairs: items[2 i] = first pair,
  * items[2 i + 1] = pairs, in no particular order; taken[v] = 1 for the transits so served (the flat
  * kernel skips their pairs).  *n_items = items wanted (those beyond `capacity` are not written and
@@ -236,8 +239,8 @@ int nd_unique_transits(const int32_t* sorted_keys, int64_t n, int32_t invalid, i
  * their degree, 4 items.  pairs_per_lane: 1 or 16, the two launch shapes the engine uses. */
 int nd_load_balancing_thresholds(int32_t thresholds[3]);
 int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,
-                     int partial_cache, int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items,
-                     uint8_t* taken, int64_t counters[5]);
+                     int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items, uint8_t* taken,
+                     int64_t counters[5]);
 
 /* Measurement, no counterpart in the reference: the rate (requests per second) at which this GPU
  * serves independent random 8-byte reads over a table of table_bytes (a power of two, 4 KiB to

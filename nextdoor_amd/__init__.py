@@ -359,7 +359,7 @@ def load_balancing_thresholds():
     return tuple(int(x) for x in out)
 
 
-def classify_runs(sorted_keys, degrees, step_size, partial_cache=True, pairs_per_lane=1, capacity=None):
+def classify_runs(sorted_keys, degrees, step_size, pairs_per_lane=1, capacity=None):
     """The load-balancing classification over a sorted key array: (items [k, 2] = first pair and
     pairs of every work item, items wanted, taken [n_vertices], counters [5])."""
     keys, degrees = _as(sorted_keys, np.int32), _as(degrees, np.int32)
@@ -368,7 +368,7 @@ def classify_runs(sorted_keys, degrees, step_size, partial_cache=True, pairs_per
     taken = np.zeros(len(degrees), np.uint8)
     counters, wanted = np.zeros(5, np.int64), C.c_int64()
     check(lib().nd_classify_runs(_ptr(keys, C.c_int32), len(keys), _ptr(degrees, C.c_int32), len(degrees), step_size,
-                                 int(partial_cache), pairs_per_lane, _ptr(items, C.c_int32), capacity,
+                                 pairs_per_lane, _ptr(items, C.c_int32), capacity,
                                  C.byref(wanted), _ptr(taken, C.c_uint8), _ptr(counters, C.c_int64)))
     return items[:min(wanted.value, capacity)], wanted.value, taken, counters
 

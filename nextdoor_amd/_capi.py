@@ -15,6 +15,7 @@ SIGNATURES = {
     "nd_last_error": (C.c_char_p, []),
     "nd_num_apps": (C.c_int, []),
     "nd_app_name": (C.c_char_p, [C.c_int]),
+    "nd_engine_abi": (C.c_int, []),
     "nd_register_app": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int]),
     "nd_graph_load": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_void_p)]),
     "nd_graph_from_edges": (C.c_int, [C.c_int32, C.c_int64, c_i32p, c_i32p, c_f32p, C.POINTER(C.c_void_p)]),
@@ -70,7 +71,7 @@ SIGNATURES = {
     "nd_sort_pairs": (C.c_int, [c_i32p, c_i32p, C.c_int64, C.c_int, c_i32p, c_i32p]),
     "nd_sort_pairs_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nd_load_balancing_thresholds": (C.c_int, [c_i32p]),
-    "nd_classify_runs": (C.c_int, [c_i32p, C.c_int64, c_i32p, C.c_int32, C.c_int, C.c_int, C.c_int, c_i32p, C.c_int64,
+    "nd_classify_runs": (C.c_int, [c_i32p, C.c_int64, c_i32p, C.c_int32, C.c_int, C.c_int, c_i32p, C.c_int64,
                                    c_i64p, C.POINTER(C.c_uint8), c_i64p]),
     "nd_collective_neighborhood": (C.c_int, [C.c_void_p, c_i32p, C.c_int64, C.c_int32, C.c_int32, c_i32p, c_i32p, c_i32p,
                                              c_f32p, C.c_int64, c_i32p]),

@@ -15,6 +15,8 @@
 // loading it (dlopen, a link dependency, ctypes.CDLL) registers the application.
 #pragma once
 
+#include <stdio.h>
+
 #include <type_traits>
 
 #include "../../include/nextdoor_amd.h"
@@ -55,12 +57,21 @@ void* make_app_engine(const char* name) {
   return engine;
 }
 
+// What nd_register_app compares: the hand-raised ND_ENGINE_ABI and the sizes of the structs a
+// shared object of apps and the library both lay out (the engine's base class, the kernel
+// parameters, the per-step bookkeeping).
+constexpr int engine_abi() {
+  return ND_ENGINE_ABI * 65536 + (int)((sizeof(EngineBase) + sizeof(StepParams) + sizeof(RunsMeta) + sizeof(PhaseTimes)) % 65536);
+}
+
 // Registers <SampleType, App> under `name` when the object is constructed (a namespace-scope
-// object: when the shared object that holds it is loaded).
+// object: when the shared object that holds it is loaded).  A refusal (name taken, other engine
+// layout) is reported on stderr: nobody looks at a static object's members.
 template <class SampleType, class App>
 struct AppRegistration {
   explicit AppRegistration(const char* name) {
-    rc = nd_register_app(name, &make_app_engine<SampleType, App>, ND_ENGINE_ABI);
+    rc = nd_register_app(name, &make_app_engine<SampleType, App>, engine_abi());
+    if (rc != 0) fprintf(stderr, "nextdoor: app '%s' was not registered: %s\n", name, nd_last_error());
   }
   int rc;
 };

@@ -258,15 +258,21 @@ const char* nd_app_name(int index) {
   return i >= 0 && i < (int)registered_apps().size() ? registered_apps()[(size_t)i].name.c_str() : nullptr;
 }
 
+int nd_engine_abi(void) { return nd::engine_abi(); }
+
 int nd_register_app(const char* name, void* (*make)(const char* name), int engine_abi) {
   return guarded([&]() -> int {
     if (!name || !*name || !make) return fail("null argument");
-    if (engine_abi != ND_ENGINE_ABI)
+    if (engine_abi != nd::engine_abi())
       return fail(std::string("app '") + name + "' was built against engine ABI " + std::to_string(engine_abi) +
-                  ", the library has " + std::to_string(ND_ENGINE_ABI), -2);
-    AppEntry taken;
-    if (find_app(name, &taken)) return fail(std::string("an app named '") + name + "' is already registered", -3);
+                  ", the library has " + std::to_string(nd::engine_abi()), -2);
+    // one lock over the look-up and the insertion: two shared objects loading at the same time
+    // cannot both find the name free
     std::lock_guard<std::mutex> lock(registry_mutex());
+    bool taken = false;
+    for (int i = 0; i < kNumBuiltInApps; ++i) taken = taken || strcmp(kApps[i].name, name) == 0;
+    for (const RegisteredApp& a : registered_apps()) taken = taken || a.name == name;
+    if (taken) return fail(std::string("an app named '") + name + "' is already registered", -3);
     registered_apps().push_back(RegisteredApp{name, make});
     return 0;
   });
@@ -757,8 +763,8 @@ int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
 }
 
 int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,
-                     int partial_cache, int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items,
-                     uint8_t* taken, int64_t counters[5]) {
+                     int pairs_per_lane, int32_t* items, int64_t capacity, int64_t* n_items, uint8_t* taken,
+                     int64_t counters[5]) {
   return guarded([&]() -> int {
     if (n < 0 || n_vertices < 1 || step_size < 1 || capacity < 1 || !degrees || !items || !n_items || !taken ||
         !counters || (n > 0 && !sorted_keys) || n >= (1ll << 31) || capacity >= (1ll << 31) ||
@@ -783,29 +789,29 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
     CAPI_HIP(d_meta.alloc(sizeof(nd::RunsMeta) * 2));
     CAPI_HIP(d_rows.alloc(sizeof(EdgePos_t) * row_ptr.size()));
     CAPI_HIP(d_items.alloc(sizeof(uint32_t) * 2 * (size_t)capacity));
-    CAPI_HIP(d_taken.alloc((size_t)n_vertices));
+    CAPI_HIP(d_taken.alloc(sizeof(uint32_t) * (size_t)n_vertices));
     constexpr size_t kCounterBytes = sizeof(nd::ClassCounters) * nd::kCounterCopies;
     CAPI_HIP(d_balance.alloc(sizeof(uint32_t) * kFoundWords + kCounterBytes));
     const uint32_t n32 = (uint32_t)n;
     CAPI_HIP(hipMemcpy(d_keys.p, sorted_keys, sizeof(uint32_t) * (size_t)n, hipMemcpyHostToDevice));
     CAPI_HIP(hipMemcpy(d_n.p, &n32, sizeof(n32), hipMemcpyHostToDevice));
     CAPI_HIP(hipMemcpy(d_rows.p, row_ptr.data(), sizeof(EdgePos_t) * row_ptr.size(), hipMemcpyHostToDevice));
-    CAPI_HIP(hipMemset(d_meta.p, 0, sizeof(nd::RunsMeta) * 2));
-    CAPI_HIP(hipMemset(d_taken.p, 0, (size_t)n_vertices));
+    nd::RunsMeta fresh[2] = {};
+    fresh[0].stamp = 1;  // the stamp that marks the transits taken at this (the only) step
+    CAPI_HIP(hipMemcpy(d_meta.p, fresh, sizeof(fresh), hipMemcpyHostToDevice));
+    CAPI_HIP(hipMemset(d_taken.p, 0, sizeof(uint32_t) * (size_t)n_vertices));
     CAPI_HIP(hipMemset(d_balance.p, 0, sizeof(uint32_t) * kFoundWords + kCounterBytes));
     nd::RunsMeta* meta = d_meta.as<nd::RunsMeta>();
     nd::ClassCounters* d_counters = (nd::ClassCounters*)(d_balance.as<uint32_t>() + kFoundWords);
     if (pairs_per_lane == 1) {
       nd::classify_run_tails<1><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
-          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint8_t>(), d_counters, partial_cache ? 1u : 0u,
-          d_balance.as<uint32_t>(), 1u);
+          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     } else {
       const int64_t per_block = 256 * nd::kClassifyItemsLarge;
       nd::classify_run_tails<nd::kClassifyItemsLarge><<<dim3((unsigned)((n + per_block - 1) / per_block)), dim3(256), 0, 0>>>(
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
-          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint8_t>(), d_counters, partial_cache ? 1u : 0u,
-          d_balance.as<uint32_t>(), 1u);
+          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     }
     CAPI_HIP(hipGetLastError());
     CAPI_HIP(hipDeviceSynchronize());
@@ -824,7 +830,9 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
     *n_items = h.n_chunks;
     const int64_t written = h.n_chunks < capacity ? (int64_t)h.n_chunks : capacity;
     CAPI_HIP(hipMemcpy(items, d_items.p, sizeof(uint32_t) * 2 * (size_t)written, hipMemcpyDeviceToHost));
-    CAPI_HIP(hipMemcpy(taken, d_taken.p, (size_t)n_vertices, hipMemcpyDeviceToHost));
+    std::vector<uint32_t> stamps((size_t)n_vertices);
+    CAPI_HIP(hipMemcpy(stamps.data(), d_taken.p, sizeof(uint32_t) * stamps.size(), hipMemcpyDeviceToHost));
+    for (int32_t v = 0; v < n_vertices; ++v) taken[v] = stamps[(size_t)v] == fresh[0].stamp ? 1 : 0;
     counters[0] = (int64_t)c.sorted_pairs;
     counters[1] = (int64_t)c.workgroup_pairs;
     counters[2] = (int64_t)c.split_pairs;

@@ -28,6 +28,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include <chrono>
 #include <memory>
@@ -397,16 +398,17 @@ __device__ __forceinline__ uint32_t flat_block_index() {
 // marker are then fetched once for all stepSize draws, whose gathers are independent and
 // overlap; several lanes per pair when pairs are few.  With the map sorted by transit,
 // neighbouring lanes share row extents and adjacency lines.
-// skip_flag (nullable): per-vertex marker of transits the workgroup kernel handles.
+// taken_stamp (nullable): per-vertex marker of the transits that work items cover at this
+// step - those whose entry equals `stamp` (RunsMeta::stamp of the step).
 // kSingleOutput: stepSize is 1 (walks); the loop over neighbours is compiled away.
 template <class SampleType, class App, bool kSingleOutput>
-__global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, const uint8_t* __restrict__ skip_flag) {
+__device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint32_t* __restrict__ taken_stamp,
+                                          uint32_t stamp) {
   if (kSingleOutput) {
     P.lanes_shift = 0;
     P.step_size = 1;
   }
   const uint64_t total = (uint64_t)(P.live_pairs ? *P.live_pairs : P.n_pairs) << P.lanes_shift;
-  const uint64_t i = (uint64_t)flat_block_index() * kFlatThreads + threadIdx.x;
   if (i >= total) return;
   CSRPartition csr = P.csr;
   const uint32_t pair = (uint32_t)(i >> P.lanes_shift);
@@ -418,11 +420,11 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
   float max_weight = 0.0f;
   if (transit != P.invalid) {
     // the marker, the row extent and the largest weight are fetched together
-    const uint8_t taken = skip_flag ? skip_flag[transit] : (uint8_t)0;
+    const uint32_t mark = taken_stamp ? taken_stamp[transit] : 0u;
     begin = csr.row_ptr[transit];
     n_edges = csr.row_ptr[transit + 1] - begin;
     max_weight = csr.max_weights[transit];
-    if (taken) return;
+    if (taken_stamp && mark == stamp) return;
   }
   if (app_uses_weights<App>::value) {
     PairedEdgeIds edges{P.paired_edges + begin};
@@ -437,6 +439,16 @@ __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P, c
       produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, nbr, n_edges,
                                                                      max_weight, edges, weights);
   }
+}
+
+// meta (with taken_stamp): the step's bookkeeping, whose stamp marks the taken transits.
+template <class SampleType, class App, bool kSingleOutput>
+__global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P,
+                                                                 const uint32_t* __restrict__ taken_stamp,
+                                                                 const RunsMeta* __restrict__ meta) {
+  const uint32_t stamp = taken_stamp ? meta->stamp : 0u;
+  flat_lane<SampleType, App, kSingleOutput>(P, (uint64_t)flat_block_index() * kFlatThreads + threadIdx.x, taken_stamp,
+                                            stamp);
 }
 
 // Walks that are not re-inverted for a while: one lane keeps its walk for a whole stretch of
@@ -517,19 +529,15 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
 
 // One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
 // transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
-// with coalesced reads and every draw of the stretch gathers from LDS.
+// with coalesced reads and every draw of the stretch gathers from LDS.  The workgroup takes
+// the items first_item, first_item + item_stride, ...
 template <class SampleType, class App>
-__global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams P,
-                                                                      const uint32_t* __restrict__ chunks,
-                                                                      const RunsMeta* __restrict__ meta,
-                                                                      uint32_t chunk_capacity,
-                                                                      uint8_t* __restrict__ skip_flag) {
+__device__ __forceinline__ void workgroup_items(StepParams& P, const uint32_t* __restrict__ chunks, uint32_t n_chunks,
+                                                uint32_t first_item, uint32_t item_stride, CSR::Edge* s_edges,
+                                                float* s_weights) {
   constexpr bool kWeights = app_uses_weights<App>::value;
-  __shared__ CSR::Edge s_edges[kCacheEdges];
-  __shared__ float s_weights[kWeights ? kCacheEdges : 1];
   CSRPartition csr = P.csr;
-  const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
-  for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+  for (uint32_t c = first_item; c < n_chunks; c += item_stride) {
     const uint32_t first_pair = chunks[2 * c];
     const uint32_t n_pairs = chunks[2 * c + 1];
     const VertexID transit = (VertexID)P.pair_keys[first_pair];
@@ -542,7 +550,6 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
       s_edges[e] = csr.edges[begin + e];
       if (kWeights) s_weights[e] = csr.weights[begin + e];
     }
-    if (threadIdx.x == 0) skip_flag[transit] = 0;  // leave the marker array clean for the next step
     __syncthreads();
     LdsBackedArray<CSR::Edge> edges{s_edges, csr.edges + begin, cached};
     LdsBackedArray<float> lds_weights{s_weights, csr.weights + begin, kWeights ? cached : 0};
@@ -554,6 +561,53 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
       produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
           P, csr, transit, first_pair + p, slot, nbr, n_edges, max_weight, edges, lds_weights);
     }
+  }
+}
+
+template <class SampleType, class App>
+__global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams P,
+                                                                      const uint32_t* __restrict__ chunks,
+                                                                      const RunsMeta* __restrict__ meta,
+                                                                      uint32_t chunk_capacity) {
+  __shared__ CSR::Edge s_edges[kCacheEdges];
+  __shared__ float s_weights[app_uses_weights<App>::value ? kCacheEdges : 1];
+  const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
+  workgroup_items<SampleType, App>(P, chunks, n_chunks, blockIdx.x, gridDim.x, s_edges, s_weights);
+}
+
+// Both classes of a load-balanced step in ONE launch: the flat lanes and the work items touch
+// disjoint pairs (a transit belongs to the work items exactly when its marker carries the step's
+// stamp, and nobody clears a marker), so nothing orders them.  The grid is made of groups of
+// kBalancedFlatBlocks flat workgroups followed by wg_per_group work-item workgroups, so that
+// both kinds start side by side from the first moment on; inside the flat part a workgroup
+// finds its pairs as in step_flat_kernel (runs of consecutive workgroups per XCD: a group is a
+// whole number of such runs for all XCDs, and wg_per_group is a multiple of the XCD count).
+// Every workgroup reserves the LDS of the adjacency cache, whichever kind it is: this launch
+// is for maps where the number of launches matters more than the flat lanes' occupancy.
+constexpr uint32_t kBalancedFlatBlocks = kXcds * kXcdRun;
+
+template <class SampleType, class App, bool kSingleOutput>
+__global__ __launch_bounds__(kStepThreads) void step_balanced_kernel(StepParams P,
+                                                                     const uint32_t* __restrict__ taken_stamp,
+                                                                     const RunsMeta* __restrict__ meta,
+                                                                     const uint32_t* __restrict__ chunks,
+                                                                     uint32_t chunk_capacity, uint32_t wg_per_group) {
+  __shared__ CSR::Edge s_edges[kCacheEdges];
+  __shared__ float s_weights[app_uses_weights<App>::value ? kCacheEdges : 1];
+  const uint32_t per_group = kBalancedFlatBlocks + wg_per_group;
+  const uint32_t group = blockIdx.x / per_group;
+  const uint32_t local = blockIdx.x - group * per_group;
+  if (local < kBalancedFlatBlocks) {
+    // the XCD this workgroup runs on is blockIdx.x % kXcds == local % kXcds
+    const uint32_t xcd = local % kXcds, turn = local / kXcds;  // turn < kXcdRun
+    const uint32_t block = group * kBalancedFlatBlocks + xcd * kXcdRun + turn;
+    flat_lane<SampleType, App, kSingleOutput>(P, (uint64_t)block * kStepThreads + threadIdx.x, taken_stamp,
+                                              meta->stamp);
+  } else {
+    const uint32_t n_groups = gridDim.x / per_group;
+    const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
+    workgroup_items<SampleType, App>(P, chunks, n_chunks, group * wg_per_group + (local - kBalancedFlatBlocks),
+                                     n_groups * wg_per_group, s_edges, s_weights);
   }
 }
 
@@ -589,6 +643,9 @@ __device__ __forceinline__ uint32_t run_start(const uint32_t* __restrict__ keys,
   return lo;
 }
 
+// The stamp after `stamp`: 1, 2, ..., 2^32 - 1, 1, ... (0 is what a cleared marker holds).
+__device__ __forceinline__ uint32_t next_stamp(uint32_t stamp) { return stamp + 1u == 0u ? 1u : stamp + 1u; }
+
 // Pairs per kernel class, summed over the load-balanced steps of a pass (what the reference's
 // printKernelTypes shows per step, src/nextdoor.cu:2117-2189).
 struct ClassCounters {
@@ -611,14 +668,11 @@ constexpr int kClassifyItemsLarge = 16;
 constexpr uint32_t kClassifyLargeFrom = 16u << 20;  // pairs
 
 // Is pair i the last of a run that the workgroup kernel should take?  Gives the run and the
-// number of work items it needs.
-// partial_cache: a transit whose adjacency is longer than the LDS cache may go to the workgroup
-// kernel too, with its first kCacheEdges edges in LDS and the rest read from memory (the
-// reference's CachedArray, src/nextdoor.cu:76-124).  refused_out (nullable): set to the run's
-// length when the run is long enough but stays with the flat kernel because of the degree.
+// number of work items it needs.  refused_out (nullable): set to the run's length when the run
+// is long enough but stays with the flat kernel because of the degree.
 __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict__ keys, uint32_t i, uint32_t n,
                                                       const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
-                                                      bool partial_cache, uint32_t* transit_out, uint32_t* start_out,
+                                                      uint32_t* transit_out, uint32_t* start_out,
                                                       uint32_t* count_out, uint32_t* n_items_out,
                                                       uint32_t* refused_out = nullptr) {
   const uint32_t transit = keys[i];
@@ -632,8 +686,7 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
   if (work < kWorkgroupWork) return false;
   const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
   if (degree == 0) return false;
-  const uint32_t staged = degree < (uint32_t)kCacheEdges ? degree : (uint32_t)kCacheEdges;
-  if ((degree > (uint32_t)kCacheEdges && !partial_cache) || (uint64_t)staged > 32ull * work) {
+  if (degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) {
     if (refused_out) *refused_out = count;
     return false;
   }
@@ -666,15 +719,20 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
                                                           RunsMeta* meta_of_next_step,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                           uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
-                                                          uint8_t* __restrict__ skip_flag,
-                                                          ClassCounters* __restrict__ counters, uint32_t partial_cache,
+                                                          uint32_t* __restrict__ taken_stamp,
+                                                          ClassCounters* __restrict__ counters,
                                                           uint32_t* __restrict__ found_by_step, uint32_t step) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t s_base;
   const uint32_t n = *n_dev;
+  const uint32_t stamp = meta->stamp;
   // the work-item counters alternate between steps: this launch clears the one the next
   // step will count into (its last reader, the previous step's workgroup kernel, is done)
-  if (blockIdx.x == 0 && threadIdx.x == 0) meta_of_next_step->n_chunks = 0;
+  // and hands the next step its stamp
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    meta_of_next_step->n_chunks = 0;
+    meta_of_next_step->stamp = next_stamp(stamp);
+  }
   if (step > 2 && found_by_step[step - 1] == 0 && found_by_step[step - 2] == 0 && step % kQuietLookEvery != 0) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&counters->sorted_pairs, (unsigned long long)n);
   const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
@@ -684,8 +742,8 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
     uint32_t refused = 0;
-    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, partial_cache != 0, &transit, &start,
-                                       &count, &n_items, &refused)) {
+    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items,
+                                       &refused)) {
       mine += n_items;
       if (n_items > 1) split_pairs += count; else single_pairs += count;
     }
@@ -731,8 +789,8 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
     // one pair per lane: the run found above is still in the registers
-    if (kClassifyItems > 1 && !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size,
-                                                               partial_cache != 0, &transit, &start, &count, &n_items)))
+    if (kClassifyItems > 1 &&
+        !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items)))
       continue;
     const bool fits = base + n_items <= chunk_capacity;
     for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
@@ -741,7 +799,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
       chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
     }
     if (fits) {
-      skip_flag[transit] = 1;
+      taken_stamp[transit] = stamp;
       found_by_step[step] = 1;  // the next step looks again
     }
     base += n_items;
@@ -800,8 +858,8 @@ __global__ __launch_bounds__(256) void small_map_place(
     uint32_t* __restrict__ state_out,
     // load balancing (classify == 0: none of it)
     uint32_t classify, RunsMeta* meta, RunsMeta* meta_of_next_step, const EdgePos_t* __restrict__ row_ptr,
-    uint32_t step_size, uint32_t* __restrict__ chunks, uint32_t chunk_capacity, uint8_t* __restrict__ skip_flag,
-    ClassCounters* __restrict__ counters, uint32_t partial_cache) {
+    uint32_t step_size, uint32_t* __restrict__ chunks, uint32_t chunk_capacity, uint32_t* __restrict__ taken_stamp,
+    ClassCounters* __restrict__ counters) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t chunk_base[1024];
   const uint32_t n_in = n_in_dev ? *n_in_dev : n_in_host;
@@ -823,6 +881,7 @@ __global__ __launch_bounds__(256) void small_map_place(
       *live_out = total;  // pairs that go on: what the step kernels of this step walk
       if (classify) {
         meta_of_next_step->n_chunks = 0;  // see classify_run_tails
+        meta_of_next_step->stamp = next_stamp(meta->stamp);
         atomicAdd(&counters->sorted_pairs, (unsigned long long)total);
       }
     }
@@ -857,8 +916,7 @@ __global__ __launch_bounds__(256) void small_map_place(
     const uint64_t work = (uint64_t)count * step_size;
     const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
     if (work >= kWorkgroupWork && degree != 0) {
-      const uint32_t staged = degree < (uint32_t)kCacheEdges ? degree : (uint32_t)kCacheEdges;
-      if ((degree > (uint32_t)kCacheEdges && !partial_cache) || (uint64_t)staged > 32ull * work) {
+      if (degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) {
         refused = count;
       } else {
         uint32_t pairs_per_chunk = kChunkOutputs / step_size;
@@ -894,7 +952,7 @@ __global__ __launch_bounds__(256) void small_map_place(
     chunks[2 * (base + g)] = start + off;
     chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
   }
-  if (base + n_items <= chunk_capacity) skip_flag[transit] = 1;
+  if (base + n_items <= chunk_capacity) taken_stamp[transit] = meta->stamp;
 }
 
 __global__ void fill_i32(int32_t* dst, size_t n, int32_t value) {
@@ -1171,6 +1229,9 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_samples_init_, sizeof(SampleType) * (size_t)n_samples_));
       ND_HIP_TRY(hipMemcpy(d_samples_init_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
                            hipMemcpyHostToDevice));
+      // what fetch_sample_states gives before the first run
+      ND_HIP_TRY(hipMemcpy(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
+                           hipMemcpyDeviceToDevice));
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     // Steps whose segment of a result row is at least a memory line long write straight
@@ -1238,19 +1299,35 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_aux_b_, sizeof(uint32_t) * max_pairs_));
     }
     ND_HIP_TRY(hipMalloc(&d_meta_, sizeof(RunsMeta) * 2));
-    ND_HIP_TRY(hipMemset(d_meta_, 0, sizeof(RunsMeta) * 2));
+    {
+      RunsMeta fresh[2] = {};
+      fresh[0].stamp = 1;  // the first load-balanced step; every classification hands the next one its stamp
+      ND_HIP_TRY(hipMemcpy(d_meta_, fresh, sizeof(fresh), hipMemcpyHostToDevice));
+    }
     ND_HIP_TRY(hipMalloc(&d_balance_, sizeof(uint32_t) * kBalanceWords));
     ND_HIP_TRY(hipMemset(d_balance_, 0, sizeof(uint32_t) * kBalanceWords));
     class_counters_ = ClassCounters();
     idle_passes_ = 0;
     balanced_steps_ = 0;
+    markers_cleared_at_ = 0;
+    schedule_counts_ = ScheduleCounts();
+    items_seen_ = false;
     ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
-    ND_HIP_TRY(hipMalloc(&d_skip_flag_, (size_t)invalid_ + 1));
-    ND_HIP_TRY(hipMemset(d_skip_flag_, 0, (size_t)invalid_ + 1));
+    ND_HIP_TRY(hipMalloc(&d_taken_stamp_, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
+    ND_HIP_TRY(hipMemset(d_taken_stamp_, 0, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
+    ND_HIP_TRY(hipStreamCreate(&side_stream_));
     ND_HIP_TRY(hipEventCreate(&ev_a_));
     ND_HIP_TRY(hipEventCreate(&ev_b_));
     ND_HIP_TRY(hipEventCreate(&ev_begin_));
     ND_HIP_TRY(hipEventCreate(&ev_end_));
+    ND_HIP_TRY(hipEventCreateWithFlags(&ev_fork_, hipEventDisableTiming));
+    ND_HIP_TRY(hipEventCreateWithFlags(&ev_join_, hipEventDisableTiming));
+    forced_schedule_ = kScheduleAuto;
+    if (const char* env = getenv("ND_STEP_SCHEDULE")) {
+      if (strcmp(env, "serial") == 0) forced_schedule_ = kScheduleSerial;
+      else if (strcmp(env, "merged") == 0) forced_schedule_ = kScheduleMerged;
+      else if (strcmp(env, "forked") == 0) forced_schedule_ = kScheduleForked;
+    }
 
     // rows staged per workgroup by the final assembly: as many as fit 64 KiB of LDS
     row_pitch_ = (uint32_t)(F | 1);
@@ -1277,6 +1354,14 @@ class Engine : public EngineBase {
       ND_HIP_TRY(hipMemcpyAsync(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
                                 hipMemcpyDeviceToDevice, stream_));
     }
+    if (balanced_steps_ - markers_cleared_at_ >= (1ull << 31)) {
+      // a marker is only ever compared with the stamp of the step that reads it; stamps repeat
+      // after 2^32 - 1 load-balanced steps, so the markers are wiped long before one can be
+      // mistaken for a fresh one
+      const size_t n = (size_t)invalid_ + 1;
+      fill_i32<<<dim3((unsigned)((n + 1023) / 1024)), dim3(1024), 0, stream_>>>((int32_t*)d_taken_stamp_, n, 0);
+      markers_cleared_at_ = balanced_steps_;
+    }
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventRecord(ev_begin_, stream_));
     const int rc = wants_launch_graph() ? replay_pass(mode) : enqueue_pass(mode);
@@ -1284,7 +1369,9 @@ class Engine : public EngineBase {
     ND_HIP_TRY(hipEventRecord(ev_end_, stream_));
     ND_HIP_TRY(hipStreamSynchronize(stream_));
     ND_HIP_TRY(hipEventElapsedTime(&times.end_to_end, ev_begin_, ev_end_));
+    schedule_counts_.passes++;
     if (balanced_this_pass_) {
+      schedule_counts_.classified_passes++;
       // after the pass and outside its timed region: what the classifications counted
       ClassCounters copies[kCounterCopies];
       ND_HIP_TRY(hipMemcpy(copies, counters_dev(), sizeof(copies), hipMemcpyDeviceToHost));
@@ -1297,6 +1384,7 @@ class Engine : public EngineBase {
         class_counters_.work_items += c.work_items;
       }
       idle_passes_ = class_counters_.work_items == 0 && class_counters_.sorted_pairs != 0 ? 1 : 0;
+      items_seen_ = class_counters_.work_items != 0;
     }
     return 0;
   }
@@ -1306,6 +1394,10 @@ class Engine : public EngineBase {
   // transits split over several work items (grid-wide), 3 = pairs in runs long enough for the
   // workgroup kernel that stayed with the flat kernel because of the transit's degree,
   // 4 = work items; the flat kernel served 0 minus 1 minus 2.
+  // Since the buffers were allocated: 5 = passes, 6 = passes whose steps were classified (a
+  // pass after one that found nothing for the workgroup class is not), 7 = load-balanced steps
+  // whose two classes ran as one launch, 8 = as two launches side by side on two streams,
+  // 9 = one after the other.
   int64_t counter(int which) const override {
     switch (which) {
       case 0: return (int64_t)class_counters_.sorted_pairs;
@@ -1313,6 +1405,11 @@ class Engine : public EngineBase {
       case 2: return (int64_t)class_counters_.split_pairs;
       case 3: return (int64_t)class_counters_.refused_pairs;
       case 4: return (int64_t)class_counters_.work_items;
+      case 5: return (int64_t)schedule_counts_.passes;
+      case 6: return (int64_t)schedule_counts_.classified_passes;
+      case 7: return (int64_t)schedule_counts_.merged_steps;
+      case 8: return (int64_t)schedule_counts_.forked_steps;
+      case 9: return (int64_t)schedule_counts_.serial_steps;
       default: return 0;
     }
   }
@@ -1397,17 +1494,14 @@ class Engine : public EngineBase {
       // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
       P.lanes_shift = 0;
       while ((1u << P.lanes_shift) < m && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted) P.lanes_shift++;
-      const unsigned flat_grid = flat_grid_for((uint64_t)n_pairs << P.lanes_shift);
+      const uint64_t flat_lanes = (uint64_t)n_pairs << P.lanes_shift;
 
       if (step == 0) {
         // roots are used in sample order (the reference also feeds step 0 an unsorted map
         // when there is more than one step, nextdoor.cu:2400 and the FIXME at 2372)
         P.pair_keys = (const uint32_t*)transits;
         P.pair_slots = nullptr;
-        tick();
-        launch_flat(P, flat_grid, nullptr);
-        tock(&times.flat_kernel);
-        times.flat_launches++;
+        if (launch_step(P, flat_lanes, false, nullptr) != 0) return -1;
       } else {
         // inversion: sort (transit, slot) by transit.  Walks sort the pairs the previous
         // step emitted (only those still alive); other apps sort the previous step's
@@ -1432,7 +1526,7 @@ class Engine : public EngineBase {
               (uint32_t)invalid_, d_counter_base_, local_start, chunk_total, n_chunks, live_now,
               d_keys_a_, d_vals_a_,
               state_travels_ ? d_aux_a_ : nullptr, balance ? 1u : 0u, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_,
-              chunk_capacity_, d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u);
+              chunk_capacity_, d_taken_stamp_, counters_dev());
           tock(&times.inversion);
           times.sort_launches += 1;
           P.pair_keys = d_keys_a_;
@@ -1441,18 +1535,7 @@ class Engine : public EngineBase {
           P.live_pairs = live_now;
           live_last = live_now;
           sorts_done++;
-          tick();
-          launch_flat(P, flat_grid, balance ? d_skip_flag_ : nullptr);
-          tock(&times.flat_kernel);
-          times.flat_launches++;
-          if (balance) {
-            tick();
-            unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
-            step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
-                P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
-            tock(&times.workgroup_kernel);
-            times.workgroup_launches++;
-          }
+          if (launch_step(P, flat_lanes, balance, meta) != 0) return -1;
         } else {
           const bool compact_only = sample_parallel || (walk_mode_ && sort_period > 1);
           const SortPlan plan = make_sort_plan(n_pairs, compact_only ? 0 : max_bits_);
@@ -1500,10 +1583,7 @@ class Engine : public EngineBase {
             times.flat_launches++;
             step += stretch - 1;
           } else if (!balance || compact_only) {
-            tick();
-            launch_flat(P, flat_grid, nullptr);
-            tock(&times.flat_kernel);
-            times.flat_launches++;
+            if (launch_step(P, flat_lanes, false, nullptr) != 0) return -1;
           } else {
             tick();
             const unsigned pair_blocks = (n_pairs + 255) / 256;
@@ -1514,23 +1594,14 @@ class Engine : public EngineBase {
               const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
               classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
                   sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                  d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
+                  d_taken_stamp_, counters_dev(), d_balance_, (uint32_t)step);
             } else {
               classify_run_tails<1><<<dim3(pair_blocks), dim3(256), 0, stream_>>>(
                   sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
-                  d_skip_flag_, counters_dev(), partial_hub_cache() ? 1u : 0u, d_balance_, (uint32_t)step);
+                  d_taken_stamp_, counters_dev(), d_balance_, (uint32_t)step);
             }
             tock(&times.load_balancing);
-            tick();
-            launch_flat(P, flat_grid, d_skip_flag_);
-            tock(&times.flat_kernel);
-            times.flat_launches++;
-            tick();
-            unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
-            step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(
-                P, d_chunks_, meta, chunk_capacity_, d_skip_flag_);
-            tock(&times.workgroup_kernel);
-            times.workgroup_launches++;
+            if (launch_step(P, flat_lanes, true, meta) != 0) return -1;
           }
         }
       }
@@ -1583,19 +1654,27 @@ class Engine : public EngineBase {
     const int parity = balanced_steps_ & 1;
     RecordedPass* pass = nullptr;
     for (RecordedPass& r : recorded_)
-      if (r.mode == mode && r.inversion_period == inversion_period && r.parity == parity) pass = &r;
+      if (r.mode == mode && r.inversion_period == inversion_period && r.parity == parity && r.items_seen == items_seen_)
+        pass = &r;
     if (!pass) {
       RecordedPass r;
       r.mode = mode;
       r.inversion_period = inversion_period;
       r.parity = parity;
+      r.items_seen = items_seen_;  // decides how the two classes of a step are launched
       const uint64_t before = balanced_steps_;
+      const ScheduleCounts counts_before = schedule_counts_;
       ND_HIP_TRY(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
       const int rc = enqueue_pass(mode);
       hipGraph_t graph = nullptr;
       const hipError_t ended = hipStreamEndCapture(stream_, &graph);
       r.balanced_steps = balanced_steps_ - before;
+      r.balanced = balanced_this_pass_;
+      r.merged_steps = schedule_counts_.merged_steps - counts_before.merged_steps;
+      r.forked_steps = schedule_counts_.forked_steps - counts_before.forked_steps;
+      r.serial_steps = schedule_counts_.serial_steps - counts_before.serial_steps;
       balanced_steps_ = before;  // advanced below, as for every replay
+      schedule_counts_ = counts_before;
       if (rc != 0 || ended != hipSuccess) {
         if (graph) (void)hipGraphDestroy(graph);
         if (rc == 0) last_error = std::string("hipStreamEndCapture: ") + hipGetErrorString(ended);
@@ -1613,6 +1692,10 @@ class Engine : public EngineBase {
     }
     times = pass->counts;  // launch counts of the recorded pass; durations stay zero
     balanced_steps_ += pass->balanced_steps;
+    balanced_this_pass_ = pass->balanced;  // the replayed pass's, not the last recorded one's
+    schedule_counts_.merged_steps += pass->merged_steps;
+    schedule_counts_.forked_steps += pass->forked_steps;
+    schedule_counts_.serial_steps += pass->serial_steps;
     ND_HIP_TRY(hipGraphLaunch(pass->exec, stream_));
     return 0;
   }
@@ -1686,26 +1769,102 @@ class Engine : public EngineBase {
       kMaxSteps + 2 + (int)(kCounterCopies * sizeof(ClassCounters) / sizeof(uint32_t));
   static constexpr int kIdleLookEvery = 8;
   ClassCounters* counters_dev() const { return (ClassCounters*)(d_balance_ + kMaxSteps + 2); }
-  // Transits whose adjacency is longer than the LDS cache stay with the flat kernel unless
-  // ND_HUB_CACHE=1 sends them to the workgroup kernel with the first kCacheEdges edges staged
-  // (the reference's CachedArray, src/nextdoor.cu:76-124).  Off because it loses: draws are
-  // uniform over the adjacency, so a hub of 10^5 edges finds a tenth of them in LDS, and on 4.2 M
-  // weighted walks the pass takes 57.7 ms with it against 37.2 ms without (the workgroup kernel
-  // then serves 9 % of the pairs in 20.7 ms); two-hop sampling gains 3 % (8.23 against 8.46 ms).
-  static bool partial_hub_cache() {
-    static const bool on = getenv("ND_HUB_CACHE") && atoi(getenv("ND_HUB_CACHE")) != 0;
-    return on;
-  }
-
   // Walks write their results in cells of two steps (StepParams::pair_cells) where a step's
   // transit is the previous step's result and the rows are regrouped by assemble_walk_rows.
   bool paired_results() const { return paired_results_; }
 
-  void launch_flat(const StepParams& P, unsigned flat_grid, const uint8_t* skip_flag) {
+  void launch_flat(const StepParams& P, uint64_t lanes, const uint32_t* taken_stamp, const RunsMeta* meta) {
+    const unsigned grid = flat_grid_for(lanes);
     if (P.step_size == 1)
-      step_flat_kernel<SampleType, App, true><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
+      step_flat_kernel<SampleType, App, true><<<dim3(grid), dim3(kFlatThreads), 0, stream_>>>(P, taken_stamp, meta);
     else
-      step_flat_kernel<SampleType, App, false><<<dim3(flat_grid), dim3(kFlatThreads), 0, stream_>>>(P, skip_flag);
+      step_flat_kernel<SampleType, App, false><<<dim3(grid), dim3(kFlatThreads), 0, stream_>>>(P, taken_stamp, meta);
+  }
+
+  // How the two classes of a load-balanced step are launched.
+  //   serial  flat kernel, then workgroup kernel, on the one stream
+  //   merged  one launch (step_balanced_kernel): for maps so small that a launch costs more
+  //           than what it computes
+  //   forked  the workgroup kernel on a second stream beside the flat kernel: for large maps,
+  //           where each keeps the occupancy of its own launch
+  // Auto: serial until a classified pass has found work items at all (a pass over a map where
+  // no transit gathers enough pairs should not pay for the second class), then by the size of
+  // the step.  ND_STEP_SCHEDULE=serial|merged|forked forces one (read when the buffers are
+  // allocated).  Results do not depend on it.
+  enum { kScheduleAuto = -1, kScheduleSerial = 0, kScheduleMerged = 1, kScheduleForked = 2 };
+  static constexpr uint64_t kMergedLanesAtMost = 1ull << 19;
+  static constexpr uint32_t kMergedWorkgroupBlocks = 16384;
+
+  int schedule_for(uint64_t lanes) const {
+    if (forced_schedule_ != kScheduleAuto) return forced_schedule_;
+    if (!items_seen_) return kScheduleSerial;
+    return lanes <= kMergedLanesAtMost ? kScheduleMerged : kScheduleForked;
+  }
+
+  // The kernels of one step over the pairs P describes.  balance: the step was classified
+  // (meta: its bookkeeping), and the transits its work items cover carry its stamp.
+  int launch_step(const StepParams& P, uint64_t lanes, bool balance, const RunsMeta* meta) {
+    if (!balance) {
+      tick();
+      launch_flat(P, lanes, nullptr, nullptr);
+      tock(&times.flat_kernel);
+      times.flat_launches++;
+      return 0;
+    }
+    const unsigned wg_grid = chunk_capacity_ < 4096u ? chunk_capacity_ : 4096u;
+    const int schedule = schedule_for(lanes);
+    if (schedule == kScheduleMerged) {
+      const uint64_t flat_blocks = (lanes + kStepThreads - 1) / kStepThreads;
+      uint64_t groups = (flat_blocks + kBalancedFlatBlocks - 1) / kBalancedFlatBlocks;
+      if (groups == 0) groups = 1;
+      const uint64_t wanted = chunk_capacity_ < kMergedWorkgroupBlocks ? chunk_capacity_ : kMergedWorkgroupBlocks;
+      uint32_t wg_per_group = (uint32_t)(((wanted + groups - 1) / groups + kXcds - 1) / kXcds * kXcds);
+      if (wg_per_group < kXcds) wg_per_group = kXcds;
+      const unsigned grid = (unsigned)(groups * (kBalancedFlatBlocks + wg_per_group));
+      tick();
+      if (P.step_size == 1)
+        step_balanced_kernel<SampleType, App, true><<<dim3(grid), dim3(kStepThreads), 0, stream_>>>(
+            P, d_taken_stamp_, meta, d_chunks_, chunk_capacity_, wg_per_group);
+      else
+        step_balanced_kernel<SampleType, App, false><<<dim3(grid), dim3(kStepThreads), 0, stream_>>>(
+            P, d_taken_stamp_, meta, d_chunks_, chunk_capacity_, wg_per_group);
+      tock(&times.flat_kernel);
+      times.flat_launches++;
+      schedule_counts_.merged_steps++;
+    } else if (schedule == kScheduleForked && !profiling) {
+      // (with per-phase events the two run one after the other, each timed undisturbed)
+      // The work items start at once on the main stream; the flat kernel, whose single-wave
+      // workgroups would fill every free slot of the machine, follows on the side stream and
+      // takes what the work items leave.
+      ND_HIP_TRY(hipEventRecord(ev_fork_, stream_));
+      ND_HIP_TRY(hipStreamWaitEvent(side_stream_, ev_fork_, 0));
+      step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
+                                                                                              chunk_capacity_);
+      {
+        const unsigned grid = flat_grid_for(lanes);
+        if (P.step_size == 1)
+          step_flat_kernel<SampleType, App, true><<<dim3(grid), dim3(kFlatThreads), 0, side_stream_>>>(P, d_taken_stamp_, meta);
+        else
+          step_flat_kernel<SampleType, App, false><<<dim3(grid), dim3(kFlatThreads), 0, side_stream_>>>(P, d_taken_stamp_, meta);
+      }
+      ND_HIP_TRY(hipEventRecord(ev_join_, side_stream_));
+      ND_HIP_TRY(hipStreamWaitEvent(stream_, ev_join_, 0));
+      times.flat_launches++;
+      times.workgroup_launches++;
+      schedule_counts_.forked_steps++;
+    } else {
+      tick();
+      launch_flat(P, lanes, d_taken_stamp_, meta);
+      tock(&times.flat_kernel);
+      times.flat_launches++;
+      tick();
+      step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
+                                                                                              chunk_capacity_);
+      tock(&times.workgroup_kernel);
+      times.workgroup_launches++;
+      if (schedule == kScheduleForked) schedule_counts_.forked_steps++; else schedule_counts_.serial_steps++;
+    }
+    return 0;
   }
 
   // workgroups of the flat kernel for this many outputs: whole groups of kXcds * kXcdRun, so
@@ -1763,13 +1922,15 @@ class Engine : public EngineBase {
     release(d_meta_);
     release(d_balance_);
     release(d_chunks_);
-    release(d_skip_flag_);
+    release(d_taken_stamp_);
     release(d_distinct_counts_);
     // whatever exists, also after an alloc that failed half way
-    for (hipEvent_t* ev : {&ev_a_, &ev_b_, &ev_begin_, &ev_end_}) {
+    for (hipEvent_t* ev : {&ev_a_, &ev_b_, &ev_begin_, &ev_end_, &ev_fork_, &ev_join_}) {
       if (*ev) (void)hipEventDestroy(*ev);
       *ev = nullptr;
     }
+    if (side_stream_) (void)hipStreamDestroy(side_stream_);
+    side_stream_ = nullptr;
     if (stream_) (void)hipStreamDestroy(stream_);
     stream_ = nullptr;
     allocated_ = false;
@@ -1795,7 +1956,9 @@ class Engine : public EngineBase {
   bool allocated_ = false;
 
   hipStream_t stream_ = nullptr;
+  hipStream_t side_stream_ = nullptr;  // the workgroup kernel of a forked step
   hipEvent_t ev_a_ = nullptr, ev_b_ = nullptr, ev_begin_ = nullptr, ev_end_ = nullptr;
+  hipEvent_t ev_fork_ = nullptr, ev_join_ = nullptr;
   VertexID_t* d_initial_ = nullptr;
   SampleType* d_samples_ = nullptr;
   SampleType* d_samples_init_ = nullptr;
@@ -1821,6 +1984,8 @@ class Engine : public EngineBase {
   bool balanced_this_pass_ = false;
   struct RecordedPass {
     int mode = 0, inversion_period = 0, parity = 0;
+    bool items_seen = false, balanced = false;
+    uint64_t merged_steps = 0, forked_steps = 0, serial_steps = 0;
     uint64_t balanced_steps = 0;  // load-balanced steps of the pass
     PhaseTimes counts;            // its launch counts
     hipGraphExec_t exec = nullptr;
@@ -1828,7 +1993,14 @@ class Engine : public EngineBase {
   std::vector<RecordedPass> recorded_;
   uint64_t balanced_steps_ = 0;        // ... counted over the life of the buffers, so the parity never repeats
   uint32_t* d_chunks_ = nullptr;
-  uint8_t* d_skip_flag_ = nullptr;
+  uint32_t* d_taken_stamp_ = nullptr;  // per vertex: the stamp of the last step whose work items covered it
+  uint64_t markers_cleared_at_ = 0;    // balanced_steps_ when the markers were last wiped
+  struct ScheduleCounts {
+    uint64_t passes = 0, classified_passes = 0, merged_steps = 0, forked_steps = 0, serial_steps = 0;
+  };
+  ScheduleCounts schedule_counts_;
+  bool items_seen_ = false;            // the last classified pass found work items
+  int forced_schedule_ = kScheduleAuto;
   int32_t* d_distinct_counts_ = nullptr;
 };
 

@@ -1366,6 +1366,9 @@ class LayerEngine : public EngineBase {
       ND_HIP_TRY(hipMalloc(&d_samples_init_, sizeof(SampleType) * (size_t)n_samples_));
       ND_HIP_TRY(hipMemcpy(d_samples_init_, samples_.data(), sizeof(SampleType) * (size_t)n_samples_,
                            hipMemcpyHostToDevice));
+      // what fetch_sample_states gives before the first run
+      ND_HIP_TRY(hipMemcpy(d_samples_, d_samples_init_, sizeof(SampleType) * (size_t)n_samples_,
+                           hipMemcpyDeviceToDevice));
       std::vector<SampleType>().swap(samples_);  // the pristine copy now lives on the device
     }
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));

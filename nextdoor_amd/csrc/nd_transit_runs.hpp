@@ -32,6 +32,8 @@ struct RunsMeta {
   uint32_t n_runs;     // unique transits in that prefix
   uint32_t n_chunks;   // work items emitted for the workgroup kernel
   uint32_t n_big_pairs;  // pairs covered by those work items
+  uint32_t stamp;      // load-balanced steps: the value that marks the transits taken by work items at
+                       // this step (see classify_run_tails in nd_engine.hpp); never 0
 };
 
 __device__ __forceinline__ bool is_run_head(const uint32_t* keys, size_t i, uint32_t invalid) {

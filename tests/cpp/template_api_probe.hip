@@ -7,7 +7,12 @@
 #include <libNextDoor_amd.hpp>
 #include <nextdoor_amd_apps.hpp>
 
-struct CallerWalkSample {};
+// what next() leaves behind for the checker: the vertex the walk last stepped from, and how
+// many times it stepped
+struct CallerWalkSample {
+  VertexID_t previous;
+  int stepsTaken;
+};
 
 // the reference's example app (example/uniformRandWalk.cu:15-93) with walks of 6 steps
 struct CallerWalkApp {
@@ -20,6 +25,8 @@ struct CallerWalkApp {
                                   WeightArray& transitEdgeWeights, const EdgePos_t numEdges,
                                   const VertexID_t neighbrID, curandState* state) {
     EdgePos_t x = RandNumGen::rand_int(state, numEdges);
+    sample->previous = *transit;
+    sample->stepsTaken++;
     return transitEdges[x];
   }
 
@@ -46,9 +53,42 @@ struct CallerWalkApp {
   template <class SampleType>
   __host__ SampleType initializeSample(CSR* graph, const VertexID_t sampleID) {
     SampleType sample;
+    sample.previous = -1;
+    sample.stepsTaken = 0;
     return sample;
   }
 };
+
+// A checker in the style of the reference's app-local ones (src/tests/singleGPU/multirw.cu:11-40,
+// src/check_results.cu:46-60): the library's rule on the sampled vertices, then the sample
+// states in nextDoorData.samples against the walks in nextDoorData.hFinalSamples.
+template <class SampleType, typename App>
+bool checkCallerWalkResult(NextDoorData<SampleType, App>& nextDoorData) {
+  if (!checkSampledVerticesResult<SampleType, App>(nextDoorData)) return false;
+  auto finalSampleSize = getFinalSampleSize<App>();
+  auto& finalSamples = nextDoorData.hFinalSamples;
+  auto& samples = nextDoorData.samples;
+  auto INVALID_VERTEX = nextDoorData.INVALID_VERTEX;
+  if (samples.size() * finalSampleSize != finalSamples.size()) {
+    printf("%zu sample states for %zu walks\n", samples.size(), finalSamples.size() / finalSampleSize);
+    return false;
+  }
+  for (size_t s = 0; s < samples.size(); s++) {
+    int taken = 0;
+    while (taken < finalSampleSize && finalSamples[s * finalSampleSize + taken] != INVALID_VERTEX) taken++;
+    // the walk stepped once per vertex it holds, the last time from the vertex before its last one
+    VertexID_t previous = -1;
+    if (taken == 1) previous = nextDoorData.initialContents[s];
+    if (taken > 1) previous = finalSamples[s * finalSampleSize + taken - 2];
+    if (samples[s].stepsTaken != taken || samples[s].previous != previous) {
+      printf("sample %zu: state {%d, %d}, walk says {%d, %d}\n", s, samples[s].previous, samples[s].stepsTaken, previous,
+             taken);
+      return false;
+    }
+  }
+  printf("sample states checked %zu\n", samples.size());
+  return true;
+}
 
 // src/tests/testBase.h:14-24, with the gtest scaffolding replaced by a function that returns the result
 #define APP_TEST_BINARY(SampleClass, AppName, App, Graph, Path, Runs, CheckResults, chkResultsFunc, KernelType, \
@@ -67,5 +107,5 @@ APP_TEST_BINARY(KHopSample, KHop, KHop3x2App, RingSP, path, 1, true,
 int main(int argc, char* argv[]) {
   if (argc > 2 && strcmp(argv[1], "--registry-app") == 0) return KHop_RingLB(argv[2]) && KHop_RingSP(argv[2]) ? 0 : 1;
   // Call the main function of NextDoor to execute the application (example/uniformRandWalk.cu:95-98)
-  return appMain<CallerWalkSample, CallerWalkApp>(argc, argv, checkSampledVerticesResult<CallerWalkSample, CallerWalkApp>);
+  return appMain<CallerWalkSample, CallerWalkApp>(argc, argv, checkCallerWalkResult<CallerWalkSample, CallerWalkApp>);
 }

@@ -77,9 +77,11 @@ def test_app_registration_refuses_what_it_cannot_run():
     maker = maker_type(lambda name: None)
     keep_alive.append(maker)
     fn = C.cast(maker, C.c_void_p)
-    abi = 2  # ND_ENGINE_ABI of include/nextdoor_amd.h
+    # the library's value: ND_ENGINE_ABI of include/nextdoor_amd.h in the upper half, struct sizes below
+    abi = L.nd_engine_abi()
     text = open(os.path.join(ROOT, "include", "nextdoor_amd.h")).read()
-    assert re.search(r"#define\s+ND_ENGINE_ABI\s+%d\b" % abi, text)
+    assert re.search(r"#define\s+ND_ENGINE_ABI\s+%d\b" % (abi >> 16), text)
+    assert L.nd_register_app(b"HostSideProbeApp", fn, abi >> 16) == -2  # the bare version number is not enough
     assert L.nd_register_app(b"HostSideProbeApp", fn, abi + 1) == -2
     assert b"engine ABI" in L.nd_last_error()
     assert L.nd_register_app(b"KHop", fn, abi) == -3

@@ -66,7 +66,7 @@ def test_unique_transits_matches_oracle(oracle, n, frac_invalid):
     assert np.array_equal(u, wu) and np.array_equal(c, wc) and np.array_equal(o, wo)
 
 
-def brute_force_classes(keys, degrees, step_size, partial_cache, thresholds):
+def brute_force_classes(keys, degrees, step_size, thresholds):
     """Which runs the workgroup kernel takes, by the stated rule, and how they are cut."""
     need_work, per_item_outputs, cache_edges = thresholds
     per_item = max(per_item_outputs // step_size, 1)
@@ -76,8 +76,7 @@ def brute_force_classes(keys, degrees, step_size, partial_cache, thresholds):
         work = int(count) * step_size
         if work < need_work or degrees[t] == 0:
             continue
-        staged = min(int(degrees[t]), cache_edges)
-        if (degrees[t] > cache_edges and not partial_cache) or staged > 32 * work:
+        if degrees[t] > cache_edges or degrees[t] > 32 * work:
             refused += int(count)
             continue
         k = -(-int(count) // per_item)
@@ -91,8 +90,8 @@ def brute_force_classes(keys, degrees, step_size, partial_cache, thresholds):
 
 
 @pytest.mark.parametrize("pairs_per_lane", [1, 16])
-@pytest.mark.parametrize("step_size,partial_cache", [(1, True), (1, False), (10, True), (25, False), (3000, True)])
-def test_run_classification_covers_every_pair_of_a_taken_transit_once(step_size, partial_cache, pairs_per_lane):
+@pytest.mark.parametrize("step_size", [1, 2, 10, 25, 3000])
+def test_run_classification_covers_every_pair_of_a_taken_transit_once(step_size, pairs_per_lane):
     # the binning of transits into kernel classes (src/nextdoor.cu:1520-1802; the reference asserts
     # the same covering at :1745-1749) against a brute-force partition of the sorted map
     rng = np.random.default_rng(11 + step_size)
@@ -108,10 +107,10 @@ def test_run_classification_covers_every_pair_of_a_taken_transit_once(step_size,
     counts[rng.integers(0, n_vertices, 6)] = rng.integers(2500, 9000, 6)
     counts[0], counts[n_vertices - 1] = 300, 2100
     keys = np.repeat(np.arange(n_vertices, dtype=np.int32), counts)
-    print("classify n", len(keys), "step size", step_size, "partial", partial_cache, "lane", pairs_per_lane, flush=True)
-    items, wanted, taken, counters = nd.classify_runs(keys, degrees, step_size, partial_cache, pairs_per_lane)
+    print("classify n", len(keys), "step size", step_size, "lane", pairs_per_lane, flush=True)
+    items, wanted, taken, counters = nd.classify_runs(keys, degrees, step_size, pairs_per_lane)
     want_taken, want_items, single, split, refused, per_item = brute_force_classes(keys, degrees, step_size,
-                                                                                   partial_cache, thresholds)
+                                                                                   thresholds)
     assert wanted == want_items == len(items)
     assert sorted(np.flatnonzero(taken).tolist()) == sorted(want_taken)
     assert counters.tolist() == [len(keys), single, split, refused, want_items]

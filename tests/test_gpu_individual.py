@@ -174,6 +174,56 @@ def test_app_matches_oracle(oracle, app, kind_name, state, gname):
     run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
 
 
+@pytest.mark.parametrize("schedule", ["serial", "merged", "forked"])
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("DeepWalkPerVertex", "DEEPWALK", False),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+    ("KHop", "KHOP", False),
+    ("KHop4x3x2", "KHOP", False),
+])
+def test_every_schedule_of_a_load_balanced_step_gives_the_oracle_bytes(oracle, app, kind_name, state, schedule,
+                                                                        monkeypatch):
+    """The two classes of a load-balanced step as one launch, side by side on two streams, or one
+    after the other: the same bytes, on a graph whose hub gathers enough samples for work items and
+    on a star, where one transit carries every sample every other step (the grid-wide case)."""
+    monkeypatch.setenv("ND_STEP_SCHEDULE", schedule)
+    g = graphs.random_graph(**GRAPHS["dense_hub"])
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, modes=(True, True))
+    n = 3000
+    leaves = np.arange(1, n)
+    star = nd.Graph.from_edges(np.concatenate([np.zeros(n - 1, int), leaves]),
+                               np.concatenate([leaves, np.zeros(n - 1, int)]),
+                               np.linspace(1, 4.9, 2 * (n - 1)).astype(np.float32))
+    run_and_compare(oracle, app, getattr(oracle, kind_name), star, check_state=state, modes=(True, False, True))
+
+
+def test_the_schedule_is_chosen_after_a_pass_that_found_work_items(oracle):
+    """Left to itself the engine runs the two classes one after the other until a classified pass
+    has found work items, then as one launch (small steps) or on two streams (large ones); the
+    counters say which, and every pass gives the oracle's bytes."""
+    g = graphs.random_graph(**GRAPHS["dense_hub"])
+    og = graphs.oracle_view(g)
+    for app, kind, small in (("UniformRandomWalk", oracle.UNIFORM_WALK, True), ("KHop40x30", oracle.KHOP, False)):
+        s = nd.Sampler(app, g, seed=SEED)
+        try:
+            want, _ = oracle.sample_individual(og, desc_for(oracle, s, kind), SEED, s.initial_contents)
+            for turn in range(3):
+                print("app", app, "turn", turn, flush=True)
+                s.do_transit_parallel(load_balancing=True)
+                assert np.array_equal(s.final_samples(), want)
+                passes, classified, merged, forked, serial = (s.counter(i) for i in range(5, 10))
+                assert (passes, classified) == (turn + 1, turn + 1) and s.counter(4) > 0
+                balanced_steps = s.steps - 1
+                assert serial == balanced_steps  # the first pass only
+                if small:
+                    assert (merged, forked) == (turn * balanced_steps, 0)
+                else:
+                    assert merged + forked == turn * balanced_steps and forked >= turn
+        finally:
+            s.close()
+
+
 def test_weighted_node2vec_instances_differ_where_the_biases_do(oracle):
     # p = 4, q = 0.5 against p = 0.5, q = 4 on a graph full of triangles: were the bias of a
     # candidate adjacent to the previous vertex mixed up with p or with 1, the two instances (or

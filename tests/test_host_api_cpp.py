@@ -78,6 +78,8 @@ def test_caller_with_an_app_of_its_own_samples_what_the_oracle_does(tmp_path):
         assert "Graph has 36 edges and 12 vertices" in out.stdout
         assert np.array_equal(np.array(parse_samples(out.stdout), np.int32), want), out.stdout
         assert "totalSampledVertices 72" in out.stdout
+        # the caller's checker read NextDoorData::samples: what next() left in every sample's state
+        assert "sample states checked 12" in out.stdout, out.stdout
     out = subprocess.run([TEMPLATE_PROBE, "--registry-app", str(graph)], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr
     assert out.stdout.count("totalSampledVertices 108") == 2  # KHop3x2App: 12 samples x (3 + 6)
