@@ -224,9 +224,11 @@ inline int getFinalSampleSize(const NextDoorDataByName& data) {
 template <class App>
 inline int getFinalSampleSize() {
   // the shape algebra of the App itself where the App is a complete type with steps() ...
+  // ... every output slot of every step: an individual app's steps start from its
+  // initialSampleSize transits (one for the reference's walk and k-hop apps)
   App app;
-  long total = 0, per_step = 1;
   const bool collective = app.samplingType() == CollectiveNeighborhood;
+  long total = 0, per_step = collective ? 1 : (long)app.initialSampleSize(nullptr);
   for (int k = 0; k < app.steps(); ++k) {
     if (collective) per_step = app.stepSize(k); else per_step *= app.stepSize(k);
     total += per_step;

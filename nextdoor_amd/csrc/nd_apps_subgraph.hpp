@@ -103,12 +103,12 @@ struct MVSSamplingAppT : nd::apps::SubgraphCommon<kBatch> {
   }
 };
 
-// ClusterGCN: step 0 passes every vertex of the sample on as the transit of step 1
-// (the reference gets the same transits from stepTransits, clusterGCNSampling.cu:95-104, and
-// uses step 0 to add up the room its list may need); at step 1 lane `neighbrID` of transit v1
-// tests the edge v1 -> vertices[neighbrID] with a binary search of v1's adjacency
-// (clusterGCNSampling.cu:46-67).  The final sample holds the 32 vertices (those with edges),
-// then INVALID.
+// ClusterGCN: an app with explicit transits, as in the reference: the transits of step 1 are
+// the sample's vertices, named by stepTransits (clusterGCNSampling.cu:89-104), whatever step 0
+// returned (the reference uses step 0 to add up the room its list may need; here it returns the
+// vertex).  At step 1 lane `neighbrID` of transit v1 tests the edge v1 -> vertices[neighbrID]
+// with a binary search of v1's adjacency (clusterGCNSampling.cu:46-67).  The final sample holds
+// the 32 vertices (those with edges), then INVALID.
 template <int kClusterVertices, int kClusters>
 struct SubGraphSamplingAppT : nd::apps::SubgraphCommon<kClusterVertices * kClusters> {
   static constexpr int kVertices = kClusterVertices * kClusters;
@@ -125,6 +125,14 @@ struct SubGraphSamplingAppT : nd::apps::SubgraphCommon<kClusterVertices * kClust
     const VertexID_t v2 = sample->state().vertices[neighbrID];
     if (utils::binarySearch(transitEdges, v2, numEdges)) sample->emit(v1, v2);
     return -1;
+  }
+
+  __host__ __device__ bool hasExplicitTransits() { return true; }
+
+  // clusterGCNSampling.cu:95-104, without the global atomic that reserves the list's room
+  template <class SampleType>
+  __device__ VertexID_t stepTransits(int, const VertexID_t, SampleType& sample, int transitIdx, curandState*) {
+    return sample.state().vertices[transitIdx];
   }
 
   // clusters are runs of 16 consecutive vertex ids (the reference's foo(),

@@ -217,6 +217,10 @@ struct StepParams {
   int32_t* pair_cells;
   uint32_t pair_cell_samples;
   void* samples;                 // SampleType[S] or nullptr
+  // Apps with explicit transits that are not walks: the (sample -> transit) map of step k+1,
+  // indexed like step_out's own array form (output slot o of this step is pair o of the next):
+  // what App::stepTransits returned for the output.  nullptr: the step's outputs are the map.
+  int32_t* explicit_out;
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
   // Walks (one transit per sample, stepSize 1 everywhere): the step kernels also emit the
   // next step's pairs in THIS step's pair order - coalesced, and without the pairs the
@@ -279,7 +283,9 @@ __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& c
                                                            // that has edges (nextdoor.cu:250-262)
   const bool explicit_transits = App().hasExplicitTransits();
   curandState rng;
-  if (runs || explicit_transits) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  // a pair whose transit is no vertex is dead, with or without explicit transits
+  const bool chooses_transit = explicit_transits && !P.is_last && transit != P.invalid;
+  if (runs || chooses_transit) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
   VertexID neighbor = P.invalid;
   if (runs) {
     const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
@@ -287,8 +293,12 @@ __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& c
     neighbor = r == -1 ? P.invalid : r;  // nextdoor.cu:288
   }
   *next_transit = neighbor;
-  if (explicit_transits && !P.is_last) {
-    const VertexID_t t = App().stepTransits(P.step + 1, sample_id, *state, (int)transit_index, &rng);
+  if (chooses_transit) {
+    // the index the reference hands over is its thread number modulo the step's transits per
+    // sample (nextdoor.cu:282: threadId % numTransits): the transit's own index where the step
+    // size is 1 (walks: 0; ClusterGCN's step 0: the vertex's place in the sample)
+    const uint32_t index = (transit_index * P.step_size + nbr) % P.transits_per_sample;
+    const VertexID_t t = App().stepTransits(P.step + 1, sample_id, *state, (int)index, &rng);
     *next_transit = t == -1 ? P.invalid : t;
   }
   return neighbor;
@@ -353,6 +363,7 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
     P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
   }
+  if (P.explicit_out) P.explicit_out[out_slot] = next_transit;
   if (P.emit_keys) {
     P.emit_keys[pair] = (uint32_t)next_transit;
     P.emit_slots[pair] = pair_slot;
@@ -1085,9 +1096,13 @@ inline int64_t step_size_at_step(int step) {
   return n;
 }
 
+// Individual apps: every output slot of every step has its place in the result row, so the
+// row holds initialSampleSize * stepSize(0) * ... * stepSize(k) entries for step k.  (The
+// reference's getFinalSampleSize, nextdoor.cu:1913-1929, starts the product at 1; that is the
+// same for its apps with one root per sample, and too short for the slots of the others.)
 template <class App>
 inline int final_sample_size() {
-  int64_t total = 0, per_step = 1;
+  int64_t total = 0, per_step = is_collective<App>() ? 1 : (int64_t)App().initialSampleSize(nullptr);
   for (int k = 0; k < App().steps(); ++k) {
     if (is_collective<App>()) per_step = App().stepSize(k); else per_step *= App().stepSize(k);
     total += per_step;
@@ -1217,6 +1232,7 @@ class Engine : public EngineBase {
     max_pairs_ = (size_t)max_pairs;
     chunk_capacity_ = (uint32_t)chunk_cap;
     const size_t F = (size_t)final_sample_size();
+    if (base != F) { last_error = "the steps' segments do not add up to the final sample size"; return -2; }
     if (host_rows) hFinalSamples.assign((size_t)n_samples_ * F, invalid_); else hFinalSamples.clear();
 
     ND_HIP_TRY(hipStreamCreate(&stream_));
@@ -1253,10 +1269,10 @@ class Engine : public EngineBase {
     walk_mode_ = init_size_ == 1 && n_steps > 1;
     for (int k = 0; k < n_steps; ++k) walk_mode_ = walk_mode_ && app.stepSize(k) == 1;
     state_travels_ = walk_mode_ && state_fits_pair<SampleType>::value;
-    if (app.hasExplicitTransits() && !walk_mode_) {
-      last_error = "explicit transits are supported for walks (one transit per sample, stepSize 1)";
-      return -2;
-    }
+    // apps that choose their transits themselves and are not walks: the next step's map is an
+    // array of its own, written next to the step's outputs
+    explicit_map_ = app.hasExplicitTransits() && !walk_mode_;
+    if (explicit_map_) ND_HIP_TRY(hipMalloc(&d_explicit_, sizeof(VertexID_t) * max_pairs_));
     if (walk_mode_) {
       ND_HIP_TRY(hipMalloc(&d_emit_keys_, sizeof(uint32_t) * max_pairs_));
       ND_HIP_TRY(hipMalloc(&d_emit_slots_, sizeof(uint32_t) * max_pairs_));
@@ -1477,6 +1493,7 @@ class Engine : public EngineBase {
       P.pair_cells = paired_results() ? d_step_out_ : nullptr;
       P.pair_cell_samples = (uint32_t)n_samples_;
       P.samples = d_samples_;
+      P.explicit_out = explicit_map_ && step + 1 < n_steps ? d_explicit_ : nullptr;
       P.paired_edges = dgraph_->paired;
       const bool emits = walk_mode_ && step + 1 < n_steps;
       P.state_travels = state_travels_;
@@ -1607,7 +1624,9 @@ class Engine : public EngineBase {
       }
       ND_HIP_TRY(hipGetLastError());
       transits = P.step_out;
-      if (rows_direct_) {
+      if (explicit_map_) {
+        transits = d_explicit_;  // one entry per output slot, no rows
+      } else if (rows_direct_) {
         transits_layout.seg_len = layout_.seg_len[step];
         transits_layout.pitch = (uint32_t)F;
       }
@@ -1804,6 +1823,11 @@ class Engine : public EngineBase {
   // The kernels of one step over the pairs P describes.  balance: the step was classified
   // (meta: its bookkeeping), and the transits its work items cover carry its stamp.
   int launch_step(const StepParams& P, uint64_t lanes, bool balance, const RunsMeta* meta) {
+    if (P.explicit_out) {
+      // the outputs of the pairs that never reach a kernel (no transit) lead nowhere
+      const size_t n = (size_t)P.n_pairs * P.step_size;
+      fill_i32<<<dim3((unsigned)((n + 1023) / 1024)), dim3(1024), 0, stream_>>>(P.explicit_out, n, P.invalid);
+    }
     if (!balance) {
       tick();
       launch_flat(P, lanes, nullptr, nullptr);
@@ -1923,6 +1947,7 @@ class Engine : public EngineBase {
     release(d_balance_);
     release(d_chunks_);
     release(d_taken_stamp_);
+    release(d_explicit_);
     release(d_distinct_counts_);
     // whatever exists, also after an alloc that failed half way
     for (hipEvent_t* ev : {&ev_a_, &ev_b_, &ev_begin_, &ev_end_, &ev_fork_, &ev_join_}) {
@@ -1969,6 +1994,8 @@ class Engine : public EngineBase {
   uint32_t* d_scratch_ = nullptr;
   uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
   bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false;
+  bool explicit_map_ = false;           // App::stepTransits fills the next step's map (apps that are not walks)
+  VertexID_t* d_explicit_ = nullptr;    // that map: the transit of every pair of the coming step
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
   // small maps: the inversion without a sort (small_map_scan, small_map_place)
   bool small_map_ = false;

@@ -107,6 +107,10 @@ struct SubgraphStepParams {
   uint64_t seed;
   uint64_t first_sample;
   uint32_t n_samples;
+  // Apps with explicit transits: what App::stepTransits returned for every output of the step,
+  // at the output's place in a second set of rows (the transits of the next step); else nullptr
+  VertexID_t* next_transit_rows;
+  int is_last;
   const void* stored;            // SampleType[n_samples]
   uint32_t units_per_step;       // units (64 lanes) of this step per sample
   uint32_t units_before_step;    // units of the earlier steps per sample
@@ -159,19 +163,32 @@ __global__ __launch_bounds__(kSubgraphThreads) void subgraph_step_kernel(Subgrap
   const VertexID* edges = csr.edges + begin;
   const float* weights = csr.weights + begin;
   const uint64_t out_slot = (P.first_sample + s) * (uint64_t)lanes_of_sample + l;
-  if (runs) {
+  // explicit transits (src/nextdoor.cu:279-289): after next(), with the same random state, the
+  // app names the transit this output stands for at the next step; only the counting run does it
+  const bool chooses_transit = !kWrite && App().hasExplicitTransits() && !P.is_last && transit != P.invalid;
+  VertexID next_transit = P.invalid;
+  if (runs || chooses_transit) {
     curandState rng;
     rng.reset(P.seed, out_slot, (uint32_t)P.step);
     EmittingSample<Stored, CountingSink> view(stored, CountingSink());
-    const VertexID r = App().template next<EmittingSample<Stored, CountingSink>, const VertexID*, const float*>(
-        P.step, &csr, &transit, (VertexID)(P.first_sample + s), &view, max_weight, edges, weights, n_edges,
-        (VertexID_t)nbr, &rng);
-    neighbor = r == -1 ? P.invalid : r;
-    count = view.emitted();
+    if (runs) {
+      const VertexID r = App().template next<EmittingSample<Stored, CountingSink>, const VertexID*, const float*>(
+          P.step, &csr, &transit, (VertexID)(P.first_sample + s), &view, max_weight, edges, weights, n_edges,
+          (VertexID_t)nbr, &rng);
+      neighbor = r == -1 ? P.invalid : r;
+      count = view.emitted();
+    }
+    if (chooses_transit) {
+      // the index the reference hands over: its thread number modulo the step's transits per sample
+      const VertexID_t t = App().stepTransits(P.step + 1, (VertexID)(P.first_sample + s), view,
+                                              (int)(l % P.transits_per_sample), &rng);
+      next_transit = t == -1 ? P.invalid : t;
+    }
   }
   if (!kWrite) {
     const uint32_t through_me = wave_inclusive_scan(count);
     if (has_lane) P.final_rows[(size_t)s * P.final_size + P.seg_base + l] = neighbor;
+    if (has_lane && P.next_transit_rows) P.next_transit_rows[(size_t)s * P.final_size + P.seg_base + l] = next_transit;
     if (live && lane == 63) counts_of_sample[unit_in_sample] = through_me;
     return;
   }
@@ -300,7 +317,6 @@ class SubgraphEngine : public EngineBase {
       last_error = "not an IndividualNeighborhood app with AdjacencyMatrix output";
       return -2;
     }
-    if (app.hasExplicitTransits()) { last_error = "apps with explicit transits are not supported"; return -2; }
     const int n_steps = app.steps();
     if (n_steps < 1 || n_steps > kMaxSteps) { last_error = "steps() must be in [1, 128]"; return -2; }
     n_samples_ = app.numSamples(csr);
@@ -352,6 +368,8 @@ class SubgraphEngine : public EngineBase {
     ND_HIP_TRY(hipMalloc(&d_stored_, sizeof(SampleType) * (size_t)n_samples_));
     ND_HIP_TRY(hipMemcpy(d_stored_, stored.data(), sizeof(SampleType) * (size_t)n_samples_, hipMemcpyHostToDevice));
     ND_HIP_TRY(hipMalloc(&d_final_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
+    if (app.hasExplicitTransits() && n_steps > 1)
+      ND_HIP_TRY(hipMalloc(&d_next_transits_, sizeof(VertexID_t) * (size_t)n_samples_ * F));
     ND_HIP_TRY(hipMalloc(&d_lengths_, per_sample));
     ND_HIP_TRY(hipMalloc(&d_list_start_, per_sample));
     units_per_sample_ = 0;
@@ -473,9 +491,12 @@ class SubgraphEngine : public EngineBase {
       P.transits = d_initial_;
       P.transit_pitch = (uint32_t)init_size_;
     } else {
-      P.transits = d_final_ + layout_.seg_base[step - 1];
+      // the previous step's outputs, or what stepTransits made of them
+      P.transits = (d_next_transits_ ? d_next_transits_ : d_final_) + layout_.seg_base[step - 1];
       P.transit_pitch = P.final_size;
     }
+    P.next_transit_rows = d_next_transits_;
+    P.is_last = step == app.steps() - 1;
     P.final_rows = d_final_;
     P.seg_base = layout_.seg_base[step];
     P.invalid = invalid_;
@@ -510,6 +531,7 @@ class SubgraphEngine : public EngineBase {
     release(d_initial_);
     release(d_stored_);
     release(d_final_);
+    release(d_next_transits_);
     release(d_lengths_);
     release(d_list_start_);
     release(d_unit_counts_);
@@ -544,6 +566,7 @@ class SubgraphEngine : public EngineBase {
   VertexID_t* d_initial_ = nullptr;
   SampleType* d_stored_ = nullptr;
   VertexID_t* d_final_ = nullptr;
+  VertexID_t* d_next_transits_ = nullptr;  // rows of the transits App::stepTransits chose (explicit transits)
   uint32_t* d_lengths_ = nullptr;
   uint32_t* d_list_start_ = nullptr;
   uint32_t* d_unit_counts_ = nullptr;

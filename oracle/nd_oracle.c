@@ -104,8 +104,9 @@ int64_t ndo_sub_warp_size_at_step(const ndo_app_desc* app, int step) {
 }
 
 int64_t ndo_final_sample_size(const ndo_app_desc* app) {
-  /* nextdoor.cu:1913-1929 */
-  int64_t total = 0, per_step = 1;
+  /* nextdoor.cu:1913-1929; individual apps: one entry per output slot, i.e. the product starts
+   * at the initial sample size (1 for the reference's walk and k-hop apps) */
+  int64_t total = 0, per_step = ndo_is_collective(app) || app->initial_size < 1 ? 1 : app->initial_size;
   for (int k = 0; k < app->steps; ++k) {
     if (ndo_is_collective(app)) per_step = app->step_size[k];
     else per_step *= app->step_size[k];
@@ -363,6 +364,69 @@ int ndo_sample_multirw(const ndo_graph* g, uint64_t seed, int64_t n_samples, int
     }
     if (last_root_idx) last_root_idx[s] = last_idx;
   }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Explicit transits with several transits per sample                         */
+/* ------------------------------------------------------------------------- */
+
+int ndo_sample_anchor_hop(const ndo_graph* g, uint64_t seed, int64_t n_samples, int64_t first_sample,
+                          int n_anchors, const int32_t* anchors, int steps, const int* step_size,
+                          int32_t* final_samples, int32_t* transits_out) {
+  if (steps <= 0 || steps > NDO_MAX_STEPS || n_anchors <= 0) return -1;
+  const int32_t invalid = g->n_vertices;
+  int64_t F = 0, widest = n_anchors, per_step = n_anchors;
+  for (int k = 0; k < steps; ++k) {
+    per_step *= step_size[k];
+    F += per_step;
+    if (per_step > widest) widest = per_step;
+  }
+  int32_t* map_a = (int32_t*)malloc(sizeof(int32_t) * (size_t)widest);
+  int32_t* map_b = (int32_t*)malloc(sizeof(int32_t) * (size_t)widest);
+  if (!map_a || !map_b) { free(map_a); free(map_b); return -2; }
+  for (int64_t s = 0; s < n_samples; ++s) {
+    const int32_t* mine = anchors + s * n_anchors;
+    int32_t* out = final_samples + s * F;
+    int32_t* prev = map_a;
+    int32_t* next = map_b;
+    for (int i = 0; i < n_anchors; ++i) prev[i] = mine[i];  /* the initial sample: the anchors */
+    int64_t T = n_anchors, seg_base = 0;
+    for (int k = 0; k < steps; ++k) {
+      const int m = step_size[k];
+      for (int64_t j = 0; j < T; ++j) {
+        const int32_t transit = prev[j];
+        if (transits_out) transits_out[s * F + seg_base + j * m] = transit;  /* the transit its outputs were drawn from */
+        for (int nbr = 0; nbr < m; ++nbr) {
+          int32_t neighbor = invalid, chosen = invalid;
+          if (transit != invalid && transit != -1) {  /* a pair without a transit is dead, and so is what follows it */
+            rng_cursor rc;
+            rc.seed = seed;
+            rc.slot = (uint64_t)(((first_sample + s) * T + j) * m + nbr);
+            rc.step = (uint32_t)k;
+            rc.draw = 0;
+            rc.st = 0;
+            const int32_t n = degree_of(g, transit);
+            if (n != 0) neighbor = g->col[g->row_ptr[transit] + next_int(&rc, n)];  /* nextdoor.cu:250-262, khop.cu:18-22 */
+            if (k != steps - 1) {
+              /* nextdoor.cu:279-289: stepTransits(k + 1) with the random state next() used and
+               * the index (thread number) % (transits per sample of this step) */
+              const int64_t index = (j * m + nbr) % T;
+              const int32_t x = next_int(&rc, n_anchors + 1);
+              if (x != n_anchors) chosen = mine[(index + x) % n_anchors];
+            }
+          }
+          out[seg_base + j * m + nbr] = neighbor;
+          next[j * m + nbr] = chosen;
+        }
+      }
+      int32_t* swap = prev; prev = next; next = swap;
+      seg_base += T * m;
+      T *= m;
+    }
+  }
+  free(map_a);
+  free(map_b);
   return 0;
 }
 

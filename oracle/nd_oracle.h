@@ -133,6 +133,23 @@ int ndo_sample_multirw(const ndo_graph* g, uint64_t seed, int64_t n_samples, int
                        int steps, int32_t* roots, int32_t* last_root_idx, int32_t* final_samples,
                        int32_t* transits_out);
 
+/* An app with explicit transits and SEVERAL transits per sample (the reference's contract allows
+ * it, nextdoor.cu:279-289; of its own apps only ClusterGCN has both, clusterGCNSampling.cu:89-104).
+ * The test application "anchor hop" (tests/cpp/user_apps.hip): a sample holds n_anchors vertices,
+ * which are its initial transits; next() is the k-hop rule (khop.cu:18-22); stepTransits(k + 1),
+ * called after next() with the same random state for every output whose transit is a vertex,
+ * draws x uniformly from [0, n_anchors] and names anchors[(index + x) % n_anchors] as the transit
+ * the output stands for at the next step, or none (x == n_anchors: that branch of the sample ends).
+ * index is what the reference passes: (thread number) % (transits per sample at step k), i.e.
+ * (j * stepSize(k) + nbr) % T_k for neighbour slot nbr of transit j.  Outputs are laid out as
+ * for every per-transit app; transits_out (nullable, same layout) gets, at the first output slot
+ * of every transit, the transit itself.  Pinned by tests that evaluate the rule draw by draw
+ * with ndo_uniform / ndo_rand_int and by adjacency to the named anchors; the values are parity
+ * unpinned by the reference, like every other app's. */
+int ndo_sample_anchor_hop(const ndo_graph* g, uint64_t seed, int64_t n_samples, int64_t first_sample,
+                          int n_anchors, const int32_t* anchors, int steps, const int* step_size,
+                          int32_t* final_samples, int32_t* transits_out);
+
 /* ---- inversion, run-length encode, scan, binning (nextdoor.cu:2924-2939, 2529-2572,
  *      1520-1802; utils.hpp:491-497) ---- */
 

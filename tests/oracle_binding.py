@@ -308,6 +308,27 @@ def sample_multirw(graph, seed, roots, steps, first_sample=0):
     return final, walkers, last, transits
 
 
+def sample_anchor_hop(graph, seed, anchors, step_sizes, first_sample=0):
+    """Returns (final [n, F], transit of every transit's first output slot [n, F], -1 elsewhere)."""
+    L = lib()
+    L.ndo_sample_anchor_hop.restype = C.c_int
+    L.ndo_sample_anchor_hop.argtypes = [C.POINTER(GraphStruct), C.c_uint64, C.c_int64, C.c_int64, C.c_int, i32p, C.c_int,
+                                        C.POINTER(C.c_int), i32p, i32p]
+    anchors = np.ascontiguousarray(anchors, dtype=np.int32)
+    n, n_anchors = anchors.shape
+    sizes = (C.c_int * len(step_sizes))(*step_sizes)
+    F, per_step = 0, n_anchors
+    for m in step_sizes:
+        per_step *= m
+        F += per_step
+    final = np.empty((n, F), np.int32)
+    transits = np.full((n, F), -1, np.int32)
+    rc = L.ndo_sample_anchor_hop(C.byref(graph.struct), seed, n, first_sample, n_anchors, _p(anchors, C.c_int32),
+                                 len(step_sizes), sizes, _p(final, C.c_int32), _p(transits, C.c_int32))
+    assert rc == 0
+    return final, transits
+
+
 def subgraph_num_samples(graph, vertices_per_sample, cap):
     return lib().ndo_subgraph_num_samples(C.byref(graph.struct), vertices_per_sample, cap)
 

@@ -45,6 +45,35 @@ def test_apps_registered_from_their_own_shared_object_match_the_oracle(app, kind
         s.close()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("gname", ["sparse", "hub"])
+def test_an_app_with_explicit_transits_and_several_transits_per_sample(gname):
+    """stepTransits decides the next step's transits (src/nextdoor.cu:279-289) for an app that is
+    not a walk: four transits per sample, step sizes 2, 3, 2; every schedule gives the oracle's bytes."""
+    nd.load_app_library(USER_APPS_LIB)
+    g = graphs.random_graph(**{"sparse": dict(n=300, mean_degree=3, seed=1, isolated_every=7),
+                               "hub": dict(n=1200, mean_degree=10, seed=2, hub=5)}[gname])
+    og = graphs.oracle_view(g)
+    s = nd.Sampler("UserAnchorHop", g, seed=SEED)
+    try:
+        assert (s.steps, s.initial_sample_size, s.final_sample_size) == (3, 4, 8 + 24 + 48)
+        anchors = s.initial_contents.reshape(-1, 4)
+        assert np.array_equal(anchors, np.stack([(np.arange(g.n_vertices) * 7 + i * 13) % g.n_vertices
+                                                 for i in range(4)], axis=1))
+        want, _ = ob.sample_anchor_hop(og, SEED, anchors, [2, 3, 2])
+        for mode in (False, True, "sample_parallel", True):
+            print("UserAnchorHop", gname, mode, flush=True)
+            if mode == "sample_parallel":
+                s.do_sample_parallel()
+            else:
+                s.do_transit_parallel(load_balancing=mode)
+            assert np.array_equal(s.final_samples(), want)
+        with pytest.raises(nd.NextDoorError):  # explicit transits: the library has no validator
+            s.check_results()
+    finally:
+        s.close()
+
+
 def write_binary_edge_list(path, src, dst, weight):
     """The reference's binary edge list: 12-byte records (int32 src, int32 dst, float32 weight),
     src/graph.hpp:42-75."""
