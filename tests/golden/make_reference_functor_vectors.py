@@ -1,8 +1,8 @@
 """Writes tests/golden/reference_functor_vectors.json: what the REFERENCE's own sampler functors
 produce on the small fixed graph of make_vectors.py.
 
-The samplers are the text of src/apps/khop/khop.cu and src/apps/randomwalks/randomWalks.cu,
-compiled from the reference tree as host C++ against this repository's App contract
+The samplers are the text of src/apps/khop/khop.cu, src/apps/randomwalks/randomWalks.cu,
+src/apps/layer/layerSampling.cu and src/apps/multiRW/multiRW.cu, compiled from the reference tree as host C++ against this repository's App contract
 (oracle/Makefile -> oracle/_ref/libreference_apps_host.so, never committed) and run by
 oracle/reference_apps_host.cpp in a plain loop over samples with this repository's slot layout
 and Philox streams.  So the numbers below are decided by the reference's next() code - its
@@ -11,9 +11,11 @@ of it.  Needs the reference tree at build time; the fixture it writes does not.
 
     make -C oracle reference && python tests/golden/make_reference_functor_vectors.py
 
-Sizes are the reference's: KHop [25, 10]; DeepWalk, PPR and Node2Vec 100 steps; two walks per
-vertex are kept (samples 0 .. 2V-1 of the 100 walks per vertex the apps ask for: a sample's
-values depend on its index and root only)."""
+Sizes are the reference's: KHop [25, 10]; Layer [10, 25]; DeepWalk, PPR and Node2Vec 100 steps; two
+walks per vertex are kept (samples 0 .. 2V-1 of the 100 walks per vertex the apps ask for: a
+sample's values depend on its index and root only); MultiRW 100 walkers and 100 steps per sample,
+the walkers starting where this repository's MultiRW app starts them (a fixed Philox stream; the
+reference draws them with rand())."""
 import ctypes as C
 import json
 import os
@@ -29,7 +31,7 @@ from tests.golden import make_vectors  # noqa: E402
 HERE = os.path.dirname(os.path.abspath(__file__))
 REF_LIB = os.path.join(ob.ORACLE_DIR, "_ref", "libreference_apps_host.so")
 SEED = 42
-APPS = {"KHop": 0, "DeepWalk": 1, "PPR": 2, "Node2Vec": 3}  # ref_sample_individual's app numbers
+APPS = {"KHop": 0, "DeepWalk": 1, "PPR": 2, "Node2Vec": 3, "Layer": 4}  # ref_sample_individual's app numbers
 
 
 def main():
@@ -46,7 +48,7 @@ def main():
         steps, sizes, n = C.c_int32(), (C.c_int32 * 128)(), C.c_int64()
         assert lib.ref_app_shape(number, V, C.byref(steps), sizes, C.byref(n)) == 0
         sizes = [sizes[k] for k in range(steps.value)]
-        n_kept = V if app == "KHop" else 2 * V
+        n_kept = V if app in ("KHop", "Layer") else 2 * V
         roots = (np.arange(n_kept) % V).astype(np.int32)
         F, per = 0, 1
         for m in sizes:
@@ -64,6 +66,19 @@ def main():
         if app == "Node2Vec":
             entry["state_t"] = t.tolist()
         out["apps"][app] = entry
+    # the multi-dimensional random walk (explicit transits)
+    lib.ref_multirw_shape.argtypes = [i32p, i32p]
+    lib.ref_sample_multirw.argtypes = [C.c_int32, C.c_int64, i32p, i32p, C.c_uint64, C.c_int64, i32p, i32p, i32p]
+    n_roots, steps = C.c_int32(), C.c_int32()
+    assert lib.ref_multirw_shape(C.byref(n_roots), C.byref(steps)) == 0
+    roots = ob.multirw_roots(V, n_roots.value, V)
+    walkers, last, final = roots.copy(), np.empty(V, np.int32), np.empty((V, steps.value), np.int32)
+    p = lambda a, ty: a.ctypes.data_as(C.POINTER(ty))  # noqa: E731
+    assert lib.ref_sample_multirw(V, len(g.col), p(g.row_ptr, C.c_int32), p(g.col, C.c_int32), SEED, V,
+                                  p(walkers, C.c_int32), p(last, C.c_int32), p(final, C.c_int32)) == 0
+    out["apps"]["MultiRW"] = {"steps": steps.value, "n_roots": n_roots.value, "roots": roots.reshape(-1).tolist(),
+                              "final": final.reshape(-1).tolist(), "shape": list(final.shape),
+                              "walkers": walkers.reshape(-1).tolist(), "last_root_idx": last.tolist()}
     path = os.path.join(HERE, "reference_functor_vectors.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

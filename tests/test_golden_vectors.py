@@ -88,7 +88,7 @@ def test_library_produces_the_committed_vectors(app):
 # from the reference's khop.cu / randomWalks.cu compiled on the CPU (see that script); neither
 # the reference tree nor that build is needed here.
 
-REFERENCE_APPS = {"KHop": "KHOP", "DeepWalk": "DEEPWALK", "PPR": "PPR", "Node2Vec": "NODE2VEC"}
+REFERENCE_APPS = {"KHop": "KHOP", "DeepWalk": "DEEPWALK", "PPR": "PPR", "Node2Vec": "NODE2VEC", "Layer": "KHOP"}
 
 
 @pytest.mark.parametrize("app", sorted(REFERENCE_APPS))
@@ -129,5 +129,38 @@ def test_library_produces_what_the_reference_functors_do(app):
                 t = s.sample_states().view(np.int32)[:kept]
                 moved = got[:, 0] != g.n_vertices
                 assert np.array_equal(t[moved], np.array(want["state_t"], np.int32)[moved])
+    finally:
+        s.close()
+
+
+def test_oracle_produces_what_the_reference_multirw_functor_does(oracle):
+    fx = load("reference_functor_vectors.json")
+    gr, want = fx["graph"], fx["apps"]["MultiRW"]
+    g = oracle.Graph(gr["row_ptr"], gr["col"], gr["weight"])
+    n, steps, n_roots = want["shape"][0], want["steps"], want["n_roots"]
+    roots = np.array(want["roots"], np.int32).reshape(n, n_roots)
+    assert np.array_equal(roots, oracle.multirw_roots(n, n_roots, g.n_vertices))
+    final, walkers, last, _ = oracle.sample_multirw(g, fx["seed"], roots, steps)
+    assert final.reshape(-1).tolist() == want["final"]
+    assert walkers.reshape(-1).tolist() == want["walkers"] and last.tolist() == want["last_root_idx"]
+
+
+@pytest.mark.gpu
+def test_library_produces_what_the_reference_multirw_functor_does():
+    import nextdoor_amd as nd
+    fx = load("reference_functor_vectors.json")
+    gr, want = fx["graph"], fx["apps"]["MultiRW"]
+    g = nd.Graph.from_csr(gr["row_ptr"], gr["col"], np.array(gr["weight"], np.float32))
+    s = nd.Sampler("MultiRW", g, seed=fx["seed"])
+    try:
+        n, n_roots = want["shape"][0], want["n_roots"]
+        assert (s.num_samples, s.steps) == (n, want["steps"])
+        for lb in (True, False):
+            print("app MultiRW lb", lb, flush=True)
+            s.do_transit_parallel(load_balancing=lb)
+            assert s.final_samples().reshape(-1).tolist() == want["final"]
+            state = s.sample_states().view(np.int32).reshape(n, n_roots + 1)
+            assert state[:, :n_roots].reshape(-1).tolist() == want["walkers"]
+            assert state[:, n_roots].tolist() == want["last_root_idx"]
     finally:
         s.close()

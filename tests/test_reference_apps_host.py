@@ -1,7 +1,8 @@
 """The oracle's restatement of the reference's samplers against the reference's own functor
 code: oracle/_ref/libreference_apps_host.so is the text of src/apps/khop/khop.cu,
-src/apps/randomwalks/randomWalks.cu and src/apps/fastgcn/fastgcnSampling.cu, compiled from the
-reference tree as host C++ against the App contract header (oracle/Makefile) and run in a plain
+src/apps/randomwalks/randomWalks.cu, src/apps/fastgcn/fastgcnSampling.cu,
+src/apps/ladies/ladiessampling.cu, src/apps/layer/layerSampling.cu and src/apps/multiRW/multiRW.cu,
+compiled from the reference tree as host C++ against the App contract header (oracle/Makefile) and run in a plain
 CPU loop with the same slot layout and random streams.  Same graph, same roots, same seed ->
 the same bytes.  Skipped where that library has not been built (no reference tree)."""
 import ctypes as C
@@ -15,7 +16,7 @@ from tests import oracle_binding as ob
 REF_LIB = os.path.join(ob.ORACLE_DIR, "_ref", "libreference_apps_host.so")
 pytestmark = pytest.mark.skipif(not os.path.exists(REF_LIB), reason="oracle/_ref is built from the reference tree")
 
-KHOP, DEEPWALK, PPR, NODE2VEC = range(4)
+KHOP, DEEPWALK, PPR, NODE2VEC, LAYER = range(5)
 SEED = 42
 i32p, f32p = C.POINTER(C.c_int32), C.POINTER(C.c_float)
 
@@ -27,6 +28,9 @@ def ref():
     lib.ref_sample_individual.argtypes = [C.c_int, C.c_int32, C.c_int64, i32p, i32p, f32p, f32p, C.c_uint64, C.c_int64,
                                           i32p, i32p, i32p]
     lib.ref_sample_fastgcn.argtypes = [C.c_int32, C.c_int64, i32p, i32p, C.c_uint64, C.c_int64, i32p, i32p, i32p, i32p]
+    lib.ref_sample_ladies.argtypes = lib.ref_sample_fastgcn.argtypes
+    lib.ref_multirw_shape.argtypes = [i32p, i32p]
+    lib.ref_sample_multirw.argtypes = [C.c_int32, C.c_int64, i32p, i32p, C.c_uint64, C.c_int64, i32p, i32p, i32p]
     return lib
 
 
@@ -80,15 +84,17 @@ GRAPHS = {
 
 @pytest.mark.parametrize("gname", list(GRAPHS))
 @pytest.mark.parametrize("app,kind,state", [(KHOP, "KHOP", False), (DEEPWALK, "DEEPWALK", False), (PPR, "PPR", False),
-                                            (NODE2VEC, "NODE2VEC", True)])
+                                            (NODE2VEC, "NODE2VEC", True), (LAYER, "KHOP", False)])
 def test_oracle_gives_what_the_reference_functors_give(ref, app, kind, state, gname):
     g = random_graph(**GRAPHS[gname])
     n = g.n_vertices
     # the reference's own sizing: k-hop one sample per vertex; the walks 100 per vertex on graphs
     # under 256 K vertices, rooted at sample index mod |V| (randomWalks.cu:23-37); a tenth of those here
     steps, sizes, n_samples, _, _ = reference_samples(ref, app, g, np.zeros(0, np.int32))
-    assert n_samples == (n if app == KHOP else 100 * n)
-    roots = np.arange(n if app == KHOP else 10 * n, dtype=np.int32) % n
+    assert n_samples == (n if app in (KHOP, LAYER) else 100 * n)
+    if app == LAYER:
+        assert sizes == [10, 25]  # layerSampling.cu:5-8
+    roots = np.arange(n if app in (KHOP, LAYER) else 10 * n, dtype=np.int32) % n
     _, _, _, want, want_t = reference_samples(ref, app, g, roots, state)
     d = ob.app_desc(getattr(ob, kind), steps, sizes)  # p = 2, q = 0.5 as the reference hard-codes them
     got, got_t = ob.sample_individual(g, d, SEED, roots)
@@ -101,9 +107,11 @@ def test_oracle_gives_what_the_reference_functors_give(ref, app, kind, state, gn
         assert np.array_equal(got_t[moved], want_t[moved])
 
 
-def test_oracle_gives_what_the_reference_fastgcn_app_gives(ref):
-    # the layer-wise app as the reference has it: 5 layers of 64 drawn uniformly from ALL
-    # vertices, the adjacency towards the previous layer recorded in the sample state
+@pytest.mark.parametrize("app", ["fastgcn", "ladies"])
+def test_oracle_gives_what_the_reference_fastgcn_app_gives(ref, app):
+    # the layer-wise apps as the reference has them (fastgcnSampling.cu and ladiessampling.cu are
+    # one text under two sets of names): 5 layers of 64 drawn uniformly from ALL vertices, the
+    # adjacency towards the previous layer recorded in the sample state
     g = random_graph(n=400, mean_degree=30, seed=3, hub=9)
     n, B, layers, n_samples = g.n_vertices, 64, 5, 12
     roots = (np.arange(n_samples * B) * 7 % n).astype(np.int32)
@@ -111,11 +119,33 @@ def test_oracle_gives_what_the_reference_fastgcn_app_gives(ref):
     final = np.empty((n_samples, layers * B), np.int32)
     rows = np.empty((n_samples, layers, B * B), np.int32)
     cols = np.empty_like(rows)
-    rc = ref.ref_sample_fastgcn(n, len(g.col), p(g.row_ptr, C.c_int32), p(g.col, C.c_int32), SEED, n_samples,
-                                p(roots, C.c_int32), p(final, C.c_int32), p(rows, C.c_int32), p(cols, C.c_int32))
+    run = ref.ref_sample_fastgcn if app == "fastgcn" else ref.ref_sample_ladies
+    rc = run(n, len(g.col), p(g.row_ptr, C.c_int32), p(g.col, C.c_int32), SEED, n_samples,
+             p(roots, C.c_int32), p(final, C.c_int32), p(rows, C.c_int32), p(cols, C.c_int32))
     assert rc == 0
     d = ob.app_desc(ob.LAYER_LITERAL, layers, [B] * layers, initial_size=B)
     got, got_rows, got_cols = ob.sample_layer_literal(g, d, SEED, roots)
     assert np.array_equal(got, final)
     assert np.array_equal(got_rows, rows) and np.array_equal(got_cols, cols)
     assert (rows != -1).any() and np.all(final[1] == n)
+
+
+def test_oracle_gives_what_the_reference_multirw_app_gives(ref):
+    # src/apps/multiRW/multiRW.cu: 100 walkers per sample, 100 steps, stepTransits picks the
+    # walker of the next step from the random state next() used; samples, walkers and lastRootIdx
+    g = random_graph(n=200, mean_degree=4, seed=8, isolated_every=9, hub=3)
+    n_roots, steps = C.c_int32(), C.c_int32()
+    assert ref.ref_multirw_shape(C.byref(n_roots), C.byref(steps)) == 0
+    assert (n_roots.value, steps.value) == (100, 100)
+    n_samples = 40
+    roots = ob.multirw_roots(n_samples, 100, g.n_vertices)
+    walkers = roots.copy()
+    last = np.empty(n_samples, np.int32)
+    final = np.empty((n_samples, 100), np.int32)
+    rc = ref.ref_sample_multirw(g.n_vertices, len(g.col), p(g.row_ptr, C.c_int32), p(g.col, C.c_int32), SEED, n_samples,
+                                p(walkers, C.c_int32), p(last, C.c_int32), p(final, C.c_int32))
+    assert rc == 0
+    got, got_walkers, got_last, _ = ob.sample_multirw(g, SEED, roots, 100)
+    assert np.array_equal(got, final)
+    assert np.array_equal(got_walkers, walkers) and np.array_equal(got_last, last)
+    assert (final == g.n_vertices).any() and (final != g.n_vertices).any()
