@@ -9,7 +9,9 @@ the timed region is the step loop only, as the reference's "End to end time"
 
 Prints one JSON line:  metric / value (sampled edges per second) / roofline (dominant
 kernel, algorithmic bytes over its measured launch time) / cpu_baseline (the CPU oracle on
-a bounded sample of the same walks, on this box's host cores).
+a bounded sample of the same walks, on this box's host cores) for that workload, and under
+"configs" the same figures, shorter runs, for all five benchmark configurations (--only: just
+the workload named with --workload).
 """
 import argparse
 import json
@@ -242,45 +244,43 @@ def algorithmic_bytes_per_pass(sampler, oracle_run, live, weighted, second_order
     return step_bytes, own_bytes, sort_bytes
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--workload", default="weighted_node2vec_rmat22", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-load-balancing", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0)
-    ap.add_argument("--skip-cpu-baseline", action="store_true")
-    ap.add_argument("--inversion-period", type=int, default=1,
-                    help="walks: invert the sample->transit map before every p-th step (1: every step, as the "
-                         "reference; 0: the engine decides); the samples do not depend on it")
-    ap.add_argument("--skip-engine-choice", action="store_true",
-                    help="walks: do not also measure the pass with the engine-chosen inversion period")
-    ap.add_argument("--seed", type=int, default=42)
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one MI355X; this build has no multi-GPU path (samples would shard "
-                 "by contiguous ranges with the graph replicated). Run with --gpus 1.")
-
+def measure(args, workload, steps, warmup, cpu_seconds, graphs, engine_choice=True):
+    """One workload: graph, sampler, warm-up, `steps` timed passes, one pass with per-phase events,
+    the CPU baseline.  Returns the result line as a dict.  graphs: cache of built graphs by spec."""
     import nextdoor_amd as nd
-    w = WORKLOADS[args.workload]
+    w = WORKLOADS[workload]
     t0 = time.perf_counter()
-    graph = make_graph(nd, w["graph"])
+    key = json.dumps(w["graph"], sort_keys=True)
+    if key not in graphs:
+        graphs.clear()  # one large graph in host memory at a time
+        graphs[key] = make_graph(nd, w["graph"])
+    graph = graphs[key]
     t_graph = time.perf_counter() - t0
+    t0 = time.perf_counter()
     sampler = nd.Sampler(w["app"], graph, seed=args.seed)
+    t_setup = time.perf_counter() - t0
     sampler.set_inversion_period(args.inversion_period)
     lb = not args.no_load_balancing
     edges_per_pass = sampler.num_samples * sampler.final_sample_size
+    skip_cpu_baseline = args.skip_cpu_baseline
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         sampler.do_transit_parallel(lb)
     wall0 = time.perf_counter()
     gpu_ms = []
-    for _ in range(args.steps):
+    for _ in range(steps):
         sampler.do_transit_parallel(lb)  # synchronises its stream before returning
         gpu_ms.append(sampler.phase_times()["end_to_end_ms"])
     wall = time.perf_counter() - wall0
-    ms_per_step = wall * 1000.0 / args.steps
+    ms_per_step = wall * 1000.0 / steps
+    per_transit = w["kind"] not in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE", "SUBGRAPH")
+    schedule = None
+    if per_transit and lb:
+        # since the buffers were allocated: passes, passes whose steps were classified (a pass after
+        # one that found no work item is not), and how the classified steps' two kernel classes ran
+        passes, classified, merged, forked, serial = (sampler.counter(i) for i in range(5, 10))
+        schedule = {"passes": passes, "lb_passes_that_classified": classified, "steps_as_one_launch": merged,
+                    "steps_on_two_streams": forked, "steps_one_kernel_after_the_other": serial}
 
     # per-kernel-family durations: one extra pass with events around every launch group
     sampler.set_profiling(True)
@@ -288,7 +288,7 @@ def main():
     prof = sampler.phase_times()
     sampler.set_profiling(False)
     kernel_classes = None
-    if w["kind"] not in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE", "SUBGRAPH") and lb:
+    if per_transit and lb:
         # pairs per kernel class over the steps of the last pass whose classification ran (the
         # reference's printKernelTypes, src/nextdoor.cu:2117-2189)
         looked, single, split, refused, items = (sampler.counter(i) for i in range(5))
@@ -300,35 +300,45 @@ def main():
     # walks, for information only (not the headline): the same pass when the engine chooses how
     # often to invert; the samples must come out the same
     adaptive = None
-    if sampler.step_size(0) == 1 and sampler.steps > 1 and args.inversion_period == 1 and not args.skip_engine_choice:
+    if sampler.step_size(0) == 1 and sampler.steps > 1 and args.inversion_period == 1 and engine_choice:
         sampler.set_inversion_period(0)
         sampler.do_transit_parallel(lb)
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             sampler.do_transit_parallel(lb)
-        ms = (time.perf_counter() - t0) * 1000.0 / args.steps
+        ms = (time.perf_counter() - t0) * 1000.0 / steps
         same = bool(np.array_equal(sampler.final_samples(), final))
         adaptive = {"ms_per_step": ms, "sampled_edges_per_s": edges_per_pass / (ms / 1000.0), "same_samples": same}
+        sampler.set_profiling(True)
+        sampler.do_transit_parallel(lb)
+        chosen = sampler.phase_times()
+        sampler.set_profiling(False)
+        adaptive["phases_ms"] = {k: round(v, 3) for k, v in chosen.items()
+                                 if k in ("inversion_ms", "flat_kernel_ms", "assemble_ms", "flat_launches", "sort_passes")}
         sampler.set_inversion_period(1)
 
     result = {
         "metric": "sampled edges/sec on 1 MI355X", "value": edges_per_pass / (ms_per_step / 1000.0),
-        "unit": "sampled edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "unit": "sampled edges/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32 ids / f32 weights", "data": "synthetic",
-        "config": {"workload": args.workload, "app": w["app"], "vertices": graph.n_vertices, "edges": graph.n_edges,
+        "config": {"workload": workload, "app": w["app"], "vertices": graph.n_vertices, "edges": graph.n_edges,
                    "samples": sampler.num_samples, "walk_steps": sampler.steps, "load_balancing": lb,
-                   "sampled_edges_per_step": edges_per_pass, "valid_outputs": valid,
+                   "sampled_edges_per_step": edges_per_pass,
+                   "value_counts": "output slots of a pass, INVALID ones included (valid_outputs of them hold a vertex)",
+                   "valid_outputs": valid,
                    "valid_sampled_edges_per_s": valid / (ms_per_step / 1000.0),
-                   "graph_build_s": round(t_graph, 1), "gpu_event_ms_per_step": float(np.mean(gpu_ms))},
+                   "graph_build_s": round(t_graph, 1), "sampler_setup_s": round(t_setup, 1),
+                   "gpu_event_ms_per_step": float(np.mean(gpu_ms))},
         "phases_ms": {k: round(v, 3) for k, v in prof.items()},
     }
     if kernel_classes:
         result["config"]["kernel_classes"] = kernel_classes
+    if schedule:
+        result["config"]["load_balancing_schedule"] = schedule
     result["config"]["inversion_period"] = args.inversion_period
     if adaptive:
         result["config"]["engine_chosen_inversion_period"] = adaptive
-
     if w["kind"] in ("FASTGCN_IMPORTANCE", "LADIES_IMPORTANCE"):
         entries, distinct = sampler.counter(0), sampler.counter(1)
         result["config"]["neighbourhood_entries"] = entries
@@ -350,18 +360,18 @@ def main():
         all_uses = mark_bytes / (prof["neighbourhood_ms"] / 1000.0) / 1e9
         result["roofline"] = {
             "bound": "hbm", "kernel": "collective_mark_binned", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload),
             "algorithmic_bytes_per_launch": from_memory / launches,
             "avg_launch_ms": prof["neighbourhood_ms"] / launches,
             "cache_served": {"bytes_per_launch_with_every_piece_use": mark_bytes / launches,
                              "GBps_with_every_piece_use": all_uses,
                              "note": "piece uses beyond the first per layer come from L2 / Infinity Cache: a cache "
                                      "throughput figure, not an HBM roofline fraction"},
-            "whole_pass": {"measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
+            "whole_pass": {"measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(workload)},
         }
-        if not args.skip_cpu_baseline:
-            result["cpu_baseline"] = cpu_baseline_layers(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
-        args.skip_cpu_baseline = True  # the walk/k-hop accounting below does not apply to layer-wise apps
+        if not skip_cpu_baseline:
+            result["cpu_baseline"] = cpu_baseline_layers(graph, sampler, w["kind"], cpu_seconds, args.seed)
+        skip_cpu_baseline = True  # the walk/k-hop accounting below does not apply to layer-wise apps
     if w["kind"] == "SUBGRAPH":
         listed = sampler.counter(0)
         result["config"]["edges_listed"] = listed
@@ -374,13 +384,13 @@ def main():
         result["roofline"] = {"bound": "hbm", "kernel": "subgraph_step_kernel (count + write passes)",
                               "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": achieved / HBM_PEAK_GBS, "traffic": None}
-        args.skip_cpu_baseline = True
+        skip_cpu_baseline = True
     if w["kind"] == "KHOP":
         counts = sampler.distinct()
         result["config"]["distinct_ms"] = sampler.phase_times()["distinct_ms"]
         result["config"]["distinct_kept"] = int(counts.sum())
-    if not args.skip_cpu_baseline:
-        base, run = cpu_baseline(graph, sampler, w["kind"], args.cpu_seconds, args.seed)
+    if not skip_cpu_baseline:
+        base, run = cpu_baseline(graph, sampler, w["kind"], cpu_seconds, args.seed)
         result["cpu_baseline"] = base
         # the reference's only CPU path over the samples is its validator (src/check_results.cu:162-299):
         # ours, over every output of the pass just sampled, on the same host cores
@@ -406,7 +416,7 @@ def main():
             "bound": "hbm", "kernel": "step_flat_kernel + step_workgroup_kernel", "achieved": achieved,
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "frac_own_algorithm": own_bytes / (step_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload),
             "algorithmic_bytes_per_launch": step_bytes / max(launches, 1),
             "own_algorithm_bytes_per_launch": own_bytes / max(launches, 1),
             "avg_launch_ms": step_ms / max(launches, 1),
@@ -414,37 +424,107 @@ def main():
             "whole_pass": {"algorithmic_bytes": step_bytes + sort_bytes, "inversion_bytes": sort_bytes,
                            "achieved_GBps": (step_bytes + sort_bytes) / (pass_ms / 1000.0) / 1e9,
                            "frac": (step_bytes + sort_bytes) / (pass_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
-                           "measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(args.workload)},
+                           "measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(workload)},
         }
         result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
-        traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
+        traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload)
         if traffic and w["kind"] != "KHOP":  # walks: the recorded figure is the flat kernel's launch
             # recorded counter traffic of one launch over this run's launch duration (flat kernel alone)
             flat_launch_s = prof["flat_kernel_ms"] / max(launches, 1) / 1000.0
             result["roofline"]["traffic_frac"] = traffic / flat_launch_s / 1e9 / HBM_PEAK_GBS
-        misses = MEASURED_L2_MISS_REQUESTS_PER_LAUNCH.get(args.workload)
+        misses = MEASURED_L2_MISS_REQUESTS_PER_LAUNCH.get(workload)
         if misses:
             # The step kernel's reads are dependent random gathers; each one that misses L2 costs a
             # 128-byte request whatever it uses.  The ceiling for such requests is measured here, on
             # this GPU, over a table of the size of the graph's arrays (rounded down to a power of two).
             graph_bytes = 4.0 * graph.n_vertices * 2 + graph.n_edges * (8.0 + 4.0 * 8.0)
             table_bytes = 1 << (int(graph_bytes).bit_length() - 1)
-            ceiling = nd.measure_gather_rate(table_bytes)
+            # the probe in every shape (1, 2, 4, 8 reads in flight per lane; workgroups of 64 and
+            # 256 lanes): the ceiling is the best of them
+            ceiling, by_shape = nd.gather_rate_ceiling(table_bytes)
             flat_ms = prof["flat_kernel_ms"] / max(launches, 1)
-            writes = MEASURED_L2_WRITE_REQUESTS_PER_LAUNCH.get(args.workload, 0.0)
+            writes = MEASURED_L2_WRITE_REQUESTS_PER_LAUNCH.get(workload, 0.0)
             result["roofline"]["l2_miss_path"] = {
                 "read_requests_per_launch": misses, "bytes_per_read_request": 128,
                 "write_requests_per_launch": writes,
                 "achieved_read_requests_per_s": misses / (flat_ms / 1000.0),
                 "achieved_requests_per_s": (misses + writes) / (flat_ms / 1000.0),
                 "ceiling_requests_per_s": ceiling, "ceiling_table_bytes": table_bytes,
-                "ceiling_kind": "independent random 8-byte reads, measured in this run",
-                "frac_of_ceiling_reads_only": misses / (flat_ms / 1000.0) / ceiling,
-                "frac_of_ceiling": (misses + writes) / (flat_ms / 1000.0) / ceiling,
+                "ceiling_kind": "independent random 8-byte reads, the best of 8 probe shapes, measured in this run",
+                "ceiling_by_shape": {f"{k}_in_flight_{lanes}_lanes": round(v / 1e9, 2) for (k, lanes), v in by_shape.items()},
+                "frac_of_ceiling": misses / (flat_ms / 1000.0) / ceiling,
+                "frac_of_ceiling_note": "read requests over the read ceiling; the launch's write requests are "
+                                        "not priced (the probe does not write)",
+                "reads_and_writes_over_read_ceiling": (misses + writes) / (flat_ms / 1000.0) / ceiling,
                 "ceiling_as_GBps": ceiling * 128 / 1e9,
             }
     del final
     sampler.close()
+    return result
+
+
+HEADLINE = "weighted_node2vec_rmat22"
+FIVE_CONFIGS = ["uniform_walk_chunglu57k", "weighted_node2vec_rmat22", "khop_rmat21", "fastgcn_importance_rmat22",
+                "ladies_importance_chunglu3m"]
+
+
+def summary(r):
+    """The per-config entry of the result line."""
+    out = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
+           "value": r["value"], "unit": r["unit"], "valid_sampled_edges_per_s": r["config"]["valid_sampled_edges_per_s"],
+           "phases_ms": r["phases_ms"]}
+    for key in ("neighbourhood_entries_per_s", "distinct_ms", "kernel_classes", "load_balancing_schedule"):
+        if key in r["config"]:
+            out[key] = r["config"][key]
+    if "engine_chosen_inversion_period" in r["config"]:
+        e = r["config"]["engine_chosen_inversion_period"]
+        out["engine_chosen_inversion_period"] = {k: e[k] for k in ("ms_per_step", "sampled_edges_per_s", "same_samples")}
+    if "roofline" in r:
+        out["roofline"] = {k: r["roofline"][k] for k in ("kernel", "bound", "frac", "achieved", "avg_launch_ms",
+                                                         "algorithmic_bytes_per_launch", "traffic") if k in r["roofline"]}
+    if "cpu_baseline" in r:
+        out["cpu_baseline"] = {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind", "sample")}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--only", action="store_true",
+                    help="measure the workload given with --workload alone; by default the other benchmark "
+                         "configurations are measured as well (shorter runs) and reported under \"configs\"")
+    ap.add_argument("--no-load-balancing", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--inversion-period", type=int, default=1,
+                    help="walks: invert the sample->transit map before every p-th step (1: every step, as the "
+                         "reference; 0: the engine decides); the samples do not depend on it")
+    ap.add_argument("--skip-engine-choice", action="store_true",
+                    help="walks: do not also measure the pass with the engine-chosen inversion period")
+    ap.add_argument("--seed", type=int, default=42)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X; this build has no multi-GPU path (samples would shard "
+                 "by contiguous ranges with the graph replicated). Run with --gpus 1.")
+
+    graphs = {}
+    result = measure(args, args.workload, args.steps, args.warmup, args.cpu_seconds, graphs,
+                     engine_choice=not args.skip_engine_choice)
+    if not args.only and args.workload == HEADLINE:
+        # the other configurations: a few timed passes each and a short CPU baseline, so that the
+        # whole run stays within minutes; the configuration that shares the headline's graph first
+        configs = {args.workload: summary(result)}
+        order = ["fastgcn_importance_rmat22", "uniform_walk_chunglu57k", "khop_rmat21", "ladies_importance_chunglu3m"]
+        for name in order:
+            t0 = time.perf_counter()
+            r = measure(args, name, min(args.steps, 5), 1, min(args.cpu_seconds, 3.0), graphs,
+                        engine_choice=not args.skip_engine_choice)
+            configs[name] = summary(r)
+            configs[name]["bench_seconds"] = round(time.perf_counter() - t0, 1)
+        result["configs"] = [configs[name] for name in FIVE_CONFIGS]
     print(json.dumps(result))
 
 

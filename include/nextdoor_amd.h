@@ -247,6 +247,12 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
  * 32 GiB; allocated and freed inside): 4 M lanes, 16 reads each, two in flight per lane.  The
  * ceiling a gather-bound step kernel is priced against next to the HBM byte peak. */
 int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s);
+/* The same with the shape of the probe chosen: reads_in_flight (1, 2, 4 or 8) independent reads
+ * issued per lane before any is used, in workgroups of workgroup_lanes (64 or 256) lanes; 16
+ * reads per lane in all.  nd_measure_gather_rate is (2, 256).  The ceiling of the path is the
+ * largest rate over the shapes. */
+int nd_measure_gather_rate_shaped(int64_t table_bytes, int reads_in_flight, int workgroup_lanes,
+                                  double* requests_per_s);
 
 /* collectiveNeighbrsSize + collectiveNeighborhood (src/nextdoor.cu:1206-1283) for n_samples
  * samples of transits_per_sample transits each (transits[s * transits_per_sample + i]):

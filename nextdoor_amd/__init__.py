@@ -383,11 +383,18 @@ def sort_pairs_noalloc(d_keys, d_vals, n, key_bits, d_keys_out, d_vals_out, stre
     check(lib().nd_sort_pairs_noalloc(d_keys, d_vals or None, n, key_bits, d_keys_out, d_vals_out, stream or None))
 
 
-def measure_gather_rate(table_bytes):
-    """Independent random 8-byte reads per second over a table of ``table_bytes`` (power of two)."""
+def measure_gather_rate(table_bytes, reads_in_flight=2, workgroup_lanes=256):
+    """Independent random 8-byte reads per second over a table of ``table_bytes`` (power of two),
+    ``reads_in_flight`` (1, 2, 4, 8) issued per lane before any is used, workgroups of 64 or 256 lanes."""
     rate = C.c_double()
-    check(lib().nd_measure_gather_rate(int(table_bytes), C.byref(rate)))
+    check(lib().nd_measure_gather_rate_shaped(int(table_bytes), reads_in_flight, workgroup_lanes, C.byref(rate)))
     return rate.value
+
+
+def gather_rate_ceiling(table_bytes):
+    """The largest rate over the probe's shapes, and the rate of every shape: (best, {(k, lanes): rate})."""
+    rates = {(k, lanes): measure_gather_rate(table_bytes, k, lanes) for k in (1, 2, 4, 8) for lanes in (64, 256)}
+    return max(rates.values()), rates
 
 
 def unique_transits(sorted_keys, invalid):

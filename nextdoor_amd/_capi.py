@@ -76,6 +76,7 @@ SIGNATURES = {
     "nd_collective_neighborhood": (C.c_int, [C.c_void_p, c_i32p, C.c_int64, C.c_int32, C.c_int32, c_i32p, c_i32p, c_i32p,
                                              c_f32p, C.c_int64, c_i32p]),
     "nd_measure_gather_rate": (C.c_int, [C.c_int64, C.POINTER(C.c_double)]),
+    "nd_measure_gather_rate_shaped": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "nd_unique_transits": (C.c_int, [c_i32p, C.c_int64, C.c_int32, c_i32p, c_i32p, c_i32p, c_i64p, c_i64p]),
 }
 

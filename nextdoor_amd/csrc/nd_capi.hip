@@ -175,7 +175,7 @@ __device__ __forceinline__ uint32_t probe_mix(uint32_t x) {
 template <int kInFlight>
 __global__ __launch_bounds__(256) void gather_rate_kernel(const uint2* __restrict__ table, uint32_t mask,
                                                          uint32_t rounds, uint32_t* sink) {
-  const uint32_t lane = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t lane = blockIdx.x * blockDim.x + threadIdx.x;
   uint32_t acc = 0, at = probe_mix(lane * 2654435761u + 1u);
   for (uint32_t r = 0; r < rounds; ++r) {
     uint2 got[kInFlight];
@@ -729,12 +729,16 @@ int nd_load_balancing_thresholds(int32_t out[3]) {
 
 // ---- measurement: what the memory system gives independent random 8-byte reads --------------
 
-int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
+int nd_measure_gather_rate_shaped(int64_t table_bytes, int reads_in_flight, int workgroup_lanes,
+                                  double* requests_per_s) {
   return guarded([&]() -> int {
     if (!requests_per_s || table_bytes < 4096 || table_bytes > (1ll << 35) || (table_bytes & (table_bytes - 1)))
       return fail("table_bytes must be a power of two between 4 KiB and 32 GiB");
-    constexpr uint32_t kLanes = 1u << 22, kRounds = 8;
-    constexpr int kInFlight = 2;
+    if (reads_in_flight != 1 && reads_in_flight != 2 && reads_in_flight != 4 && reads_in_flight != 8)
+      return fail("reads_in_flight must be 1, 2, 4 or 8");
+    if (workgroup_lanes != 64 && workgroup_lanes != 256) return fail("workgroup_lanes must be 64 or 256");
+    constexpr uint32_t kLanes = 1u << 22;
+    const uint32_t rounds = 16u / (uint32_t)reads_in_flight < 2u ? 2u : 16u / (uint32_t)reads_in_flight;  // 16 reads per lane
     DeviceBuffer table, sink;
     CAPI_HIP(table.alloc((size_t)table_bytes));
     CAPI_HIP(sink.alloc(sizeof(uint32_t) * kLanes));
@@ -743,10 +747,16 @@ int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
     CAPI_HIP(hipEventCreate(&begin));
     hipError_t e = hipEventCreate(&end);
     float best_ms = 0.0f;
+    const dim3 grid(kLanes / (uint32_t)workgroup_lanes), block((uint32_t)workgroup_lanes);
+    const uint32_t mask = (uint32_t)(table_bytes / 8 - 1);
     for (int rep = 0; e == hipSuccess && rep < 3; ++rep) {  // the first launch warms the translation caches
       e = hipEventRecord(begin, nullptr);
-      gather_rate_kernel<kInFlight><<<dim3(kLanes / 256), dim3(256)>>>(table.as<uint2>(), (uint32_t)(table_bytes / 8 - 1),
-                                                                       kRounds, sink.as<uint32_t>());
+      switch (reads_in_flight) {
+        case 1: gather_rate_kernel<1><<<grid, block>>>(table.as<uint2>(), mask, rounds, sink.as<uint32_t>()); break;
+        case 2: gather_rate_kernel<2><<<grid, block>>>(table.as<uint2>(), mask, rounds, sink.as<uint32_t>()); break;
+        case 4: gather_rate_kernel<4><<<grid, block>>>(table.as<uint2>(), mask, rounds, sink.as<uint32_t>()); break;
+        default: gather_rate_kernel<8><<<grid, block>>>(table.as<uint2>(), mask, rounds, sink.as<uint32_t>()); break;
+      }
       if (e == hipSuccess) e = hipGetLastError();
       if (e == hipSuccess) e = hipEventRecord(end, nullptr);
       if (e == hipSuccess) e = hipEventSynchronize(end);
@@ -757,9 +767,13 @@ int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
     (void)hipEventDestroy(begin);
     if (end) (void)hipEventDestroy(end);
     CAPI_HIP(e);
-    *requests_per_s = (double)kLanes * kRounds * kInFlight / ((double)best_ms / 1000.0);
+    *requests_per_s = (double)kLanes * rounds * reads_in_flight / ((double)best_ms / 1000.0);
     return 0;
   });
+}
+
+int nd_measure_gather_rate(int64_t table_bytes, double* requests_per_s) {
+  return nd_measure_gather_rate_shaped(table_bytes, 2, 256, requests_per_s);
 }
 
 int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degrees, int32_t n_vertices, int step_size,
