@@ -204,6 +204,11 @@ void nd_free_device_memory(void);
  * states, src/rand_num_gen.cuh:117-122). */
 int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, int64_t n_slots,
                            int draws_per_slot, float* out);
+/* The same for a step of the given stepSize: steps that draw several outputs per transit
+ * (step_size > 1) use the grouped form of the stream, in which the first draw of four consecutive
+ * output slots comes from one Philox block (nd_philox.hpp); step_size 1 is nd_philox_fill_uniform. */
+int nd_philox_fill_step(uint64_t seed, uint32_t step, int step_size, uint64_t first_slot, int64_t n_slots,
+                        int draws_per_slot, float* out);
 /* cub::DeviceRadixSort::SortPairs as called at src/nextdoor.cu:2930-2933: stable sort of
  * (key, value) by the low key_bits bits.  vals == NULL: value = index. */
 int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_bits, int32_t* keys_out,

@@ -337,9 +337,11 @@ class SamplingModule:
 
 # ---- building blocks (device kernels behind host buffers) ---------------------------------
 
-def philox_fill_uniform(seed, step, first_slot, n_slots, draws_per_slot=1):
+def philox_fill_uniform(seed, step, first_slot, n_slots, draws_per_slot=1, step_size=1):
+    """The random numbers of a step as a buffer: draws_per_slot uniforms for each of n_slots output
+    slots from first_slot on.  step_size > 1: the grouped form of the stream such steps use."""
     out = np.empty(n_slots * draws_per_slot, dtype=np.float32)
-    check(lib().nd_philox_fill_uniform(seed, step, first_slot, n_slots, draws_per_slot, _ptr(out, C.c_float)))
+    check(lib().nd_philox_fill_step(seed, step, step_size, first_slot, n_slots, draws_per_slot, _ptr(out, C.c_float)))
     return out.reshape(n_slots, draws_per_slot)
 
 

@@ -68,6 +68,7 @@ SIGNATURES = {
     "nd_final_samples_array": (c_i32p, []),
     "nd_free_device_memory": (None, []),
     "nd_philox_fill_uniform": (C.c_int, [C.c_uint64, C.c_uint32, C.c_uint64, C.c_int64, C.c_int, c_f32p]),
+    "nd_philox_fill_step": (C.c_int, [C.c_uint64, C.c_uint32, C.c_int, C.c_uint64, C.c_int64, C.c_int, c_f32p]),
     "nd_sort_pairs": (C.c_int, [c_i32p, c_i32p, C.c_int64, C.c_int, c_i32p, c_i32p]),
     "nd_sort_pairs_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nd_load_balancing_thresholds": (C.c_int, [c_i32p]),

@@ -157,11 +157,12 @@ struct DeviceBuffer {
 };
 
 __global__ void philox_fill_kernel(uint64_t seed, uint32_t step, uint64_t first_slot, size_t n_slots,
-                                   int draws_per_slot, float* out) {
+                                   int draws_per_slot, int grouped, float* out) {
   const size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (slot >= n_slots) return;
   nd::RandState rng;
-  rng.reset(seed, first_slot + slot, step);
+  if (grouped) rng.reset_grouped(seed, first_slot + slot, step);
+  else rng.reset(seed, first_slot + slot, step);
   for (int d = 0; d < draws_per_slot; ++d) out[slot * draws_per_slot + d] = rng.next_uniform();
 }
 
@@ -638,7 +639,13 @@ const int32_t* nd_final_samples_array(void) {
 
 int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, int64_t n_slots, int draws_per_slot,
                            float* out) {
+  return nd_philox_fill_step(seed, step, 1, first_slot, n_slots, draws_per_slot, out);
+}
+
+int nd_philox_fill_step(uint64_t seed, uint32_t step, int step_size, uint64_t first_slot, int64_t n_slots,
+                        int draws_per_slot, float* out) {
   return guarded([&]() -> int {
+    if (step_size < 1) return fail("bad argument");
     if (n_slots < 0 || draws_per_slot < 1 || (n_slots > 0 && !out)) return fail("bad argument");
     if (n_slots == 0) return 0;
     DeviceBuffer d;
@@ -646,7 +653,7 @@ int nd_philox_fill_uniform(uint64_t seed, uint32_t step, uint64_t first_slot, in
     CAPI_HIP(d.alloc(bytes));
     philox_fill_kernel<<<dim3((unsigned)((n_slots + 255) / 256)), dim3(256), 0, 0>>>(seed, step, first_slot,
                                                                                     (size_t)n_slots, draws_per_slot,
-                                                                                    d.as<float>());
+                                                                                    step_size > 1 ? 1 : 0, d.as<float>());
     CAPI_HIP(hipGetLastError());
     CAPI_HIP(hipMemcpy(out, d.p, bytes, hipMemcpyDeviceToHost));
     return 0;
@@ -802,7 +809,7 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
     CAPI_HIP(d_n.alloc(sizeof(uint32_t)));
     CAPI_HIP(d_meta.alloc(sizeof(nd::RunsMeta) * 2));
     CAPI_HIP(d_rows.alloc(sizeof(EdgePos_t) * row_ptr.size()));
-    CAPI_HIP(d_items.alloc(sizeof(uint32_t) * 2 * (size_t)capacity));
+    CAPI_HIP(d_items.alloc(sizeof(nd::WorkItem) * (size_t)capacity));
     CAPI_HIP(d_taken.alloc(sizeof(uint32_t) * (size_t)n_vertices));
     constexpr size_t kCounterBytes = sizeof(nd::ClassCounters) * nd::kCounterCopies;
     CAPI_HIP(d_balance.alloc(sizeof(uint32_t) * kFoundWords + kCounterBytes));
@@ -820,12 +827,12 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
     if (pairs_per_lane == 1) {
       nd::classify_run_tails<1><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, 0>>>(
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
-          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
+          d_items.as<nd::WorkItem>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     } else {
       const int64_t per_block = 256 * nd::kClassifyItemsLarge;
       nd::classify_run_tails<nd::kClassifyItemsLarge><<<dim3((unsigned)((n + per_block - 1) / per_block)), dim3(256), 0, 0>>>(
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
-          d_items.as<uint32_t>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
+          d_items.as<nd::WorkItem>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     }
     CAPI_HIP(hipGetLastError());
     CAPI_HIP(hipDeviceSynchronize());
@@ -843,7 +850,16 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
     // the kernel counts every item it wants; those beyond the capacity were not written
     *n_items = h.n_chunks;
     const int64_t written = h.n_chunks < capacity ? (int64_t)h.n_chunks : capacity;
-    CAPI_HIP(hipMemcpy(items, d_items.p, sizeof(uint32_t) * 2 * (size_t)written, hipMemcpyDeviceToHost));
+    std::vector<nd::WorkItem> records((size_t)written);
+    CAPI_HIP(hipMemcpy(records.data(), d_items.p, sizeof(nd::WorkItem) * (size_t)written, hipMemcpyDeviceToHost));
+    for (int64_t i = 0; i < written; ++i) {
+      const nd::WorkItem& r = records[(size_t)i];
+      // what the item says of its transit is what the caller's arrays say
+      if (r.transit != sorted_keys[r.first_pair] || r.begin != row_ptr[(size_t)r.transit] || r.n_edges != degrees[r.transit])
+        return fail("internal error: a work item does not describe its transit");
+      items[2 * i] = (int32_t)r.first_pair;
+      items[2 * i + 1] = (int32_t)r.n_pairs;
+    }
     std::vector<uint32_t> stamps((size_t)n_vertices);
     CAPI_HIP(hipMemcpy(stamps.data(), d_taken.p, sizeof(uint32_t) * stamps.size(), hipMemcpyDeviceToHost));
     for (int32_t v = 0; v < n_vertices; ++v) taken[v] = stamps[(size_t)v] == fresh[0].stamp ? 1 : 0;

@@ -191,6 +191,9 @@ struct StepParams {
   int step;
   uint32_t step_size;            // m_k
   uint32_t lanes_shift;          // flat kernel: 2^lanes_shift lanes share the outputs of a pair
+  uint32_t groups_per_pair;      // step_size > 1: the groups of four consecutive output slots (one
+                                 // Philox block each for the first draw, nd_philox.hpp) the outputs
+                                 // of a pair can touch at most; a lane works through whole groups
   uint32_t transits_per_sample;  // T_k
   uint32_t seg_base;             // offset of this step's segment inside a final sample
   uint32_t final_size;           // F
@@ -273,11 +276,14 @@ constexpr uint32_t kChunkOutputs = ND_CHUNK_OUTPUTS;
 // next() for one output and, for apps with explicit transits, stepTransits() for the step
 // after it (nextdoor.cu:279-289: the random state is the one next() used).  Returns the
 // sampled vertex; *next_transit is the transit the pair has at the next step.
+// grouped: the step draws several outputs per transit, and first_word is the output's word of
+// its group's shared block (the grouped form of the stream, nd_philox.hpp).
 template <class SampleType, class App, class EdgeArray, class WeightArray>
 __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t sample,
                                             uint32_t transit_index, uint64_t out_slot, uint32_t nbr,
                                             EdgePos_t n_edges, float max_weight, EdgeArray& edges,
-                                            WeightArray& weights, SampleType* state, VertexID* next_transit) {
+                                            WeightArray& weights, SampleType* state, VertexID* next_transit,
+                                            bool grouped, uint32_t first_word) {
   const VertexID sample_id = (VertexID)(P.first_sample + sample);
   const bool runs = transit != P.invalid && n_edges != 0;  // next() only runs for a real transit
                                                            // that has edges (nextdoor.cu:250-262)
@@ -285,7 +291,10 @@ __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& c
   curandState rng;
   // a pair whose transit is no vertex is dead, with or without explicit transits
   const bool chooses_transit = explicit_transits && !P.is_last && transit != P.invalid;
-  if (runs || chooses_transit) rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  if (runs || chooses_transit) {
+    if (grouped) rng.reset_with_first(P.seed, P.first_slot + out_slot, (uint32_t)P.step, first_word);
+    else rng.reset(P.seed, P.first_slot + out_slot, (uint32_t)P.step);
+  }
   VertexID neighbor = P.invalid;
   if (runs) {
     const VertexID r = App().template next<SampleType, EdgeArray, WeightArray>(
@@ -323,12 +332,13 @@ __device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t 
 
 // pair: index of the pair in the order the step kernels walk them (sorted by transit, or
 // the raw map at step 0).
+// First half: next() (and stepTransits) for the output; nothing of the step's results is stored.
 template <class SampleType, class App, class EdgeArray, class WeightArray>
-__device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
-                                               uint32_t pair_slot, uint32_t nbr, EdgePos_t n_edges, float max_weight,
-                                               EdgeArray& edges, WeightArray& weights) {
+__device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
+                                               uint32_t pair_slot, uint32_t sample, uint32_t nbr, EdgePos_t n_edges,
+                                               float max_weight, EdgeArray& edges, WeightArray& weights, bool grouped,
+                                               uint32_t first_word, VertexID* neighbor_out, VertexID* next_transit_out) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
-  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
   const uint32_t transit_index = pair_slot - sample * P.transits_per_sample;
   VertexID neighbor = P.invalid, next_transit = P.invalid;
   bool travelled = false;
@@ -339,7 +349,7 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
       uint32_t bits = P.pair_state ? P.pair_state[pair] : ((const uint32_t*)P.samples)[sample];
       __builtin_memcpy(&state, &bits, sizeof(uint32_t));
       neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                          edges, weights, &state, &next_transit);
+                                          edges, weights, &state, &next_transit, grouped, first_word);
       __builtin_memcpy(&bits, &state, sizeof(uint32_t));
       if (P.emit_state) P.emit_state[pair] = bits;
       // a walk that ends here leaves the stream of pairs: its state goes home
@@ -351,12 +361,22 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
     if constexpr (std::is_empty<SampleType>::value) {
       SampleType no_state;
       neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                          edges, weights, &no_state, &next_transit);
+                                          edges, weights, &no_state, &next_transit, grouped, first_word);
     } else {
       neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
-                                          edges, weights, (SampleType*)P.samples + sample, &next_transit);
+                                          edges, weights, (SampleType*)P.samples + sample, &next_transit, grouped,
+                                          first_word);
     }
   }
+  *neighbor_out = neighbor;
+  *next_transit_out = next_transit;
+}
+
+// Second half: the output goes to its place in the step's results, and what the next step
+// needs of it to the next step's map.
+__device__ __forceinline__ void store_output(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
+                                             uint32_t sample, uint32_t nbr, VertexID neighbor, VertexID next_transit) {
+  const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   if (P.pair_cells) {
     store_walk_result(P, sample, transit, neighbor);
   } else {
@@ -373,6 +393,54 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
       P.emit_ranks[pair] = atomicAdd(&P.emit_counts[first + (pair & (copies - 1u))], 1u);
     }
   }
+}
+
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
+                                               uint32_t pair_slot, uint32_t nbr, EdgePos_t n_edges, float max_weight,
+                                               EdgeArray& edges, WeightArray& weights) {
+  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
+  VertexID neighbor, next_transit;
+  compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, sample, nbr, n_edges,
+                                                          max_weight, edges, weights, false, 0u, &neighbor,
+                                                          &next_transit);
+  store_output(P, transit, pair, pair_slot, sample, nbr, neighbor, next_transit);
+}
+
+// The outputs of a pair that fall into group `gi` of the pair's groups of four consecutive
+// (global) output slots: one shared Philox block, then up to four outputs.  For steps with
+// step_size > 1.
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ void produce_group(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
+                                              uint32_t pair_slot, uint32_t gi, EdgePos_t n_edges, float max_weight,
+                                              EdgeArray& edges, WeightArray& weights) {
+  const uint64_t first = P.first_slot + (uint64_t)pair_slot * P.step_size;  // global slot of the pair's output 0
+  const uint64_t group = (first >> 2) + gi;
+  const uint64_t lo = group * 4 > first ? group * 4 : first;
+  const uint64_t end = first + P.step_size;
+  const uint64_t hi = group * 4 + 4 < end ? group * 4 + 4 : end;
+  if (lo >= hi) return;
+  PhiloxBlock block = PhiloxBlock();
+  // next() draws for a real transit with edges; stepTransits for any real transit (run_app)
+  if (transit != P.invalid && (n_edges != 0 || (App().hasExplicitTransits() && !P.is_last)))
+    block = grouped_first_block(P.seed, group, (uint32_t)P.step);
+  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
+  // all draws first, then all stores: the up to four gathers of the group are under way
+  // together instead of each waiting behind the store of the one before
+  VertexID neighbor[4], next_transit[4];
+#pragma unroll
+  for (uint32_t q = 0; q < 4; ++q) {
+    neighbor[q] = next_transit[q] = P.invalid;
+    if (lo + q < hi)
+      compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, sample,
+                                                              (uint32_t)(lo + q - first), n_edges, max_weight, edges,
+                                                              weights, true, block_word(block, (uint32_t)(lo + q) & 3u),
+                                                              &neighbor[q], &next_transit[q]);
+  }
+#pragma unroll
+  for (uint32_t q = 0; q < 4; ++q)
+    if (lo + q < hi)
+      store_output(P, transit, pair, pair_slot, sample, (uint32_t)(lo + q - first), neighbor[q], next_transit[q]);
 }
 
 // inversion_period == 0: walks are inverted before every step when there are at least this
@@ -437,18 +505,29 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
     max_weight = csr.max_weights[transit];
     if (taken_stamp && mark == stamp) return;
   }
+  // one output (walks), or the pair's groups of four output slots first_nbr, first_nbr + stride, ...
   if (app_uses_weights<App>::value) {
     PairedEdgeIds edges{P.paired_edges + begin};
     PairedEdgeWeights weights{P.paired_edges + begin};
-    for (uint32_t nbr = first_nbr; nbr < P.step_size; nbr += nbr_stride)
-      produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, nbr, n_edges,
+    if (kSingleOutput) {
+      produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, 0, n_edges,
                                                                         max_weight, edges, weights);
+    } else {
+      for (uint32_t gi = first_nbr; gi < P.groups_per_pair; gi += nbr_stride)
+        produce_group<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, gi, n_edges,
+                                                                         max_weight, edges, weights);
+    }
   } else {
     const CSR::Edge* edges = csr.edges + begin;
     const float* weights = csr.weights + begin;
-    for (uint32_t nbr = first_nbr; nbr < P.step_size; nbr += nbr_stride)
-      produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, nbr, n_edges,
+    if (kSingleOutput) {
+      produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, 0, n_edges,
                                                                      max_weight, edges, weights);
+    } else {
+      for (uint32_t gi = first_nbr; gi < P.groups_per_pair; gi += nbr_stride)
+        produce_group<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, gi, n_edges,
+                                                                      max_weight, edges, weights);
+    }
   }
 }
 
@@ -538,24 +617,48 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
   }
 }
 
+// A work item of the workgroup class: a stretch of pairs on one transit, with what the
+// classification knew of the transit, so that the workgroup that takes the item goes from this
+// one record straight to the adjacency (one 32-byte fetch instead of a chain of three
+// dependent ones: item, transit of its first pair, row extent).
+struct alignas(16) WorkItem {
+  uint32_t first_pair, n_pairs;
+  int32_t transit;
+  EdgePos_t begin, n_edges;  // the transit's row extent
+  uint32_t unused[3];
+};
+
 // One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
 // transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
 // with coalesced reads and every draw of the stretch gathers from LDS.  The workgroup takes
 // the items first_item, first_item + item_stride, ...
 template <class SampleType, class App>
-__device__ __forceinline__ void workgroup_items(StepParams& P, const uint32_t* __restrict__ chunks, uint32_t n_chunks,
+__device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* __restrict__ chunks, uint32_t n_chunks,
                                                 uint32_t first_item, uint32_t item_stride, CSR::Edge* s_edges,
                                                 float* s_weights) {
   constexpr bool kWeights = app_uses_weights<App>::value;
   CSRPartition csr = P.csr;
+  WorkItem item = WorkItem();
+  if (first_item < n_chunks) item = chunks[first_item];
   for (uint32_t c = first_item; c < n_chunks; c += item_stride) {
-    const uint32_t first_pair = chunks[2 * c];
-    const uint32_t n_pairs = chunks[2 * c + 1];
-    const VertexID transit = (VertexID)P.pair_keys[first_pair];
-    const EdgePos_t begin = csr.row_ptr[transit];
-    const EdgePos_t n_edges = csr.row_ptr[transit + 1] - begin;
-    const float max_weight = csr.max_weights[transit];
+    // the record of the item after this one is fetched while this one is worked on
+    WorkItem coming = item;
+    if (c + item_stride < n_chunks) coming = chunks[c + item_stride];
+    const uint32_t first_pair = item.first_pair;
+    const uint32_t n_pairs = item.n_pairs;
+    const VertexID transit = (VertexID)item.transit;
+    const EdgePos_t begin = item.begin;
+    const EdgePos_t n_edges = item.n_edges;
+    const float max_weight = csr.max_weights[transit];  // every next() is handed it, hint or no hint
     const EdgePos_t cached = n_edges < kCacheEdges ? n_edges : kCacheEdges;
+    // Lanes per pair: one, or the power of two (at most the groups of four output slots a pair
+    // has) that the item's pairs leave room for in the workgroup; lane `sub` of a pair takes the
+    // pair's groups sub, sub + L, ...  The slot of a lane's first pair is fetched together with
+    // the adjacency, not after it.
+    uint32_t lanes_shift = 0;
+    while ((1u << lanes_shift) < P.groups_per_pair && (n_pairs << (lanes_shift + 1)) <= (uint32_t)kStepThreads) lanes_shift++;
+    const uint32_t lanes = n_pairs << lanes_shift;
+    uint32_t slot = threadIdx.x < lanes ? P.pair_slots[first_pair + (threadIdx.x >> lanes_shift)] : 0u;
     __syncthreads();  // the previous work item is done with the cache
     for (EdgePos_t e = threadIdx.x; e < cached; e += kStepThreads) {
       s_edges[e] = csr.edges[begin + e];
@@ -564,20 +667,25 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const uint32_t* _
     __syncthreads();
     LdsBackedArray<CSR::Edge> edges{s_edges, csr.edges + begin, cached};
     LdsBackedArray<float> lds_weights{s_weights, csr.weights + begin, kWeights ? cached : 0};
-    const uint32_t outputs = n_pairs * P.step_size;
-    for (uint32_t o = threadIdx.x; o < outputs; o += kStepThreads) {
-      const uint32_t p = P.step_size == 1 ? o : o / P.step_size;
-      const uint32_t nbr = o - p * P.step_size;
-      const uint32_t slot = P.pair_slots[first_pair + p];
-      produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
-          P, csr, transit, first_pair + p, slot, nbr, n_edges, max_weight, edges, lds_weights);
+    for (uint32_t t = threadIdx.x; t < lanes; t += kStepThreads) {
+      const uint32_t p = t >> lanes_shift;
+      if (t != threadIdx.x) slot = P.pair_slots[first_pair + p];
+      if (P.groups_per_pair == 0) {  // one output per pair
+        produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
+            P, csr, transit, first_pair + p, slot, 0, n_edges, max_weight, edges, lds_weights);
+      } else {
+        for (uint32_t gi = t & ((1u << lanes_shift) - 1u); gi < P.groups_per_pair; gi += 1u << lanes_shift)
+          produce_group<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
+              P, csr, transit, first_pair + p, slot, gi, n_edges, max_weight, edges, lds_weights);
+      }
     }
+    item = coming;
   }
 }
 
 template <class SampleType, class App>
 __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams P,
-                                                                      const uint32_t* __restrict__ chunks,
+                                                                      const WorkItem* __restrict__ chunks,
                                                                       const RunsMeta* __restrict__ meta,
                                                                       uint32_t chunk_capacity) {
   __shared__ CSR::Edge s_edges[kCacheEdges];
@@ -601,7 +709,7 @@ template <class SampleType, class App, bool kSingleOutput>
 __global__ __launch_bounds__(kStepThreads) void step_balanced_kernel(StepParams P,
                                                                      const uint32_t* __restrict__ taken_stamp,
                                                                      const RunsMeta* __restrict__ meta,
-                                                                     const uint32_t* __restrict__ chunks,
+                                                                     const WorkItem* __restrict__ chunks,
                                                                      uint32_t chunk_capacity, uint32_t wg_per_group) {
   __shared__ CSR::Edge s_edges[kCacheEdges];
   __shared__ float s_weights[app_uses_weights<App>::value ? kCacheEdges : 1];
@@ -685,7 +793,8 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
                                                       const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
                                                       uint32_t* transit_out, uint32_t* start_out,
                                                       uint32_t* count_out, uint32_t* n_items_out,
-                                                      uint32_t* refused_out = nullptr) {
+                                                      uint32_t* refused_out = nullptr, EdgePos_t* begin_out = nullptr,
+                                                      EdgePos_t* degree_out = nullptr) {
   const uint32_t transit = keys[i];
   if (i + 1 != n && keys[i + 1] == transit) return false;  // not the last pair of its run
   // pairs a run needs for the workgroup kernel; a shorter run is ruled out with one read
@@ -695,12 +804,15 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
   const uint32_t count = i + 1 - start;
   const uint64_t work = (uint64_t)count * step_size;
   if (work < kWorkgroupWork) return false;
-  const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
+  const EdgePos_t begin = row_ptr[transit];
+  const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - begin);
   if (degree == 0) return false;
   if (degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) {
     if (refused_out) *refused_out = count;
     return false;
   }
+  if (begin_out) *begin_out = begin;
+  if (degree_out) *degree_out = (EdgePos_t)degree;
   uint32_t pairs_per_chunk = kChunkOutputs / step_size;
   if (pairs_per_chunk == 0) pairs_per_chunk = 1;
   *transit_out = transit;
@@ -729,7 +841,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
                                                           const uint32_t* __restrict__ n_dev, RunsMeta* meta,
                                                           RunsMeta* meta_of_next_step,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
-                                                          uint32_t* __restrict__ chunks, uint32_t chunk_capacity,
+                                                          WorkItem* __restrict__ chunks, uint32_t chunk_capacity,
                                                           uint32_t* __restrict__ taken_stamp,
                                                           ClassCounters* __restrict__ counters,
                                                           uint32_t* __restrict__ found_by_step, uint32_t step) {
@@ -748,13 +860,14 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&counters->sorted_pairs, (unsigned long long)n);
   const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
   uint32_t transit, start, count, n_items;
+  EdgePos_t begin = 0, degree = 0;
   uint32_t mine = 0;
   uint32_t single_pairs = 0, split_pairs = 0, refused_pairs = 0;
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
     uint32_t refused = 0;
     if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items,
-                                       &refused)) {
+                                       &refused, &begin, &degree)) {
       mine += n_items;
       if (n_items > 1) split_pairs += count; else single_pairs += count;
     }
@@ -801,13 +914,19 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
     const uint64_t i = first + k;
     // one pair per lane: the run found above is still in the registers
     if (kClassifyItems > 1 &&
-        !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items)))
+        !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items,
+                                         nullptr, &begin, &degree)))
       continue;
     const bool fits = base + n_items <= chunk_capacity;
     for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
       const uint32_t off = g * pairs_per_chunk;
-      chunks[2 * (base + g)] = start + off;
-      chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+      WorkItem item = WorkItem();
+      item.first_pair = start + off;
+      item.n_pairs = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+      item.transit = (int32_t)transit;
+      item.begin = begin;
+      item.n_edges = degree;
+      chunks[base + g] = item;
     }
     if (fits) {
       taken_stamp[transit] = stamp;
@@ -869,7 +988,7 @@ __global__ __launch_bounds__(256) void small_map_place(
     uint32_t* __restrict__ state_out,
     // load balancing (classify == 0: none of it)
     uint32_t classify, RunsMeta* meta, RunsMeta* meta_of_next_step, const EdgePos_t* __restrict__ row_ptr,
-    uint32_t step_size, uint32_t* __restrict__ chunks, uint32_t chunk_capacity, uint32_t* __restrict__ taken_stamp,
+    uint32_t step_size, WorkItem* __restrict__ chunks, uint32_t chunk_capacity, uint32_t* __restrict__ taken_stamp,
     ClassCounters* __restrict__ counters) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t chunk_base[1024];
@@ -923,9 +1042,12 @@ __global__ __launch_bounds__(256) void small_map_place(
   }
   if (!classify) return;
   // the run's class, decided by its first pair (rules of workgroup_run_ends_at)
+  EdgePos_t begin = 0;
+  uint32_t degree = 0;
   if (head) {
     const uint64_t work = (uint64_t)count * step_size;
-    const uint32_t degree = (uint32_t)(row_ptr[transit + 1] - row_ptr[transit]);
+    begin = row_ptr[transit];
+    degree = (uint32_t)(row_ptr[transit + 1] - begin);
     if (work >= kWorkgroupWork && degree != 0) {
       if (degree > (uint32_t)kCacheEdges || (uint64_t)degree > 32ull * work) {
         refused = count;
@@ -960,8 +1082,13 @@ __global__ __launch_bounds__(256) void small_map_place(
   if (pairs_per_chunk == 0) pairs_per_chunk = 1;
   for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
     const uint32_t off = g * pairs_per_chunk;
-    chunks[2 * (base + g)] = start + off;
-    chunks[2 * (base + g) + 1] = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+    WorkItem item = WorkItem();
+    item.first_pair = start + off;
+    item.n_pairs = count - off < pairs_per_chunk ? count - off : pairs_per_chunk;
+    item.transit = (int32_t)transit;
+    item.begin = begin;
+    item.n_edges = (EdgePos_t)degree;
+    chunks[base + g] = item;
   }
   if (base + n_items <= chunk_capacity) taken_stamp[transit] = meta->stamp;
 }
@@ -1328,7 +1455,7 @@ class Engine : public EngineBase {
     markers_cleared_at_ = 0;
     schedule_counts_ = ScheduleCounts();
     items_seen_ = false;
-    ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(uint32_t) * 2 * (size_t)chunk_capacity_));
+    ND_HIP_TRY(hipMalloc(&d_chunks_, sizeof(WorkItem) * (size_t)chunk_capacity_));
     ND_HIP_TRY(hipMalloc(&d_taken_stamp_, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
     ND_HIP_TRY(hipMemset(d_taken_stamp_, 0, sizeof(uint32_t) * ((size_t)invalid_ + 1)));
     ND_HIP_TRY(hipStreamCreate(&side_stream_));
@@ -1509,8 +1636,17 @@ class Engine : public EngineBase {
       uint32_t* live_now = d_live_ + (sorts_done & 1);  // pairs the inversion of this step keeps
       // lanes of the flat kernel per pair: one when the pairs alone fill the machine, else
       // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
+      // groups of four consecutive output slots a pair's outputs can touch: the pair's first
+      // slot is a multiple of m, so its place in its group is one of (i * m) % 4
+      P.groups_per_pair = 0;
+      if (m > 1)
+        for (uint32_t i = 0; i < 4; ++i) {
+          const uint32_t groups = ((i * m) % 4 + m - 1) / 4 + 1;
+          if (groups > P.groups_per_pair) P.groups_per_pair = groups;
+        }
       P.lanes_shift = 0;
-      while ((1u << P.lanes_shift) < m && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted) P.lanes_shift++;
+      while ((1u << P.lanes_shift) < P.groups_per_pair && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted)
+        P.lanes_shift++;
       const uint64_t flat_lanes = (uint64_t)n_pairs << P.lanes_shift;
 
       if (step == 0) {
@@ -2019,7 +2155,7 @@ class Engine : public EngineBase {
   };
   std::vector<RecordedPass> recorded_;
   uint64_t balanced_steps_ = 0;        // ... counted over the life of the buffers, so the parity never repeats
-  uint32_t* d_chunks_ = nullptr;
+  WorkItem* d_chunks_ = nullptr;
   uint32_t* d_taken_stamp_ = nullptr;  // per vertex: the stamp of the last step whose work items covered it
   uint64_t markers_cleared_at_ = 0;    // balanced_steps_ when the markers were last wiped
   struct ScheduleCounts {

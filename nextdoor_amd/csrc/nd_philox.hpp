@@ -12,6 +12,16 @@
 //
 // `slot` is the global index of the output being produced at `step`:
 // ((sample * transitsPerSample + transitIdx) * stepSize + neighbourIdx).
+//
+// Steps that draw several outputs per transit (stepSize > 1: k-hop) use the GROUPED form of the
+// stream: four consecutive output slots share one block for their first draw,
+//   draw 0 of (slot, step)      = word (slot & 3) of block(slot >> 2, step | 2^31, 0)
+//   draw d >= 1 of (slot, step) = draw d - 1 of the slot's own stream above,
+// because such a step takes one draw per output (a uniform pick) and would otherwise spend a
+// whole ten-round block on one word of it: the lane that produces the outputs of a transit
+// computes one block per four of them.  (The multiplications of Philox are what a k-hop step
+// waits for: 40 quarter-rate 32-bit multiplies per block.)  Walk steps (stepSize 1) draw several
+// numbers per output and keep the plain form.
 #pragma once
 
 #include <stdint.h>
@@ -61,11 +71,26 @@ ND_HD float u32_to_unit_float(uint32_t word) {
   return (float)(word >> 8) * 5.9604644775390625e-08f;  // 2^-24, exact
 }
 
+constexpr uint32_t kGroupedStepFlag = 0x80000000u;
+
+// The block the slots 4 * group .. 4 * group + 3 share for their first draw at a grouped step.
+ND_HD PhiloxBlock grouped_first_block(uint64_t seed, uint64_t group, uint32_t step) {
+  return philox4x32_10((uint32_t)group, (uint32_t)(group >> 32), step | kGroupedStepFlag, 0u, (uint32_t)seed,
+                       (uint32_t)(seed >> 32));
+}
+
+// Word i (0..3) of a block, by comparisons: an index into the array would put it in memory.
+ND_HD uint32_t block_word(const PhiloxBlock& b, uint32_t i) {
+  return i == 0 ? b.w[0] : i == 1 ? b.w[1] : i == 2 ? b.w[2] : b.w[3];
+}
+
 // Cursor over the draws of one (slot, step).  This is the object an App's next()
 // receives as its random-state handle.
 struct RandState {
-  uint32_t slot_lo, slot_hi, step, draw;
+  uint32_t slot_lo, slot_hi, step, draw;  // draw: draws taken from the slot's own stream
   uint32_t key0, key1;
+  uint32_t first_word;  // grouped form: the word of the shared block, until it is drawn
+  uint32_t has_first;
   // The words of the current Philox block that have not been drawn yet, next one first.  A
   // draw takes word0 and moves the others up: no word is ever picked by an index, so the state
   // stays in registers (an array indexed by the draw number, or selects among its members,
@@ -80,9 +105,27 @@ struct RandState {
     key0 = (uint32_t)seed;
     key1 = (uint32_t)(seed >> 32);
     word0 = word1 = word2 = word3 = 0;
+    first_word = 0;
+    has_first = 0;
+  }
+
+  // Grouped form, the first draw given: the caller holds the shared block of the slot's group.
+  ND_HD void reset_with_first(uint64_t seed, uint64_t slot, uint32_t step_, uint32_t first) {
+    reset(seed, slot, step_);
+    first_word = first;
+    has_first = 1;
+  }
+
+  // Grouped form, computing the shared block here (host loops, one-off uses).
+  ND_HD void reset_grouped(uint64_t seed, uint64_t slot, uint32_t step_) {
+    reset_with_first(seed, slot, step_, block_word(grouped_first_block(seed, slot >> 2, step_), (uint32_t)slot & 3u));
   }
 
   ND_HD uint32_t next_word() {
+    if (has_first) {
+      has_first = 0;
+      return first_word;
+    }
     if ((draw & 3u) == 0) {
       const PhiloxBlock b = philox4x32_10(slot_lo, slot_hi, step, draw >> 2, key0, key1);
       word0 = b.w[0];
@@ -106,6 +149,12 @@ ND_HD float uniform_at(uint64_t seed, uint64_t slot, uint32_t step, uint32_t dra
   PhiloxBlock b = philox4x32_10((uint32_t)slot, (uint32_t)(slot >> 32), step, draw >> 2,
                                 (uint32_t)seed, (uint32_t)(seed >> 32));
   return u32_to_unit_float(b.w[draw & 3u]);
+}
+
+// Draw `draw` of the grouped form.
+ND_HD float grouped_uniform_at(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw) {
+  if (draw == 0) return u32_to_unit_float(block_word(grouped_first_block(seed, slot >> 2, step), (uint32_t)slot & 3u));
+  return uniform_at(seed, slot, step, draw - 1);
 }
 
 // min((int)(u * n), n - 1): the reference's RandNumGen::rand_int

@@ -50,15 +50,23 @@ int32_t ndo_rand_int(float u, int32_t n) {
   return id < n - 1 ? id : n - 1;
 }
 
+float ndo_uniform_grouped(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw) {
+  /* steps with stepSize > 1: the first draw of four consecutive slots comes from one block */
+  if (draw == 0) return ndo_uniform(seed, slot >> 2, step | 0x80000000u, (uint32_t)(slot & 3u));
+  return ndo_uniform(seed, slot, step, draw - 1);
+}
+
 /* A cursor over the draws of one (slot, step): what the device RandState is. */
 typedef struct {
   uint64_t seed, slot;
   uint32_t step, draw;
   ndo_stats* st;
+  int grouped;  /* the step's stepSize is > 1 */
 } rng_cursor;
 
 static float next_uniform(rng_cursor* c) {
-  float u = ndo_uniform(c->seed, c->slot, c->step, c->draw);
+  float u = c->grouped ? ndo_uniform_grouped(c->seed, c->slot, c->step, c->draw)
+                       : ndo_uniform(c->seed, c->slot, c->step, c->draw);
   c->draw++;
   if (c->st) c->st->draws++;
   return u;
@@ -292,6 +300,7 @@ int ndo_sample_individual(const ndo_graph* g, const ndo_app_desc* app, uint64_t 
             rc.step = (uint32_t)k;
             rc.draw = 0;
             rc.st = st;
+            rc.grouped = m > 1;
             int32_t r = next_individual(g, app, k, transit, &t_state, &rc);
             neighbor = (r == -1) ? invalid : r;  /* nextdoor.cu:288 */
           }
@@ -348,6 +357,7 @@ int ndo_sample_multirw(const ndo_graph* g, uint64_t seed, int64_t n_samples, int
       rc.step = (uint32_t)k;
       rc.draw = 0;
       rc.st = 0;
+      rc.grouped = 0;
       int32_t neighbor = invalid;
       if (transit != invalid && degree_of(g, transit) != 0) {
         const int32_t n = degree_of(g, transit);
@@ -406,6 +416,7 @@ int ndo_sample_anchor_hop(const ndo_graph* g, uint64_t seed, int64_t n_samples, 
             rc.step = (uint32_t)k;
             rc.draw = 0;
             rc.st = 0;
+            rc.grouped = m > 1;
             const int32_t n = degree_of(g, transit);
             if (n != 0) neighbor = g->col[g->row_ptr[transit] + next_int(&rc, n)];  /* nextdoor.cu:250-262, khop.cu:18-22 */
             if (k != steps - 1) {
@@ -669,7 +680,7 @@ int ndo_sample_layer_literal(const ndo_graph* g, const ndo_app_desc* app, uint64
         if (transits[0] != invalid && transits[0] != -1) {
           rng_cursor rc;
           rc.seed = seed; rc.slot = (uint64_t)((first_sample + s) * m + nbr); rc.step = (uint32_t)k;
-          rc.draw = 0; rc.st = 0;
+          rc.draw = 0; rc.st = 0; rc.grouped = 0;
           const int32_t id = next_int(&rc, g->n_vertices);
           for (int i = 0; i < B; ++i) {
             const int has = ndo_has_edge(g, transits[i], id);

@@ -80,6 +80,12 @@ void ndo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
  * (slot_lo, slot_hi, step, draw >> 2) and key (seed_lo, seed_hi), mapped to [0,1) as
  * (word >> 8) * 2^-24.  pinned by KAT + range/closed-form tests. */
 float ndo_uniform(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw);
+/* The form of the stream at steps whose stepSize is > 1 (one draw per output, a uniform pick):
+ * draw 0 of four consecutive slots comes from one block,
+ *   draw 0 = ndo_uniform(seed, slot >> 2, step | 2^31, slot & 3),  draw d >= 1 = ndo_uniform(seed, slot, step, d - 1).
+ * The engine's definition (nd_philox.hpp), like the plain form; the block function under both is
+ * pinned by the Random123 vectors. */
+float ndo_uniform_grouped(uint64_t seed, uint64_t slot, uint32_t step, uint32_t draw);
 
 /* RandNumGen::rand_int (rand_num_gen.cuh:117-122): min((int)(u*n), n-1) in float.
  * pinned by closed-form cases incl. the u*n == n rounding case. */

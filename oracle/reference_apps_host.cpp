@@ -66,7 +66,9 @@ int sample_individual(HostGraph& g, uint64_t seed, int64_t n_samples, const int3
           // next() only runs for a real transit that has edges (src/nextdoor.cu:250-262)
           if (transit != invalid && transit != -1 && g.view.get_n_edges_for_vertex(transit) != 0) {
             curandState rng;
-            rng.reset(seed, (uint64_t)((s * T + j) * m + nbr), (uint32_t)k);
+            // steps that draw several outputs per transit use the grouped form of the stream
+            if (m > 1) rng.reset_grouped(seed, (uint64_t)((s * T + j) * m + nbr), (uint32_t)k);
+            else rng.reset(seed, (uint64_t)((s * T + j) * m + nbr), (uint32_t)k);
             const CSR::Edge* edges = g.view.get_edges(transit);
             const float* weights = g.view.get_weights(transit);
             const VertexID r = app.template next<SampleType, const CSR::Edge*, const float*>(

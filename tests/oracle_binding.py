@@ -52,6 +52,8 @@ def lib():
         L.ndo_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
         L.ndo_uniform.restype = C.c_float
         L.ndo_uniform.argtypes = [C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32]
+        L.ndo_uniform_grouped.restype = C.c_float
+        L.ndo_uniform_grouped.argtypes = [C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32]
         L.ndo_rand_int.restype = C.c_int32
         L.ndo_rand_int.argtypes = [C.c_float, C.c_int32]
         for name in ("ndo_step_size_at_step", "ndo_number_of_transits", "ndo_sub_warp_size_at_step"):
@@ -155,6 +157,11 @@ def philox(ctr, key):
 
 def uniform(seed, slot, step, draw):
     return lib().ndo_uniform(seed, slot, step, draw)
+
+
+def uniform_grouped(seed, slot, step, draw):
+    """The stream of steps with stepSize > 1 (first draw shared by four consecutive slots)."""
+    return lib().ndo_uniform_grouped(seed, slot, step, draw)
 
 
 def rand_int(u, n):

@@ -15,6 +15,12 @@ def test_philox_fill_matches_oracle(oracle):
         for d in range(6):
             assert got[slot, d] == oracle.uniform(seed, first + slot, step, d)
     assert got.min() >= 0.0 and got.max() < 1.0
+    # the buffer of a step that draws several outputs per transit: the grouped form of the stream
+    first = (1 << 33) + 6  # not a multiple of four: the first group is cut
+    got = nd.philox_fill_uniform(seed, step, first, 1000, 3, step_size=10)
+    for slot in list(range(0, 12)) + list(range(12, 1000, 37)):
+        for d in range(3):
+            assert got[slot, d] == oracle.uniform_grouped(seed, first + slot, step, d)
 
 
 SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 4095, 4096, 4097, 12289, 1000003]

@@ -93,7 +93,7 @@ def test_khop_closed_form_and_layout(oracle):
             if not adj[s]:
                 want = n
             else:
-                u = oracle.uniform(SEED, s * m0 + nbr, 0, 0)
+                u = oracle.uniform_grouped(SEED, s * m0 + nbr, 0, 0)  # step sizes > 1: the grouped stream
                 want = sorted(adj[s])[rint(u, len(adj[s]))]
             hop0.append(want)
             assert final[s, nbr] == want
@@ -102,7 +102,7 @@ def test_khop_closed_form_and_layout(oracle):
                 if t == n or not adj[t]:
                     want = n
                 else:
-                    u = oracle.uniform(SEED, (s * m0 + j) * m1 + nbr, 1, 0)
+                    u = oracle.uniform_grouped(SEED, (s * m0 + j) * m1 + nbr, 1, 0)
                     want = sorted(adj[t])[rint(u, len(adj[t]))]
                 assert final[s, m0 + j * m1 + nbr] == want
 

@@ -102,10 +102,10 @@ def anchor_hop_by_hand(oracle, g, seed, anchors, step_sizes, sample):
                 if transit != V:
                     adj = adjacency(g, transit)
                     if len(adj):
-                        neighbor = int(adj[oracle.rand_int(oracle.uniform(seed, slot, k, draw), len(adj))])
+                        neighbor = int(adj[oracle.rand_int(oracle.uniform_grouped(seed, slot, k, draw), len(adj))])
                         draw += 1
                     if k != len(step_sizes) - 1:
-                        x = oracle.rand_int(oracle.uniform(seed, slot, k, draw), len(anchors) + 1)
+                        x = oracle.rand_int(oracle.uniform_grouped(seed, slot, k, draw), len(anchors) + 1)
                         if x != len(anchors):
                             chosen = int(anchors[((j * m + nbr) % T + x) % len(anchors)])
                 out.append(neighbor)

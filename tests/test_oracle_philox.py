@@ -56,3 +56,22 @@ def test_rand_int_closed_forms(oracle):
             assert got == want and 0 <= got <= n - 1
     # curand_uniform can return exactly 1.0; the clamp is what keeps the index in range
     assert oracle.rand_int(1.0, 17) == 16
+
+
+def test_grouped_stream_is_the_plain_stream_rearranged(oracle):
+    """Steps with stepSize > 1 take the first draw of four consecutive output slots from one
+    block - counter (slot >> 2, step | 2^31, 0), word slot & 3 - and every later draw from the
+    slot's own stream, one position earlier.  Stated on ndo_uniform, which the known-answer
+    vectors pin: nothing new is computed, only which word goes where."""
+    seed = 0x299f31d0a4093822
+    for slot in [0, 1, 2, 3, 4, 5, 7, 250, 251, (1 << 34) + 6, (1 << 34) + 7]:
+        for step in (0, 1, 99):
+            assert oracle.uniform_grouped(seed, slot, step, 0) == oracle.uniform(seed, slot >> 2, step | (1 << 31), slot & 3)
+            for d in range(1, 7):
+                assert oracle.uniform_grouped(seed, slot, step, d) == oracle.uniform(seed, slot, step, d - 1)
+    # the four slots of a group draw the four words of ONE block, which no slot's own stream uses
+    firsts = [oracle.uniform_grouped(seed, 8 + i, 3, 0) for i in range(4)]
+    assert len(set(firsts)) == 4
+    assert firsts == [oracle.uniform(seed, 2, 3 | (1 << 31), i) for i in range(4)]
+    us = np.array([oracle.uniform_grouped(42, s, 1, 0) for s in range(4000)], dtype=np.float64)
+    assert us.min() >= 0.0 and us.max() < 1.0 and abs(us.mean() - 0.5) < 0.02
