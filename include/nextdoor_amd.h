@@ -218,8 +218,11 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
  * DEVICE arrays, enqueued on `stream` (a hipStream_t; NULL = the default stream) without
  * waiting for it, with all working memory in a fixed array inside the library
  * (ND_SORT_PAIRS_NOALLOC_MAX pairs at most: 8.5 MiB per GPU, held until the process ends).
- * Calls no hipMalloc / hipFree / memset.  d_vals == NULL: value = index.  The output arrays
- * must not be the input arrays.  More than ND_SORT_PAIRS_NOALLOC_MAX pairs: returns -2.  All
+ * Calls no hipMalloc / hipFree / memset.  d_vals == NULL: value = index.  No output array may
+ * overlap an input array or the other output array (returns -3).  The first call on a device asks
+ * the runtime for the address of the working array (hipGetSymbolAddress, which may load the
+ * library's code object): make that call outside graph capture; nd_sampler_set_graph on the
+ * device does it as well.  More than ND_SORT_PAIRS_NOALLOC_MAX pairs: returns -2.  All
  * calls on one GPU share the working array: calls that overlap on one GPU (two streams, two
  * host threads) race; calls on one stream are ordered by the stream. */
 #define ND_SORT_PAIRS_NOALLOC_MAX 1048576

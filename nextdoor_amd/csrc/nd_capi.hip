@@ -368,6 +368,12 @@ int nd_sampler_set_graph(nd_sampler* s, const nd_graph* g) {
     int n_devices = 0;
     if (hipGetDeviceCount(&n_devices) != hipSuccess || n_devices < 1) return fail("no HIP device available");
     s->graph = g;
+    {
+      // the address of nd_sort_pairs_noalloc's working array on this device, asked for here so
+      // that a later first call of it under graph capture has nothing left to set up
+      uint32_t* unused = nullptr;
+      (void)scratch_on_current_device(&unused);
+    }
     const int rc = s->engine->set_graph(g);
     return rc == 0 ? 0 : fail(s->engine->last_error, rc);
   });
@@ -702,7 +708,18 @@ int nd_sort_pairs_noalloc(const int32_t* d_keys, const int32_t* d_vals, int64_t 
       return fail("nd_sort_pairs_noalloc sorts at most " + std::to_string(kNoAllocMaxPairs) + " pairs, " +
                   std::to_string(n) + " given (use nd_sort_pairs)", -2);
     if (n == 0) return 0;
-    if (d_keys_out == d_keys || (d_vals && d_vals_out == d_vals)) return fail("the sort is not in place");
+    {
+      // no array of the call may share a byte with another one it is written while read:
+      // the outputs with each other and with the inputs
+      const size_t bytes = sizeof(int32_t) * (size_t)n;
+      auto overlap = [bytes](const void* a, const void* b) {
+        const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
+        return a && b && x < y + bytes && y < x + bytes;
+      };
+      if (overlap(d_keys_out, d_vals_out) || overlap(d_keys_out, d_keys) || overlap(d_keys_out, d_vals) ||
+          overlap(d_vals_out, d_keys) || overlap(d_vals_out, d_vals))
+        return fail("the sort is not in place: input and output arrays must not overlap", -3);
+    }
     uint32_t* work = nullptr;
     CAPI_HIP(scratch_on_current_device(&work));
     const nd::SortPlan plan = nd::make_sort_plan((size_t)n, key_bits);

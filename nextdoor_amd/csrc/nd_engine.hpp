@@ -30,6 +30,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <chrono>
 #include <memory>
 #include <string>
@@ -94,7 +95,7 @@ class HostArray {
         size_ = data_ ? n : 0;
       }
     }
-    for (size_t i = 0; i < size_; ++i) data_[i] = value;
+    std::fill_n(data_, size_, value);
   }
   void clear() {
     if (data_) {
@@ -407,40 +408,88 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
   store_output(P, transit, pair, pair_slot, sample, nbr, neighbor, next_transit);
 }
 
+// Four consecutive ids of a result, at an address that is a multiple of four bytes only.
+struct __attribute__((packed, aligned(4))) FourIds {
+  VertexID a, b, c, d;
+};
+
 // The outputs of a pair that fall into group `gi` of the pair's groups of four consecutive
 // (global) output slots: one shared Philox block, then up to four outputs.  For steps with
-// step_size > 1.
+// step_size > 1.  In two halves, so that a lane that works through several groups can have
+// the gathers of the next group under way while the results of this one are stored.
+struct GroupOutputs {
+  uint64_t first, lo, hi;  // global slots: the pair's output 0, the group's outputs [lo, hi)
+  uint32_t sample;
+  VertexID neighbor[4], next_transit[4];
+};
+
 template <class SampleType, class App, class EdgeArray, class WeightArray>
-__device__ __forceinline__ void produce_group(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
+__device__ __forceinline__ void compute_group(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
                                               uint32_t pair_slot, uint32_t gi, EdgePos_t n_edges, float max_weight,
-                                              EdgeArray& edges, WeightArray& weights) {
+                                              EdgeArray& edges, WeightArray& weights, GroupOutputs* out) {
   const uint64_t first = P.first_slot + (uint64_t)pair_slot * P.step_size;  // global slot of the pair's output 0
   const uint64_t group = (first >> 2) + gi;
   const uint64_t lo = group * 4 > first ? group * 4 : first;
   const uint64_t end = first + P.step_size;
   const uint64_t hi = group * 4 + 4 < end ? group * 4 + 4 : end;
+  out->first = first;
+  out->lo = lo;
+  out->hi = hi;
   if (lo >= hi) return;
   PhiloxBlock block = PhiloxBlock();
   // next() draws for a real transit with edges; stepTransits for any real transit (run_app)
   if (transit != P.invalid && (n_edges != 0 || (App().hasExplicitTransits() && !P.is_last)))
     block = grouped_first_block(P.seed, group, (uint32_t)P.step);
-  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
-  // all draws first, then all stores: the up to four gathers of the group are under way
-  // together instead of each waiting behind the store of the one before
-  VertexID neighbor[4], next_transit[4];
+  out->sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
+  // all draws of the group before any store: its up to four gathers are under way together
 #pragma unroll
   for (uint32_t q = 0; q < 4; ++q) {
-    neighbor[q] = next_transit[q] = P.invalid;
+    out->neighbor[q] = out->next_transit[q] = P.invalid;
     if (lo + q < hi)
-      compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, sample,
+      compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, out->sample,
                                                               (uint32_t)(lo + q - first), n_edges, max_weight, edges,
                                                               weights, true, block_word(block, (uint32_t)(lo + q) & 3u),
-                                                              &neighbor[q], &next_transit[q]);
+                                                              &out->neighbor[q], &out->next_transit[q]);
+  }
+}
+
+__device__ __forceinline__ void store_group(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
+                                            const GroupOutputs& g) {
+  if (g.lo >= g.hi) return;
+  if (g.hi - g.lo == 4 && !P.pair_cells && !P.explicit_out && !P.emit_keys) {
+    // a whole group whose outputs are all there is to store: the four ids are neighbours in
+    // the step's results (word aligned, not more), and go out as one 16-byte store
+    const uint32_t per_sample = P.transits_per_sample * P.step_size;
+    const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + (g.lo - g.first);
+    FourIds* dst = reinterpret_cast<FourIds*>(P.step_out + (size_t)g.sample * P.out_pitch +
+                                              (size_t)(out_slot - (uint64_t)g.sample * per_sample));
+    *dst = FourIds{g.neighbor[0], g.neighbor[1], g.neighbor[2], g.neighbor[3]};
+    return;
   }
 #pragma unroll
   for (uint32_t q = 0; q < 4; ++q)
-    if (lo + q < hi)
-      store_output(P, transit, pair, pair_slot, sample, (uint32_t)(lo + q - first), neighbor[q], next_transit[q]);
+    if (g.lo + q < g.hi)
+      store_output(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.lo + q - g.first), g.neighbor[q],
+                   g.next_transit[q]);
+}
+
+// The groups first, first + stride, ... of a pair, the draws of a group made before the
+// results of the group before it are stored.
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ void produce_groups(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
+                                               uint32_t pair_slot, uint32_t first_group, uint32_t stride,
+                                               EdgePos_t n_edges, float max_weight, EdgeArray& edges,
+                                               WeightArray& weights) {
+  GroupOutputs held;
+  held.first = held.lo = held.hi = 0;  // nothing held yet
+  for (uint32_t gi = first_group; gi < P.groups_per_pair; gi += stride) {
+    GroupOutputs now;
+    compute_group<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, gi, n_edges, max_weight,
+                                                           edges, weights, &now);
+    store_group(P, transit, pair, pair_slot, held);
+    held = now;
+  }
+  store_group(P, transit, pair, pair_slot, held);
 }
 
 // inversion_period == 0: walks are inverted before every step when there are at least this
@@ -513,9 +562,8 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
       produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, 0, n_edges,
                                                                         max_weight, edges, weights);
     } else {
-      for (uint32_t gi = first_nbr; gi < P.groups_per_pair; gi += nbr_stride)
-        produce_group<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, gi, n_edges,
-                                                                         max_weight, edges, weights);
+      produce_groups<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, first_nbr,
+                                                                        nbr_stride, n_edges, max_weight, edges, weights);
     }
   } else {
     const CSR::Edge* edges = csr.edges + begin;
@@ -524,9 +572,8 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
       produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, 0, n_edges,
                                                                      max_weight, edges, weights);
     } else {
-      for (uint32_t gi = first_nbr; gi < P.groups_per_pair; gi += nbr_stride)
-        produce_group<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, gi, n_edges,
-                                                                      max_weight, edges, weights);
+      produce_groups<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, first_nbr,
+                                                                     nbr_stride, n_edges, max_weight, edges, weights);
     }
   }
 }
@@ -628,6 +675,35 @@ struct alignas(16) WorkItem {
   uint32_t unused[3];
 };
 
+// The first `count` (at most kCacheEdges) words of `src` into LDS by the whole workgroup.  A
+// lane takes four consecutive words per round (one 16-byte load from a word-aligned address)
+// and has the loads of ALL its rounds under way before it writes the first to LDS: a loop of
+// "load one word, wait, write it" costs a memory round trip per 256 words - for a
+// 2000-edge adjacency eight trips one after the other, and the workgroup class spent most of
+// its time there.
+template <class T>
+__device__ __forceinline__ void stage_into_lds(const T* __restrict__ src, T* lds, EdgePos_t count) {
+  static_assert(sizeof(T) == 4, "32-bit words");
+  struct __attribute__((packed, aligned(4))) FourWords { uint32_t a, b, c, d; };
+  constexpr int kRounds = kCacheEdges / (kStepThreads * 4);
+  FourWords held[kRounds];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const EdgePos_t e = (EdgePos_t)(r * kStepThreads + threadIdx.x) * 4;
+    if (e + 4 <= count) held[r] = *reinterpret_cast<const FourWords*>(src + e);
+  }
+  // the up to three words after the last whole four
+  const EdgePos_t rest = count & ~(EdgePos_t)3;
+  T last = T();
+  if ((EdgePos_t)threadIdx.x < count - rest) last = src[rest + threadIdx.x];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const EdgePos_t e = (EdgePos_t)(r * kStepThreads + threadIdx.x) * 4;
+    if (e + 4 <= count) *reinterpret_cast<uint4*>(lds + e) = make_uint4(held[r].a, held[r].b, held[r].c, held[r].d);
+  }
+  if ((EdgePos_t)threadIdx.x < count - rest) lds[rest + threadIdx.x] = last;
+}
+
 // One workgroup per work item = a stretch of pairs that sit on the SAME transit.  The
 // transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
 // with coalesced reads and every draw of the stretch gathers from LDS.  The workgroup takes
@@ -638,17 +714,25 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
                                                 float* s_weights) {
   constexpr bool kWeights = app_uses_weights<App>::value;
   CSRPartition csr = P.csr;
-  WorkItem item = WorkItem();
-  if (first_item < n_chunks) item = chunks[first_item];
+  // the five words of an item that are used, as scalars (the same for every lane)
+  uint32_t first_pair = 0, n_pairs = 0;
+  VertexID transit = 0;
+  EdgePos_t begin = 0, n_edges = 0;
+  auto fetch = [&](uint32_t c, uint32_t* fp, uint32_t* np, VertexID* t, EdgePos_t* b, EdgePos_t* ne) {
+    *fp = chunks[c].first_pair;
+    *np = chunks[c].n_pairs;
+    *t = (VertexID)chunks[c].transit;
+    *b = chunks[c].begin;
+    *ne = chunks[c].n_edges;
+  };
+  if (first_item < n_chunks) fetch(first_item, &first_pair, &n_pairs, &transit, &begin, &n_edges);
   for (uint32_t c = first_item; c < n_chunks; c += item_stride) {
     // the record of the item after this one is fetched while this one is worked on
-    WorkItem coming = item;
-    if (c + item_stride < n_chunks) coming = chunks[c + item_stride];
-    const uint32_t first_pair = item.first_pair;
-    const uint32_t n_pairs = item.n_pairs;
-    const VertexID transit = (VertexID)item.transit;
-    const EdgePos_t begin = item.begin;
-    const EdgePos_t n_edges = item.n_edges;
+    uint32_t coming_first_pair = 0, coming_n_pairs = 0;
+    VertexID coming_transit = 0;
+    EdgePos_t coming_begin = 0, coming_n_edges = 0;
+    if (c + item_stride < n_chunks)
+      fetch(c + item_stride, &coming_first_pair, &coming_n_pairs, &coming_transit, &coming_begin, &coming_n_edges);
     const float max_weight = csr.max_weights[transit];  // every next() is handed it, hint or no hint
     const EdgePos_t cached = n_edges < kCacheEdges ? n_edges : kCacheEdges;
     // Lanes per pair: one, or the power of two (at most the groups of four output slots a pair
@@ -660,10 +744,8 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
     const uint32_t lanes = n_pairs << lanes_shift;
     uint32_t slot = threadIdx.x < lanes ? P.pair_slots[first_pair + (threadIdx.x >> lanes_shift)] : 0u;
     __syncthreads();  // the previous work item is done with the cache
-    for (EdgePos_t e = threadIdx.x; e < cached; e += kStepThreads) {
-      s_edges[e] = csr.edges[begin + e];
-      if (kWeights) s_weights[e] = csr.weights[begin + e];
-    }
+    stage_into_lds(csr.edges + begin, s_edges, cached);
+    if (kWeights) stage_into_lds(csr.weights + begin, s_weights, cached);
     __syncthreads();
     LdsBackedArray<CSR::Edge> edges{s_edges, csr.edges + begin, cached};
     LdsBackedArray<float> lds_weights{s_weights, csr.weights + begin, kWeights ? cached : 0};
@@ -674,12 +756,16 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
         produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
             P, csr, transit, first_pair + p, slot, 0, n_edges, max_weight, edges, lds_weights);
       } else {
-        for (uint32_t gi = t & ((1u << lanes_shift) - 1u); gi < P.groups_per_pair; gi += 1u << lanes_shift)
-          produce_group<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
-              P, csr, transit, first_pair + p, slot, gi, n_edges, max_weight, edges, lds_weights);
+        produce_groups<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
+            P, csr, transit, first_pair + p, slot, t & ((1u << lanes_shift) - 1u), 1u << lanes_shift, n_edges,
+            max_weight, edges, lds_weights);
       }
     }
-    item = coming;
+    first_pair = coming_first_pair;
+    n_pairs = coming_n_pairs;
+    transit = coming_transit;
+    begin = coming_begin;
+    n_edges = coming_n_edges;
   }
 }
 
@@ -688,8 +774,8 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
                                                                       const WorkItem* __restrict__ chunks,
                                                                       const RunsMeta* __restrict__ meta,
                                                                       uint32_t chunk_capacity) {
-  __shared__ CSR::Edge s_edges[kCacheEdges];
-  __shared__ float s_weights[app_uses_weights<App>::value ? kCacheEdges : 1];
+  __shared__ __align__(16) CSR::Edge s_edges[kCacheEdges];  // filled with 16-byte stores
+  __shared__ __align__(16) float s_weights[app_uses_weights<App>::value ? kCacheEdges : 4];
   const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
   workgroup_items<SampleType, App>(P, chunks, n_chunks, blockIdx.x, gridDim.x, s_edges, s_weights);
 }
@@ -711,8 +797,8 @@ __global__ __launch_bounds__(kStepThreads) void step_balanced_kernel(StepParams 
                                                                      const RunsMeta* __restrict__ meta,
                                                                      const WorkItem* __restrict__ chunks,
                                                                      uint32_t chunk_capacity, uint32_t wg_per_group) {
-  __shared__ CSR::Edge s_edges[kCacheEdges];
-  __shared__ float s_weights[app_uses_weights<App>::value ? kCacheEdges : 1];
+  __shared__ __align__(16) CSR::Edge s_edges[kCacheEdges];  // filled with 16-byte stores
+  __shared__ __align__(16) float s_weights[app_uses_weights<App>::value ? kCacheEdges : 4];
   const uint32_t per_group = kBalancedFlatBlocks + wg_per_group;
   const uint32_t group = blockIdx.x / per_group;
   const uint32_t local = blockIdx.x - group * per_group;

@@ -104,3 +104,33 @@ def test_an_app_whose_factory_gives_nothing_is_an_error():
     g = nextdoor_amd.Graph.from_edges([0, 1], [1, 0])
     with pytest.raises(nextdoor_amd.NextDoorError, match="returned no engine"):
         nextdoor_amd.Sampler("HostSideProbeApp", g)
+
+
+def test_the_sort_that_allocates_nothing_refuses_bad_calls_before_it_touches_a_device():
+    """nd_sort_pairs_noalloc checks its arguments on the host first: too many pairs, and any
+    overlap between the arrays of a call (equal pointers, an output inside an input's range,
+    the two outputs inside each other), are refused with a message.  The addresses below are
+    never dereferenced: every call here is refused before a HIP call is made."""
+    import nextdoor_amd as nd
+    L = nd._capi.lib()
+    base = 1 << 40
+    n = 1000
+
+    def call(keys, vals, n_pairs, keys_out, vals_out):
+        return L.nd_sort_pairs_noalloc(keys, vals, n_pairs, 20, keys_out, vals_out, None), L.nd_last_error().decode()
+
+    rc, why = call(base, None, nd.SORT_PAIRS_NOALLOC_MAX + 1, base + (1 << 30), base + (2 << 30))
+    assert rc == -2 and "at most" in why
+    far = [base + i * (1 << 20) for i in range(4)]
+    for keys, vals, keys_out, vals_out in [
+            (far[0], far[1], far[0], far[3]),              # keys sorted in place
+            (far[0], far[1], far[2], far[1]),              # values sorted in place
+            (far[0], far[1], far[2], far[2]),              # both outputs one array
+            (far[0], far[1], far[2], far[2] + 4 * n - 4),  # the outputs share their last / first word
+            (far[0], far[1], far[0] + 4 * (n - 1), far[3]),  # an output starts inside an input
+            (far[0], far[1], far[1] - 4, far[3]),          # an output ends inside an input
+    ]:
+        rc, why = call(keys, vals, n, keys_out, vals_out)
+        assert rc == -3 and "overlap" in why, (keys, vals, keys_out, vals_out, rc, why)
+    assert call(None, None, 0, None, None)[0] == 0  # nothing to sort
+    assert call(None, None, 5, far[2], far[3])[0] != 0  # no input
