@@ -1051,8 +1051,9 @@ __global__ __launch_bounds__(256) void small_map_scan(uint32_t* __restrict__ cou
   const uint32_t first = blockIdx.x * kSmallMapChunk + threadIdx.x * 4u;
   uint32_t c[4];
 #pragma unroll
+  for (int k = 0; k < 4; ++k) c[k] = first + k < n_counters ? counts[first + k] : 0u;
+#pragma unroll
   for (int k = 0; k < 4; ++k) {
-    c[k] = first + k < n_counters ? counts[first + k] : 0u;
     if (c[k]) counts[first + k] = 0;  // ready for the pairs the coming step emits
   }
   uint32_t block_total;
@@ -1078,8 +1079,17 @@ __global__ __launch_bounds__(256) void small_map_place(
     ClassCounters* __restrict__ counters) {
   __shared__ uint32_t s_wave[kScanThreads / kWave];
   __shared__ uint32_t chunk_base[1024];
-  const uint32_t n_in = n_in_dev ? *n_in_dev : n_in_host;
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  // the pair's own words do not wait for the chunk scan; n_in_host bounds the arrays
+  uint32_t transit = invalid, rank = 0, slot = 0, state = 0;
+  if (i < n_in_host) {
+    transit = emit_keys[i];
+    rank = emit_ranks[i];
+    slot = emit_slots[i];
+    if (state_out) state = emit_state[i];
+  }
+  const uint32_t n_in = n_in_dev ? *n_in_dev : n_in_host;
+  if (i >= n_in) transit = invalid;
   {
     // where every chunk starts among the placed pairs
     uint32_t t[4];
@@ -1102,19 +1112,17 @@ __global__ __launch_bounds__(256) void small_map_place(
       }
     }
   }
-  uint32_t transit = invalid, start = 0, count = 0, n_items = 0, refused = 0;
+  uint32_t start = 0, count = 0, n_items = 0, refused = 0;
   bool head = false;
-  if (i < n_in) {
-    transit = emit_keys[i];
+  {
     if (transit != invalid) {
-      const uint32_t rank = emit_ranks[i];
       const uint32_t first_copy = counter_base[transit];
       const uint32_t beyond = counter_base[transit + 1];  // the counter after the last one exists
       const uint32_t mine = first_copy + (i & (beyond - first_copy - 1u));
       const uint32_t pos = chunk_base[mine / kSmallMapChunk] + local_start[mine] + rank;
       keys_out[pos] = transit;
-      slots_out[pos] = emit_slots[i];
-      if (state_out) state_out[pos] = emit_state[i];
+      slots_out[pos] = slot;
+      if (state_out) state_out[pos] = state;
       if (rank == 0) {
         // the first pair of the first copy that counted any is the first pair of the run
         const uint32_t run_start = chunk_base[first_copy / kSmallMapChunk] + local_start[first_copy];

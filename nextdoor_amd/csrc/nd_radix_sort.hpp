@@ -69,13 +69,18 @@ __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* 
   __syncthreads();
   if (n_dev) n = *n_dev;
   const size_t tile_start = (size_t)blockIdx.x * kSortTile;
+  // all of a lane's keys are fetched before the first is counted: with the count inside the
+  // loop every key waited for the one before it (eight memory round trips one after the other)
+  uint32_t mine[kSortItems];
 #pragma unroll
   for (int it = 0; it < kSortItems; ++it) {
     const size_t idx = tile_start + (size_t)it * kSortThreads + threadIdx.x;
-    if (idx < n) {
-      const uint32_t k = keys[layout.at(idx)];
-      if (k != drop_key) atomicAdd(&s_hist[(k >> shift) & mask], 1u);
-    }
+    mine[it] = idx < n ? keys[layout.at(idx)] : drop_key;
+  }
+#pragma unroll
+  for (int it = 0; it < kSortItems; ++it) {
+    const size_t idx = tile_start + (size_t)it * kSortThreads + threadIdx.x;
+    if (idx < n && mine[it] != drop_key) atomicAdd(&s_hist[(mine[it] >> shift) & mask], 1u);
   }
   __syncthreads();
   if (threadIdx.x <= mask) hist[(size_t)threadIdx.x * num_tiles + blockIdx.x] = s_hist[threadIdx.x];
@@ -91,14 +96,33 @@ __global__ __launch_bounds__(kSortThreads) void radix_row_scan(uint32_t* __restr
   const uint32_t per_thread = (num_tiles + kSortThreads - 1) / kSortThreads;
   const uint32_t begin = threadIdx.x * per_thread;
   const uint32_t end = begin + per_thread < num_tiles ? begin + per_thread : num_tiles;
+  // a stretch of at most kHeld counts stays in registers: its loads are all under way at once
+  // and the second sweep reads nothing
+  constexpr uint32_t kHeld = 8;
+  uint32_t held[kHeld];
   uint32_t sum = 0;
-  for (uint32_t i = begin; i < end; ++i) sum += row[i];
+  if (per_thread <= kHeld) {
+#pragma unroll
+    for (uint32_t k = 0; k < kHeld; ++k) held[k] = k < per_thread && begin + k < end ? row[begin + k] : 0u;
+#pragma unroll
+    for (uint32_t k = 0; k < kHeld; ++k) sum += held[k];
+  } else {
+    for (uint32_t i = begin; i < end; ++i) sum += row[i];
+  }
   uint32_t total;
   uint32_t running = block_exclusive_scan_256(sum, s_scan_tmp, &total);
-  for (uint32_t i = begin; i < end; ++i) {
-    const uint32_t c = row[i];
-    row[i] = running;
-    running += c;
+  if (per_thread <= kHeld) {
+#pragma unroll
+    for (uint32_t k = 0; k < kHeld; ++k) {
+      if (k < per_thread && begin + k < end) row[begin + k] = running;
+      running += held[k];
+    }
+  } else {
+    for (uint32_t i = begin; i < end; ++i) {
+      const uint32_t c = row[i];
+      row[i] = running;
+      running += c;
+    }
   }
   if (threadIdx.x == 0) row_totals[blockIdx.x] = total;
 }
