@@ -187,6 +187,10 @@ class EngineBase {
 // Step kernels
 // ---------------------------------------------------------------------------------------
 
+// Steps an app may have for its INVALID outputs to be written by the step kernels instead of
+// a fill of the whole result.
+constexpr int kMaxFillLevels = 8;
+
 struct StepParams {
   CSRPartition csr;
   int step;
@@ -225,6 +229,16 @@ struct StepParams {
   // indexed like step_out's own array form (output slot o of this step is pair o of the next):
   // what App::stepTransits returned for the output.  nullptr: the step's outputs are the map.
   int32_t* explicit_out;
+  // Results written straight into the rows, with nothing filled in beforehand: an output that
+  // is INVALID (and a pair with no transit or no edges, for all its outputs) leads nowhere at
+  // the later steps, whose pairs the inversion drops - no kernel ever reaches the slots that
+  // descend from it, so whoever writes the INVALID writes them too.  Level 0 is this step
+  // (offset 0, one slot per output), level l the l-th step after it: output q of a sample owns
+  // slots [q * fill_mult[l], (q + 1) * fill_mult[l]) at step_out + fill_off[l] of its row.
+  // fill_levels == 0: the result was filled before the pass, nothing of this is done.
+  uint32_t fill_levels;
+  uint32_t fill_off[kMaxFillLevels];
+  uint32_t fill_mult[kMaxFillLevels];
   const EdgeRecord* paired_edges; // interleaved (dst, weight) copy of the edges, or nullptr
   // Walks (one transit per sample, stepSize 1 everywhere): the step kernels also emit the
   // next step's pairs in THIS step's pair order - coalesced, and without the pairs the
@@ -373,6 +387,38 @@ __device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition
   *next_transit_out = next_transit;
 }
 
+// Output q (index inside the sample's segment of this step) is INVALID: so is everything the
+// later steps would have drawn from it (StepParams::fill_levels).
+__device__ __forceinline__ void fill_below(const StepParams& P, uint32_t sample, uint32_t q) {
+  int32_t* row = P.step_out + (size_t)sample * P.out_pitch;
+#pragma unroll
+  for (int l = 1; l < kMaxFillLevels; ++l) {
+    if ((uint32_t)l < P.fill_levels) {
+      int32_t* dst = row + P.fill_off[l] + (size_t)q * P.fill_mult[l];
+      for (uint32_t x = 0; x < P.fill_mult[l]; ++x) dst[x] = P.invalid;
+    }
+  }
+}
+
+// All outputs of a pair (slot pair_slot) are INVALID - it has no transit, or the transit has no
+// edge: its m outputs and what descends from them are contiguous stretches of the sample's row,
+// written by the lanes of the wavefront that are still at work: `helper` is the lane's number
+// among them, `helpers` how many they are.
+__device__ __forceinline__ void fill_dead_pair(const StepParams& P, uint32_t pair_slot, uint32_t helper,
+                                               uint32_t helpers) {
+  const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
+  const uint32_t q0 = (pair_slot - sample * P.transits_per_sample) * P.step_size;
+  int32_t* row = P.step_out + (size_t)sample * P.out_pitch;
+#pragma unroll
+  for (int l = 0; l < kMaxFillLevels; ++l) {
+    if ((uint32_t)l < P.fill_levels) {
+      int32_t* dst = row + P.fill_off[l] + (size_t)q0 * P.fill_mult[l];
+      const uint32_t n = P.step_size * P.fill_mult[l];
+      for (uint32_t x = helper; x < n; x += helpers) dst[x] = P.invalid;
+    }
+  }
+}
+
 // Second half: the output goes to its place in the step's results, and what the next step
 // needs of it to the next step's map.
 __device__ __forceinline__ void store_output(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
@@ -382,7 +428,9 @@ __device__ __forceinline__ void store_output(const StepParams& P, VertexID trans
     store_walk_result(P, sample, transit, neighbor);
   } else {
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
-    P.step_out[(size_t)sample * P.out_pitch + (size_t)(out_slot - (uint64_t)sample * per_sample)] = neighbor;
+    const uint32_t q = (uint32_t)(out_slot - (uint64_t)sample * per_sample);
+    P.step_out[(size_t)sample * P.out_pitch + q] = neighbor;
+    if (P.fill_levels > 1 && neighbor == P.invalid) fill_below(P, sample, q);
   }
   if (P.explicit_out) P.explicit_out[out_slot] = next_transit;
   if (P.emit_keys) {
@@ -461,9 +509,14 @@ __device__ __forceinline__ void store_group(const StepParams& P, VertexID transi
     // the step's results (word aligned, not more), and go out as one 16-byte store
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
     const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + (g.lo - g.first);
-    FourIds* dst = reinterpret_cast<FourIds*>(P.step_out + (size_t)g.sample * P.out_pitch +
-                                              (size_t)(out_slot - (uint64_t)g.sample * per_sample));
+    const uint32_t q = (uint32_t)(out_slot - (uint64_t)g.sample * per_sample);
+    FourIds* dst = reinterpret_cast<FourIds*>(P.step_out + (size_t)g.sample * P.out_pitch + q);
     *dst = FourIds{g.neighbor[0], g.neighbor[1], g.neighbor[2], g.neighbor[3]};
+    if (P.fill_levels > 1) {
+#pragma unroll
+      for (uint32_t x = 0; x < 4; ++x)
+        if (g.neighbor[x] == P.invalid) fill_below(P, g.sample, q + x);
+    }
     return;
   }
 #pragma unroll
@@ -553,6 +606,23 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
     n_edges = csr.row_ptr[transit + 1] - begin;
     max_weight = csr.max_weights[transit];
     if (taken_stamp && mark == stamp) return;
+  }
+  if (P.fill_levels != 0) {
+    // pairs all of whose outputs are INVALID: no draw, the wavefront writes their stretches
+    const bool dead = transit == P.invalid || n_edges == 0;
+    uint64_t todo = __ballot(dead && first_nbr == 0);
+    if (todo) {
+      // lanes past the last pair, or whose transit a work item covers, have left already
+      const uint64_t at_work = __ballot(1);
+      const uint32_t helper = (uint32_t)__popcll(at_work & ((1ull << (threadIdx.x & (kWave - 1))) - 1ull));
+      const uint32_t helpers = (uint32_t)__popcll(at_work);
+      while (todo) {
+        const int src = __ffsll((unsigned long long)todo) - 1;
+        todo &= todo - 1;
+        fill_dead_pair(P, __shfl(slot, src, kWave), helper, helpers);
+      }
+    }
+    if (dead) return;
   }
   // one output (walks), or the pair's groups of four output slots first_nbr, first_nbr + stride, ...
   if (app_uses_weights<App>::value) {
@@ -1565,6 +1635,11 @@ class Engine : public EngineBase {
       else if (strcmp(env, "merged") == 0) forced_schedule_ = kScheduleMerged;
       else if (strcmp(env, "forked") == 0) forced_schedule_ = kScheduleForked;
     }
+    // ND_MARK_UNWRITTEN=1: a pass whose kernels write every slot of the result themselves first
+    // sets the result to a value that is neither a vertex nor INVALID, so that a slot no kernel
+    // wrote shows in the result instead of keeping what an earlier pass left there (for tests)
+    mark_unwritten_ = false;
+    if (const char* env = getenv("ND_MARK_UNWRITTEN")) mark_unwritten_ = strcmp(env, "1") == 0;
 
     // rows staged per workgroup by the final assembly: as many as fit 64 KiB of LDS
     row_pitch_ = (uint32_t)(F | 1);
@@ -1675,11 +1750,14 @@ class Engine : public EngineBase {
     if (balance)
       fill_i32<<<dim3((kBalanceWords + 255) / 256), dim3(256), 0, stream_>>>((int32_t*)d_balance_, kBalanceWords, 0);
     // pairs whose transit is INVALID are dropped by the inversion and never reach a step
-    // kernel: their outputs keep this fill
-    {
+    // kernel: their outputs keep this fill - unless the step kernels write the rows themselves
+    // and, with every INVALID, what descends from it (StepParams::fill_levels)
+    const bool kernels_fill = rows_direct_ && !explicit_map_ && !walk_mode_ && n_steps <= kMaxFillLevels;
+    if (!kernels_fill || mark_unwritten_) {
+      const int32_t value = kernels_fill ? invalid_ + 1 : invalid_;
       const size_t n_out = (size_t)n_samples_ * (paired_results() ? (F + 1) / 2 * 2 : F);
       fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(
-          rows_direct_ ? d_final_ : d_step_out_, n_out, invalid_);
+          rows_direct_ ? d_final_ : d_step_out_, n_out, value);
     }
 
     uint32_t transits_per_sample = (uint32_t)init_size_;
@@ -1715,6 +1793,16 @@ class Engine : public EngineBase {
       P.pair_cell_samples = (uint32_t)n_samples_;
       P.samples = d_samples_;
       P.explicit_out = explicit_map_ && step + 1 < n_steps ? d_explicit_ : nullptr;
+      P.fill_levels = 0;
+      if (kernels_fill) {
+        uint32_t mult = 1;
+        for (int later = step; later < n_steps; ++later) {
+          if (later > step) mult *= (uint32_t)app.stepSize(later);
+          P.fill_off[P.fill_levels] = layout_.seg_base[later] - layout_.seg_base[step];
+          P.fill_mult[P.fill_levels] = mult;
+          P.fill_levels++;
+        }
+      }
       P.paired_edges = dgraph_->paired;
       const bool emits = walk_mode_ && step + 1 < n_steps;
       P.state_travels = state_travels_;
@@ -2223,7 +2311,7 @@ class Engine : public EngineBase {
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
   uint32_t* d_live_ = nullptr;          // pairs the inversion kept (real transits); two words, alternating by step
-  bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false;
+  bool walk_mode_ = false, state_travels_ = false, rows_direct_ = false, mark_unwritten_ = false;
   bool explicit_map_ = false;           // App::stepTransits fills the next step's map (apps that are not walks)
   VertexID_t* d_explicit_ = nullptr;    // that map: the transit of every pair of the coming step
   uint32_t *d_emit_keys_ = nullptr, *d_emit_slots_ = nullptr, *d_emit_state_ = nullptr;  // next step's pairs
