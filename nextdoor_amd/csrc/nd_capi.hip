@@ -846,8 +846,9 @@ int nd_classify_runs(const int32_t* sorted_keys, int64_t n, const int32_t* degre
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
           d_items.as<nd::WorkItem>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     } else {
-      const int64_t per_block = 256 * nd::kClassifyItemsLarge;
-      nd::classify_run_tails<nd::kClassifyItemsLarge><<<dim3((unsigned)((n + per_block - 1) / per_block)), dim3(256), 0, 0>>>(
+      const int64_t per_block = nd::kClassifyThreadsLarge * nd::kClassifyItemsLarge;
+      nd::classify_run_tails<nd::kClassifyItemsLarge, nd::kClassifyThreadsLarge>
+          <<<dim3((unsigned)((n + per_block - 1) / per_block)), dim3(nd::kClassifyThreadsLarge), 0, 0>>>(
           d_keys.as<uint32_t>(), d_n.as<uint32_t>(), meta, meta + 1, d_rows.as<EdgePos_t>(), (uint32_t)step_size,
           d_items.as<nd::WorkItem>(), (uint32_t)capacity, d_taken.as<uint32_t>(), d_counters, d_balance.as<uint32_t>(), 1u);
     }

@@ -27,10 +27,11 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
 }
 
 // Exclusive scan of one value per thread across a 256-thread workgroup.
-// s_wave_totals must hold 4 uint32.  Returns the exclusive prefix; *block_total gets
+// s_wave_totals must hold one uint32 per wavefront of the workgroup (kThreads / 64; 4 for the
+// 256-thread form).  Returns the exclusive prefix; *block_total gets
 // the sum over the workgroup.  Contains two barriers.
-__device__ __forceinline__ uint32_t block_exclusive_scan_256(uint32_t v, uint32_t* s_wave_totals,
-                                                             uint32_t* block_total) {
+template <int kThreads>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave_totals, uint32_t* block_total) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const uint32_t incl = wave_inclusive_scan(v);
@@ -38,7 +39,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan_256(uint32_t v, uint32_
   __syncthreads();
   uint32_t before = 0, total = 0;
 #pragma unroll
-  for (int w = 0; w < kScanThreads / kWave; ++w) {
+  for (int w = 0; w < kThreads / kWave; ++w) {
     const uint32_t t = s_wave_totals[w];
     if (w < wave) before += t;
     total += t;
@@ -46,6 +47,11 @@ __device__ __forceinline__ uint32_t block_exclusive_scan_256(uint32_t v, uint32_
   __syncthreads();
   *block_total = total;
   return before + incl - v;
+}
+
+__device__ __forceinline__ uint32_t block_exclusive_scan_256(uint32_t v, uint32_t* s_wave_totals,
+                                                             uint32_t* block_total) {
+  return block_exclusive_scan<kScanThreads>(v, s_wave_totals, block_total);
 }
 
 __global__ __launch_bounds__(kScanThreads) void scan_tile_totals(const uint32_t* __restrict__ in, size_t n,

@@ -940,24 +940,19 @@ constexpr uint32_t kDirectSegment = 16;  // ids: segments this long are written 
 // Consecutive pairs per lane of classify_run_tails: many for large maps (fewer atomics),
 // one for small ones (the launch is latency bound: 3.4 vs 1.8 ms over the 99 steps of 4.2 M walks).
 constexpr int kClassifyItemsLarge = 16;
+// (workgroups of 1024 lanes, for a quarter of the atomics that claim work items: 0.34 ms
+// against 0.24 on 5.2e7 pairs - the launch waits for its slowest lanes, not for the atomics)
+constexpr int kClassifyThreadsLarge = 256;
 constexpr uint32_t kClassifyLargeFrom = 16u << 20;  // pairs
 
-// Is pair i the last of a run that the workgroup kernel should take?  Gives the run and the
-// number of work items it needs.  refused_out (nullable): set to the run's length when the run
-// is long enough but stays with the flat kernel because of the degree.
-__device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict__ keys, uint32_t i, uint32_t n,
-                                                      const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
-                                                      uint32_t* transit_out, uint32_t* start_out,
-                                                      uint32_t* count_out, uint32_t* n_items_out,
-                                                      uint32_t* refused_out = nullptr, EdgePos_t* begin_out = nullptr,
-                                                      EdgePos_t* degree_out = nullptr) {
-  const uint32_t transit = keys[i];
-  if (i + 1 != n && keys[i + 1] == transit) return false;  // not the last pair of its run
-  // pairs a run needs for the workgroup kernel; a shorter run is ruled out with one read
-  const uint32_t needed = (kWorkgroupWork + step_size - 1) / step_size;
-  if (i + 1 < needed || keys[i + 1 - needed] != transit) return false;
-  const uint32_t start = run_start(keys, i + 1 - needed, transit);
-  const uint32_t count = i + 1 - start;
+// A run of `count` pairs on `transit` that starts at pair `start`: should the workgroup kernel
+// take it?  Gives the run and the number of work items it needs.  refused_out (nullable): set to
+// the run's length when the run is long enough but stays with the flat kernel because of the degree.
+__device__ __forceinline__ bool workgroup_takes_run(uint32_t transit, uint32_t start, uint32_t count,
+                                                    const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
+                                                    uint32_t* transit_out, uint32_t* start_out, uint32_t* count_out,
+                                                    uint32_t* n_items_out, uint32_t* refused_out = nullptr,
+                                                    EdgePos_t* begin_out = nullptr, EdgePos_t* degree_out = nullptr) {
   const uint64_t work = (uint64_t)count * step_size;
   if (work < kWorkgroupWork) return false;
   const EdgePos_t begin = row_ptr[transit];
@@ -978,6 +973,21 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
   return true;
 }
 
+// Pair i, on `transit`, is the last of its run, whose start is not known: the same question.
+__device__ __forceinline__ bool workgroup_run_of_tail(const uint32_t* __restrict__ keys, uint32_t i, uint32_t transit,
+                                                      const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
+                                                      uint32_t* transit_out, uint32_t* start_out,
+                                                      uint32_t* count_out, uint32_t* n_items_out,
+                                                      uint32_t* refused_out = nullptr, EdgePos_t* begin_out = nullptr,
+                                                      EdgePos_t* degree_out = nullptr) {
+  // pairs a run needs for the workgroup kernel; a shorter run is ruled out with one read
+  const uint32_t needed = (kWorkgroupWork + step_size - 1) / step_size;
+  if (i + 1 < needed || keys[i + 1 - needed] != transit) return false;
+  const uint32_t start = run_start(keys, i + 1 - needed, transit);
+  return workgroup_takes_run(transit, start, i + 1 - start, row_ptr, step_size, transit_out, start_out, count_out,
+                             n_items_out, refused_out, begin_out, degree_out);
+}
+
 // Every lane looks at kClassifyItems consecutive pairs.  The work items of a workgroup's
 // runs are claimed with ONE atomic per workgroup or wavefront (atomics on a single counter are served
 // one after the other, ~10 ns each: one per run cost 3 ms on 1.5e5 qualifying runs); their
@@ -992,8 +1002,8 @@ __device__ __forceinline__ bool workgroup_run_ends_at(const uint32_t* __restrict
 // a step's classification decides never changes a result, only which kernel draws it.
 constexpr uint32_t kQuietLookEvery = 4;
 
-template <int kClassifyItems>
-__global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __restrict__ keys,
+template <int kClassifyItems, int kThreads = 256>
+__global__ __launch_bounds__(kThreads) void classify_run_tails(const uint32_t* __restrict__ keys,
                                                           const uint32_t* __restrict__ n_dev, RunsMeta* meta,
                                                           RunsMeta* meta_of_next_step,
                                                           const EdgePos_t* __restrict__ row_ptr, uint32_t step_size,
@@ -1001,7 +1011,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
                                                           uint32_t* __restrict__ taken_stamp,
                                                           ClassCounters* __restrict__ counters,
                                                           uint32_t* __restrict__ found_by_step, uint32_t step) {
-  __shared__ uint32_t s_wave[kScanThreads / kWave];
+  __shared__ uint32_t s_wave[kThreads / kWave];
   __shared__ uint32_t s_base;
   const uint32_t n = *n_dev;
   const uint32_t stamp = meta->stamp;
@@ -1014,16 +1024,73 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   }
   if (step > 2 && found_by_step[step - 1] == 0 && found_by_step[step - 2] == 0 && step % kQuietLookEvery != 0) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&counters->sorted_pairs, (unsigned long long)n);
-  const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kClassifyItems;
+  const uint64_t first = ((uint64_t)blockIdx.x * kThreads + threadIdx.x) * kClassifyItems;
   uint32_t transit, start, count, n_items;
   EdgePos_t begin = 0, degree = 0;
+  // the first run the lane found stays in registers for the second sweep (few lanes find two)
+  int kept_k = -1;
+  uint32_t kept_transit = 0, kept_start = 0, kept_count = 0, kept_items = 0;
+  EdgePos_t kept_begin = 0, kept_degree = 0;
   uint32_t mine = 0;
   uint32_t single_pairs = 0, split_pairs = 0, refused_pairs = 0;
+  // the lane's keys and the one after them, fetched together (16 bytes at a time where the lane
+  // has a multiple of four keys and all of them exist): only the last pair of a run reads more
+  uint32_t held[kClassifyItems + 1];
+  if (kClassifyItems % 4 == 0 && first + kClassifyItems < n && (reinterpret_cast<uintptr_t>(keys) & 15u) == 0) {
+#pragma unroll
+    for (int k = 0; k < kClassifyItems; k += 4) {
+      const uint4 four = *reinterpret_cast<const uint4*>(keys + first + k);
+      held[k] = four.x;
+      held[k + 1] = four.y;
+      held[k + 2] = four.z;
+      held[k + 3] = four.w;
+    }
+    held[kClassifyItems] = keys[first + kClassifyItems];
+  } else {
+#pragma unroll
+    for (int k = 0; k <= kClassifyItems; ++k) held[k] = first + k < n ? keys[first + k] : 0u;
+  }
+  uint32_t tails = 0;  // bit k: pair first + k is the last of its run
+#pragma unroll
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
+    if (i < n && (i + 1 == n || held[k + 1] != held[k])) tails |= 1u << k;
+  }
+  // Where the run that a lane's first tail closes starts: after the last tail of the lanes
+  // before it in the wavefront (their keys are the ones just before the lane's own).  Only a
+  // run that began before the wavefront's first key is searched for in memory.
+  uint32_t start_known;  // 0: not known; else the start of the run the next tail closes
+  {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    uint32_t after_last = tails ? (uint32_t)first + (31u - (uint32_t)__clz(tails)) + 1u : 0u;
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint32_t other = __shfl_up(after_last, d, kWave);
+      if (lane >= (uint32_t)d && other > after_last) after_last = other;
+    }
+    start_known = __shfl_up(after_last, 1, kWave);
+    if (lane == 0) start_known = 0;
+  }
+#pragma unroll
+  for (int k = 0; k < kClassifyItems; ++k) {
     uint32_t refused = 0;
-    if (i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items,
-                                       &refused, &begin, &degree)) {
+    if (((tails >> k) & 1u) == 0) continue;
+    const uint32_t i = (uint32_t)(first + k);
+    const bool takes = start_known != 0
+                           ? workgroup_takes_run(held[k], start_known, i + 1 - start_known, row_ptr, step_size,
+                                                 &transit, &start, &count, &n_items, &refused, &begin, &degree)
+                           : workgroup_run_of_tail(keys, i, held[k], row_ptr, step_size, &transit, &start, &count,
+                                                   &n_items, &refused, &begin, &degree);
+    start_known = i + 1;
+    if (takes) {
+      if (kept_k < 0) {
+        kept_k = k;
+        kept_transit = transit;
+        kept_start = start;
+        kept_count = count;
+        kept_items = n_items;
+        kept_begin = begin;
+        kept_degree = degree;
+      }
       mine += n_items;
       if (n_items > 1) split_pairs += count; else single_pairs += count;
     }
@@ -1039,7 +1106,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
       items += __shfl_xor(items, d, kWave);
     }
     if ((threadIdx.x & (kWave - 1)) == 0) {
-      ClassCounters* mine_c = counters + ((blockIdx.x * (256 / kWave) + threadIdx.x / kWave) % kCounterCopies);
+      ClassCounters* mine_c = counters + ((blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave) % kCounterCopies);
       if (single_pairs) atomicAdd(&mine_c->workgroup_pairs, (unsigned long long)single_pairs);
       if (split_pairs) atomicAdd(&mine_c->split_pairs, (unsigned long long)split_pairs);
       if (refused_pairs) atomicAdd(&mine_c->refused_pairs, (unsigned long long)refused_pairs);
@@ -1057,7 +1124,7 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
     base = __shfl(wave_base, kWave - 1, kWave) + incl - mine;
   } else {
     uint32_t block_total;
-    base = block_exclusive_scan_256(mine, s_wave, &block_total);
+    base = block_exclusive_scan<kThreads>(mine, s_wave, &block_total);
     if (block_total == 0) return;  // the same for every lane of the workgroup
     if (threadIdx.x == 0) s_base = atomicAdd(&meta->n_chunks, block_total);
     __syncthreads();
@@ -1069,10 +1136,20 @@ __global__ __launch_bounds__(256) void classify_run_tails(const uint32_t* __rest
   for (int k = 0; k < kClassifyItems; ++k) {
     const uint64_t i = first + k;
     // one pair per lane: the run found above is still in the registers
-    if (kClassifyItems > 1 &&
-        !(i < n && workgroup_run_ends_at(keys, (uint32_t)i, n, row_ptr, step_size, &transit, &start, &count, &n_items,
-                                         nullptr, &begin, &degree)))
-      continue;
+    if (kClassifyItems > 1) {
+      if (k == kept_k) {
+        transit = kept_transit;
+        start = kept_start;
+        count = kept_count;
+        n_items = kept_items;
+        begin = kept_begin;
+        degree = kept_degree;
+      } else if (!(k > kept_k && ((tails >> k) & 1u) != 0 &&
+                   workgroup_run_of_tail(keys, (uint32_t)i, keys[i], row_ptr, step_size, &transit, &start, &count,
+                                         &n_items, nullptr, &begin, &degree))) {
+        continue;
+      }
+    }
     const bool fits = base + n_items <= chunk_capacity;
     for (uint32_t g = 0; g < n_items && base + g < chunk_capacity; ++g) {
       const uint32_t off = g * pairs_per_chunk;
@@ -1205,7 +1282,7 @@ __global__ __launch_bounds__(256) void small_map_place(
     }
   }
   if (!classify) return;
-  // the run's class, decided by its first pair (rules of workgroup_run_ends_at)
+  // the run's class, decided by its first pair (rules of workgroup_run_of_tail)
   EdgePos_t begin = 0;
   uint32_t degree = 0;
   if (head) {
@@ -1926,8 +2003,10 @@ class Engine : public EngineBase {
             RunsMeta* meta_next = d_meta_ + ((balanced_steps_ + 1) & 1);
             balanced_steps_++;
             if (n_pairs >= kClassifyLargeFrom) {
-              const unsigned tail_blocks = (n_pairs + 256 * kClassifyItemsLarge - 1) / (256 * kClassifyItemsLarge);
-              classify_run_tails<kClassifyItemsLarge><<<dim3(tail_blocks), dim3(256), 0, stream_>>>(
+              const unsigned per_block = kClassifyThreadsLarge * kClassifyItemsLarge;
+              const unsigned tail_blocks = (n_pairs + per_block - 1) / per_block;
+              classify_run_tails<kClassifyItemsLarge, kClassifyThreadsLarge>
+                  <<<dim3(tail_blocks), dim3(kClassifyThreadsLarge), 0, stream_>>>(
                   sorted_keys, live_now, meta, meta_next, dgraph_->row_ptr(), m, d_chunks_, chunk_capacity_,
                   d_taken_stamp_, counters_dev(), d_balance_, (uint32_t)step);
             } else {
