@@ -2024,8 +2024,7 @@ class Engine : public EngineBase {
       if (explicit_map_) {
         transits = d_explicit_;  // one entry per output slot, no rows
       } else if (rows_direct_) {
-        transits_layout.seg_len = layout_.seg_len[step];
-        transits_layout.pitch = (uint32_t)F;
+        transits_layout.rows(layout_.seg_len[step], (uint32_t)F);
       }
       transits_per_sample *= m;
     }

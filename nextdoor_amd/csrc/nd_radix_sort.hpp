@@ -50,8 +50,22 @@ __device__ __forceinline__ int tile_offset(int wave, int it, int lane) {
 struct KeyLayout {
   uint32_t seg_len = 0;  // 0: contiguous
   uint32_t pitch = 0;
+  uint64_t magic = 0;    // floor(2^64 / seg_len) + 1 (2^64 / seg_len for a power of two): i / seg_len is the
+                         // upper half of i * magic for every i below 2^32, without a division per key
+  void rows(uint32_t segment, uint32_t row_pitch) {
+    seg_len = segment;
+    pitch = row_pitch;
+    magic = segment ? ~0ull / segment + 1ull : 0ull;
+  }
   __host__ __device__ size_t at(size_t i) const {
-    return seg_len ? (i / seg_len) * (size_t)pitch + i % seg_len : i;
+    if (seg_len == 0) return i;
+    if (seg_len == 1) return i * (size_t)pitch;  // (no 64-bit magic for 1)
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint64_t row = __umul64hi((uint64_t)i, magic);  // i < 2^32: the sorts take at most 2^32 - 1 keys
+#else
+    const uint64_t row = i / seg_len;
+#endif
+    return row * (size_t)pitch + (i - row * seg_len);
   }
 };
 
