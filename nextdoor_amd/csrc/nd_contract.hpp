@@ -195,22 +195,19 @@ __host__ __device__ __forceinline__ bool binarySearch(F& array, T x, int size) {
 
 namespace nd {
 
-// Adjacency of the current transit staged in LDS: entries [0, cached) come from LDS,
-// the rest from HBM.  One of the two EdgeArray / WeightArray types an App::next is
-// instantiated with (the other is a plain pointer); only operator[] is required
-// (the reference's CachedArray, src/nextdoor.cu:76-124, plays this role).
-// The LDS half is held as a pointer in the LDS address space, so reads of it are plain LDS
-// loads and no generic-pointer test is generated.
+// Adjacency of the current transit staged in LDS, all of it (a transit whose adjacency does
+// not fit is not given to the workgroup class).  One of the EdgeArray / WeightArray types an
+// App::next is instantiated with (the other is a plain pointer); only operator[] is required
+// (the reference's CachedArray, src/nextdoor.cu:76-124, plays this role).  The array is held
+// as a pointer in the LDS address space, so reads of it are plain LDS loads: no generic-pointer
+// test, and no branch to a copy in memory whose possible load every LDS read would wait for.
 #if defined(__HIPCC__)
 template <typename T>
-struct LdsBackedArray {
+struct LdsArray {
   typedef const __attribute__((address_space(3))) T* LdsPointer;
   LdsPointer lds;
-  const T* global;
-  EdgePos_t cached;
-  __device__ __forceinline__ LdsBackedArray(const T* lds_array, const T* global_array, EdgePos_t n_cached)
-      : lds((LdsPointer)lds_array), global(global_array), cached(n_cached) {}
-  __device__ __forceinline__ T operator[](EdgePos_t i) const { return i < cached ? lds[i] : global[i]; }
+  __device__ __forceinline__ explicit LdsArray(const T* lds_array) : lds((LdsPointer)lds_array) {}
+  __device__ __forceinline__ T operator[](EdgePos_t i) const { return lds[i]; }
 };
 #endif
 

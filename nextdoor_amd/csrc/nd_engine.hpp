@@ -280,8 +280,13 @@ constexpr int kStepThreads = 256;
 #define ND_FLAT_THREADS 64
 #endif
 constexpr int kFlatThreads = ND_FLAT_THREADS;
-// LDS adjacency cache of the workgroup kernel, in edges.
-constexpr int kCacheEdges = 8192;
+// LDS adjacency cache of the workgroup kernel, in edges (k-hop pass with 8192 / 6144 / 4096: 3.58 / 3.75 /
+// 3.87 ms - a smaller cache lets more workgroups share a compute unit, but hands the flat kernel
+// more of the hubs than that wins).
+#ifndef ND_CACHE_EDGES
+#define ND_CACHE_EDGES 8192
+#endif
+constexpr int kCacheEdges = ND_CACHE_EDGES;
 // A transit goes to the workgroup kernel when at least this many outputs are drawn from it.
 constexpr uint32_t kWorkgroupWork = 256;
 // Outputs one work item of the workgroup kernel covers at most; larger runs are split
@@ -389,6 +394,8 @@ __device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition
 
 // Output q (index inside the sample's segment of this step) is INVALID: so is everything the
 // later steps would have drawn from it (StepParams::fill_levels).
+// (Inlined although it is rare and repeated at every store: a call from a step kernel costs the
+// kernel its register allocation - the k-hop pass took 9.9 ms instead of 3.5 with this out of line.)
 __device__ __forceinline__ void fill_below(const StepParams& P, uint32_t sample, uint32_t q) {
   int32_t* row = P.step_out + (size_t)sample * P.out_pitch;
 #pragma unroll
@@ -466,9 +473,11 @@ struct __attribute__((packed, aligned(4))) FourIds {
 // step_size > 1.  In two halves, so that a lane that works through several groups can have
 // the gathers of the next group under way while the results of this one are stored.
 struct GroupOutputs {
-  uint64_t first, lo, hi;  // global slots: the pair's output 0, the group's outputs [lo, hi)
+  uint64_t first;     // global slot of the pair's output 0
+  uint64_t base;      // global slot of the group's word 0 (a multiple of four)
+  uint32_t from, to;  // the words [from, to) of the group belong to the pair
   uint32_t sample;
-  VertexID neighbor[4], next_transit[4];
+  VertexID neighbor[4], next_transit[4];  // by word
 };
 
 template <class SampleType, class App, class EdgeArray, class WeightArray>
@@ -477,38 +486,40 @@ __device__ __forceinline__ void compute_group(const StepParams& P, CSRPartition&
                                               EdgeArray& edges, WeightArray& weights, GroupOutputs* out) {
   const uint64_t first = P.first_slot + (uint64_t)pair_slot * P.step_size;  // global slot of the pair's output 0
   const uint64_t group = (first >> 2) + gi;
-  const uint64_t lo = group * 4 > first ? group * 4 : first;
+  const uint64_t base = group * 4;
   const uint64_t end = first + P.step_size;
-  const uint64_t hi = group * 4 + 4 < end ? group * 4 + 4 : end;
   out->first = first;
-  out->lo = lo;
-  out->hi = hi;
-  if (lo >= hi) return;
+  out->base = base;
+  out->from = base < first ? (uint32_t)(first - base) : 0u;
+  out->to = base + 4 <= end ? 4u : (end > base ? (uint32_t)(end - base) : 0u);
+  if (out->from >= out->to) return;
   PhiloxBlock block = PhiloxBlock();
   // next() draws for a real transit with edges; stepTransits for any real transit (run_app)
   if (transit != P.invalid && (n_edges != 0 || (App().hasExplicitTransits() && !P.is_last)))
-    block = grouped_first_block(P.seed, group, (uint32_t)P.step);
+    block = grouped_first_block_scalar_seed(P.seed, group, (uint32_t)P.step);
   out->sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
-  // all draws of the group before any store: its up to four gathers are under way together
+  // all draws of the group before any store: its up to four gathers are under way together.
+  // Word w of the block belongs to slot base + w: which word an output takes is known when
+  // the loop is unrolled, nothing is selected at run time.
 #pragma unroll
-  for (uint32_t q = 0; q < 4; ++q) {
-    out->neighbor[q] = out->next_transit[q] = P.invalid;
-    if (lo + q < hi)
+  for (uint32_t w = 0; w < 4; ++w) {
+    out->neighbor[w] = out->next_transit[w] = P.invalid;
+    if (w >= out->from && w < out->to)
       compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, out->sample,
-                                                              (uint32_t)(lo + q - first), n_edges, max_weight, edges,
-                                                              weights, true, block_word(block, (uint32_t)(lo + q) & 3u),
-                                                              &out->neighbor[q], &out->next_transit[q]);
+                                                              (uint32_t)(base + w - first), n_edges, max_weight, edges,
+                                                              weights, true, block.w[w], &out->neighbor[w],
+                                                              &out->next_transit[w]);
   }
 }
 
 __device__ __forceinline__ void store_group(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
                                             const GroupOutputs& g) {
-  if (g.lo >= g.hi) return;
-  if (g.hi - g.lo == 4 && !P.pair_cells && !P.explicit_out && !P.emit_keys) {
+  if (g.from >= g.to) return;
+  if (g.from == 0 && g.to == 4 && !P.pair_cells && !P.explicit_out && !P.emit_keys) {
     // a whole group whose outputs are all there is to store: the four ids are neighbours in
     // the step's results (word aligned, not more), and go out as one 16-byte store
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
-    const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + (g.lo - g.first);
+    const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + (g.base - g.first);
     const uint32_t q = (uint32_t)(out_slot - (uint64_t)g.sample * per_sample);
     FourIds* dst = reinterpret_cast<FourIds*>(P.step_out + (size_t)g.sample * P.out_pitch + q);
     *dst = FourIds{g.neighbor[0], g.neighbor[1], g.neighbor[2], g.neighbor[3]};
@@ -520,10 +531,10 @@ __device__ __forceinline__ void store_group(const StepParams& P, VertexID transi
     return;
   }
 #pragma unroll
-  for (uint32_t q = 0; q < 4; ++q)
-    if (g.lo + q < g.hi)
-      store_output(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.lo + q - g.first), g.neighbor[q],
-                   g.next_transit[q]);
+  for (uint32_t w = 0; w < 4; ++w)
+    if (w >= g.from && w < g.to)
+      store_output(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.base + w - g.first), g.neighbor[w],
+                   g.next_transit[w]);
 }
 
 // The groups first, first + stride, ... of a pair, the draws of a group made before the
@@ -534,7 +545,8 @@ __device__ __forceinline__ void produce_groups(const StepParams& P, CSRPartition
                                                EdgePos_t n_edges, float max_weight, EdgeArray& edges,
                                                WeightArray& weights) {
   GroupOutputs held;
-  held.first = held.lo = held.hi = 0;  // nothing held yet
+  held.first = held.base = 0;
+  held.from = held.to = 0;  // nothing held yet
   for (uint32_t gi = first_group; gi < P.groups_per_pair; gi += stride) {
     GroupOutputs now;
     compute_group<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, gi, n_edges, max_weight,
@@ -750,7 +762,9 @@ struct alignas(16) WorkItem {
 // and has the loads of ALL its rounds under way before it writes the first to LDS: a loop of
 // "load one word, wait, write it" costs a memory round trip per 256 words - for a
 // 2000-edge adjacency eight trips one after the other, and the workgroup class spent most of
-// its time there.
+// its time there.  (Holding the words of the NEXT work item in registers while the workgroup
+// draws from this one's adjacency was measured too: 31 more registers per lane, four wavefronts
+// per SIMD instead of five, and the k-hop launch 9 % slower.)
 template <class T>
 __device__ __forceinline__ void stage_into_lds(const T* __restrict__ src, T* lds, EdgePos_t count) {
   static_assert(sizeof(T) == 4, "32-bit words");
@@ -807,8 +821,10 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
     const EdgePos_t cached = n_edges < kCacheEdges ? n_edges : kCacheEdges;
     // Lanes per pair: one, or the power of two (at most the groups of four output slots a pair
     // has) that the item's pairs leave room for in the workgroup; lane `sub` of a pair takes the
-    // pair's groups sub, sub + L, ...  The slot of a lane's first pair is fetched together with
-    // the adjacency, not after it.
+    // pair's groups sub, sub + L, ...  (Dealing the (pair, group) tasks of an item to the lanes
+    // one by one keeps more lanes busy - 94 instead of 59 % for 100 pairs of three groups - and
+    // was slower: 1.23 against 1.17 ms for the k-hop launch, which does not wait for its lanes.)
+    // The slot of a lane's first pair is fetched together with the adjacency, not after it.
     uint32_t lanes_shift = 0;
     while ((1u << lanes_shift) < P.groups_per_pair && (n_pairs << (lanes_shift + 1)) <= (uint32_t)kStepThreads) lanes_shift++;
     const uint32_t lanes = n_pairs << lanes_shift;
@@ -817,18 +833,23 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
     stage_into_lds(csr.edges + begin, s_edges, cached);
     if (kWeights) stage_into_lds(csr.weights + begin, s_weights, cached);
     __syncthreads();
-    LdsBackedArray<CSR::Edge> edges{s_edges, csr.edges + begin, cached};
-    LdsBackedArray<float> lds_weights{s_weights, csr.weights + begin, kWeights ? cached : 0};
+    // the classification hands over no transit whose adjacency exceeds the cache
+    LdsArray<CSR::Edge> edges{s_edges};
+    typedef typename std::conditional<kWeights, LdsArray<float>, const float*>::type Weights;
+    Weights weights_of_transit = [&]() {
+      if constexpr (kWeights) return LdsArray<float>{s_weights};
+      else return csr.weights + begin;
+    }();
     for (uint32_t t = threadIdx.x; t < lanes; t += kStepThreads) {
       const uint32_t p = t >> lanes_shift;
       if (t != threadIdx.x) slot = P.pair_slots[first_pair + p];
       if (P.groups_per_pair == 0) {  // one output per pair
-        produce_output<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
-            P, csr, transit, first_pair + p, slot, 0, n_edges, max_weight, edges, lds_weights);
+        produce_output<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot, 0, n_edges,
+                                                                      max_weight, edges, weights_of_transit);
       } else {
-        produce_groups<SampleType, App, LdsBackedArray<CSR::Edge>, LdsBackedArray<float>>(
-            P, csr, transit, first_pair + p, slot, t & ((1u << lanes_shift) - 1u), 1u << lanes_shift, n_edges,
-            max_weight, edges, lds_weights);
+        produce_groups<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot,
+                                                                      t & ((1u << lanes_shift) - 1u), 1u << lanes_shift,
+                                                                      n_edges, max_weight, edges, weights_of_transit);
       }
     }
     first_pair = coming_first_pair;

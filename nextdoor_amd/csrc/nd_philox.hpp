@@ -79,6 +79,24 @@ ND_HD PhiloxBlock grouped_first_block(uint64_t seed, uint64_t group, uint32_t st
                        (uint32_t)(seed >> 32));
 }
 
+// The same for a seed that is the same for every lane (a kernel argument).  The ten round keys
+// are then scalars, and the compiler, seeing that they never change, computes all twenty words
+// once per kernel and keeps them - more scalar registers than a step kernel has to spare, so
+// they end up parked in lanes of a vector register and every use is a vector-pipe read (a fifth
+// of the block's vector instructions).  The empty statement makes the key opaque at this point:
+// the rounds add their constants on the scalar unit as they go.
+ND_HD PhiloxBlock grouped_first_block_scalar_seed(uint64_t seed, uint64_t group, uint32_t step) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // (read from the first lane: a no-op for a value that is in scalar registers already, and
+  // what makes it one where the compiler has moved the kernel's arguments to vector registers)
+  uint32_t k0 = __builtin_amdgcn_readfirstlane((uint32_t)seed), k1 = __builtin_amdgcn_readfirstlane((uint32_t)(seed >> 32));
+  asm volatile("" : "+s"(k0), "+s"(k1));
+  return philox4x32_10((uint32_t)group, (uint32_t)(group >> 32), step | kGroupedStepFlag, 0u, k0, k1);
+#else
+  return grouped_first_block(seed, group, step);
+#endif
+}
+
 // Word i (0..3) of a block, by comparisons: an index into the array would put it in memory.
 ND_HD uint32_t block_word(const PhiloxBlock& b, uint32_t i) {
   return i == 0 ? b.w[0] : i == 1 ? b.w[1] : i == 2 ? b.w[2] : b.w[3];
