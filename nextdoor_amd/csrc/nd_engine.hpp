@@ -501,6 +501,39 @@ __device__ __forceinline__ void compute_group(const StepParams& P, CSRPartition&
   // all draws of the group before any store: its up to four gathers are under way together.
   // Word w of the block belongs to slot base + w: which word an output takes is known when
   // the loop is unrolled, nothing is selected at run time.
+  if (std::is_empty<SampleType>::value && !App().hasExplicitTransits()) {
+    // An app without sample state draws nothing but its result: all four words are drawn, whether
+    // the pair owns them or not, and those it does not own are dropped afterwards.  Without a
+    // branch around each draw the four gathers are issued one after the other and waited for
+    // once; with it, each waited for its own (and for the stores of the group before).
+    // (Looking at what next() returned only after the stores of the lane's previous group have
+    // been issued, so that the gathers do not queue behind those stores: no gain, 1.26 against
+    // 1.24 ms for the k-hop flat launches.)
+    VertexID drawn[4] = {P.invalid, P.invalid, P.invalid, P.invalid};
+    if (transit != P.invalid && n_edges != 0) {  // next() only runs for a real transit that has edges (run_app)
+      const VertexID sample_id = (VertexID)(P.first_sample + out->sample);
+      VertexID at = transit;
+      SampleType no_state;
+      VertexID r[4];
+#pragma unroll
+      for (uint32_t w = 0; w < 4; ++w) {
+        const bool owned = w >= out->from && w < out->to;
+        curandState rng;
+        rng.reset_with_first(P.seed, base + w, (uint32_t)P.step, block.w[w]);
+        r[w] = App().template next<SampleType, EdgeArray, WeightArray>(
+            P.step, &csr, &at, sample_id, &no_state, max_weight, edges, weights, n_edges,
+            (VertexID_t)(owned ? (uint32_t)(base + w - first) : 0u), &rng);
+      }
+#pragma unroll
+      for (uint32_t w = 0; w < 4; ++w) drawn[w] = r[w] == -1 ? P.invalid : r[w];  // nextdoor.cu:288
+    }
+#pragma unroll
+    for (uint32_t w = 0; w < 4; ++w) {
+      const bool owned = w >= out->from && w < out->to;
+      out->neighbor[w] = out->next_transit[w] = owned ? drawn[w] : P.invalid;
+    }
+    return;
+  }
 #pragma unroll
   for (uint32_t w = 0; w < 4; ++w) {
     out->neighbor[w] = out->next_transit[w] = P.invalid;
