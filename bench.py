@@ -26,31 +26,42 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes one launch of the dominant kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
-# this script (profiles/step_kernels_<workload>_hbm_traffic.md; counters scaled by a plain copy of
-# known size).  None where no such run has been recorded.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 1.119e9,     # step_flat_kernel
-    "uniform_walk_chunglu57k": 6.233e6,      # step_flat_kernel
-    "khop_rmat21": 3.265e9,                  # step kernels of one hop (2 x flat 2.024e9 + workgroup 2.482e9, over 2 hops)
-    "fastgcn_importance_rmat22": 5.28e9,     # collective_mark_binned, average over its 2 launches per pass
-    "ladies_importance_chunglu3m": 6.727e10,  # collective_mark_binned, average over its 2 launches per pass
-}
-# HBM bytes of all kernels of one pass, same source.
-MEASURED_TRAFFIC_BYTES_PER_PASS = {
-    "weighted_node2vec_rmat22": 149.1e9, "uniform_walk_chunglu57k": 1.31e9, "khop_rmat21": 13.54e9,
-    "fastgcn_importance_rmat22": 16.44e9, "ladies_importance_chunglu3m": 161.15e9,
+# What rocprofv3 counter runs of this script recorded (the summaries under profiles/; a test compares
+# these constants with the tables there).  Per profile: the dominant kernel(s), the HBM bytes one
+# launch of it moves (FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of known size:
+# profiles/step_kernels_<profile>_hbm_traffic.md) and the HBM bytes of all kernels of a pass; where
+# recorded, the read and write requests one launch sends past L2 (TCC_EA0_RDREQ_sum - every one of
+# them 128 bytes - and TCC_EA0_WRREQ_sum: profiles/step_kernels_<profile>_l2_requests.md).
+MEASURED = {
+    "weighted_node2vec_rmat22": {
+        "kernels": {"nd::step_flat_kernel": 1.122e9}, "bytes_per_pass": 149.35e9,
+        "read_requests": {"nd::step_flat_kernel": 8.235e6}, "write_requests": {"nd::step_flat_kernel": 1.672e6}},
+    # the same workload with --inversion-period 0 (the engine's choice: walks keep their lanes)
+    "weighted_node2vec_rmat22_period0": {
+        "kernels": {"nd::walk_stretch_kernel": 3.675e10}, "bytes_per_pass": 152.72e9,
+        "read_requests": {"nd::walk_stretch_kernel": 2.843e8}, "write_requests": {"nd::walk_stretch_kernel": 6.466e6}},
+    "uniform_walk_chunglu57k": {"kernels": {"nd::step_balanced_kernel": 6.046e6}, "bytes_per_pass": 1.31e9},
+    # both kernel classes of a hop; the flat kernel is launched for both hops, the workgroup kernel for the second
+    "khop_rmat21": {"kernels": {"nd::step_flat_kernel": 1.208e9, "nd::step_workgroup_kernel": 2.402e9},
+                    "bytes_per_pass": 9.00e9},
+    # collective_mark_binned, average over its 2 launches per pass
+    "fastgcn_importance_rmat22": {"kernels": {"nd::collective_mark_binned": 5.274e9}, "bytes_per_pass": 16.43e9},
+    "ladies_importance_chunglu3m": {"kernels": {"nd::collective_mark_binned": 6.735e10}, "bytes_per_pass": 161.30e9},
 }
 
-# Read requests one launch of the dominant kernel sends past L2 (rocprofv3 TCC_EA0_RDREQ_sum, every
-# one of them 128 bytes: profiles/step_kernels_<workload>_l2_requests.md).  None where not recorded.
-MEASURED_L2_MISS_REQUESTS_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 8.21e6,      # step_flat_kernel
-}
-# Write requests of the same launch to memory (TCC_EA0_WRREQ_sum, same summary).
-MEASURED_L2_WRITE_REQUESTS_PER_LAUNCH = {
-    "weighted_node2vec_rmat22": 1.67e6,      # step_flat_kernel; 0.46 M of them 64-byte, the rest 32-byte
-}
+
+def _one(values):
+    return next(iter(values.values()))
+
+
+# HBM bytes per launch of the dominant kernel (k-hop: the step kernels of one hop = the two flat
+# launches and the workgroup launch of a pass, over its 2 hops)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {name: _one(m["kernels"]) for name, m in MEASURED.items() if len(m["kernels"]) == 1}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH["khop_rmat21"] = (2 * MEASURED["khop_rmat21"]["kernels"]["nd::step_flat_kernel"] +
+                                                     MEASURED["khop_rmat21"]["kernels"]["nd::step_workgroup_kernel"]) / 2
+MEASURED_TRAFFIC_BYTES_PER_PASS = {name: m["bytes_per_pass"] for name, m in MEASURED.items()}
+MEASURED_L2_MISS_REQUESTS_PER_LAUNCH = {name: _one(m["read_requests"]) for name, m in MEASURED.items() if "read_requests" in m}
+MEASURED_L2_WRITE_REQUESTS_PER_LAUNCH = {name: _one(m["write_requests"]) for name, m in MEASURED.items() if "write_requests" in m}
 
 WORKLOADS = {
     # name: (app, graph factory kwargs)
@@ -358,9 +369,20 @@ def measure(args, workload, steps, warmup, cpu_seconds, graphs, engine_choice=Tr
         # thousand pieces are served by the caches and are reported apart, not as HBM bytes
         achieved = from_memory / (prof["neighbourhood_ms"] / 1000.0) / 1e9
         all_uses = mark_bytes / (prof["neighbourhood_ms"] / 1000.0) / 1e9
+        # what the recorded counters say the launch is bound by: its measured HBM traffic over this
+        # run's launch time.  The LADIES form streams (entries in, keys out: near half of the HBM
+        # peak); the FastGCN form moves a fifth of the peak - its hubs' pieces and adjacencies come
+        # from the caches, and a workgroup spends its time in the chain of searches, LDS table and
+        # barriers it goes through per stretch of the vertex range
+        recorded = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload)
+        traffic_gbps = recorded / (prof["neighbourhood_ms"] / launches / 1000.0) / 1e9 if recorded else None
+        bound = "hbm" if traffic_gbps is None or traffic_gbps / HBM_PEAK_GBS >= 0.3 else \
+            "latency (dependent steps per stretch of the vertex range; the caches serve the hubs)"
         result["roofline"] = {
-            "bound": "hbm", "kernel": "collective_mark_binned", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload),
+            "bound": bound, "kernel": "collective_mark_binned", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": recorded,
+            "measured_traffic_GBps": traffic_gbps,
+            "measured_traffic_frac": traffic_gbps / HBM_PEAK_GBS if traffic_gbps else None,
             "algorithmic_bytes_per_launch": from_memory / launches,
             "avg_launch_ms": prof["neighbourhood_ms"] / launches,
             "cache_served": {"bytes_per_launch_with_every_piece_use": mark_bytes / launches,
@@ -427,6 +449,23 @@ def measure(args, workload, steps, warmup, cpu_seconds, graphs, engine_choice=Tr
                            "measured_traffic": MEASURED_TRAFFIC_BYTES_PER_PASS.get(workload)},
         }
         result["config"]["bytes_per_sampled_edge"] = (step_bytes + sort_bytes) / edges_per_pass
+        if adaptive:
+            # the same accounting for the pass with the engine-chosen inversion period: the step
+            # kernels' algorithmic bytes are those of the algorithm, whatever the schedule
+            chosen_ms = adaptive["phases_ms"]["flat_kernel_ms"]
+            chosen_launches = max(adaptive["phases_ms"]["flat_launches"], 1)
+            period0 = MEASURED.get(workload + "_period0")
+            adaptive["roofline"] = {
+                "bound": "hbm", "kernel": "walk_stretch_kernel (and step_flat_kernel for step 0)",
+                "achieved": step_bytes / (chosen_ms / 1000.0) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": step_bytes / (chosen_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
+                "algorithmic_bytes_per_launch": step_bytes / chosen_launches,
+                "avg_launch_ms": chosen_ms / chosen_launches,
+                "traffic": _one(period0["kernels"]) if period0 else None,
+                "whole_pass": {"measured_traffic": period0["bytes_per_pass"] if period0 else None,
+                               "measured_traffic_GBps": period0["bytes_per_pass"] / (adaptive["ms_per_step"] / 1000.0) / 1e9
+                               if period0 else None},
+            }
         traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload)
         if traffic and w["kind"] != "KHOP":  # walks: the recorded figure is the flat kernel's launch
             # recorded counter traffic of one launch over this run's launch duration (flat kernel alone)
@@ -458,6 +497,18 @@ def measure(args, workload, steps, warmup, cpu_seconds, graphs, engine_choice=Tr
                 "reads_and_writes_over_read_ceiling": (misses + writes) / (flat_ms / 1000.0) / ceiling,
                 "ceiling_as_GBps": ceiling * 128 / 1e9,
             }
+            period0 = MEASURED.get(workload + "_period0")
+            if adaptive and "roofline" in adaptive and period0 and "read_requests" in period0:
+                # the stretch kernel against the same ceiling: its recorded requests per launch (the
+                # average over a pass's stretches) times the stretches of this pass, over the time
+                # of the pass's step kernels (which includes the one flat launch of step 0)
+                stretches = max(adaptive["phases_ms"]["flat_launches"] - 1, 1)
+                reads = _one(period0["read_requests"]) * stretches
+                chosen_s = adaptive["phases_ms"]["flat_kernel_ms"] / 1000.0
+                adaptive["roofline"]["l2_miss_path"] = {
+                    "read_requests_per_pass": reads, "write_requests_per_pass": _one(period0["write_requests"]) * stretches,
+                    "achieved_read_requests_per_s": reads / chosen_s, "ceiling_requests_per_s": ceiling,
+                    "frac_of_ceiling": reads / chosen_s / ceiling}
     del final
     sampler.close()
     return result
@@ -479,6 +530,9 @@ def summary(r):
     if "engine_chosen_inversion_period" in r["config"]:
         e = r["config"]["engine_chosen_inversion_period"]
         out["engine_chosen_inversion_period"] = {k: e[k] for k in ("ms_per_step", "sampled_edges_per_s", "same_samples")}
+        if "roofline" in e:
+            out["engine_chosen_inversion_period"]["roofline"] = {k: e["roofline"][k] for k in ("kernel", "frac", "avg_launch_ms",
+                                                                                              "algorithmic_bytes_per_launch")}
     if "roofline" in r:
         out["roofline"] = {k: r["roofline"][k] for k in ("kernel", "bound", "frac", "achieved", "avg_launch_ms",
                                                          "algorithmic_bytes_per_launch", "traffic") if k in r["roofline"]}
