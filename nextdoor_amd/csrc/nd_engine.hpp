@@ -224,6 +224,10 @@ struct StepParams {
   // one scattered store per two steps instead of two.  nullptr: step_out as described above.
   int32_t* pair_cells;
   uint32_t pair_cell_samples;
+  // With the cells: walk_cells[s] = how many cells of walk s hold results, written once per pass
+  // by the step at which the walk ends (its result is INVALID, or it is the last step).  The
+  // regrouping reads only those cells, so nothing fills the cells before a pass.
+  uint32_t* walk_cells;
   void* samples;                 // SampleType[S] or nullptr
   // Apps with explicit transits that are not walks: the (sample -> transit) map of step k+1,
   // indexed like step_out's own array form (output slot o of this step is pair o of the next):
@@ -336,6 +340,12 @@ __device__ __forceinline__ VertexID run_app(const StepParams& P, CSRPartition& c
 // The result of a walk's step into the cells two steps share (StepParams::pair_cells).  An even
 // step leaves its result to the odd step that follows - a walk that ends at the even step has
 // INVALID there, which the cell holds already - unless it is the last step of all.
+// Cells of a walk that hold results when the walk ends at `step`: an odd step has just written
+// cell (step - 1) / 2; an even step writes its cell only when it is the last step of all.
+__device__ __forceinline__ uint32_t walk_cells_at_end(int step, bool last_of_all) {
+  return (step & 1) ? (uint32_t)(step + 1) / 2u : (uint32_t)step / 2u + (last_of_all ? 1u : 0u);
+}
+
 __device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t sample, VertexID transit,
                                                   VertexID neighbor, int step) {
   int32_t* cell = P.pair_cells + ((size_t)(step >> 1) * P.pair_cell_samples + sample) * 2;
@@ -344,6 +354,7 @@ __device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t 
   } else if (P.is_last) {
     cell[0] = neighbor;
   }
+  if (P.walk_cells && (P.is_last || neighbor == P.invalid)) P.walk_cells[sample] = walk_cells_at_end(step, P.is_last);
 }
 __device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t sample, VertexID transit,
                                                   VertexID neighbor) {
@@ -755,6 +766,8 @@ __global__ __launch_bounds__(kFlatThreads) void walk_stretch_kernel(StepParams P
       int32_t* cell = P.pair_cells + ((size_t)(step >> 1) * P.pair_cell_samples + slot) * 2;
       if (step & 1) *reinterpret_cast<int2*>(cell) = make_int2(transit, neighbor);
       else if (step == last_step) cell[0] = neighbor;
+      if (P.walk_cells && (step == last_step || neighbor == P.invalid))
+        P.walk_cells[slot] = walk_cells_at_end(step, step == last_step);
     } else {
       P.step_out[(size_t)k * out_stride + slot] = neighbor;
     }
@@ -1457,7 +1470,8 @@ __global__ __launch_bounds__(256) void assemble_final_rows(const int32_t* __rest
 __global__ __launch_bounds__(256) void assemble_walk_rows(const int32_t* __restrict__ step_out,
                                                           int32_t* __restrict__ final_samples, uint32_t n_samples,
                                                           uint32_t n_steps, uint32_t row_pitch,
-                                                          uint32_t samples_per_block, uint32_t paired) {
+                                                          uint32_t samples_per_block, uint32_t paired,
+                                                          const uint32_t* __restrict__ walk_cells, int32_t invalid) {
   extern __shared__ int32_t s_rows[];
   const uint32_t s0 = blockIdx.x * samples_per_block;
   const uint32_t nb = n_samples - s0 < samples_per_block ? n_samples - s0 : samples_per_block;
@@ -1467,8 +1481,10 @@ __global__ __launch_bounds__(256) void assemble_walk_rows(const int32_t* __restr
     if (s >= nb) continue;
     if (paired) {
       const int2* cells = reinterpret_cast<const int2*>(step_out);
+      // (walk_cells: the cells beyond the walk's last one were never written)
+      const uint32_t written = walk_cells ? walk_cells[s0 + s] : ~0u;
       for (uint32_t j = wave; 2u * j < n_steps; j += 4u) {
-        const int2 c = cells[(size_t)j * n_samples + s0 + s];
+        const int2 c = j < written ? cells[(size_t)j * n_samples + s0 + s] : make_int2(invalid, invalid);
         s_rows[s * row_pitch + 2u * j] = c.x;
         if (2u * j + 1u < n_steps) s_rows[s * row_pitch + 2u * j + 1u] = c.y;
       }
@@ -1784,6 +1800,7 @@ class Engine : public EngineBase {
     }
     paired_results_ = walk_mode_ && !rows_direct_ && rows_per_block_ > 0 && !App().hasExplicitTransits() &&
                       !(getenv("ND_PAIRED_RESULTS") && atoi(getenv("ND_PAIRED_RESULTS")) == 0);
+    if (paired_results_) ND_HIP_TRY(hipMalloc(&d_walk_cells_, sizeof(uint32_t) * (size_t)n_samples_));
     allocated_ = true;
     return 0;
   }
@@ -1884,8 +1901,11 @@ class Engine : public EngineBase {
     // kernel: their outputs keep this fill - unless the step kernels write the rows themselves
     // and, with every INVALID, what descends from it (StepParams::fill_levels)
     const bool kernels_fill = rows_direct_ && !explicit_map_ && !walk_mode_ && n_steps <= kMaxFillLevels;
-    if (!kernels_fill || mark_unwritten_) {
-      const int32_t value = kernels_fill ? invalid_ + 1 : invalid_;
+    // walks whose results go into cells of two steps: the regrouping reads only the cells a walk
+    // has written (StepParams::walk_cells)
+    const bool no_fill = kernels_fill || paired_results();
+    if (!no_fill || mark_unwritten_) {
+      const int32_t value = no_fill ? invalid_ + 1 : invalid_;
       const size_t n_out = (size_t)n_samples_ * (paired_results() ? (F + 1) / 2 * 2 : F);
       fill_i32<<<dim3((unsigned)((n_out + 1023) / 1024)), dim3(1024), 0, stream_>>>(
           rows_direct_ ? d_final_ : d_step_out_, n_out, value);
@@ -1922,6 +1942,7 @@ class Engine : public EngineBase {
       }
       P.pair_cells = paired_results() ? d_step_out_ : nullptr;
       P.pair_cell_samples = (uint32_t)n_samples_;
+      P.walk_cells = paired_results() ? d_walk_cells_ : nullptr;
       P.samples = d_samples_;
       P.explicit_out = explicit_map_ && step + 1 < n_steps ? d_explicit_ : nullptr;
       P.fill_levels = 0;
@@ -2092,7 +2113,8 @@ class Engine : public EngineBase {
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
       assemble_walk_rows<<<dim3(blocks), dim3(256), lds, stream_>>>(d_step_out_, d_final_, (uint32_t)n_samples_,
                                                                     (uint32_t)n_steps, row_pitch_, rows_per_block_,
-                                                                    paired_results() ? 1u : 0u);
+                                                                    paired_results() ? 1u : 0u,
+                                                                    paired_results() ? d_walk_cells_ : nullptr, invalid_);
     } else if (rows_per_block_ > 0) {
       const unsigned blocks = (unsigned)((n_samples_ + rows_per_block_ - 1) / rows_per_block_);
       const size_t lds = (size_t)rows_per_block_ * row_pitch_ * sizeof(int32_t);
@@ -2378,6 +2400,7 @@ class Engine : public EngineBase {
     release(d_samples_init_);
     release(d_final_);
     release(d_step_out_);
+    release(d_walk_cells_);
     release(d_keys_a_);
     release(d_vals_a_);
     release(d_keys_b_);
@@ -2439,6 +2462,7 @@ class Engine : public EngineBase {
   SampleType* d_samples_init_ = nullptr;
   VertexID_t* d_final_ = nullptr;
   VertexID_t* d_step_out_ = nullptr;
+  uint32_t* d_walk_cells_ = nullptr;  // cells of every walk that hold results (StepParams::walk_cells)
   uint32_t *d_keys_a_ = nullptr, *d_vals_a_ = nullptr, *d_keys_b_ = nullptr, *d_vals_b_ = nullptr;
   uint32_t* d_hist_ = nullptr;
   uint32_t* d_scratch_ = nullptr;
