@@ -217,7 +217,7 @@ int nd_sort_pairs(const int32_t* keys, const int32_t* vals, int64_t n, int key_b
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): nd_sort_pairs on
  * DEVICE arrays, enqueued on `stream` (a hipStream_t; NULL = the default stream) without
  * waiting for it, with all working memory in a fixed array inside the library
- * (ND_SORT_PAIRS_NOALLOC_MAX pairs at most: 8.5 MiB per GPU, held until the process ends).
+ * (ND_SORT_PAIRS_NOALLOC_MAX pairs at most: 8.4 MiB per GPU, held until the process ends).
  * Calls no hipMalloc / hipFree / memset.  d_vals == NULL: value = index.  No output array may
  * overlap an input array or the other output array (returns -3).  The first call on a device asks
  * the runtime for the address of the working array (hipGetSymbolAddress, which may load the
