@@ -403,6 +403,11 @@ __device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition
   *next_transit_out = next_transit;
 }
 
+// Four consecutive ids of a result, at an address that is a multiple of four bytes only.
+struct __attribute__((packed, aligned(4))) FourIds {
+  VertexID a, b, c, d;
+};
+
 // Output q (index inside the sample's segment of this step) is INVALID: so is everything the
 // later steps would have drawn from it (StepParams::fill_levels).
 // (Inlined although it is rare and repeated at every store: a call from a step kernel costs the
@@ -432,7 +437,11 @@ __device__ __forceinline__ void fill_dead_pair(const StepParams& P, uint32_t pai
     if ((uint32_t)l < P.fill_levels) {
       int32_t* dst = row + P.fill_off[l] + (size_t)q0 * P.fill_mult[l];
       const uint32_t n = P.step_size * P.fill_mult[l];
-      for (uint32_t x = helper; x < n; x += helpers) dst[x] = P.invalid;
+      // 16 bytes per lane and store (the address is a multiple of four bytes only), then the rest
+      const uint32_t fours = n / 4u;
+      for (uint32_t x = helper; x < fours; x += helpers)
+        *reinterpret_cast<FourIds*>(dst + 4u * x) = FourIds{P.invalid, P.invalid, P.invalid, P.invalid};
+      for (uint32_t x = 4u * fours + helper; x < n; x += helpers) dst[x] = P.invalid;
     }
   }
 }
@@ -473,11 +482,6 @@ __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition
                                                           &next_transit);
   store_output(P, transit, pair, pair_slot, sample, nbr, neighbor, next_transit);
 }
-
-// Four consecutive ids of a result, at an address that is a multiple of four bytes only.
-struct __attribute__((packed, aligned(4))) FourIds {
-  VertexID a, b, c, d;
-};
 
 // The outputs of a pair that fall into group `gi` of the pair's groups of four consecutive
 // (global) output slots: one shared Philox block, then up to four outputs.  For steps with
