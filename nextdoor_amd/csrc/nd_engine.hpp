@@ -612,8 +612,16 @@ __device__ __forceinline__ void produce_groups(const StepParams& P, CSRPartition
 constexpr double kWalksPerVertexForInversion = 4.0;
 constexpr int kSparseInversionPeriod = 32;
 
-// Lanes the flat kernel wants before it gives a lane all the outputs of a pair.
+// Lanes the flat kernel wants before it gives a lane all the outputs of a pair: enough to fill
+// the machine where the map is sorted by transit (neighbouring lanes then share their transit's
+// lines, and what a lane fetches once per pair - transit, slot, row extent - is spread over all
+// the pair's outputs), many more at step 0, where the roots come in sample order, every lane's
+// gathers miss the caches and a lane that draws all 25 outputs of a root keeps its wavefront
+// alive seven round trips long.  Measured on the two hops of 2.1 M k-hop samples (flat launches,
+// ms): 2^20 at both steps 1.26; roots 2^23 (4 lanes per root) 1.12; roots 2^25 (8 lanes) 1.08;
+// 2^26 at both steps (2 lanes per pair at the second hop) 1.21; 2^27 (4 lanes) 1.52.
 constexpr uint64_t kFlatLanesWanted = 1ull << 20;
+constexpr uint64_t kFlatLanesWantedForRoots = 1ull << 25;
 
 constexpr uint32_t kXcds = 8;
 // Consecutive workgroups (in sorted-pair order) one XCD handles before the next XCD takes over.
@@ -1983,7 +1991,8 @@ class Engine : public EngineBase {
           if (groups > P.groups_per_pair) P.groups_per_pair = groups;
         }
       P.lanes_shift = 0;
-      while ((1u << P.lanes_shift) < P.groups_per_pair && ((uint64_t)n_pairs << P.lanes_shift) < kFlatLanesWanted)
+      const uint64_t lanes_wanted = step == 0 ? kFlatLanesWantedForRoots : kFlatLanesWanted;
+      while ((1u << P.lanes_shift) < P.groups_per_pair && ((uint64_t)n_pairs << P.lanes_shift) < lanes_wanted)
         P.lanes_shift++;
       const uint64_t flat_lanes = (uint64_t)n_pairs << P.lanes_shift;
 
