@@ -605,6 +605,21 @@ __device__ __forceinline__ void produce_groups(const StepParams& P, CSRPartition
   store_group(P, transit, pair, pair_slot, held);
 }
 
+// The same without holding a group back: for the workgroup class, whose draws come from LDS
+// and have no memory latency to hide behind the stores of the group before.
+template <class SampleType, class App, class EdgeArray, class WeightArray>
+__device__ __forceinline__ void produce_groups_in_turn(const StepParams& P, CSRPartition& csr, VertexID transit,
+                                                       uint32_t pair, uint32_t pair_slot, uint32_t first_group,
+                                                       uint32_t stride, EdgePos_t n_edges, float max_weight,
+                                                       EdgeArray& edges, WeightArray& weights) {
+  for (uint32_t gi = first_group; gi < P.groups_per_pair; gi += stride) {
+    GroupOutputs now;
+    compute_group<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, gi, n_edges, max_weight,
+                                                           edges, weights, &now);
+    store_group(P, transit, pair, pair_slot, now);
+  }
+}
+
 // inversion_period == 0: walks are inverted before every step when there are at least this
 // many walks per vertex, else every kSparseInversionPeriod steps (measured on 4.2 M weighted
 // node2vec walks over 4.2 M vertices: 45.3 ms per 100 steps inverting every step, 38.0 every
@@ -905,7 +920,7 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
         produce_output<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot, 0, n_edges,
                                                                       max_weight, edges, weights_of_transit);
       } else {
-        produce_groups<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot,
+        produce_groups_in_turn<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot,
                                                                       t & ((1u << lanes_shift) - 1u), 1u << lanes_shift,
                                                                       n_edges, max_weight, edges, weights_of_transit);
       }
