@@ -42,8 +42,8 @@ MEASURED = {
         "read_requests": {"nd::walk_stretch_kernel": 2.843e8}, "write_requests": {"nd::walk_stretch_kernel": 6.536e6}},
     "uniform_walk_chunglu57k": {"kernels": {"nd::step_balanced_kernel": 6.059e6}, "bytes_per_pass": 1.29e9},
     # both kernel classes of a hop; the flat kernel is launched for both hops, the workgroup kernel for the second
-    "khop_rmat21": {"kernels": {"nd::step_flat_kernel": 1.095e9, "nd::step_workgroup_kernel": 2.404e9},
-                    "bytes_per_pass": 8.78e9},
+    "khop_rmat21": {"kernels": {"nd::step_flat_kernel": 1.096e9, "nd::step_workgroup_kernel": 2.388e9},
+                    "bytes_per_pass": 8.76e9},
     # collective_mark_binned, average over its 2 launches per pass
     "fastgcn_importance_rmat22": {"kernels": {"nd::collective_mark_binned": 5.27e9}, "bytes_per_pass": 16.42e9},
     "ladies_importance_chunglu3m": {"kernels": {"nd::collective_mark_binned": 6.73e10}, "bytes_per_pass": 161.18e9},
