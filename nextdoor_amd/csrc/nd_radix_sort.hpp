@@ -105,44 +105,37 @@ __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* 
 }
 
 // One workgroup per digit: exclusive scan of the digit's row of the table (over tiles) in
-// place, and the row total.
+// place, and the row total.  The row is taken in stretches of kSortThreads * kHeld counts: a
+// thread holds kHeld consecutive counts of a stretch in registers (their loads are all under
+// way at once, and the sweep that writes the prefixes reads nothing), the workgroup scans the
+// threads' sums, and the stretch's total is carried to the next stretch.
 __global__ __launch_bounds__(kSortThreads) void radix_row_scan(uint32_t* __restrict__ hist, uint32_t num_tiles,
                                                                uint32_t* __restrict__ row_totals) {
   __shared__ uint32_t s_scan_tmp[kSortWaves];
   uint32_t* row = hist + (size_t)blockIdx.x * num_tiles;
-  // thread t owns a contiguous stretch of the row
-  const uint32_t per_thread = (num_tiles + kSortThreads - 1) / kSortThreads;
-  const uint32_t begin = threadIdx.x * per_thread;
-  const uint32_t end = begin + per_thread < num_tiles ? begin + per_thread : num_tiles;
-  // a stretch of at most kHeld counts stays in registers: its loads are all under way at once
-  // and the second sweep reads nothing
   constexpr uint32_t kHeld = 8;
-  uint32_t held[kHeld];
-  uint32_t sum = 0;
-  if (per_thread <= kHeld) {
+  uint32_t carry = 0;
+  for (uint32_t stretch = 0; stretch < num_tiles; stretch += kSortThreads * kHeld) {
+    // a short row is spread over all threads rather than packed into the first few
+    const uint32_t left = num_tiles - stretch;
+    const uint32_t per_thread = left >= kSortThreads * kHeld ? kHeld : (left + kSortThreads - 1) / kSortThreads;
+    const uint32_t begin = stretch + threadIdx.x * per_thread;
+    uint32_t held[kHeld];
+    uint32_t sum = 0;
 #pragma unroll
-    for (uint32_t k = 0; k < kHeld; ++k) held[k] = k < per_thread && begin + k < end ? row[begin + k] : 0u;
+    for (uint32_t k = 0; k < kHeld; ++k) held[k] = k < per_thread && begin + k < num_tiles ? row[begin + k] : 0u;
 #pragma unroll
     for (uint32_t k = 0; k < kHeld; ++k) sum += held[k];
-  } else {
-    for (uint32_t i = begin; i < end; ++i) sum += row[i];
-  }
-  uint32_t total;
-  uint32_t running = block_exclusive_scan_256(sum, s_scan_tmp, &total);
-  if (per_thread <= kHeld) {
+    uint32_t total;
+    uint32_t running = carry + block_exclusive_scan_256(sum, s_scan_tmp, &total);
 #pragma unroll
     for (uint32_t k = 0; k < kHeld; ++k) {
-      if (k < per_thread && begin + k < end) row[begin + k] = running;
+      if (k < per_thread && begin + k < num_tiles) row[begin + k] = running;
       running += held[k];
     }
-  } else {
-    for (uint32_t i = begin; i < end; ++i) {
-      const uint32_t c = row[i];
-      row[i] = running;
-      running += c;
-    }
+    carry += total;
   }
-  if (threadIdx.x == 0) row_totals[blockIdx.x] = total;
+  if (threadIdx.x == 0) row_totals[blockIdx.x] = carry;
 }
 
 // aux_in / aux_out (kAux): a second 32-bit payload that travels with the pair.  It goes
