@@ -75,6 +75,8 @@ struct KeyLayout {
 
 // n_dev (nullable): element count kept in device memory; overrides n when given.
 // drop_key: keys equal to it are left out of the sort (kPadKey: nothing is left out).
+// (A workgroup counting four consecutive tiles, so that a digit's four counts leave as one 16-byte
+// store instead of four pieces of four lines: 0.86 -> 0.85 ms of inversion on 5.2e7 pairs; not kept.)
 template <int kSortItems>
 __global__ __launch_bounds__(kSortThreads) void radix_histogram(const uint32_t* __restrict__ keys, size_t n,
                                                                 const uint32_t* __restrict__ n_dev, int shift,
