@@ -142,52 +142,68 @@ __global__ __launch_bounds__(kSortThreads) void radix_row_scan(uint32_t* __restr
 
 // aux_in / aux_out (kAux): a second 32-bit payload that travels with the pair.  It goes
 // through the LDS staging area of the values in a second round, after the keys and values
-// of the tile have been written, so the workgroup needs no more LDS than without it.
+// of the tile have been written, so that the workgroup needs no more LDS than without it.
+// kSortItems is the keys per lane of the histogram's 256-lane workgroups; this kernel runs the
+// same tile with kScatterThreads lanes, each taking kSortItems * 256 / kScatterThreads keys: the
+// ranking of a lane's keys is a chain of ballots per key, one key after the other, and with
+// twice the lanes the chain is half as long.  Inversion of the 100-step pass over 4.2 M walks: 256
+// lanes 10.2 ms, 512 lanes 9.4 ms (with tiles of 2048 / 3072 keys: 11.0 / 9.7), 1024 lanes 10.8-11.8.
+#ifndef ND_SCATTER_THREADS
+#define ND_SCATTER_THREADS 512
+#endif
+constexpr int kScatterThreads = ND_SCATTER_THREADS;
+constexpr int kScatterWaves = kScatterThreads / kWave;
+
 template <int kSortItems, bool kIotaValues, bool kAux>
-__global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __restrict__ keys_in,
-                                                              const uint32_t* __restrict__ vals_in,
-                                                              const uint32_t* __restrict__ aux_in,
-                                                              uint32_t* __restrict__ keys_out,
-                                                              uint32_t* __restrict__ vals_out,
-                                                              uint32_t* __restrict__ aux_out, size_t n,
-                                                              const uint32_t* __restrict__ n_dev, int shift,
-                                                              uint32_t mask, int digit_bits, uint32_t drop_key,
-                                                              const uint32_t* __restrict__ scanned_hist,
-                                                              const uint32_t* __restrict__ row_totals,
-                                                              uint32_t num_tiles, uint32_t* __restrict__ kept_out,
-                                                              KeyLayout layout) {
+__global__ __launch_bounds__(kScatterThreads) void radix_scatter(const uint32_t* __restrict__ keys_in,
+                                                                 const uint32_t* __restrict__ vals_in,
+                                                                 const uint32_t* __restrict__ aux_in,
+                                                                 uint32_t* __restrict__ keys_out,
+                                                                 uint32_t* __restrict__ vals_out,
+                                                                 uint32_t* __restrict__ aux_out, size_t n,
+                                                                 const uint32_t* __restrict__ n_dev, int shift,
+                                                                 uint32_t mask, int digit_bits, uint32_t drop_key,
+                                                                 const uint32_t* __restrict__ scanned_hist,
+                                                                 const uint32_t* __restrict__ row_totals,
+                                                                 uint32_t num_tiles, uint32_t* __restrict__ kept_out,
+                                                                 KeyLayout layout) {
   constexpr int kSortTile = kSortThreads * kSortItems;
+  static_assert(kSortTile % kScatterThreads == 0, "the tile is a whole number of keys per lane");
+  constexpr int kItems = kSortTile / kScatterThreads;  // keys per lane here
   __shared__ uint32_t s_keys[kSortTile];
   __shared__ uint32_t s_vals[kSortTile];
-  __shared__ uint32_t s_wave_count[kSortWaves][kRadix];
+  __shared__ uint32_t s_wave_count[kScatterWaves][kRadix];
   __shared__ uint32_t s_digit_base[kRadix];
   __shared__ uint32_t s_global_base[kRadix];
-  __shared__ uint32_t s_scan_tmp[kSortWaves];
+  __shared__ uint32_t s_scan_tmp[kScatterWaves];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
+  const bool digit_lane = tid < kRadix;  // lanes that own a digit in the per-digit steps
   if (n_dev) n = *n_dev;
   const size_t tile_start = (size_t)blockIdx.x * kSortTile;
   if (tile_start >= n && !(kept_out && blockIdx.x == 0)) return;
   // first position of every digit in the output: exclusive scan of the row totals
   uint32_t kept_total;
-  const uint32_t digit_first = block_exclusive_scan_256((uint32_t)tid <= mask ? row_totals[tid] : 0u, s_scan_tmp,
-                                                        &kept_total);
+  const uint32_t digit_first = block_exclusive_scan<kScatterThreads>(
+      digit_lane && (uint32_t)tid <= mask ? row_totals[tid] : 0u, s_scan_tmp, &kept_total);
   // number of keys the whole sort keeps; published once
   if (kept_out && blockIdx.x == 0 && tid == 0) kept_out[0] = kept_total;
   if (tile_start >= n) return;
   const uint32_t in_tile = (uint32_t)((n - tile_start) < (size_t)kSortTile ? (n - tile_start) : (size_t)kSortTile);
 
+  if (digit_lane) {
 #pragma unroll
-  for (int w = 0; w < kSortWaves; ++w) s_wave_count[w][tid] = 0;
+    for (int w = 0; w < kScatterWaves; ++w) s_wave_count[w][tid] = 0;
+  }
   __syncthreads();
 
-  uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], aux[kAux ? kSortItems : 1];
-  bool live[kSortItems];
+  uint32_t key[kItems], val[kItems], rank[kItems], aux[kAux ? kItems : 1];
+  bool live[kItems];
 #pragma unroll
-  for (int it = 0; it < kSortItems; ++it) {
-    const uint32_t off = (uint32_t)tile_offset<kSortItems>(wave, it, lane);
+  for (int it = 0; it < kItems; ++it) {
+    const uint32_t off = (uint32_t)tile_offset<kItems>(wave, it, lane);
     const bool inside = off < in_tile;
     key[it] = inside ? keys_in[layout.at(tile_start + off)] : kPadKey;
     live[it] = inside && key[it] != drop_key;
@@ -198,7 +214,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
 
   const uint64_t lanes_below = (1ull << lane) - 1ull;
 #pragma unroll
-  for (int it = 0; it < kSortItems; ++it) {
+  for (int it = 0; it < kItems; ++it) {
     const uint32_t digit = (key[it] >> shift) & mask;
     // peers = live lanes of this wave holding the same digit
     uint64_t peers = __ballot(live[it]);
@@ -218,21 +234,25 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   // per digit: turn the per-wave counts into exclusive prefixes over waves, then scan
   // the tile totals over digits.
   uint32_t digit_total = 0;
+  if (digit_lane) {
 #pragma unroll
-  for (int w = 0; w < kSortWaves; ++w) {
-    const uint32_t c = s_wave_count[w][tid];
-    s_wave_count[w][tid] = digit_total;
-    digit_total += c;
+    for (int w = 0; w < kScatterWaves; ++w) {
+      const uint32_t c = s_wave_count[w][tid];
+      s_wave_count[w][tid] = digit_total;
+      digit_total += c;
+    }
   }
   uint32_t live_in_tile;
-  const uint32_t digit_base = block_exclusive_scan_256(digit_total, s_scan_tmp, &live_in_tile);
-  s_digit_base[tid] = digit_base;
-  if ((uint32_t)tid <= mask)
-    s_global_base[tid] = digit_first + scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
+  const uint32_t digit_base = block_exclusive_scan<kScatterThreads>(digit_total, s_scan_tmp, &live_in_tile);
+  if (digit_lane) {
+    s_digit_base[tid] = digit_base;
+    if ((uint32_t)tid <= mask)
+      s_global_base[tid] = digit_first + scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
+  }
   __syncthreads();
 
 #pragma unroll
-  for (int it = 0; it < kSortItems; ++it) {
+  for (int it = 0; it < kItems; ++it) {
     if (live[it]) {
       const uint32_t digit = (key[it] >> shift) & mask;
       const uint32_t pos = s_digit_base[digit] + s_wave_count[wave][digit] + rank[it];
@@ -243,7 +263,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   }
   __syncthreads();
 
-  for (uint32_t p = tid; p < live_in_tile; p += kSortThreads) {
+  for (uint32_t p = tid; p < live_in_tile; p += kScatterThreads) {
     const uint32_t k = s_keys[p];
     const uint32_t out = s_global_base[(k >> shift) & mask] + p;
     keys_out[out] = k;
@@ -252,11 +272,11 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter(const uint32_t* __
   if (kAux) {
     __syncthreads();
 #pragma unroll
-    for (int it = 0; it < kSortItems; ++it) {
+    for (int it = 0; it < kItems; ++it) {
       if (live[it]) s_vals[rank[it]] = aux[it];
     }
     __syncthreads();
-    for (uint32_t p = tid; p < live_in_tile; p += kSortThreads) {
+    for (uint32_t p = tid; p < live_in_tile; p += kScatterThreads) {
       const uint32_t out = s_global_base[(s_keys[p] >> shift) & mask] + p;
       aux_out[out] = s_vals[p];
     }
@@ -332,16 +352,17 @@ inline void sort_pass(const SortPlan& plan, const SortJob& job, const uint32_t* 
   radix_histogram<kSortItems><<<grid, block, 0, stream>>>(src_k, plan.n, n_dev, shift, mask, drop, job.hist,
                                                           plan.num_tiles, layout);
   radix_row_scan<<<dim3(mask + 1), block, 0, stream>>>(job.hist, plan.num_tiles, job.scratch);
+  const dim3 scatter_block(kScatterThreads);
   if (src_v == nullptr)
-    radix_scatter<kSortItems, true, false><<<grid, block, 0, stream>>>(src_k, nullptr, nullptr, dst_k, dst_v, nullptr,
+    radix_scatter<kSortItems, true, false><<<grid, scatter_block, 0, stream>>>(src_k, nullptr, nullptr, dst_k, dst_v, nullptr,
                                                                        plan.n, n_dev, shift, mask, bits, drop, job.hist,
                                                                        job.scratch, plan.num_tiles, kept_out, layout);
   else if (src_x == nullptr)
-    radix_scatter<kSortItems, false, false><<<grid, block, 0, stream>>>(src_k, src_v, nullptr, dst_k, dst_v, nullptr,
+    radix_scatter<kSortItems, false, false><<<grid, scatter_block, 0, stream>>>(src_k, src_v, nullptr, dst_k, dst_v, nullptr,
                                                                         plan.n, n_dev, shift, mask, bits, drop,
                                                                         job.hist, job.scratch, plan.num_tiles, kept_out, layout);
   else
-    radix_scatter<kSortItems, false, true><<<grid, block, 0, stream>>>(src_k, src_v, src_x, dst_k, dst_v, dst_x, plan.n,
+    radix_scatter<kSortItems, false, true><<<grid, scatter_block, 0, stream>>>(src_k, src_v, src_x, dst_k, dst_v, dst_x, plan.n,
                                                                        n_dev, shift, mask, bits, drop, job.hist,
                                                                        job.scratch, plan.num_tiles, kept_out, layout);
 }
