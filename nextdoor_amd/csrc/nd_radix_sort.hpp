@@ -142,7 +142,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_row_scan(uint32_t* __restr
 
 // aux_in / aux_out (kAux): a second 32-bit payload that travels with the pair.  It goes
 // through the LDS staging area of the values in a second round, after the keys and values
-// of the tile have been written, so that the workgroup needs no more LDS than without it.
+// of the tile have been written, so that the workgroup needs no more LDS than without it (with a
+// staging area of its own and one round: inversion of the 4.2 M-walk pass 9.4 -> 10.5 ms).
 // kSortItems is the keys per lane of the histogram's 256-lane workgroups; this kernel runs the
 // same tile with kScatterThreads lanes, each taking kSortItems * 256 / kScatterThreads keys: the
 // ranking of a lane's keys is a chain of ballots per key, one key after the other, and with
