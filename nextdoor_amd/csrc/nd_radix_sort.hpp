@@ -193,6 +193,9 @@ __global__ __launch_bounds__(kScatterThreads) void radix_scatter(const uint32_t*
   if (kept_out && blockIdx.x == 0 && tid == 0) kept_out[0] = kept_total;
   if (tile_start >= n) return;
   const uint32_t in_tile = (uint32_t)((n - tile_start) < (size_t)kSortTile ? (n - tile_start) : (size_t)kSortTile);
+  // where the tile's keys of a digit go among all keys of that digit: fetched now, with the keys,
+  // not after the ranking, where it would be one more round trip
+  const uint32_t before_tile = digit_lane && (uint32_t)tid <= mask ? scanned_hist[(size_t)tid * num_tiles + blockIdx.x] : 0u;
 
   if (digit_lane) {
 #pragma unroll
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(kScatterThreads) void radix_scatter(const uint32_t*
   if (digit_lane) {
     s_digit_base[tid] = digit_base;
     if ((uint32_t)tid <= mask)
-      s_global_base[tid] = digit_first + scanned_hist[(size_t)tid * num_tiles + blockIdx.x] - digit_base;
+      s_global_base[tid] = digit_first + before_tile - digit_base;
   }
   __syncthreads();
 
