@@ -40,7 +40,7 @@ MEASURED = {
     "weighted_node2vec_rmat22_period0": {
         "kernels": {"nd::walk_stretch_kernel": 3.676e10}, "bytes_per_pass": 150.95e9,
         "read_requests": {"nd::walk_stretch_kernel": 2.843e8}, "write_requests": {"nd::walk_stretch_kernel": 6.536e6}},
-    "uniform_walk_chunglu57k": {"kernels": {"nd::step_balanced_kernel": 6.046e6}, "bytes_per_pass": 1.29e9},
+    "uniform_walk_chunglu57k": {"kernels": {"nd::step_flat_kernel": 1.224e7}, "bytes_per_pass": 1.27e9},
     # both kernel classes of a hop; the flat kernel is launched for both hops, the workgroup kernel for the second
     "khop_rmat21": {"kernels": {"nd::step_flat_kernel": 1.096e9, "nd::step_workgroup_kernel": 2.39e9},
                     "bytes_per_pass": 8.75e9},
@@ -298,6 +298,10 @@ def measure(args, workload, steps, warmup, cpu_seconds, graphs, engine_choice=Tr
     sampler.do_transit_parallel(lb)
     prof = sampler.phase_times()
     sampler.set_profiling(False)
+    if schedule is not None and sampler.step_size(0) == 1 and sampler.steps > 1 and prof["sort_passes"] == 0:
+        # a walk over a small map: the kernel that emits a pair places it for the next step, one
+        # launch per step, every pair with the flat lanes - nothing is sorted or classified
+        schedule["small_map_placed_as_emitted"] = True
     kernel_classes = None
     if per_transit and lb:
         # pairs per kernel class over the steps of the last pass whose classification ran (the

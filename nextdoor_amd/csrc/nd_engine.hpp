@@ -264,6 +264,21 @@ struct StepParams {
   uint32_t* emit_counts;
   uint32_t* emit_ranks;
   const uint32_t* emit_counter_base;
+  // Small maps placed as they are emitted (nullptr: not in use): counter c owns the places
+  // [emit_place_start[c], emit_place_start[c + 1]) of the next step's pair arrays - room for
+  // about twice the walks it expects - and a pair whose rank fits goes straight there; the few
+  // that do not fit take a place past emit_spill_first, handed out by the counter *emit_spill.
+  // The next step's lanes walk ALL places, the empty ones hold INVALID: the map is inverted, with
+  // gaps, by the kernel that produced it, and a step is one launch.
+  const uint32_t* emit_place_start;
+  uint32_t* emit_spill;
+  uint32_t emit_spill_first;
+  // ... and the other side of it: the lane that takes a pair from such an array marks its place
+  // empty again, and the first lanes clear the counters the pairs were placed by, so that the
+  // arrays and counters are ready when they are written the step after next (two sets alternate).
+  uint32_t* taken_keys;       // == pair_keys, writable; nullptr: the pairs are a dense list
+  uint32_t* taken_counts;     // the counters behind pair_keys, the spill counter after the last
+  uint32_t taken_n_counts;
 };
 
 // A SampleType small enough to travel with its pair through the inversion.
@@ -364,11 +379,14 @@ __device__ __forceinline__ void store_walk_result(const StepParams& P, uint32_t 
 // pair: index of the pair in the order the step kernels walk them (sorted by transit, or
 // the raw map at step 0).
 // First half: next() (and stepTransits) for the output; nothing of the step's results is stored.
-template <class SampleType, class App, class EdgeArray, class WeightArray>
+// kStateOut: the state that travels with the pair is handed to the caller, who knows where the
+// pair goes (store_output<true>), instead of being written next to the pair's index.
+template <class SampleType, class App, class EdgeArray, class WeightArray, bool kStateOut = false>
 __device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
                                                uint32_t pair_slot, uint32_t sample, uint32_t nbr, EdgePos_t n_edges,
                                                float max_weight, EdgeArray& edges, WeightArray& weights, bool grouped,
-                                               uint32_t first_word, VertexID* neighbor_out, VertexID* next_transit_out) {
+                                               uint32_t first_word, VertexID* neighbor_out, VertexID* next_transit_out,
+                                               uint32_t* state_out = nullptr) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   const uint32_t transit_index = pair_slot - sample * P.transits_per_sample;
   VertexID neighbor = P.invalid, next_transit = P.invalid;
@@ -382,7 +400,8 @@ __device__ __forceinline__ void compute_output(const StepParams& P, CSRPartition
       neighbor = run_app<SampleType, App>(P, csr, transit, sample, transit_index, out_slot, nbr, n_edges, max_weight,
                                           edges, weights, &state, &next_transit, grouped, first_word);
       __builtin_memcpy(&bits, &state, sizeof(uint32_t));
-      if (P.emit_state) P.emit_state[pair] = bits;
+      if (kStateOut) *state_out = bits;
+      else if (P.emit_state) P.emit_state[pair] = bits;
       // a walk that ends here leaves the stream of pairs: its state goes home
       if (P.is_last || next_transit == P.invalid) ((uint32_t*)P.samples)[sample] = bits;
       travelled = true;
@@ -448,10 +467,18 @@ __device__ __forceinline__ void fill_dead_pair(const StepParams& P, uint32_t pai
 
 // Second half: the output goes to its place in the step's results, and what the next step
 // needs of it to the next step's map.
+// kPlaces: the flat kernel of walks over small maps (flat_lane's kPlaces), whose lanes place the
+// pair for the next step themselves (StepParams::emit_place_start) and then also store its
+// travelling state.
+// kWalkStep: the step may be a walk's (one output per pair); cells shared by two steps and
+// emitted pairs exist only there, and the code of steps that draw several outputs per pair is
+// compiled without them (the k-hop kernels are slower by a tenth with that code merely present).
+template <bool kPlaces = false, bool kWalkStep = true>
 __device__ __forceinline__ void store_output(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
-                                             uint32_t sample, uint32_t nbr, VertexID neighbor, VertexID next_transit) {
+                                             uint32_t sample, uint32_t nbr, VertexID neighbor, VertexID next_transit,
+                                             uint32_t state_bits = 0) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
-  if (P.pair_cells) {
+  if (kWalkStep && P.pair_cells) {
     store_walk_result(P, sample, transit, neighbor);
   } else {
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
@@ -460,27 +487,40 @@ __device__ __forceinline__ void store_output(const StepParams& P, VertexID trans
     if (P.fill_levels > 1 && neighbor == P.invalid) fill_below(P, sample, q);
   }
   if (P.explicit_out) P.explicit_out[out_slot] = next_transit;
-  if (P.emit_keys) {
-    P.emit_keys[pair] = (uint32_t)next_transit;
-    P.emit_slots[pair] = pair_slot;
+  if (kWalkStep && P.emit_keys) {
+    uint32_t at = pair;
     if (P.emit_counts && next_transit != P.invalid) {
       const uint32_t first = P.emit_counter_base[next_transit];
       const uint32_t copies = P.emit_counter_base[next_transit + 1] - first;
-      P.emit_ranks[pair] = atomicAdd(&P.emit_counts[first + (pair & (copies - 1u))], 1u);
+      const uint32_t counter = first + (pair & (copies - 1u));
+      const uint32_t rank = atomicAdd(&P.emit_counts[counter], 1u);
+      if (kPlaces && P.emit_place_start) {
+        const uint32_t place = P.emit_place_start[counter];
+        at = place + rank < P.emit_place_start[counter + 1] ? place + rank : P.emit_spill_first + atomicAdd(P.emit_spill, 1u);
+      } else {
+        P.emit_ranks[pair] = rank;
+      }
+    }
+    // placed pairs: a walk that has ended takes no place (the empty places hold INVALID already)
+    if (!(kPlaces && P.emit_place_start) || next_transit != P.invalid) {
+      P.emit_keys[at] = (uint32_t)next_transit;
+      P.emit_slots[at] = pair_slot;
+      if (kPlaces && P.emit_state) P.emit_state[at] = state_bits;
     }
   }
 }
 
-template <class SampleType, class App, class EdgeArray, class WeightArray>
+template <class SampleType, class App, class EdgeArray, class WeightArray, bool kPlaces = false>
 __device__ __forceinline__ void produce_output(const StepParams& P, CSRPartition& csr, VertexID transit, uint32_t pair,
                                                uint32_t pair_slot, uint32_t nbr, EdgePos_t n_edges, float max_weight,
                                                EdgeArray& edges, WeightArray& weights) {
   const uint32_t sample = P.transits_per_sample == 1 ? pair_slot : pair_slot / P.transits_per_sample;
   VertexID neighbor, next_transit;
-  compute_output<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, sample, nbr, n_edges,
-                                                          max_weight, edges, weights, false, 0u, &neighbor,
-                                                          &next_transit);
-  store_output(P, transit, pair, pair_slot, sample, nbr, neighbor, next_transit);
+  uint32_t state_bits = 0;
+  compute_output<SampleType, App, EdgeArray, WeightArray, kPlaces>(P, csr, transit, pair, pair_slot, sample, nbr,
+                                                                   n_edges, max_weight, edges, weights, false, 0u,
+                                                                   &neighbor, &next_transit, &state_bits);
+  store_output<kPlaces>(P, transit, pair, pair_slot, sample, nbr, neighbor, next_transit, state_bits);
 }
 
 // The outputs of a pair that fall into group `gi` of the pair's groups of four consecutive
@@ -563,7 +603,7 @@ __device__ __forceinline__ void compute_group(const StepParams& P, CSRPartition&
 __device__ __forceinline__ void store_group(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
                                             const GroupOutputs& g) {
   if (g.from >= g.to) return;
-  if (g.from == 0 && g.to == 4 && !P.pair_cells && !P.explicit_out && !P.emit_keys) {
+  if (g.from == 0 && g.to == 4 && !P.explicit_out) {
     // a whole group whose outputs are all there is to store: the four ids are neighbours in
     // the step's results (word aligned, not more), and go out as one 16-byte store
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
@@ -581,8 +621,8 @@ __device__ __forceinline__ void store_group(const StepParams& P, VertexID transi
 #pragma unroll
   for (uint32_t w = 0; w < 4; ++w)
     if (w >= g.from && w < g.to)
-      store_output(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.base + w - g.first), g.neighbor[w],
-                   g.next_transit[w]);
+      store_output<false, false>(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.base + w - g.first), g.neighbor[w],
+                                 g.next_transit[w]);
 }
 
 // The groups first, first + stride, ... of a pair, the draws of a group made before the
@@ -665,12 +705,19 @@ __device__ __forceinline__ uint32_t flat_block_index() {
 // taken_stamp (nullable): per-vertex marker of the transits that work items cover at this
 // step - those whose entry equals `stamp` (RunsMeta::stamp of the step).
 // kSingleOutput: stepSize is 1 (walks); the loop over neighbours is compiled away.
-template <class SampleType, class App, bool kSingleOutput>
+// kPlaces: a walk over a small map whose pairs are placed as they are emitted
+// (StepParams::emit_place_start, taken_keys); a kernel of its own, so that the others are
+// compiled without it.
+template <class SampleType, class App, bool kSingleOutput, bool kPlaces = false>
 __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint32_t* __restrict__ taken_stamp,
                                           uint32_t stamp) {
   if (kSingleOutput) {
     P.lanes_shift = 0;
     P.step_size = 1;
+  }
+  if (kPlaces && P.taken_keys) {
+    // pairs placed as they were emitted: nobody reads their counters during this step
+    if (i < P.taken_n_counts) P.taken_counts[i] = 0;
   }
   const uint64_t total = (uint64_t)(P.live_pairs ? *P.live_pairs : P.n_pairs) << P.lanes_shift;
   if (i >= total) return;
@@ -678,7 +725,14 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
   const uint32_t pair = (uint32_t)(i >> P.lanes_shift);
   const uint32_t first_nbr = (uint32_t)i & ((1u << P.lanes_shift) - 1u);
   const uint32_t nbr_stride = 1u << P.lanes_shift;
-  const VertexID transit = (VertexID)P.pair_keys[pair];
+  VertexID transit;
+  if (kPlaces && P.taken_keys) {
+    transit = (VertexID)P.taken_keys[pair];
+    if (transit == P.invalid) return;  // an empty place
+    P.taken_keys[pair] = (uint32_t)P.invalid;
+  } else {
+    transit = (VertexID)P.pair_keys[pair];
+  }
   const uint32_t slot = P.pair_slots ? P.pair_slots[pair] : pair;
   EdgePos_t n_edges = 0, begin = 0;
   float max_weight = 0.0f;
@@ -712,8 +766,8 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
     PairedEdgeIds edges{P.paired_edges + begin};
     PairedEdgeWeights weights{P.paired_edges + begin};
     if (kSingleOutput) {
-      produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, 0, n_edges,
-                                                                        max_weight, edges, weights);
+      produce_output<SampleType, App, PairedEdgeIds, PairedEdgeWeights, kPlaces>(P, csr, transit, pair, slot, 0, n_edges,
+                                                                                 max_weight, edges, weights);
     } else {
       produce_groups<SampleType, App, PairedEdgeIds, PairedEdgeWeights>(P, csr, transit, pair, slot, first_nbr,
                                                                         nbr_stride, n_edges, max_weight, edges, weights);
@@ -722,8 +776,8 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
     const CSR::Edge* edges = csr.edges + begin;
     const float* weights = csr.weights + begin;
     if (kSingleOutput) {
-      produce_output<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, 0, n_edges,
-                                                                     max_weight, edges, weights);
+      produce_output<SampleType, App, const CSR::Edge*, const float*, kPlaces>(P, csr, transit, pair, slot, 0, n_edges,
+                                                                              max_weight, edges, weights);
     } else {
       produce_groups<SampleType, App, const CSR::Edge*, const float*>(P, csr, transit, pair, slot, first_nbr,
                                                                      nbr_stride, n_edges, max_weight, edges, weights);
@@ -732,13 +786,13 @@ __device__ __forceinline__ void flat_lane(StepParams& P, uint64_t i, const uint3
 }
 
 // meta (with taken_stamp): the step's bookkeeping, whose stamp marks the taken transits.
-template <class SampleType, class App, bool kSingleOutput>
+template <class SampleType, class App, bool kSingleOutput, bool kPlaces = false>
 __global__ __launch_bounds__(kFlatThreads) void step_flat_kernel(StepParams P,
                                                                  const uint32_t* __restrict__ taken_stamp,
                                                                  const RunsMeta* __restrict__ meta) {
   const uint32_t stamp = taken_stamp ? meta->stamp : 0u;
-  flat_lane<SampleType, App, kSingleOutput>(P, (uint64_t)flat_block_index() * kFlatThreads + threadIdx.x, taken_stamp,
-                                            stamp);
+  flat_lane<SampleType, App, kSingleOutput, kPlaces>(P, (uint64_t)flat_block_index() * kFlatThreads + threadIdx.x,
+                                                     taken_stamp, stamp);
 }
 
 // Walks that are not re-inverted for a while: one lane keeps its walk for a whole stretch of
@@ -865,7 +919,8 @@ __device__ __forceinline__ void stage_into_lds(const T* __restrict__ src, T* lds
 // transit's adjacency (and weights, when the app draws by weight) is staged once into LDS
 // with coalesced reads and every draw of the stretch gathers from LDS.  The workgroup takes
 // the items first_item, first_item + item_stride, ...
-template <class SampleType, class App>
+// kSingleOutput: the step draws one output per pair; each form is compiled without the other.
+template <class SampleType, class App, bool kSingleOutput>
 __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* __restrict__ chunks, uint32_t n_chunks,
                                                 uint32_t first_item, uint32_t item_stride, CSR::Edge* s_edges,
                                                 float* s_weights) {
@@ -899,7 +954,8 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
     // was slower: 1.23 against 1.17 ms for the k-hop launch, which does not wait for its lanes.)
     // The slot of a lane's first pair is fetched together with the adjacency, not after it.
     uint32_t lanes_shift = 0;
-    while ((1u << lanes_shift) < P.groups_per_pair && (n_pairs << (lanes_shift + 1)) <= (uint32_t)kStepThreads) lanes_shift++;
+    if (!kSingleOutput)
+      while ((1u << lanes_shift) < P.groups_per_pair && (n_pairs << (lanes_shift + 1)) <= (uint32_t)kStepThreads) lanes_shift++;
     const uint32_t lanes = n_pairs << lanes_shift;
     uint32_t slot = threadIdx.x < lanes ? P.pair_slots[first_pair + (threadIdx.x >> lanes_shift)] : 0u;
     __syncthreads();  // the previous work item is done with the cache
@@ -916,7 +972,7 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
     for (uint32_t t = threadIdx.x; t < lanes; t += kStepThreads) {
       const uint32_t p = t >> lanes_shift;
       if (t != threadIdx.x) slot = P.pair_slots[first_pair + p];
-      if (P.groups_per_pair == 0) {  // one output per pair
+      if (kSingleOutput) {
         produce_output<SampleType, App, LdsArray<CSR::Edge>, Weights>(P, csr, transit, first_pair + p, slot, 0, n_edges,
                                                                       max_weight, edges, weights_of_transit);
       } else {
@@ -933,7 +989,7 @@ __device__ __forceinline__ void workgroup_items(StepParams& P, const WorkItem* _
   }
 }
 
-template <class SampleType, class App>
+template <class SampleType, class App, bool kSingleOutput>
 __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams P,
                                                                       const WorkItem* __restrict__ chunks,
                                                                       const RunsMeta* __restrict__ meta,
@@ -941,7 +997,7 @@ __global__ __launch_bounds__(kStepThreads) void step_workgroup_kernel(StepParams
   __shared__ __align__(16) CSR::Edge s_edges[kCacheEdges];  // filled with 16-byte stores
   __shared__ __align__(16) float s_weights[app_uses_weights<App>::value ? kCacheEdges : 4];
   const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
-  workgroup_items<SampleType, App>(P, chunks, n_chunks, blockIdx.x, gridDim.x, s_edges, s_weights);
+  workgroup_items<SampleType, App, kSingleOutput>(P, chunks, n_chunks, blockIdx.x, gridDim.x, s_edges, s_weights);
 }
 
 // Both classes of a load-balanced step in ONE launch: the flat lanes and the work items touch
@@ -975,8 +1031,9 @@ __global__ __launch_bounds__(kStepThreads) void step_balanced_kernel(StepParams 
   } else {
     const uint32_t n_groups = gridDim.x / per_group;
     const uint32_t n_chunks = meta->n_chunks < chunk_capacity ? meta->n_chunks : chunk_capacity;
-    workgroup_items<SampleType, App>(P, chunks, n_chunks, group * wg_per_group + (local - kBalancedFlatBlocks),
-                                     n_groups * wg_per_group, s_edges, s_weights);
+    workgroup_items<SampleType, App, kSingleOutput>(P, chunks, n_chunks,
+                                                    group * wg_per_group + (local - kBalancedFlatBlocks),
+                                                    n_groups * wg_per_group, s_edges, s_weights);
   }
 }
 
@@ -1279,11 +1336,25 @@ __global__ __launch_bounds__(kThreads) void classify_run_tails(const uint32_t* _
 // order inside a run is the order the atomics were served in; results do not depend on it
 // (randomness is keyed by the slot).  The counters of a transit (StepParams::emit_counter_base)
 // are consecutive, so its run is still one stretch of the placed pairs.
+//
+// Where the places are not many times the pairs, the two placing launches go too: every counter
+// owns a fixed stretch of the next step's pair arrays, with room for twice the walks it expects
+// from its share of the edge ends, and the emitting lane writes its pair straight to stretch
+// start + rank (StepParams::emit_place_start; the few pairs whose rank does not fit take a place
+// after all stretches).  The next step's launch has a lane for every place and skips the empty
+// ones; the lane that takes a pair marks its place empty again and the first lanes clear the
+// counters, so two sets of arrays alternate without a launch of their own.  A step is then one
+// launch (8.4 us on 56,944 walks, against 18.2 us for the three launches of count, place and
+// step); every pair goes to the flat lanes - the transits many walks share keep their adjacency
+// in the caches of a map this small - so nothing is classified.  ND_SMALL_MAP=1 keeps the two
+// placing launches, ND_SMALL_MAP=0 the sort.
 constexpr uint32_t kSmallMapPairs = 1u << 17;
 constexpr uint32_t kSmallMapCounters = 1u << 20;  // counters of all vertices at most
 constexpr uint32_t kSmallMapWalksPerCounter = 16;   // a vertex expected to take more walks per step gets copies
 constexpr uint32_t kSmallMapMaxCopies = 256;
 constexpr uint32_t kSmallMapChunk = 1024;  // counters per workgroup of small_map_scan; at most 1024 chunks
+constexpr uint32_t kSmallMapSparePlaces = 4;    // places of a counter beyond twice the walks it expects
+constexpr size_t kSmallMapPlacesPerPair = 12;   // placing at emission: places of all counters per pair at most
 
 __global__ __launch_bounds__(256) void small_map_scan(uint32_t* __restrict__ counts, uint32_t n_counters,
                                                       uint32_t* __restrict__ local_start,
@@ -1749,7 +1820,7 @@ class Engine : public EngineBase {
         !(getenv("ND_SMALL_MAP") && atoi(getenv("ND_SMALL_MAP")) == 0)) {
       const size_t V = (size_t)graph_->get_n_vertices();
       const double per_edge = graph_->col.empty() ? 0.0 : (double)max_pairs_ / (double)graph_->col.size();
-      std::vector<uint32_t> base(V + 1), edges_into(V, 0);
+      std::vector<uint32_t> base(V + 1), edges_into(V, 0), place_start(1, 0u);
       for (const CSR::Edge dst : graph_->col) edges_into[(size_t)dst]++;
       uint64_t at = 0;
       for (size_t v = 0; v < V; ++v) {
@@ -1758,13 +1829,40 @@ class Engine : public EngineBase {
         uint32_t copies = 1;
         while (copies < kSmallMapMaxCopies && (double)(copies * kSmallMapWalksPerCounter) < walks) copies <<= 1;
         at += copies;
+        // places of each of its counters when the pairs are placed as they are emitted: twice
+        // the walks it expects and a few more
+        const uint32_t places = (uint32_t)(2.0 * walks / copies) + kSmallMapSparePlaces;
+        for (uint32_t c = 0; c < copies; ++c) place_start.push_back(place_start.back() + places);
       }
       base[V] = (uint32_t)at;
       small_counters_ = (size_t)at + 1;  // one more, so that every run has an end to read
+      place_start.push_back(place_start.back());  // ... which owns no place
       small_map_ = small_counters_ < kSmallMapCounters;
       if (small_map_) {
         ND_HIP_TRY(hipMalloc(&d_counter_base_, sizeof(uint32_t) * base.size()));
         ND_HIP_TRY(hipMemcpy(d_counter_base_, base.data(), sizeof(uint32_t) * base.size(), hipMemcpyHostToDevice));
+      }
+      // Placing at emission walks every place at every step: only where the places are not many
+      // times the pairs (ND_SMALL_MAP=1 keeps the two placing launches).
+      small_placed_ = small_map_ && (size_t)place_start.back() <= kSmallMapPlacesPerPair * max_pairs_ &&
+                      !(getenv("ND_SMALL_MAP") && atoi(getenv("ND_SMALL_MAP")) == 1);
+      if (small_placed_) {
+        placed_spill_first_ = place_start.back();
+        placed_places_ = (size_t)placed_spill_first_ + max_pairs_;  // every pair could spill
+        ND_HIP_TRY(hipMalloc(&d_place_start_, sizeof(uint32_t) * place_start.size()));
+        ND_HIP_TRY(hipMemcpy(d_place_start_, place_start.data(), sizeof(uint32_t) * place_start.size(),
+                             hipMemcpyHostToDevice));
+        for (int b = 0; b < 2; ++b) {
+          ND_HIP_TRY(hipMalloc(&d_placed_keys_[b], sizeof(uint32_t) * placed_places_));
+          ND_HIP_TRY(hipMalloc(&d_placed_slots_[b], sizeof(uint32_t) * placed_places_));
+          ND_HIP_TRY(hipMemset(d_placed_slots_[b], 0, sizeof(uint32_t) * placed_places_));
+          if (state_fits_pair<SampleType>::value) {
+            ND_HIP_TRY(hipMalloc(&d_placed_state_[b], sizeof(uint32_t) * placed_places_));
+            ND_HIP_TRY(hipMemset(d_placed_state_[b], 0, sizeof(uint32_t) * placed_places_));
+          }
+          ND_HIP_TRY(hipMalloc(&d_placed_counts_[b], sizeof(uint32_t) * (small_counters_ + 1)));
+        }
+        placed_dirty_ = true;  // cleared by the first pass that uses them
       }
     }
     if (small_map_) {
@@ -1917,6 +2015,22 @@ class Engine : public EngineBase {
     // passes that do not classify (nor launch the workgroup kernel); every kIdleLookEvery-th
     // pass looks again.  Results do not depend on it.
     bool balance = mode == kTransitParallelLoadBalanced && n_steps > 1 && !(walk_mode_ && sort_period > 1);
+    // small maps inverted at every step, the pairs placed by the kernel that emits them: one launch
+    // per step, every pair with the flat lanes (what a hub's adjacency is, is in the caches)
+    const bool placed = small_placed_ && sort_period == 1 && !sample_parallel;
+    if (placed) {
+      balance = false;
+      if (placed_dirty_) {
+        // a pass that did not get to its end left pairs or counts behind
+        for (int b = 0; b < 2; ++b) {
+          fill_i32<<<dim3((unsigned)((placed_places_ + 1023) / 1024)), dim3(1024), 0, stream_>>>(
+              (int32_t*)d_placed_keys_[b], placed_places_, invalid_);
+          fill_i32<<<dim3((unsigned)((small_counters_ + 1 + 1023) / 1024)), dim3(1024), 0, stream_>>>(
+              (int32_t*)d_placed_counts_[b], small_counters_ + 1, 0);
+        }
+      }
+      placed_dirty_ = true;
+    }
     if (balance && !wants_launch_graph() && idle_passes_ > 0 && idle_passes_ % kIdleLookEvery != 0) {
       balance = false;
       idle_passes_++;
@@ -1994,6 +2108,23 @@ class Engine : public EngineBase {
       P.emit_counts = emits && counted ? d_small_ : nullptr;
       P.emit_ranks = emits && counted ? d_emit_ranks_ : nullptr;
       P.emit_counter_base = d_counter_base_;
+      P.emit_place_start = nullptr;
+      P.emit_spill = nullptr;
+      P.emit_spill_first = 0;
+      P.taken_keys = nullptr;
+      P.taken_counts = nullptr;
+      P.taken_n_counts = 0;
+      if (placed && emits) {
+        const int to = step & 1;  // step k writes set k % 2 and reads the other
+        P.emit_keys = d_placed_keys_[to];
+        P.emit_slots = d_placed_slots_[to];
+        P.emit_state = state_travels_ ? d_placed_state_[to] : nullptr;
+        P.emit_counts = d_placed_counts_[to];
+        P.emit_ranks = nullptr;
+        P.emit_place_start = d_place_start_;
+        P.emit_spill = d_placed_counts_[to] + small_counters_;
+        P.emit_spill_first = placed_spill_first_;
+      }
       uint32_t* live_now = d_live_ + (sorts_done & 1);  // pairs the inversion of this step keeps
       // lanes of the flat kernel per pair: one when the pairs alone fill the machine, else
       // the power of two (at most the step size, rounded up) that brings the lanes to ~2^20
@@ -2024,7 +2155,19 @@ class Engine : public EngineBase {
         // Walks that invert only now and then gain nothing from the transit order (few of them
         // share a transit, and the order is stale one step later): they only drop the walks
         // that have ended, keeping slot order, in which the writes of a step's results coalesce.
-        if (counted) {
+        if (placed) {
+          // small map, placed by the previous step's kernel: every place is a lane
+          const int from = (step - 1) & 1;
+          P.pair_keys = d_placed_keys_[from];
+          P.pair_slots = d_placed_slots_[from];
+          P.pair_state = state_travels_ ? d_placed_state_[from] : nullptr;
+          P.n_pairs = (uint32_t)placed_places_;
+          P.taken_keys = d_placed_keys_[from];
+          P.taken_counts = d_placed_counts_[from];
+          P.taken_n_counts = (uint32_t)small_counters_ + 1;
+          const uint64_t lanes = placed_places_ > small_counters_ + 1 ? placed_places_ : small_counters_ + 1;
+          if (launch_step(P, lanes, false, nullptr) != 0) return -1;
+        } else if (counted) {
           // small map: the previous step's kernels have counted the pairs per transit
           const uint32_t n_keys = (uint32_t)small_counters_;
           const uint32_t n_chunks = (n_keys + kSmallMapChunk - 1) / kSmallMapChunk;
@@ -2161,6 +2304,7 @@ class Engine : public EngineBase {
     }
     tock(&times.assemble);
     ND_HIP_TRY(hipGetLastError());
+    if (placed) placed_dirty_ = false;  // the last step has taken every pair and cleared the counters behind it
     return 0;
   }
 
@@ -2295,9 +2439,20 @@ class Engine : public EngineBase {
   // transit is the previous step's result and the rows are regrouped by assemble_walk_rows.
   bool paired_results() const { return paired_results_; }
 
+  void launch_workgroup(const StepParams& P, unsigned grid, const RunsMeta* meta) {
+    if (P.step_size == 1)
+      step_workgroup_kernel<SampleType, App, true><<<dim3(grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
+                                                                                                   chunk_capacity_);
+    else
+      step_workgroup_kernel<SampleType, App, false><<<dim3(grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
+                                                                                                    chunk_capacity_);
+  }
+
   void launch_flat(const StepParams& P, uint64_t lanes, const uint32_t* taken_stamp, const RunsMeta* meta) {
     const unsigned grid = flat_grid_for(lanes);
-    if (P.step_size == 1)
+    if (P.emit_place_start || P.taken_keys)
+      step_flat_kernel<SampleType, App, true, true><<<dim3(grid), dim3(kFlatThreads), 0, stream_>>>(P, taken_stamp, meta);
+    else if (P.step_size == 1)
       step_flat_kernel<SampleType, App, true><<<dim3(grid), dim3(kFlatThreads), 0, stream_>>>(P, taken_stamp, meta);
     else
       step_flat_kernel<SampleType, App, false><<<dim3(grid), dim3(kFlatThreads), 0, stream_>>>(P, taken_stamp, meta);
@@ -2369,8 +2524,7 @@ class Engine : public EngineBase {
       // takes what the work items leave.
       ND_HIP_TRY(hipEventRecord(ev_fork_, stream_));
       ND_HIP_TRY(hipStreamWaitEvent(side_stream_, ev_fork_, 0));
-      step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
-                                                                                              chunk_capacity_);
+      launch_workgroup(P, wg_grid, meta);
       {
         const unsigned grid = flat_grid_for(lanes);
         if (P.step_size == 1)
@@ -2389,8 +2543,7 @@ class Engine : public EngineBase {
       tock(&times.flat_kernel);
       times.flat_launches++;
       tick();
-      step_workgroup_kernel<SampleType, App><<<dim3(wg_grid), dim3(kStepThreads), 0, stream_>>>(P, d_chunks_, meta,
-                                                                                              chunk_capacity_);
+      launch_workgroup(P, wg_grid, meta);
       tock(&times.workgroup_kernel);
       times.workgroup_launches++;
       if (schedule == kScheduleForked) schedule_counts_.forked_steps++; else schedule_counts_.serial_steps++;
@@ -2446,6 +2599,14 @@ class Engine : public EngineBase {
     release(d_emit_keys_);
     release(d_emit_slots_);
     release(d_emit_ranks_);
+    release(d_place_start_);
+    for (int b = 0; b < 2; ++b) {
+      release(d_placed_keys_[b]);
+      release(d_placed_slots_[b]);
+      release(d_placed_state_[b]);
+      release(d_placed_counts_[b]);
+    }
+    small_placed_ = false;
     release(d_small_);
     release(d_counter_base_);
     release(d_emit_state_);
@@ -2512,6 +2673,14 @@ class Engine : public EngineBase {
   uint32_t* d_counter_base_ = nullptr;  // first counter of every vertex
   uint32_t* d_emit_ranks_ = nullptr;
   uint32_t* d_small_ = nullptr;  // counters, their starts inside a chunk, chunk totals
+  // small maps whose pairs are placed as they are emitted (StepParams::emit_place_start): two
+  // sets of pair arrays with gaps and of counters, one written while the other is read
+  bool small_placed_ = false, placed_dirty_ = false;
+  uint32_t placed_spill_first_ = 0;
+  size_t placed_places_ = 0;
+  uint32_t* d_place_start_ = nullptr;
+  uint32_t *d_placed_keys_[2] = {nullptr, nullptr}, *d_placed_slots_[2] = {nullptr, nullptr};
+  uint32_t *d_placed_state_[2] = {nullptr, nullptr}, *d_placed_counts_[2] = {nullptr, nullptr};
   uint32_t *d_aux_a_ = nullptr, *d_aux_b_ = nullptr;  // ping-pong of the travelling state
   RunsMeta* d_meta_ = nullptr;          // two work-item counters, alternating between load-balanced steps
   uint32_t* d_balance_ = nullptr;       // which steps' classifications found a run; the pass's ClassCounters

@@ -198,12 +198,15 @@ def test_every_schedule_of_a_load_balanced_step_gives_the_oracle_bytes(oracle, a
     run_and_compare(oracle, app, getattr(oracle, kind_name), star, check_state=state, modes=(True, False, True))
 
 
-def test_the_schedule_is_chosen_after_a_pass_that_found_work_items(oracle):
+def test_the_schedule_is_chosen_after_a_pass_that_found_work_items(oracle, monkeypatch):
     """Left to itself the engine runs the two classes one after the other until a classified pass
     has found work items, then as one launch (small steps) or on two streams (large ones); the
     counters say which, and every pass gives the oracle's bytes."""
     g = graphs.random_graph(**GRAPHS["dense_hub"])
     og = graphs.oracle_view(g)
+    # the small walk with the two placing launches, which classify; left to itself a map this
+    # small is placed by the kernel that emits it and every pair goes to the flat lanes
+    monkeypatch.setenv("ND_SMALL_MAP", "1")
     for app, kind, small in (("UniformRandomWalk", oracle.UNIFORM_WALK, True), ("KHop40x30", oracle.KHOP, False)):
         s = nd.Sampler(app, g, seed=SEED)
         try:
@@ -390,12 +393,14 @@ def test_a_new_graph_needs_a_new_alloc(oracle, app):
 ])
 def test_both_inversions_of_a_small_map_give_the_oracle_bytes(oracle, app, kind_name, state, monkeypatch):
     """Walks over a small map are inverted without a sort (counts per next transit, taken while
-    the pairs are emitted); ND_SMALL_MAP=0 sends the same map through the radix sort.  Also the
+    the pairs are emitted): the emitting kernel places the pairs itself, or (ND_SMALL_MAP=1) two
+    launches place them; ND_SMALL_MAP=0 sends the same map through the radix sort.  Also the
     largest map that still takes the first route, and a hub that gathers every walk."""
     g = graphs.random_graph(n=3000, mean_degree=8, seed=23, hub=7, isolated_every=13)
-    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
-    monkeypatch.setenv("ND_SMALL_MAP", "0")
-    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, modes=(False, True, True))
+    for route in ("1", "0"):
+        monkeypatch.setenv("ND_SMALL_MAP", route)
+        run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state)
     monkeypatch.delenv("ND_SMALL_MAP")
     if app == "UniformRandomWalk":
         n = 1 << 17  # as many pairs as the small-map route takes; one more vertex takes the other route
@@ -406,10 +411,11 @@ def test_both_inversions_of_a_small_map_give_the_oracle_bytes(oracle, app, kind_
             run_and_compare(oracle, app, getattr(oracle, kind_name), big, check_state=state, modes=(True,))
 
 
-def test_small_map_inversion_classifies_every_run_by_the_rules(oracle):
-    """The placing launch of the small-map inversion decides the load-balancing class of every
-    run from the counts; what it reports (nd_sampler_counter) is what the rules give for the
-    transits the oracle's walks are on, step by step."""
+def test_small_map_inversion_classifies_every_run_by_the_rules(oracle, monkeypatch):
+    """The placing launch of the small-map inversion (ND_SMALL_MAP=1) decides the load-balancing
+    class of every run from the counts; what it reports (nd_sampler_counter) is what the rules
+    give for the transits the oracle's walks are on, step by step."""
+    monkeypatch.setenv("ND_SMALL_MAP", "1")
     work_from, item_outputs, cache_edges = nd.load_balancing_thresholds()
     # a hub that fits the LDS cache, one that does not, and a sparse rest
     n = 20000
