@@ -476,7 +476,7 @@ __device__ __forceinline__ void fill_dead_pair(const StepParams& P, uint32_t pai
 template <bool kPlaces = false, bool kWalkStep = true>
 __device__ __forceinline__ void store_output(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
                                              uint32_t sample, uint32_t nbr, VertexID neighbor, VertexID next_transit,
-                                             uint32_t state_bits = 0) {
+                                             uint32_t state_bits = 0, bool chooses_transits = true) {
   const uint64_t out_slot = (uint64_t)pair_slot * P.step_size + nbr;
   if (kWalkStep && P.pair_cells) {
     store_walk_result(P, sample, transit, neighbor);
@@ -486,7 +486,8 @@ __device__ __forceinline__ void store_output(const StepParams& P, VertexID trans
     P.step_out[(size_t)sample * P.out_pitch + q] = neighbor;
     if (P.fill_levels > 1 && neighbor == P.invalid) fill_below(P, sample, q);
   }
-  if (P.explicit_out) P.explicit_out[out_slot] = next_transit;
+  // (chooses_transits: App::hasExplicitTransits(), where the caller knows the app)
+  if (chooses_transits && P.explicit_out) P.explicit_out[out_slot] = next_transit;
   if (kWalkStep && P.emit_keys) {
     uint32_t at = pair;
     if (P.emit_counts && next_transit != P.invalid) {
@@ -600,10 +601,12 @@ __device__ __forceinline__ void compute_group(const StepParams& P, CSRPartition&
   }
 }
 
+template <class App>
 __device__ __forceinline__ void store_group(const StepParams& P, VertexID transit, uint32_t pair, uint32_t pair_slot,
                                             const GroupOutputs& g) {
   if (g.from >= g.to) return;
-  if (g.from == 0 && g.to == 4 && !P.explicit_out) {
+  const bool chooses_transits = App().hasExplicitTransits();  // a constant of the app
+  if (g.from == 0 && g.to == 4 && !(chooses_transits && P.explicit_out)) {
     // a whole group whose outputs are all there is to store: the four ids are neighbours in
     // the step's results (word aligned, not more), and go out as one 16-byte store
     const uint32_t per_sample = P.transits_per_sample * P.step_size;
@@ -622,7 +625,7 @@ __device__ __forceinline__ void store_group(const StepParams& P, VertexID transi
   for (uint32_t w = 0; w < 4; ++w)
     if (w >= g.from && w < g.to)
       store_output<false, false>(P, transit, pair, pair_slot, g.sample, (uint32_t)(g.base + w - g.first), g.neighbor[w],
-                                 g.next_transit[w]);
+                                 g.next_transit[w], 0u, chooses_transits);
 }
 
 // The groups first, first + stride, ... of a pair, the draws of a group made before the
@@ -639,10 +642,10 @@ __device__ __forceinline__ void produce_groups(const StepParams& P, CSRPartition
     GroupOutputs now;
     compute_group<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, gi, n_edges, max_weight,
                                                            edges, weights, &now);
-    store_group(P, transit, pair, pair_slot, held);
+    store_group<App>(P, transit, pair, pair_slot, held);
     held = now;
   }
-  store_group(P, transit, pair, pair_slot, held);
+  store_group<App>(P, transit, pair, pair_slot, held);
 }
 
 // The same without holding a group back: for the workgroup class, whose draws come from LDS
@@ -656,7 +659,7 @@ __device__ __forceinline__ void produce_groups_in_turn(const StepParams& P, CSRP
     GroupOutputs now;
     compute_group<SampleType, App, EdgeArray, WeightArray>(P, csr, transit, pair, pair_slot, gi, n_edges, max_weight,
                                                            edges, weights, &now);
-    store_group(P, transit, pair, pair_slot, now);
+    store_group<App>(P, transit, pair, pair_slot, now);
   }
 }
 
