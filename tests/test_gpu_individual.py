@@ -411,6 +411,25 @@ def test_both_inversions_of_a_small_map_give_the_oracle_bytes(oracle, app, kind_
             run_and_compare(oracle, app, getattr(oracle, kind_name), big, check_state=state, modes=(True,))
 
 
+@pytest.mark.parametrize("app,kind_name,state", [
+    ("UniformRandomWalk", "UNIFORM_WALK", False),
+    ("WeightedNode2Vec", "WEIGHTED_NODE2VEC", True),
+])
+def test_placed_pairs_that_find_no_place_spill(oracle, app, kind_name, state):
+    """A small map whose pairs are placed by the kernel that emits them gives every vertex room for
+    about twice the walks its share of the edge ends lets it expect.  Here that expectation is as
+    wrong as it can be: every walk funnels through 16 vertices into ONE vertex that only 16 edges
+    point to (room for a few dozen pairs), every third step, so nearly all pairs take the places
+    past the counters' own."""
+    n = 3000
+    rest = np.arange(17, n)
+    src = np.concatenate([rest, np.arange(1, 17), np.zeros(len(rest), np.int64)])
+    dst = np.concatenate([1 + rest % 16, np.zeros(16, np.int64), rest])
+    weights = (1.0 + (np.arange(len(src)) % 7)).astype(np.float32)
+    g = nd.Graph.from_edges(src, dst, weights, n_vertices=n)
+    run_and_compare(oracle, app, getattr(oracle, kind_name), g, check_state=state, modes=(True, False, True))
+
+
 def test_small_map_inversion_classifies_every_run_by_the_rules(oracle, monkeypatch):
     """The placing launch of the small-map inversion (ND_SMALL_MAP=1) decides the load-balancing
     class of every run from the counts; what it reports (nd_sampler_counter) is what the rules
