@@ -872,25 +872,21 @@ __global__ __launch_bounds__(kSumThreads) void bitmap_group_sums(const uint32_t*
   for (uint32_t s = first_sample + wave; s < end_sample; s += kSumThreads / kWave) {
     const uint4* words = (const uint4*)(bitmap + (size_t)s * words_per_sample + (size_t)part * kPartWords + lane * kGroupWords);
     const uint4 a = words[0], b = words[1];
-    const uint64_t w[kGroupWords / 2] = {a.x | ((uint64_t)a.y << 32), a.z | ((uint64_t)a.w << 32),
-                                         b.x | ((uint64_t)b.y << 32), b.z | ((uint64_t)b.w << 32)};
+    // word by word: finding and clearing the lowest set bit of a 32-bit word is three vector
+    // instructions, of a 64-bit one eight, and the launch is bound by instruction issue
+    const uint32_t w[kGroupWords] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     uint64_t sum = 0;
     uint32_t count = 0;
 #pragma unroll
-    for (uint32_t k = 0; k < kGroupWords / 2; ++k) {
-      uint64_t bits = w[k];
-      count += (uint32_t)__popcll(bits);
-      const uint32_t* from = mine + k * 64u;
+    for (uint32_t k = 0; k < kGroupWords; ++k) {
+      uint32_t bits = w[k];
+      count += (uint32_t)__popc(bits);
+      const uint32_t* from = mine + k * 32u;
       while (bits) {
-        // two lookups under way per round
-        const uint32_t i0 = (uint32_t)__ffsll((unsigned long long)bits) - 1u;
-        bits &= bits - 1ull;
-        const bool second = bits != 0;
-        const uint32_t i1 = second ? (uint32_t)__ffsll((unsigned long long)bits) - 1u : i0;
-        bits &= bits - 1ull;  // 0 stays 0
+        const uint32_t i0 = (uint32_t)__ffs((int)bits) - 1u;
+        bits &= bits - 1u;
         const uint64_t d0 = from[i0];
-        const uint64_t d1 = second ? from[i1] : 0u;
-        sum += d0 * d0 + d1 * d1;
+        sum += d0 * d0;
       }
     }
     const uint64_t through = wave_inclusive_scan_u64(sum);
