@@ -43,7 +43,7 @@ MEASURED = {
     "uniform_walk_chunglu57k": {"kernels": {"nd::step_flat_kernel": 1.224e7}, "bytes_per_pass": 1.27e9},
     # both kernel classes of a hop; the flat kernel is launched for both hops, the workgroup kernel for the second
     "khop_rmat21": {"kernels": {"nd::step_flat_kernel": 1.088e9, "nd::step_workgroup_kernel": 2.385e9},
-                    "bytes_per_pass": 8.73e9},
+                    "bytes_per_pass": 8.45e9},
     # collective_mark_binned, average over its 2 launches per pass
     "fastgcn_importance_rmat22": {"kernels": {"nd::collective_mark_binned": 5.268e9}, "bytes_per_pass": 16.41e9},
     "ladies_importance_chunglu3m": {"kernels": {"nd::collective_mark_binned": 6.752e10}, "bytes_per_pass": 161.61e9},

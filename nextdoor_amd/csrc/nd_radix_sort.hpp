@@ -25,7 +25,7 @@ namespace nd {
 constexpr int kSortThreads = 256;
 constexpr int kSortWaves = kSortThreads / kWave;
 // Keys per lane and tile: 10 (2560 pairs per workgroup) for sorts that are latency bound,
-// 16 (4096 pairs) for large ones, where fewer, larger tiles keep the digit table small.
+// 32 (8192 pairs) for large ones, where fewer, larger tiles keep the digit table small.
 // Measured: inversion of a 100-step pass over 4.2 M walks 12.3 ms with 16, 11.5 ms with 8,
 // 14.7 ms with 4; sorts of ~1e8 entries are 12 % slower with 8 than with 16.  Again, after the
 // kernels had their loads batched: 13.96 / 11.50 / 10.80 / 10.24 / 10.62 ms with 4 / 6 / 8 / 10 / 12.
@@ -33,7 +33,12 @@ constexpr int kSortWaves = kSortThreads / kWave;
 #define ND_SORT_ITEMS_SMALL 10
 #endif
 constexpr int kSortItemsSmall = ND_SORT_ITEMS_SMALL;
-constexpr int kSortItemsLarge = 16;
+// (5.2e7 pairs of the k-hop pass, three digit passes, with 12 / 16 / 20 / 24 / 28 / 32 keys per lane of the
+// histogram kernel: 0.85 / 0.83 / 0.83 / 0.81 / 0.81 / 0.80 ms)
+#ifndef ND_SORT_ITEMS_LARGE
+#define ND_SORT_ITEMS_LARGE 32
+#endif
+constexpr int kSortItemsLarge = ND_SORT_ITEMS_LARGE;
 constexpr size_t kSortLargeFrom = (size_t)16 << 20;  // pairs
 constexpr int kSortMaxTile = kSortThreads * kSortItemsLarge;
 constexpr int kRadixBits = 8;
