@@ -47,6 +47,22 @@ def test_sort_pairs_matches_stable_sort(oracle, bits):
         assert np.array_equal(ko2, wk) and np.array_equal(vo2, np.argsort(keys, kind="stable").astype(np.int32))
 
 
+def test_sort_of_more_than_16_mi_pairs_matches_stable_sort():
+    """Sorts of at least 2^24 pairs run with larger tiles than the sizes above: a ragged last tile,
+    a heavy last bucket, given values and generated ones."""
+    n, bits = (16 << 20) + 4097, 23
+    rng = np.random.default_rng(5)
+    keys = rng.integers(0, 1 << bits, n).astype(np.int32)
+    keys[rng.integers(0, n, n // 5)] = (1 << bits) - 1
+    vals = rng.integers(0, 1 << 31, n).astype(np.int32)
+    order = np.argsort(keys, kind="stable")
+    print("sort n", n, "bits", bits, flush=True)
+    ko, vo = nd.sort_pairs(keys, vals, bits)
+    assert np.array_equal(ko, keys[order]) and np.array_equal(vo, vals[order])
+    ko, vo = nd.sort_pairs(keys, None, bits)
+    assert np.array_equal(ko, keys[order]) and np.array_equal(vo, order.astype(np.int32))
+
+
 def test_sort_ignores_bits_above_key_bits():
     keys = np.array([0x105, 0x003, 0x204, 0x001], np.int32)
     ko, vo = nd.sort_pairs(keys, None, 8)
